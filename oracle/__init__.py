@@ -1,0 +1,162 @@
+"""ctypes front-end of the CPU oracle (``oracle/adr_oracle.c``).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, by ``__graft_entry__.smoke()`` and by the
+``cpu_baseline`` leg of ``bench.py`` as the checker / baseline.  The product package
+(``adrastea_amd``) never imports this module.
+
+fp16 data is exchanged as ``numpy.float16`` arrays (viewed as ``uint16`` for the C side).
+All element strides follow the reference convention (``adrastea_models/src/kernels.rs:864-887``):
+``x`` = last dim, ``y`` = second-to-last, ``z`` = batch, counted in elements.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+
+LOAD_IDENTITY, LOAD_SCALE = 0, 1
+(STORE_IDENTITY, STORE_GELU_BIAS, STORE_BETA_GELU_BIAS, STORE_BETA_BIAS, STORE_SCALE, STORE_ADD,
+ STORE_QUICK_GELU_BIAS) = range(7)
+MASK_NONE, MASK_CAUSAL = 0, 1
+FAITHFUL, EXACT = 0, 1
+
+
+def build(force: bool = False) -> str:
+    """Compile liboracle.so (and the reference code objects when the checkout exists)."""
+    src = os.path.join(_HERE, "adr_oracle.c")
+    stale = (not os.path.exists(_LIB_PATH)) or os.path.getmtime(_LIB_PATH) < os.path.getmtime(src)
+    if force or stale:
+        subprocess.check_call(["make", "-s", "-C", _HERE, os.path.join(_HERE, "liboracle.so")])
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        L = C.CDLL(_LIB_PATH)
+        u16p, u8p, f32p, f64p = (C.POINTER(C.c_uint16), C.POINTER(C.c_uint8),
+                                 C.POINTER(C.c_float), C.POINTER(C.c_double))
+        L.adr_o_h2f.restype = C.c_float
+        L.adr_o_h2f.argtypes = [C.c_uint16]
+        L.adr_o_f2h.restype = C.c_uint16
+        L.adr_o_f2h.argtypes = [C.c_float]
+        L.adr_o_d2h.restype = C.c_uint16
+        L.adr_o_d2h.argtypes = [C.c_double]
+        L.adr_o_hmul.restype = C.c_uint16
+        L.adr_o_hmul.argtypes = [C.c_uint16, C.c_uint16]
+        L.adr_o_hadd.restype = C.c_uint16
+        L.adr_o_hadd.argtypes = [C.c_uint16, C.c_uint16]
+        L.adr_o_h2f_n.argtypes = [f32p, u16p, C.c_int64]
+        L.adr_o_f2h_n.argtypes = [u16p, f32p, C.c_int64]
+        L.adr_o_d2h_n.argtypes = [u16p, f64p, C.c_int64]
+        L.adr_o_matmul_f16.restype = C.c_int
+        L.adr_o_matmul_f16.argtypes = ([u16p, u16p, u16p] + [C.c_int] * 13 +
+                                       [u16p, C.c_float, C.c_float, C.c_uint32, C.c_uint32,
+                                        C.c_uint32, C.c_int, C.c_int])
+        L.adr_o_matmul_nt_f16.argtypes = [u16p, u16p, u16p, C.c_int, C.c_int, C.c_int, C.c_float,
+                                          C.c_int]
+        for name in ("adr_o_matmul_nt_fp16u8", "adr_o_matmul_nt_fp16u8_naive"):
+            getattr(L, name).argtypes = [u16p, u16p, u8p, u16p, C.c_int, C.c_int, C.c_int,
+                                         C.c_int, C.c_float, C.c_int]
+        L.adr_o_dequantize_absmax_u8.argtypes = [u16p, u8p, u16p, C.c_int, C.c_int, C.c_int]
+        L.adr_o_quantize_absmax_u8.argtypes = [u8p, u16p, u16p, C.c_int, C.c_int, C.c_int]
+        L.adr_o_dequant_table.argtypes = [u16p]
+        _lib = L
+    return _lib
+
+
+def _p16(a):
+    return a.ctypes.data_as(C.POINTER(C.c_uint16))
+
+
+def _p8(a):
+    return a.ctypes.data_as(C.POINTER(C.c_uint8))
+
+
+def _as_f16_flat(a) -> np.ndarray:
+    a = np.ascontiguousarray(a)
+    assert a.dtype == np.float16, a.dtype
+    return a.reshape(-1)
+
+
+def matmul_f16(out_buf, lhs_buf, rhs_buf, batches, m, k, n, so, sl, sr, bias=None, beta=0.0,
+               scale=1.0, store=STORE_IDENTITY, load=LOAD_IDENTITY, mask=MASK_NONE,
+               mode=FAITHFUL, threads=1, offsets=(0, 0, 0)):
+    """Run the oracle matmul on flat fp16 buffers.
+
+    ``so``/``sl``/``sr`` are ``(stride_x, stride_y, stride_z)`` triples in elements and
+    ``offsets`` the element offsets of output/lhs/rhs inside their buffers.  ``out_buf`` is
+    updated in place (and returned); it must be a contiguous 1-d float16 array.
+    """
+    assert out_buf.dtype == np.float16 and out_buf.flags.c_contiguous and out_buf.ndim == 1
+    lhs_buf, rhs_buf = _as_f16_flat(lhs_buf), _as_f16_flat(rhs_buf)
+    if bias is not None:
+        bias = _as_f16_flat(bias)
+    o_u, l_u, r_u = out_buf.view(np.uint16), lhs_buf.view(np.uint16), rhs_buf.view(np.uint16)
+    rc = lib().adr_o_matmul_f16(
+        _p16(o_u[offsets[0]:]), _p16(l_u[offsets[1]:]), _p16(r_u[offsets[2]:]), batches, m, k, n,
+        so[0], so[1], so[2], sl[0], sl[1], sl[2], sr[0], sr[1], sr[2],
+        _p16(bias.view(np.uint16)) if bias is not None else None, float(beta), float(scale),
+        int(store), int(load), int(mask), int(mode), int(threads))
+    if rc != 0:
+        raise ValueError("oracle: unsupported store/load/mask combination or missing bias")
+    return out_buf
+
+
+def matmul_nt_f16(out, lhs, rhs, beta=0.0, threads=1):
+    m, p = lhs.shape
+    n = rhs.shape[0]
+    assert out.shape == (m, n) and out.flags.c_contiguous and out.dtype == np.float16
+    lhs, rhs = np.ascontiguousarray(lhs), np.ascontiguousarray(rhs)
+    lib().adr_o_matmul_nt_f16(_p16(out.view(np.uint16)), _p16(lhs.view(np.uint16)),
+                              _p16(rhs.view(np.uint16)), m, p, n, float(beta), threads)
+    return out
+
+
+def matmul_nt_fp16u8(out, lhs, rhs_q, scales, block_size, beta=0.0, threads=1, naive=False):
+    m, p = lhs.shape
+    n = rhs_q.shape[0]
+    assert out.shape == (m, n) and out.flags.c_contiguous and out.dtype == np.float16
+    assert rhs_q.dtype == np.uint8 and scales.dtype == np.float16
+    assert scales.shape == (n, p // block_size)
+    lhs, rhs_q, scales = map(np.ascontiguousarray, (lhs, rhs_q, scales))
+    fn = lib().adr_o_matmul_nt_fp16u8_naive if naive else lib().adr_o_matmul_nt_fp16u8
+    fn(_p16(out.view(np.uint16)), _p16(lhs.view(np.uint16)), _p8(rhs_q),
+       _p16(scales.view(np.uint16)), m, p, n, block_size, float(beta), threads)
+    return out
+
+
+def dequantize_absmax_u8(q, scales, block_size):
+    rows, cols = q.shape
+    q, scales = np.ascontiguousarray(q), np.ascontiguousarray(scales)
+    assert scales.shape == (rows, cols // block_size) and scales.dtype == np.float16
+    out = np.empty((rows, cols), np.float16)
+    lib().adr_o_dequantize_absmax_u8(_p16(out.view(np.uint16)), _p8(q),
+                                     _p16(scales.view(np.uint16)), rows, cols, block_size)
+    return out
+
+
+def quantize_absmax_u8(x, block_size):
+    rows, cols = x.shape
+    x = np.ascontiguousarray(x)
+    assert x.dtype == np.float16 and cols % block_size == 0
+    q = np.empty((rows, cols), np.uint8)
+    scales = np.empty((rows, cols // block_size), np.float16)
+    lib().adr_o_quantize_absmax_u8(_p8(q), _p16(scales.view(np.uint16)), _p16(x.view(np.uint16)),
+                                   rows, cols, block_size)
+    return q, scales
+
+
+def dequant_table():
+    out = np.empty(256 * 65536, np.uint16)
+    lib().adr_o_dequant_table(_p16(out))
+    return out.reshape(256, 65536)
