@@ -1,0 +1,65 @@
+"""ctypes binding of libadrastea_kernels_hip.so (declarations: include/adrastea_kernels.h)."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libadrastea_kernels_hip.so")
+
+# every symbol include/adrastea_kernels.h declares
+SYMBOLS = (
+    "adr_matmul_f16", "adr_matmul_f16_slow", "adr_matmul_f16_raw", "adr_matmul_nt_f16",
+    "adr_matmul_nt_fp16u8", "adr_dequantize_absmax_u8", "adr_quantize_absmax_u8",
+    "adr_dequantize_absmax_uint8", "adr_quantize_absmax_uint8", "adr_matmul_f16_plan",
+    "adr_matmul_nt_fp16u8_plan", "adr_strerror", "adr_abi_version",
+)
+
+ADR_OK, ADR_EINVAL_SHAPE, ADR_EINVAL_ENUM, ADR_ENOTIMPL, ADR_ENULL, ADR_EDIVISIBILITY = (
+    0, -1, -2, -3, -4, -5)
+
+
+class TensorDesc(C.Structure):
+    """adr_tensor_desc: index 0 is the innermost dimension (kernels.rs:28-47)."""
+    _fields_ = [("ptr", C.c_void_p), ("dims", C.c_uint32), ("shape", C.c_uint32 * 7),
+                ("strides", C.c_uint32 * 7)]
+
+
+_lib = None
+
+
+def lib():
+    """The loaded library.  Raises if it has not been built: there is no fallback path."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m adrastea_amd.build` "
+            "(hipcc, gfx950); adrastea_amd has no CPU or PyTorch fallback")
+    L = C.CDLL(LIB_PATH)
+    vp, i32, u32, f32 = C.c_void_p, C.c_int32, C.c_uint32, C.c_float
+    mm = [vp, vp, vp, vp] + [i32] * 13 + [vp, f32, f32, u32, u32, u32]
+    L.adr_matmul_f16.argtypes = mm
+    L.adr_matmul_f16_slow.argtypes = mm
+    L.adr_matmul_f16_raw.argtypes = [vp, vp, vp, vp] + [i32] * 13
+    L.adr_matmul_nt_f16.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32]
+    L.adr_matmul_nt_fp16u8.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, f32]
+    L.adr_dequantize_absmax_u8.argtypes = [vp, vp, vp, vp, i32, i32, i32]
+    L.adr_quantize_absmax_u8.argtypes = [vp, vp, vp, vp, i32, i32, i32]
+    L.adr_dequantize_absmax_uint8.argtypes = [vp, TensorDesc, TensorDesc, TensorDesc]
+    L.adr_quantize_absmax_uint8.argtypes = [vp, TensorDesc, TensorDesc, TensorDesc]
+    L.adr_matmul_f16_plan.argtypes = [C.c_char_p, i32] + [i32] * 13 + [u32, u32, u32]
+    L.adr_matmul_nt_fp16u8_plan.argtypes = [C.c_char_p, i32, i32, i32, i32, i32]
+    L.adr_strerror.argtypes = [C.c_int]
+    L.adr_strerror.restype = C.c_char_p
+    L.adr_abi_version.restype = C.c_int
+    for name in SYMBOLS:
+        if name not in ("adr_strerror",):
+            getattr(L, name).restype = C.c_int
+    _lib = L
+    return L
+
+
+def strerror(code: int) -> str:
+    return lib().adr_strerror(code).decode()

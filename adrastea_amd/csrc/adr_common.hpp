@@ -1,0 +1,136 @@
+// Shared device/host definitions of the gfx950 matmul kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/adrastea_kernels.h"
+
+namespace adr {
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+
+// The 22 matmul arguments (adrastea_models/src/kernels.rs:864-887) as one POD.
+struct MatmulArgs {
+  half_t* output;
+  const half_t* lhs;
+  const half_t* rhs;
+  int batches, m, k, n;
+  int stride_ox, stride_oy, stride_oz;
+  int stride_lx, stride_ly, stride_lz;
+  int stride_rx, stride_ry, stride_rz;
+  const half_t* bias;
+  float beta;
+  float scale;
+  uint32_t store, load, mask;
+  // u8-quantised right operand (adr_matmul_nt_fp16u8): rhs is then unused
+  const uint8_t* rhs_q;
+  const half_t* scales;
+  int block_size;
+};
+
+// Internal store operator of the contiguous NT entry points (matmul_nt_wmma_16x128x256.cu:63-66):
+// out = fp16(acc + beta * out), the accumulator is NOT narrowed first.  Not part of the ABI enum.
+constexpr uint32_t STORE_ACC_BETA = 7;
+
+__device__ __forceinline__ half_t bits_to_half(uint16_t b) { return __builtin_bit_cast(half_t, b); }
+__device__ __forceinline__ uint16_t half_to_bits(half_t h) { return __builtin_bit_cast(uint16_t, h); }
+
+// Store operators (adrastea_kernels/cpp/matmul.cu:418-491).  `acc` is the fp32 accumulator;
+// it is narrowed to fp16 first because every reference operator takes a __half argument
+// (matmul.cu:47-52, 64-71, 80-87).  `prev` is the element already in the output; callers
+// load it only for the operators that read it (needs_prev()).
+struct Epilogue {
+  const half_t* bias;
+  float beta;
+  half_t hscale;
+  uint32_t store;
+
+  __host__ __device__ static bool needs_prev(uint32_t store) {
+    return store == ADR_STORE_ADD || store == ADR_STORE_BETA_BIAS ||
+           store == ADR_STORE_BETA_GELU_BIAS || store == STORE_ACC_BETA;
+  }
+  __host__ __device__ static bool needs_bias(uint32_t store) {
+    return store == ADR_STORE_BETA_BIAS || store == ADR_STORE_BETA_GELU_BIAS ||
+           store == ADR_STORE_QUICK_GELU_BIAS;
+  }
+
+  __device__ __forceinline__ half_t apply(float acc, half_t prev, half_t bias_x) const {
+    if (store == STORE_ACC_BETA) return (half_t)(acc + beta * (float)prev);
+    half_t s16 = (half_t)acc;
+    switch (store) {
+      default:
+      case ADR_STORE_IDENTITY:
+        return s16;
+      case ADR_STORE_SCALE:
+        return s16 * hscale;
+      case ADR_STORE_ADD:
+        return s16 + prev;
+      case ADR_STORE_BETA_BIAS: {
+        float v = (float)s16 + (float)bias_x;
+        return (half_t)(v + beta * (float)prev);
+      }
+      case ADR_STORE_QUICK_GELU_BIAS: {
+        float v = (float)s16 + (float)bias_x;
+        return (half_t)(v * (1.0f / (1.0f + expf(-1.702f * v))));
+      }
+      case ADR_STORE_BETA_GELU_BIAS: {
+        float v = (float)s16 + (float)bias_x;
+        float g = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+        return (half_t)(g + beta * (float)prev);
+      }
+    }
+  }
+};
+
+__device__ __forceinline__ half_t neg_inf_half() { return bits_to_half(0xFC00u); }
+
+// Four u8 weights (one dword) -> four fp16 values (q - 127.5) * s with ONE rounding each, the
+// reference's dequantisation (adrastea_kernels/cpp/quantize.cu:53-54) bit for bit:
+// 0x6000 | (q << 1) is the fp16 number 512 + q (the step at 512 is 0.5); subtracting 639.5
+// gives q - 127.5 exactly, and an fp16 multiply rounds the exact product once -- the same
+// value as narrowing the (exact) fp32 product.  fp16 denormals are never flushed on gfx950.
+__device__ __forceinline__ void dequant4(uint32_t w, half2_t s2, half2_t& lo, half2_t& hi) {
+  uint32_t p01 = __builtin_amdgcn_perm(0u, w, 0x0c010c00u);  // 0x00 b1 00 b0
+  uint32_t p23 = __builtin_amdgcn_perm(0u, w, 0x0c030c02u);  // 0x00 b3 00 b2
+  p01 = (p01 << 1) | 0x60006000u;
+  p23 = (p23 << 1) | 0x60006000u;
+  const half2_t bias = {(half_t)639.5f, (half_t)639.5f};
+  lo = (__builtin_bit_cast(half2_t, p01) - bias) * s2;
+  hi = (__builtin_bit_cast(half2_t, p23) - bias) * s2;
+}
+
+// Eight consecutive u8 weights sharing one scale -> eight fp16 values in memory order.
+__device__ __forceinline__ half8_t dequant8(uint32_t w0, uint32_t w1, half2_t s2) {
+  half2_t a, b, c, d;
+  dequant4(w0, s2, a, b);
+  dequant4(w1, s2, c, d);
+  half8_t r;
+  r[0] = a[0]; r[1] = a[1]; r[2] = b[0]; r[3] = b[1];
+  r[4] = c[0]; r[5] = c[1]; r[6] = d[0]; r[7] = d[1];
+  return r;
+}
+
+// Launchers implemented in the kernel translation units; all return a hipError_t.
+hipError_t launch_matmul_general(hipStream_t stream, const MatmulArgs& a);
+// Returns true and fills `name` when the MFMA kernel family covers these arguments.
+bool mfma_gemm_supported(const MatmulArgs& a, const char** name);
+hipError_t launch_mfma_gemm(hipStream_t stream, const MatmulArgs& a);
+
+hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, const uint8_t* rhs,
+                          const half_t* scales, int m, int p, int n, int block_size, float beta);
+const char* gemm_u8_plan(int m, int p, int n, int block_size);
+
+hipError_t launch_dequantize(hipStream_t stream, adr_tensor_desc out, adr_tensor_desc scales,
+                             adr_tensor_desc in);
+hipError_t launch_quantize(hipStream_t stream, adr_tensor_desc out, adr_tensor_desc scales,
+                           adr_tensor_desc in);
+
+}  // namespace adr

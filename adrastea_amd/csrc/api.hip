@@ -1,0 +1,216 @@
+// extern "C" entry points: argument validation, kernel selection, launch.
+// Declarations and the reference interface each one replaces: include/adrastea_kernels.h.
+#include <string.h>
+
+#include "adr_common.hpp"
+
+using namespace adr;
+
+namespace {
+
+constexpr int ABI_VERSION = 1;
+
+int validate_matmul(const MatmulArgs& a, bool check_ptrs) {
+  if (a.store > ADR_STORE_QUICK_GELU_BIAS || a.load > ADR_LOAD_SCALE || a.mask > ADR_MASK_CAUSAL)
+    return ADR_EINVAL_ENUM;
+  if (a.store == ADR_STORE_GELU_BIAS) return ADR_ENOTIMPL;
+  if (a.batches < 0 || a.m < 0 || a.n < 0 || a.k < 0) return ADR_EINVAL_SHAPE;
+  if (check_ptrs) {
+    if (a.batches && a.m && a.n) {
+      if (!a.output || (a.k && (!a.lhs || !a.rhs))) return ADR_ENULL;
+      if (Epilogue::needs_bias(a.store) && !a.bias) return ADR_ENULL;
+    }
+  }
+  return ADR_OK;
+}
+
+MatmulArgs pack(uint16_t* output, const uint16_t* lhs, const uint16_t* rhs, int32_t batches,
+                int32_t m, int32_t k, int32_t n, int32_t stride_ox, int32_t stride_oy,
+                int32_t stride_oz, int32_t stride_lx, int32_t stride_ly, int32_t stride_lz,
+                int32_t stride_rx, int32_t stride_ry, int32_t stride_rz, const uint16_t* bias,
+                float beta, float scale, uint32_t store, uint32_t load, uint32_t mask) {
+  MatmulArgs a{};
+  a.output = (half_t*)output;
+  a.lhs = (const half_t*)lhs;
+  a.rhs = (const half_t*)rhs;
+  a.batches = batches; a.m = m; a.k = k; a.n = n;
+  a.stride_ox = stride_ox; a.stride_oy = stride_oy; a.stride_oz = stride_oz;
+  a.stride_lx = stride_lx; a.stride_ly = stride_ly; a.stride_lz = stride_lz;
+  a.stride_rx = stride_rx; a.stride_ry = stride_ry; a.stride_rz = stride_rz;
+  a.bias = (const half_t*)bias;
+  a.beta = beta;
+  a.scale = scale;
+  a.store = store; a.load = load; a.mask = mask;
+  return a;
+}
+
+bool empty(const MatmulArgs& a) { return a.batches == 0 || a.m == 0 || a.n == 0; }
+
+int run_matmul(hipStream_t stream, const MatmulArgs& a, bool allow_fast) {
+  if (empty(a)) return ADR_OK;
+  const char* name;
+  if (allow_fast && mfma_gemm_supported(a, &name)) return (int)launch_mfma_gemm(stream, a);
+  return (int)launch_matmul_general(stream, a);  // also the k == 0 case: store(0)
+}
+
+adr_tensor_desc desc2d(const void* ptr, int rows, int cols) {
+  adr_tensor_desc d{};
+  d.ptr = (void*)ptr;
+  d.dims = 2;
+  d.shape[0] = (uint32_t)cols; d.shape[1] = (uint32_t)rows;
+  d.strides[0] = 1; d.strides[1] = (uint32_t)cols;
+  return d;
+}
+
+int validate_quant(const adr_tensor_desc& wide, const adr_tensor_desc& scales,
+                   const adr_tensor_desc& other) {
+  if (!wide.ptr || !scales.ptr || !other.ptr) return ADR_ENULL;
+  if (wide.dims != 2 || scales.dims != 2 || other.dims != 2) return ADR_EINVAL_SHAPE;
+  if (wide.shape[0] != other.shape[0] || wide.shape[1] != other.shape[1] ||
+      scales.shape[1] != wide.shape[1])
+    return ADR_EINVAL_SHAPE;
+  if (scales.shape[0] == 0 || wide.shape[0] % scales.shape[0] != 0) return ADR_EDIVISIBILITY;
+  return ADR_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int adr_abi_version(void) { return ABI_VERSION; }
+
+const char* adr_strerror(int code) {
+  switch (code) {
+    case ADR_OK: return "success";
+    case ADR_EINVAL_SHAPE: return "invalid shape or size";
+    case ADR_EINVAL_ENUM: return "store/load/mask operator out of range";
+    case ADR_ENOTIMPL: return "MatmulStoreOp::GeluBias has no device implementation";
+    case ADR_ENULL: return "null tensor pointer or missing bias";
+    case ADR_EDIVISIBILITY: return "size not divisible by block_size / unsupported block_size";
+    case ADR_EUNSUPPORTED_DEVICE: return "current device is not gfx950";
+    default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
+  }
+}
+
+int adr_matmul_f16(adr_stream_t stream, uint16_t* output, const uint16_t* lhs, const uint16_t* rhs,
+                   int32_t batches, int32_t m, int32_t k, int32_t n, int32_t stride_ox,
+                   int32_t stride_oy, int32_t stride_oz, int32_t stride_lx, int32_t stride_ly,
+                   int32_t stride_lz, int32_t stride_rx, int32_t stride_ry, int32_t stride_rz,
+                   const uint16_t* bias, float beta, float scale, uint32_t store, uint32_t load,
+                   uint32_t mask) {
+  MatmulArgs a = pack(output, lhs, rhs, batches, m, k, n, stride_ox, stride_oy, stride_oz,
+                      stride_lx, stride_ly, stride_lz, stride_rx, stride_ry, stride_rz, bias, beta,
+                      scale, store, load, mask);
+  if (int rc = validate_matmul(a, true)) return rc;
+  return run_matmul((hipStream_t)stream, a, true);
+}
+
+int adr_matmul_f16_slow(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
+                        const uint16_t* rhs, int32_t batches, int32_t m, int32_t k, int32_t n,
+                        int32_t stride_ox, int32_t stride_oy, int32_t stride_oz, int32_t stride_lx,
+                        int32_t stride_ly, int32_t stride_lz, int32_t stride_rx, int32_t stride_ry,
+                        int32_t stride_rz, const uint16_t* bias, float beta, float scale,
+                        uint32_t store, uint32_t load, uint32_t mask) {
+  MatmulArgs a = pack(output, lhs, rhs, batches, m, k, n, stride_ox, stride_oy, stride_oz,
+                      stride_lx, stride_ly, stride_lz, stride_rx, stride_ry, stride_rz, bias, beta,
+                      scale, store, load, mask);
+  if (int rc = validate_matmul(a, true)) return rc;
+  return run_matmul((hipStream_t)stream, a, false);
+}
+
+int adr_matmul_f16_raw(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
+                       const uint16_t* rhs, int32_t batches, int32_t m, int32_t k, int32_t n,
+                       int32_t stride_ox, int32_t stride_oy, int32_t stride_oz, int32_t stride_lx,
+                       int32_t stride_ly, int32_t stride_lz, int32_t stride_rx, int32_t stride_ry,
+                       int32_t stride_rz) {
+  return adr_matmul_f16(stream, output, lhs, rhs, batches, m, k, n, stride_ox, stride_oy,
+                        stride_oz, stride_lx, stride_ly, stride_lz, stride_rx, stride_ry, stride_rz,
+                        nullptr, 0.0f, 1.0f, ADR_STORE_IDENTITY, ADR_LOAD_IDENTITY, ADR_MASK_NONE);
+}
+
+int adr_matmul_f16_plan(char* name, int32_t cap, int32_t batches, int32_t m, int32_t k, int32_t n,
+                        int32_t stride_ox, int32_t stride_oy, int32_t stride_oz, int32_t stride_lx,
+                        int32_t stride_ly, int32_t stride_lz, int32_t stride_rx, int32_t stride_ry,
+                        int32_t stride_rz, uint32_t store, uint32_t load, uint32_t mask) {
+  MatmulArgs a = pack(nullptr, nullptr, nullptr, batches, m, k, n, stride_ox, stride_oy, stride_oz,
+                      stride_lx, stride_ly, stride_lz, stride_rx, stride_ry, stride_rz, nullptr,
+                      0.0f, 1.0f, store, load, mask);
+  if (int rc = validate_matmul(a, false)) return rc;
+  const char* chosen = "none (empty)";
+  if (!empty(a) && !mfma_gemm_supported(a, &chosen)) chosen = "matmul_general";
+  if (name && cap > 0) {
+    strncpy(name, chosen, (size_t)cap - 1);
+    name[cap - 1] = 0;
+  }
+  return ADR_OK;
+}
+
+int adr_matmul_nt_f16(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
+                      const uint16_t* rhs, int32_t m, int32_t p, int32_t n, float beta) {
+  if (m < 0 || p < 0 || n < 0) return ADR_EINVAL_SHAPE;
+  if (m == 0 || n == 0) return ADR_OK;
+  if (!output || (p && (!lhs || !rhs))) return ADR_ENULL;
+  MatmulArgs a = pack(output, lhs, rhs, 1, m, p, n, 1, n, 0, 1, p, 0, p, 1, 0, nullptr, beta, 1.0f,
+                      STORE_ACC_BETA, ADR_LOAD_IDENTITY, ADR_MASK_NONE);
+  return run_matmul((hipStream_t)stream, a, true);
+}
+
+int adr_matmul_nt_fp16u8(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
+                         const uint8_t* rhs, const uint16_t* scales, int32_t m, int32_t p,
+                         int32_t n, int32_t block_size, float beta) {
+  if (m < 0 || p < 0 || n < 0 || block_size <= 0) return ADR_EINVAL_SHAPE;
+  if (p % block_size != 0) return ADR_EDIVISIBILITY;
+  if (m == 0 || n == 0) return ADR_OK;
+  if (!output || (p && (!lhs || !rhs || !scales))) return ADR_ENULL;
+  return (int)launch_gemm_u8((hipStream_t)stream, (half_t*)output, (const half_t*)lhs, rhs,
+                             (const half_t*)scales, m, p, n, block_size, beta);
+}
+
+int adr_matmul_nt_fp16u8_plan(char* name, int32_t cap, int32_t m, int32_t p, int32_t n,
+                              int32_t block_size) {
+  if (m < 0 || p < 0 || n < 0 || block_size <= 0) return ADR_EINVAL_SHAPE;
+  if (p % block_size != 0) return ADR_EDIVISIBILITY;
+  const char* chosen = (m == 0 || n == 0) ? "none (empty)" : gemm_u8_plan(m, p, n, block_size);
+  if (name && cap > 0) {
+    strncpy(name, chosen, (size_t)cap - 1);
+    name[cap - 1] = 0;
+  }
+  return ADR_OK;
+}
+
+int adr_dequantize_absmax_uint8(adr_stream_t stream, adr_tensor_desc output,
+                                adr_tensor_desc scales, adr_tensor_desc input) {
+  if (int rc = validate_quant(output, scales, input)) return rc;
+  if (output.shape[0] == 0 || output.shape[1] == 0) return ADR_OK;
+  return (int)launch_dequantize((hipStream_t)stream, output, scales, input);
+}
+
+int adr_quantize_absmax_uint8(adr_stream_t stream, adr_tensor_desc output, adr_tensor_desc scales,
+                              adr_tensor_desc input) {
+  if (int rc = validate_quant(output, scales, input)) return rc;
+  if (output.shape[0] == 0 || output.shape[1] == 0) return ADR_OK;
+  return (int)launch_quantize((hipStream_t)stream, output, scales, input);
+}
+
+int adr_dequantize_absmax_u8(adr_stream_t stream, uint16_t* output, const uint8_t* q,
+                             const uint16_t* scales, int32_t rows, int32_t cols,
+                             int32_t block_size) {
+  if (rows < 0 || cols < 0 || block_size <= 0) return ADR_EINVAL_SHAPE;
+  if (cols % block_size != 0) return ADR_EDIVISIBILITY;
+  if (rows == 0 || cols == 0) return ADR_OK;
+  return adr_dequantize_absmax_uint8(stream, desc2d(output, rows, cols),
+                                     desc2d(scales, rows, cols / block_size),
+                                     desc2d(q, rows, cols));
+}
+
+int adr_quantize_absmax_u8(adr_stream_t stream, uint8_t* q, uint16_t* scales,
+                           const uint16_t* input, int32_t rows, int32_t cols, int32_t block_size) {
+  if (rows < 0 || cols < 0 || block_size <= 0) return ADR_EINVAL_SHAPE;
+  if (cols % block_size != 0) return ADR_EDIVISIBILITY;
+  if (rows == 0 || cols == 0) return ADR_OK;
+  return adr_quantize_absmax_uint8(stream, desc2d(q, rows, cols),
+                                   desc2d(scales, rows, cols / block_size),
+                                   desc2d(input, rows, cols));
+}
+
+}  // extern "C"

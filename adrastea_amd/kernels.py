@@ -1,0 +1,282 @@
+"""Host-side matmul interface, mirroring ``adrastea_models/src/kernels.rs``.
+
+``CommonKernels.matmul_f16`` / ``matmul_f16_slow`` keep the reference's names, argument meaning
+and error behaviour (kernels.rs:206-213, 753-890): views in, options by value, shape mismatches
+raise ``AssertionError`` (the reference ``assert_eq!``-panics), device/launcher errors raise
+``AdrasteaError`` (the reference returns ``anyhow::Error``).  ``lower_matmul`` is the pure
+lowering of views + options to the 22-scalar argument tuple of the C ABI.
+
+The u8 entry points have no Rust caller in the reference (llama.rs:28-29); their methods here
+follow the device kernels' argument lists (matmul_nt_fp16u8.cu:4-12, quantize.cu:3-5,46-48).
+"""
+from __future__ import annotations
+
+import ctypes as C
+import threading
+from dataclasses import dataclass, field
+from typing import Optional, Tuple
+
+from . import _ffi
+from .tensor import TensorLayout, TensorView
+
+
+class AdrasteaError(RuntimeError):
+    def __init__(self, code: int, what: str):
+        super().__init__(f"{what}: {_ffi.strerror(code)} (code {code})")
+        self.code = code
+
+
+# ---- option enums (kernels.rs:81-167) ------------------------------------------------------
+
+class MatmulMask:
+    NONE = 0
+    CAUSAL = 1
+
+
+@dataclass(frozen=True)
+class MatmulLoad:
+    op: int = 0          # MatmulLoadOp: Identity = 0, Scale = 1
+    scale: float = 1.0
+
+    @staticmethod
+    def Identity() -> "MatmulLoad":
+        return MatmulLoad(0, 1.0)
+
+    @staticmethod
+    def Scale(scale: float) -> "MatmulLoad":
+        return MatmulLoad(1, float(scale))
+
+    def lower(self) -> int:
+        return self.op
+
+
+@dataclass(frozen=True)
+class MatmulStore:
+    op: int = 0          # MatmulStoreOp, kernels.rs:103-112
+    beta: float = 0.0
+    scale: Optional[float] = None
+    bias: Optional[TensorView] = None
+
+    @staticmethod
+    def Identity() -> "MatmulStore":
+        return MatmulStore(0)
+
+    @staticmethod
+    def GeluBias(bias) -> "MatmulStore":
+        return MatmulStore(1, bias=bias)
+
+    @staticmethod
+    def BetaGeluBias(beta: float, bias) -> "MatmulStore":
+        return MatmulStore(2, beta=float(beta), bias=bias)
+
+    @staticmethod
+    def BetaBias(beta: float, bias) -> "MatmulStore":
+        return MatmulStore(3, beta=float(beta), bias=bias)
+
+    @staticmethod
+    def Scale(scale: float) -> "MatmulStore":
+        return MatmulStore(4, scale=float(scale))
+
+    @staticmethod
+    def Add() -> "MatmulStore":
+        return MatmulStore(5)
+
+    @staticmethod
+    def QuickGeluBias(bias) -> "MatmulStore":
+        return MatmulStore(6, bias=bias)
+
+    def lower(self) -> int:
+        return self.op
+
+
+@dataclass(frozen=True)
+class MatmulOptions:
+    """Builder with the reference's method names (kernels.rs:143-167)."""
+    load_: MatmulLoad = field(default_factory=MatmulLoad.Identity)
+    store_: MatmulStore = field(default_factory=MatmulStore.Identity)
+    mask_: int = MatmulMask.NONE
+
+    @staticmethod
+    def new() -> "MatmulOptions":
+        return MatmulOptions()
+
+    def load(self, load: MatmulLoad) -> "MatmulOptions":
+        return MatmulOptions(load, self.store_, self.mask_)
+
+    def store(self, store: MatmulStore) -> "MatmulOptions":
+        return MatmulOptions(self.load_, store, self.mask_)
+
+    def mask(self, mask: int) -> "MatmulOptions":
+        return MatmulOptions(self.load_, self.store_, mask)
+
+
+# ---- lowering (kernels.rs:821-890) -----------------------------------------------------------
+
+@dataclass(frozen=True)
+class LoweredMatmul:
+    batches: int
+    m: int
+    k: int
+    n: int
+    stride_o: Tuple[int, int, int]   # (x, y, z)
+    stride_l: Tuple[int, int, int]
+    stride_r: Tuple[int, int, int]
+    beta: float
+    scale: float
+    store: int
+    load: int
+    mask: int
+
+    def scalars(self):
+        return (self.batches, self.m, self.k, self.n, *self.stride_o, *self.stride_l,
+                *self.stride_r)
+
+
+def _xyz(layout: TensorLayout) -> Tuple[int, int, int]:
+    # batch stride 0 for rank-2 operands: they are broadcast over the batches (kernels.rs:868-880)
+    return (layout.stride(-1), layout.stride(-2), layout.stride(-3) if len(layout.dims) > 2 else 0)
+
+
+def lower_matmul(output: TensorLayout, left: TensorLayout, right: TensorLayout,
+                 options: MatmulOptions) -> LoweredMatmul:
+    assert left.size(-1) == right.size(-2), "K mismatch"      # kernels.rs:825
+    assert output.size(-2) == left.size(-2), "M mismatch"     # kernels.rs:826
+    assert output.size(-1) == right.size(-1), "N mismatch"    # kernels.rs:827
+    scale = options.load_.scale if options.load_.op == 1 else 1.0
+    if options.store_.op == 4:
+        scale *= options.store_.scale                          # one float for both (:837-843)
+    beta = options.store_.beta if options.store_.op in (2, 3) else 0.0
+    batches = output.size(-3) if len(output.dims) > 2 else 1
+    return LoweredMatmul(batches, left.size(-2), left.size(-1), right.size(-1), _xyz(output),
+                         _xyz(left), _xyz(right), beta, scale, options.store_.lower(),
+                         options.load_.lower(), options.mask_)
+
+
+# ---- the kernel interface ----------------------------------------------------------------------
+
+class CommonKernels:
+    """The matmul subset of the reference trait (kernels.rs:169-229)."""
+
+    def matmul_f16(self, output: TensorView, left: TensorView, right: TensorView,
+                   options: MatmulOptions) -> None:
+        raise NotImplementedError
+
+    def matmul_f16_slow(self, output: TensorView, left: TensorView, right: TensorView,
+                        options: MatmulOptions) -> None:
+        raise NotImplementedError
+
+
+def _current_stream() -> int:
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
+class GpuKernels(CommonKernels):
+    """Launches through the C ABI on torch's current HIP stream.  Holds no mutable state."""
+
+    def __init__(self):
+        self._lib = _ffi.lib()
+        import torch
+        if not torch.cuda.is_available():
+            raise RuntimeError("adrastea_amd.GpuKernels needs a GPU; there is no CPU fallback")
+
+    def _matmul(self, fn, what, output, left, right, options):
+        low = lower_matmul(output.layout, left.layout, right.layout, options)
+        bias = options.store_.bias
+        rc = fn(_current_stream(), output.data_ptr(), left.data_ptr(), right.data_ptr(),
+                *low.scalars(), bias.data_ptr() if bias is not None else None, low.beta,
+                low.scale, low.store, low.load, low.mask)
+        if rc != 0:
+            raise AdrasteaError(rc, what)
+
+    def matmul_f16(self, output, left, right, options=MatmulOptions()):
+        self._matmul(self._lib.adr_matmul_f16, "matmul_f16", output, left, right, options)
+
+    def matmul_f16_slow(self, output, left, right, options=MatmulOptions()):
+        self._matmul(self._lib.adr_matmul_f16_slow, "matmul_f16_slow", output, left, right,
+                     options)
+
+    # -- contiguous NT forms (device signatures only in the reference) --
+    def matmul_nt_f16(self, output, lhs, rhs, beta: float = 0.0):
+        m, p = lhs.shape
+        n = rhs.shape[0]
+        assert rhs.shape[1] == p and tuple(output.shape) == (m, n)
+        assert output.is_contiguous() and lhs.is_contiguous() and rhs.is_contiguous()
+        rc = self._lib.adr_matmul_nt_f16(_current_stream(), output.data_ptr(), lhs.data_ptr(),
+                                         rhs.data_ptr(), m, p, n, beta)
+        if rc != 0:
+            raise AdrasteaError(rc, "matmul_nt_f16")
+
+    def matmul_nt_fp16u8(self, output, lhs, rhs_q, scales, block_size: int, beta: float = 0.0):
+        m, p = lhs.shape
+        n = rhs_q.shape[0]
+        assert rhs_q.shape[1] == p and tuple(output.shape) == (m, n)
+        assert tuple(scales.shape) == (n, p // block_size)
+        assert all(t.is_contiguous() for t in (output, lhs, rhs_q, scales))
+        rc = self._lib.adr_matmul_nt_fp16u8(_current_stream(), output.data_ptr(), lhs.data_ptr(),
+                                            rhs_q.data_ptr(), scales.data_ptr(), m, p, n,
+                                            block_size, beta)
+        if rc != 0:
+            raise AdrasteaError(rc, "matmul_nt_fp16u8")
+
+    def dequantize_absmax_uint8(self, output, scales, q):
+        rows, cols = q.shape
+        block_size = cols // scales.shape[1]
+        rc = self._lib.adr_dequantize_absmax_u8(_current_stream(), output.data_ptr(),
+                                                q.data_ptr(), scales.data_ptr(), rows, cols,
+                                                block_size)
+        if rc != 0:
+            raise AdrasteaError(rc, "dequantize_absmax_uint8")
+
+    def quantize_absmax_uint8(self, q, scales, x):
+        rows, cols = x.shape
+        block_size = cols // scales.shape[1]
+        rc = self._lib.adr_quantize_absmax_u8(_current_stream(), q.data_ptr(), scales.data_ptr(),
+                                              x.data_ptr(), rows, cols, block_size)
+        if rc != 0:
+            raise AdrasteaError(rc, "quantize_absmax_uint8")
+
+
+def descriptor(view: TensorView) -> _ffi.TensorDesc:
+    """TensorGpuDescriptor::from (kernels.rs:38-55): dims and strides reversed, innermost first."""
+    d = _ffi.TensorDesc()
+    d.ptr = view.data_ptr()
+    d.dims = len(view.layout.dims)
+    for i, (dim, stride) in enumerate(zip(reversed(view.layout.dims),
+                                          reversed(view.layout.strides))):
+        d.shape[i] = dim
+        d.strides[i] = stride
+    return d
+
+
+def plan_matmul(output: TensorLayout, left: TensorLayout, right: TensorLayout,
+                options: MatmulOptions = MatmulOptions()) -> str:
+    """Name of the kernel adr_matmul_f16 selects for these layouts (no device needed)."""
+    low = lower_matmul(output, left, right, options)
+    buf = C.create_string_buffer(64)
+    rc = _ffi.lib().adr_matmul_f16_plan(buf, 64, *low.scalars(), low.store, low.load, low.mask)
+    if rc != 0:
+        raise AdrasteaError(rc, "matmul_f16_plan")
+    return buf.value.decode()
+
+
+class MatmulTracer(CommonKernels):
+    """Decorator recording the set of (left, right, output) layouts seen by the matmuls, then
+    forwarding (kernels.rs:231-359)."""
+
+    def __init__(self, inner: CommonKernels):
+        self.inner = inner
+        self._lock = threading.Lock()
+        self.shapes = set()
+
+    def _record(self, output, left, right):
+        with self._lock:
+            self.shapes.add((left.layout, right.layout, output.layout))
+
+    def matmul_f16(self, output, left, right, options=MatmulOptions()):
+        self._record(output, left, right)
+        self.inner.matmul_f16(output, left, right, options)
+
+    def matmul_f16_slow(self, output, left, right, options=MatmulOptions()):
+        self._record(output, left, right)
+        self.inner.matmul_f16_slow(output, left, right, options)

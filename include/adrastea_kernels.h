@@ -1,0 +1,172 @@
+/*
+ * adrastea_kernels -- C ABI of the gfx950 (MI355X) matmul kernels.
+ *
+ * This is the boundary a Rust `extern "C"` block in adrastea_kernels binds.  Every entry
+ * point takes plain pointers and scalars, launches asynchronously on the given HIP stream
+ * (NULL = the null stream, which is what the reference uses: `stream: None`,
+ * adrastea_models/src/kernels.rs:862), never synchronises, never allocates, and returns
+ * 0 on success, a positive hipError_t, or a negative ADR_E* code.  Invalid requests are
+ * rejected on the host; no entry point traps on the device.
+ *
+ * fp16 data is passed as uint16_t bit patterns (Rust `half::f16` is repr(transparent) u16).
+ * All strides are in ELEMENTS.  `x` is the last tensor dimension, `y` the second to last,
+ * `z` the batch dimension (kernels.rs:864-887).
+ */
+#ifndef ADRASTEA_KERNELS_H
+#define ADRASTEA_KERNELS_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* A hipStream_t, declared opaquely so that this header needs no HIP include. */
+typedef void* adr_stream_t;
+
+/* Error codes (negative; positive values are hipError_t). */
+enum {
+  ADR_OK = 0,
+  ADR_EINVAL_SHAPE = -1,   /* negative / zero-incompatible sizes, offsets beyond int32 */
+  ADR_EINVAL_ENUM = -2,    /* store / load / mask value out of range */
+  ADR_ENOTIMPL = -3,       /* MatmulStoreOp::GeluBias = 1: lowers from Rust
+                              (kernels.rs:125) but has no device case in the reference
+                              (matmul.cu:450-491 -> NYI trap); rejected here instead */
+  ADR_ENULL = -4,          /* null tensor pointer, or a bias operator without a bias */
+  ADR_EDIVISIBILITY = -5,  /* u8 kernels: p % block_size != 0 or block_size not supported */
+  ADR_EUNSUPPORTED_DEVICE = -6 /* the current device is not gfx950 */
+};
+
+/* adrastea_models/src/kernels.rs:81-135, adrastea_kernels/cpp/matmul.cu:26-36 */
+enum { ADR_LOAD_IDENTITY = 0, ADR_LOAD_SCALE = 1 };
+enum {
+  ADR_STORE_IDENTITY = 0,
+  ADR_STORE_GELU_BIAS = 1,
+  ADR_STORE_BETA_GELU_BIAS = 2,
+  ADR_STORE_BETA_BIAS = 3,
+  ADR_STORE_SCALE = 4,
+  ADR_STORE_ADD = 5,
+  ADR_STORE_QUICK_GELU_BIAS = 6
+};
+enum { ADR_MASK_NONE = 0, ADR_MASK_CAUSAL = 1 };
+
+/*
+ * Replaces the launch of `matmul_f16_fast` in GpuKernels::matmul_f16
+ * (adrastea_models/src/kernels.rs:821-890; device adrastea_kernels/cpp/matmul.cu:504-513).
+ * Same 22 arguments in the same order as the Rust tuple (kernels.rs:864-887), preceded by
+ * the stream.  Launch geometry and LDS size are chosen inside.
+ *
+ *   O[b,y,x] = store( sum_k load(L[b,y,k]) * load(R[b,k,x]) ),  mask(x, y) -> -inf
+ *
+ * fp16 operands, fp32 accumulation, fp16 result.  The accumulator is narrowed to fp16
+ * before the store operator, as in the reference (matmul.cu:47-52, 64-71).
+ */
+int adr_matmul_f16(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
+                   const uint16_t* rhs, int32_t batches, int32_t m, int32_t k, int32_t n,
+                   int32_t stride_ox, int32_t stride_oy, int32_t stride_oz, int32_t stride_lx,
+                   int32_t stride_ly, int32_t stride_lz, int32_t stride_rx, int32_t stride_ry,
+                   int32_t stride_rz, const uint16_t* bias, float beta, float scale,
+                   uint32_t store, uint32_t load, uint32_t mask);
+
+/*
+ * Replaces the launch of the naive `matmul_f16` in GpuKernels::matmul_f16_slow
+ * (kernels.rs:753-819; device matmul.cu:195-222, 493-502).  One thread per output element,
+ * any strides; reproduces the reference arithmetic step for step (fp16-rounded products,
+ * sequential fp32 sum).  It is the correctness path the fast kernels are compared with.
+ */
+int adr_matmul_f16_slow(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
+                        const uint16_t* rhs, int32_t batches, int32_t m, int32_t k, int32_t n,
+                        int32_t stride_ox, int32_t stride_oy, int32_t stride_oz,
+                        int32_t stride_lx, int32_t stride_ly, int32_t stride_lz,
+                        int32_t stride_rx, int32_t stride_ry, int32_t stride_rz,
+                        const uint16_t* bias, float beta, float scale, uint32_t store,
+                        uint32_t load, uint32_t mask);
+
+/* `matmul_f16_raw` (matmul.cu:515-517): identity operators, the 16 common arguments. */
+int adr_matmul_f16_raw(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
+                       const uint16_t* rhs, int32_t batches, int32_t m, int32_t k, int32_t n,
+                       int32_t stride_ox, int32_t stride_oy, int32_t stride_oz,
+                       int32_t stride_lx, int32_t stride_ly, int32_t stride_lz,
+                       int32_t stride_rx, int32_t stride_ry, int32_t stride_rz);
+
+/*
+ * fp16 NT GEMM, contiguous operands: out[m,n] = lhs[m,p] . rhs[n,p]^T + beta * out[m,n].
+ * Argument list of `matmul_nt_wmma_16x128x256` / `matmul_nt_wmma_128x64x64`
+ * (adrastea_kernels/cpp/matmul_nt_wmma_16x128x256.cu:8-14); their m%16 / n%128 / p%256
+ * divisibility requirements do not apply here.
+ */
+int adr_matmul_nt_f16(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
+                      const uint16_t* rhs, int32_t m, int32_t p, int32_t n, float beta);
+
+/*
+ * u8-quantised-weight NT GEMM / GEMV with the dequantisation fused into the weight load.
+ * Argument list of `matmul_nt_fp16u8` and `matmul_nt_wmma_16x128x256_fp16u8`
+ * (adrastea_kernels/cpp/matmul_nt_fp16u8.cu:4-12, matmul_nt_wmma_16x128x256_fp16u8.cu:12-20):
+ *
+ *   w[c,i]   = fp16( (float(rhs[c,i]) - 127.5f) * float(scales[c, i / block_size]) )
+ *   out[r,c] = fp16( sum_i lhs[r,i] * w[c,i]  +  beta * out[r,c] )      (fp32 accumulation)
+ *
+ * lhs [m,p] fp16, rhs [n,p] u8, scales [n, p/block_size] fp16, out [m,n] fp16, all contiguous.
+ * Any m >= 1 and n >= 1; p % block_size == 0; block_size a multiple of 8.
+ */
+int adr_matmul_nt_fp16u8(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
+                         const uint8_t* rhs, const uint16_t* scales, int32_t m, int32_t p,
+                         int32_t n, int32_t block_size, float beta);
+
+/*
+ * Flat-pointer forms of `dequantize_absmax_uint8` / `quantize_absmax_uint8`
+ * (adrastea_kernels/cpp/quantize.cu:46-56 and :3-44) for contiguous [rows, cols] tensors with
+ * scales [rows, cols / block_size]:
+ *   dequantise: out = fp16((float(q) - 127.5f) * float(scale))
+ *   quantise:   scale = fp16(absmax / 127.5f); q = u8(round(127.5f + x / float(scale)))
+ */
+int adr_dequantize_absmax_u8(adr_stream_t stream, uint16_t* output, const uint8_t* q,
+                             const uint16_t* scales, int32_t rows, int32_t cols,
+                             int32_t block_size);
+int adr_quantize_absmax_u8(adr_stream_t stream, uint8_t* q, uint16_t* scales,
+                           const uint16_t* input, int32_t rows, int32_t cols,
+                           int32_t block_size);
+
+/*
+ * The by-value tensor descriptor the reference passes to its quantise kernels
+ * (TensorGpuDescriptor, adrastea_models/src/kernels.rs:28-61; device TensorView<T>,
+ * adrastea_kernels/cpp/compat.h:40-45).  Index 0 is the INNERMOST dimension.
+ */
+typedef struct adr_tensor_desc {
+  void* ptr;
+  uint32_t dims;
+  uint32_t shape[7];
+  uint32_t strides[7];
+} adr_tensor_desc;
+
+/* Descriptor forms with the reference's argument order (quantize.cu:3-5, 46-48).  2-d
+ * tensors, any strides; block_size = output.shape[0] / scales.shape[0]. */
+int adr_dequantize_absmax_uint8(adr_stream_t stream, adr_tensor_desc output,
+                                adr_tensor_desc scales, adr_tensor_desc input);
+int adr_quantize_absmax_uint8(adr_stream_t stream, adr_tensor_desc output,
+                              adr_tensor_desc scales, adr_tensor_desc input);
+
+/*
+ * Diagnostics (no counterpart in the reference).
+ *
+ * adr_matmul_f16_plan: writes the name of the kernel adr_matmul_f16 would launch for these
+ * arguments into `name` (at most `cap` bytes, NUL-terminated) without touching the device.
+ * Same validation and return codes as adr_matmul_f16 minus the pointer checks.
+ */
+int adr_matmul_f16_plan(char* name, int32_t cap, int32_t batches, int32_t m, int32_t k,
+                        int32_t n, int32_t stride_ox, int32_t stride_oy, int32_t stride_oz,
+                        int32_t stride_lx, int32_t stride_ly, int32_t stride_lz,
+                        int32_t stride_rx, int32_t stride_ry, int32_t stride_rz, uint32_t store,
+                        uint32_t load, uint32_t mask);
+int adr_matmul_nt_fp16u8_plan(char* name, int32_t cap, int32_t m, int32_t p, int32_t n,
+                              int32_t block_size);
+
+/* Human-readable text for an ADR_E* code or hipError_t. */
+const char* adr_strerror(int code);
+/* ABI version of this library (bumped on any signature change). */
+int adr_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ADRASTEA_KERNELS_H */

@@ -1,0 +1,408 @@
+"""GPU parity of the fp16 matmul entry points (through the C ABI) against the CPU oracle, the
+reference's own naive kernel (oracle/_ref, when built) and an fp32/fp64 GEMM.
+
+Bars: bit-exact where the arithmetic is exactly determined (dyadic inputs, fp16-only operators,
+mask pattern, the step-for-step slow kernel); max relative error <= 1e-2 against an fp32/fp64
+GEMM on random inputs (the stated tolerance of this path: fp16 output, fp32 accumulation).
+"""
+import itertools
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import rng, randn_f16, ulp_diff_f16, max_rel_err, largest_address, view
+from gpu_common import to_dev, to_np, raw_matmul, oracle_matmul, plan
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2  # max relative error vs an fp32/fp64 GEMM (fp16 output, fp32 accumulation)
+
+
+def dyadic(g, shape):
+    return (g.integers(-256, 257, size=shape) / 64.0).astype(np.float16)
+
+
+def nt_strides(M, K, N):
+    # output row-major, lhs row-major, rhs = W[N,K].permute([1,0])
+    return (1, N, 0), (1, K, 0), (K, 1, 0)
+
+
+@pytest.fixture(scope="module")
+def ref():
+    import refgpu
+    if not refgpu.available():
+        pytest.skip("oracle/_ref code objects not built")
+    return refgpu.RefKernels()
+
+
+# ------------------------------------------------------------------ slow (step-for-step) kernel
+
+STORES_EXACT = [oracle.STORE_IDENTITY, oracle.STORE_SCALE, oracle.STORE_ADD]
+STORES_F32 = [oracle.STORE_BETA_BIAS, oracle.STORE_QUICK_GELU_BIAS, oracle.STORE_BETA_GELU_BIAS]
+
+
+def _random_layout_case(g, B, M, K, N):
+    perms = list(itertools.permutations(range(3)))
+
+    def layout(shape, perm, pad):
+        strides, s = [0, 0, 0], pad
+        for d in reversed(perm):
+            strides[d] = s
+            s *= shape[d] + 1
+        return strides
+    po, pl, pr = (perms[i] for i in g.integers(0, 6, size=3))
+    so3 = layout((B, M, N), po, 1)
+    sl3 = layout((B, M, K), pl, int(g.integers(1, 3)))
+    sr3 = layout((B, K, N), pr, int(g.integers(1, 3)))
+    return so3, sl3, sr3
+
+
+@pytest.mark.parametrize("store", STORES_EXACT + STORES_F32)
+@pytest.mark.parametrize("load", [oracle.LOAD_IDENTITY, oracle.LOAD_SCALE])
+@pytest.mark.parametrize("mask", [oracle.MASK_NONE, oracle.MASK_CAUSAL])
+def test_slow_kernel_matches_faithful_oracle(store, load, mask):
+    g = rng(100 + store * 10 + load * 2 + mask)
+    B, M, K, N = 3, 19, 45, 21
+    so3, sl3, sr3 = _random_layout_case(g, B, M, K, N)
+    lbuf = randn_f16(g, largest_address((B, M, K), sl3) + 4)
+    rbuf = randn_f16(g, largest_address((B, K, N), sr3) + 3, 0.2)
+    obuf = randn_f16(g, largest_address((B, M, N), so3) + 2)
+    bias = randn_f16(g, N)
+    so, sl, sr = (so3[2], so3[1], so3[0]), (sl3[2], sl3[1], sl3[0]), (sr3[2], sr3[1], sr3[0])
+    kw = dict(beta=0.6, scale=0.37, store=store, load=load, mask=mask, offsets=(1, 3, 2))
+    want = oracle_matmul(obuf, lbuf, rbuf, B, M, K, N, so, sl, sr, bias=bias,
+                         mode=oracle.FAITHFUL, **kw)
+    o_t, l_t, r_t, b_t = to_dev(obuf), to_dev(lbuf), to_dev(rbuf), to_dev(bias)
+    rc = raw_matmul("adr_matmul_f16_slow", o_t, l_t, r_t, B, M, K, N, so, sl, sr, bias_t=b_t, **kw)
+    assert rc == 0
+    got = to_np(o_t)
+    if store in STORES_EXACT:
+        assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    else:
+        # fp32 epilogue: the device may fuse a multiply-add or use its own expf/tanhf
+        assert np.max(ulp_diff_f16(got, want)) <= 2
+
+
+@pytest.mark.parametrize("store", STORES_EXACT + STORES_F32)
+@pytest.mark.parametrize("mask", [oracle.MASK_NONE, oracle.MASK_CAUSAL])
+def test_oracle_and_slow_kernel_match_reference_naive_kernel(ref, store, mask):
+    """The reference's own matmul_f16 kernel, compiled for gfx950, on the same inputs: pins the
+    C restatement (faithful mode) and the slow kernel to the real thing."""
+    g = rng(200 + store * 2 + mask)
+    B, M, K, N = 2, 37, 70, 41
+    so3, sl3, sr3 = _random_layout_case(g, B, M, K, N)
+    lbuf = randn_f16(g, largest_address((B, M, K), sl3) + 1)
+    rbuf = randn_f16(g, largest_address((B, K, N), sr3) + 1, 0.2)
+    obuf = randn_f16(g, largest_address((B, M, N), so3) + 1)
+    bias = randn_f16(g, N)
+    so, sl, sr = (so3[2], so3[1], so3[0]), (sl3[2], sl3[1], sl3[0]), (sr3[2], sr3[1], sr3[0])
+    kw = dict(beta=-0.4, scale=0.2, store=store, load=oracle.LOAD_IDENTITY, mask=mask)
+    l_t, r_t, b_t = to_dev(lbuf), to_dev(rbuf), to_dev(bias)
+    o_ref = to_dev(obuf)
+    ref.matmul_f16(o_ref.data_ptr(), l_t.data_ptr(), r_t.data_ptr(), B, M, K, N, so, sl, sr,
+                   bias_ptr=b_t.data_ptr(), **kw)
+    torch.cuda.synchronize()
+    want = to_np(o_ref)
+    o_t = to_dev(obuf)
+    assert raw_matmul("adr_matmul_f16_slow", o_t, l_t, r_t, B, M, K, N, so, sl, sr, bias_t=b_t,
+                      **kw) == 0
+    got = to_np(o_t)
+    orc = oracle_matmul(obuf, lbuf, rbuf, B, M, K, N, so, sl, sr, bias=bias, mode=oracle.FAITHFUL,
+                        **kw)
+    if store in STORES_EXACT:
+        assert np.array_equal(orc.view(np.uint16), want.view(np.uint16))
+        assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    else:
+        assert np.max(ulp_diff_f16(orc, want)) <= 2
+        assert np.max(ulp_diff_f16(got, want)) <= 2
+
+
+def test_reference_tiled_kernel_agrees_with_its_naive_kernel(ref):
+    """matmul_f16_fast (the production kernel of the reference) sums in the same k order with the
+    same fp16 products: the two reference kernels, and therefore the oracle, must agree."""
+    g = rng(210)
+    B, M, K, N = 2, 50, 75, 70  # K % 32 != 0 exercises its scalar tail loop
+    so, sl, sr = (1, N, M * N), (1, K, M * K), (K, 1, K * N)
+    l, r = randn_f16(g, B * M * K), randn_f16(g, B * K * N, 0.2)
+    l_t, r_t = to_dev(l), to_dev(r)
+    o1, o2 = to_dev(np.zeros(B * M * N, np.float16)), to_dev(np.zeros(B * M * N, np.float16))
+    ref.matmul_f16(o1.data_ptr(), l_t.data_ptr(), r_t.data_ptr(), B, M, K, N, so, sl, sr)
+    ref.matmul_f16_fast(o2.data_ptr(), l_t.data_ptr(), r_t.data_ptr(), B, M, K, N, so, sl, sr)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_np(o1).view(np.uint16), to_np(o2).view(np.uint16))
+
+
+# ------------------------------------------------------------------ fast (MFMA) path
+
+SHAPES = [
+    # (B, M, K, N): tails in every dimension, every tile configuration
+    (1, 77, 768, 2304),     # BASELINE config 1 (CLIP text QKV)
+    (1, 64, 64, 64),
+    (1, 1, 8, 1),
+    (1, 33, 72, 130),
+    (1, 300, 200, 520),
+    (1, 515, 136, 1100),
+    (3, 129, 96, 257),
+    (1, 2056, 256, 1024),   # config-2-like M tail with the large tile
+]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_fast_nt_bit_exact_on_dyadic_inputs(shape):
+    B, M, K, N = shape
+    g = rng(300 + M + N)
+    so, sl, sr = (1, N, M * N), (1, K, M * K), (K, 1, K * N)
+    assert plan(B, M, K, N, so, sl, sr).startswith("gemm_nt_mfma")
+    # k/64 values in [-1/8, 1/8]: sums of up to 768 products stay exact in fp32
+    l = (g.integers(-8, 9, size=B * M * K) / 64.0).astype(np.float16)
+    r = (g.integers(-8, 9, size=B * K * N) / 64.0).astype(np.float16)
+    o_t = to_dev(np.full(B * M * N, 9.0, np.float16))
+    assert raw_matmul("adr_matmul_f16", o_t, to_dev(l), to_dev(r), B, M, K, N, so, sl, sr) == 0
+    want = np.einsum("bmk,bnk->bmn", l.reshape(B, M, K).astype(np.float64),
+                     r.reshape(B, N, K).astype(np.float64)).astype(np.float32).astype(np.float16)
+    assert np.array_equal(to_np(o_t).reshape(B, M, N).view(np.uint16), want.view(np.uint16))
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_fast_nt_random_within_tolerance_and_close_to_oracle(shape):
+    B, M, K, N = shape
+    g = rng(400 + M + N)
+    so, sl, sr = (1, N, M * N), (1, K, M * K), (K, 1, K * N)
+    l, r = randn_f16(g, B * M * K), randn_f16(g, B * K * N, K ** -0.5)
+    o_t = to_dev(np.zeros(B * M * N, np.float16))
+    assert raw_matmul("adr_matmul_f16", o_t, to_dev(l), to_dev(r), B, M, K, N, so, sl, sr) == 0
+    got = to_np(o_t).reshape(B, M, N)
+    ref64 = np.einsum("bmk,bnk->bmn", l.reshape(B, M, K).astype(np.float64),
+                      r.reshape(B, N, K).astype(np.float64))
+    assert max_rel_err(got, ref64) <= TOL
+    # exact products + fp32 accumulation: within one fp16 step of the correctly rounded result
+    assert np.max(ulp_diff_f16(got, ref64.astype(np.float16))) <= 1 or max_rel_err(got, ref64) <= 2e-3
+
+
+@pytest.mark.parametrize("store", STORES_EXACT + STORES_F32)
+@pytest.mark.parametrize("mask", [oracle.MASK_NONE, oracle.MASK_CAUSAL])
+def test_fast_nt_epilogues_match_oracle(store, mask):
+    g = rng(500 + store * 2 + mask)
+    B, M, K, N = 2, 150, 64, 200
+    so, sl, sr = (1, N, M * N), (1, K, M * K), (K, 1, K * N)
+    assert plan(B, M, K, N, so, sl, sr, store=store, mask=mask).startswith("gemm_nt_mfma")
+    l = (g.integers(-16, 17, size=B * M * K) / 16.0).astype(np.float16)
+    r = (g.integers(-16, 17, size=B * K * N) / 16.0).astype(np.float16)
+    prev, bias = randn_f16(g, B * M * N), randn_f16(g, N)
+    kw = dict(beta=0.7, scale=0.2, store=store, load=oracle.LOAD_IDENTITY, mask=mask)
+    want = oracle_matmul(prev, l, r, B, M, K, N, so, sl, sr, bias=bias, mode=oracle.EXACT, **kw)
+    o_t = to_dev(prev)
+    assert raw_matmul("adr_matmul_f16", o_t, to_dev(l), to_dev(r), B, M, K, N, so, sl, sr,
+                      bias_t=to_dev(bias), **kw) == 0
+    got = to_np(o_t)
+    if store in STORES_EXACT:
+        assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    else:
+        assert np.max(ulp_diff_f16(got, want)) <= 2
+    if mask == oracle.MASK_CAUSAL:
+        y, x = np.mgrid[0:M, 0:N]
+        assert np.all(got.reshape(B, M, N).view(np.uint16)[:, x > y] == 0xFC00)
+
+
+def test_fast_nt_load_scale():
+    g = rng(520)
+    B, M, K, N = 1, 100, 128, 90
+    so, sl, sr = (1, N, 0), (1, K, 0), (K, 1, 0)
+    l, r = randn_f16(g, M * K), randn_f16(g, K * N, 0.1)
+    scale = 64.0 ** -0.25  # Whisper's d_head^-0.25 (whisper.rs:424-430)
+    want = oracle_matmul(np.zeros(M * N, np.float16), l, r, B, M, K, N, so, sl, sr,
+                         load=oracle.LOAD_SCALE, scale=scale, mode=oracle.EXACT)
+    o_t = to_dev(np.zeros(M * N, np.float16))
+    assert raw_matmul("adr_matmul_f16", o_t, to_dev(l), to_dev(r), B, M, K, N, so, sl, sr,
+                      load=oracle.LOAD_SCALE, scale=scale) == 0
+    assert np.max(ulp_diff_f16(to_np(o_t), want)) <= 1
+
+
+def test_attention_views_qk_and_pv():
+    """llama.rs:534-554 with S=160, 4 heads, head_dim 64: QK^T with Scale + Causal on the
+    interleaved-head views, then P.V into the strided output view."""
+    g = rng(530)
+    S, H, D = 160, 4, 64
+    HD = H * D
+    q, k, v = (dyadic(g, S * HD) for _ in range(3))
+    scale = 1.0 / np.sqrt(D)
+    so, sl, sr = (1, S, S * S), (1, HD, D), (HD, 1, D)
+    assert plan(H, S, D, S, so, sl, sr, store=4, mask=1).startswith("gemm_nt_mfma")
+    kw = dict(store=oracle.STORE_SCALE, scale=scale, mask=oracle.MASK_CAUSAL)
+    want = oracle_matmul(np.zeros(H * S * S, np.float16), q, k, H, S, D, S, so, sl, sr,
+                         mode=oracle.EXACT, **kw)
+    qk_t = to_dev(np.zeros(H * S * S, np.float16))
+    assert raw_matmul("adr_matmul_f16", qk_t, to_dev(q), to_dev(k), H, S, D, S, so, sl, sr, **kw) == 0
+    assert np.array_equal(to_np(qk_t).view(np.uint16), want.view(np.uint16))
+    # P.V: probabilities k/64 in [0, 1/8]
+    p = (g.integers(0, 9, size=H * S * S) / 64.0).astype(np.float16)
+    so, sl, sr = (1, HD, D), (1, S, S * S), (1, HD, D)
+    # the general kernel rounds each product to fp16 like the reference; a tiled kernel does not
+    mode = oracle.FAITHFUL if plan(H, S, S, D, so, sl, sr) == "matmul_general" else oracle.EXACT
+    want = oracle_matmul(np.zeros(S * HD, np.float16), p, v, H, S, S, D, so, sl, sr, mode=mode)
+    o_t = to_dev(np.zeros(S * HD, np.float16))
+    assert raw_matmul("adr_matmul_f16", o_t, to_dev(p), to_dev(v), H, S, S, D, so, sl, sr) == 0
+    assert np.array_equal(to_np(o_t).view(np.uint16), want.view(np.uint16))
+
+
+def test_row_and_batch_strides_with_padding_on_the_fast_path():
+    g = rng(540)
+    B, M, K, N = 2, 70, 96, 150
+    ly, rx, oy = K + 8, K + 16, N + 5
+    lz, rz, oz = M * ly + 8, N * rx + 24, M * oy + 3
+    so, sl, sr = (1, oy, oz), (1, ly, lz), (rx, 1, rz)
+    assert plan(B, M, K, N, so, sl, sr).startswith("gemm_nt_mfma")
+    lbuf, rbuf = dyadic(g, B * lz + 8), dyadic(g, B * rz + 8)
+    obuf = np.full(B * oz + 8, 5.0, np.float16)
+    want = oracle_matmul(obuf, lbuf, rbuf, B, M, K, N, so, sl, sr, mode=oracle.EXACT,
+                         offsets=(3, 8, 8))
+    o_t = to_dev(obuf)
+    assert raw_matmul("adr_matmul_f16", o_t, to_dev(lbuf), to_dev(rbuf), B, M, K, N, so, sl, sr,
+                      offsets=(3, 8, 8)) == 0
+    assert np.array_equal(to_np(o_t).view(np.uint16), want.view(np.uint16))  # gaps untouched too
+
+
+def test_unsupported_layouts_fall_back_and_stay_correct():
+    g = rng(550)
+    B, M, K, N = 1, 40, 50, 30   # K % 8 != 0
+    so, sl, sr = (1, N, 0), (1, K, 0), (K, 1, 0)
+    assert plan(B, M, K, N, so, sl, sr) == "matmul_general"
+    l, r = dyadic(g, M * K), dyadic(g, K * N)
+    want = oracle_matmul(np.zeros(M * N, np.float16), l, r, B, M, K, N, so, sl, sr,
+                         mode=oracle.FAITHFUL)
+    o_t = to_dev(np.zeros(M * N, np.float16))
+    assert raw_matmul("adr_matmul_f16", o_t, to_dev(l), to_dev(r), B, M, K, N, so, sl, sr) == 0
+    assert np.array_equal(to_np(o_t).view(np.uint16), want.view(np.uint16))
+    # misaligned base pointer on an otherwise supported layout
+    K = 64
+    l, r = dyadic(g, M * K + 8), dyadic(g, K * N + 8)
+    sl, sr = (1, K, 0), (K, 1, 0)
+    want = oracle_matmul(np.zeros(M * N, np.float16), l, r, B, M, K, N, so, sl, sr,
+                         mode=oracle.FAITHFUL, offsets=(0, 1, 3))
+    o_t = to_dev(np.zeros(M * N, np.float16))
+    assert raw_matmul("adr_matmul_f16", o_t, to_dev(l), to_dev(r), B, M, K, N, so, sl, sr,
+                      offsets=(0, 1, 3)) == 0
+    assert np.array_equal(to_np(o_t).view(np.uint16), want.view(np.uint16))
+
+
+def test_matmul_nt_f16_entry_point():
+    from adrastea_amd import GpuKernels
+    g = rng(560)
+    M, K, N = 48, 256, 200
+    a, b, prev = dyadic(g, (M, K)), dyadic(g, (N, K)), randn_f16(g, (M, N))
+    for beta in (0.0, 0.5):
+        want = prev.copy()
+        oracle.matmul_nt_f16(want, a, b, beta=beta)
+        o_t = to_dev(prev)
+        GpuKernels().matmul_nt_f16(o_t, to_dev(a), to_dev(b), beta=beta)
+        assert np.max(ulp_diff_f16(to_np(o_t), want)) <= (0 if beta == 0.0 else 1)
+
+
+# ------------------------------------------------------------------ host API and error behaviour
+
+def test_gpukernels_interface_and_errors():
+    from adrastea_amd import (GpuKernels, TensorView, MatmulOptions, MatmulStore, MatmulMask,
+                              AdrasteaError, MatmulTracer)
+    g = rng(570)
+    S, D = 96, 64
+    kern = MatmulTracer(GpuKernels())
+    x, w = dyadic(g, (S, D)), dyadic(g, (D, D))
+    x_t, w_t = to_dev(x), to_dev(w)
+    out = torch.zeros(S, D, dtype=torch.float16, device="cuda")
+    kern.matmul_f16(TensorView.of(out), TensorView.of(x_t), TensorView.of(w_t).permute([1, 0]),
+                    MatmulOptions.new())
+    want = (x.astype(np.float64) @ w.astype(np.float64).T).astype(np.float32).astype(np.float16)
+    assert np.array_equal(to_np(out), want)
+    assert len(kern.shapes) == 1
+    with pytest.raises(AssertionError):   # K mismatch: the reference assert_eq!-panics
+        kern.matmul_f16(TensorView.of(out), TensorView.of(x_t), TensorView.of(w_t[:, :32]),
+                        MatmulOptions.new())
+    bias = torch.zeros(D, dtype=torch.float16, device="cuda")
+    with pytest.raises(AdrasteaError) as e:  # GeluBias: device NYI in the reference
+        kern.matmul_f16(TensorView.of(out), TensorView.of(x_t), TensorView.of(w_t).permute([1, 0]),
+                        MatmulOptions.new().store(MatmulStore.GeluBias(TensorView.of(bias))))
+    assert e.value.code == -3
+    with pytest.raises(AdrasteaError) as e:  # bias operator without a bias
+        kern.matmul_f16(TensorView.of(out), TensorView.of(x_t), TensorView.of(w_t).permute([1, 0]),
+                        MatmulOptions.new().store(MatmulStore.BetaBias(1.0, None)))
+    assert e.value.code == -4
+    o_t = to_dev(np.zeros(4, np.float16))
+    assert raw_matmul("adr_matmul_f16", o_t, o_t, o_t, 1, 2, 2, 2, (1, 2, 0), (1, 2, 0), (1, 2, 0),
+                      store=9) == -2
+    assert raw_matmul("adr_matmul_f16", o_t, o_t, o_t, 1, -2, 2, 2, (1, 2, 0), (1, 2, 0),
+                      (1, 2, 0)) == -1
+    # empty problems are a no-op, k == 0 stores store(0)
+    assert raw_matmul("adr_matmul_f16", o_t, o_t, o_t, 1, 0, 2, 2, (1, 2, 0), (1, 2, 0), (1, 2, 0)) == 0
+    o_t = to_dev(np.full(4, 3.0, np.float16))
+    assert raw_matmul("adr_matmul_f16", o_t, o_t, o_t, 1, 2, 0, 2, (1, 2, 0), (1, 2, 0), (1, 2, 0)) == 0
+    assert np.all(to_np(o_t) == 0)
+
+
+# ------------------------------------------------------------------ BASELINE sizes: properties
+
+FULL = [
+    # name, B, M, K, N  (fp16 NT weights)
+    ("clip_mlp_up", 1, 2056, 1024, 4096),
+    ("clip_mlp_down", 1, 2056, 4096, 1024),
+    ("llama_qkv", 1, 2048, 4096, 12288),
+    ("llama_o", 1, 2048, 4096, 4096),
+    ("llama_gate", 1, 2048, 4096, 11008),
+    ("llama_down", 1, 2048, 11008, 4096),
+]
+
+
+@pytest.mark.parametrize("case", FULL, ids=[c[0] for c in FULL])
+def test_full_size_gemm_against_fp32_gemm_and_slow_kernel(case):
+    """At BASELINE sizes: max relative error <= 1e-2 against an fp32 GEMM of the same fp16
+    inputs (torch, on the device, as the independent fp32 reference), and agreement with the
+    step-for-step slow kernel on a band of rows."""
+    _, B, M, K, N = case
+    gen = torch.Generator(device="cuda").manual_seed(42)
+    a = torch.randn(M, K, generator=gen, device="cuda").half()
+    w = (torch.randn(N, K, generator=gen, device="cuda") * K ** -0.5).half()
+    out = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+    so, sl, sr = nt_strides(M, K, N)
+    assert raw_matmul("adr_matmul_f16", out, a, w, 1, M, K, N, so, sl, sr) == 0
+    ref32 = a.float() @ w.float().t()
+    rms = ref32.pow(2).mean().sqrt()
+    rel = ((out.float() - ref32).abs() / torch.maximum(ref32.abs(), rms)).max().item()
+    assert rel <= TOL, rel
+    rows = 64
+    slow = torch.zeros(rows, N, dtype=torch.float16, device="cuda")
+    assert raw_matmul("adr_matmul_f16_slow", slow, a[M - rows:], w, 1, rows, K, N, so, sl, sr) == 0
+    rel = ((out[M - rows:].float() - slow.float()).abs() /
+           torch.maximum(slow.float().abs(), rms)).max().item()
+    assert rel <= TOL, rel
+
+
+def test_full_size_attention_products():
+    """BASELINE config 4: 32 heads, head_dim 128, seq 2048.  QK^T scaled by 1/sqrt(128) with the
+    causal mask; P.V with softmaxed scores.  Checked per head against an fp32 batched GEMM."""
+    S, H, D = 2048, 32, 128
+    HD = H * D
+    gen = torch.Generator(device="cuda").manual_seed(43)
+    q, k, v = (torch.randn(S, HD, generator=gen, device="cuda").half() for _ in range(3))
+    qk = torch.zeros(H, S, S, dtype=torch.float16, device="cuda")
+    so, sl, sr = (1, S, S * S), (1, HD, D), (HD, 1, D)
+    scale = 1.0 / np.sqrt(D)
+    assert raw_matmul("adr_matmul_f16", qk, q, k, H, S, D, S, so, sl, sr,
+                      store=oracle.STORE_SCALE, scale=scale, mask=oracle.MASK_CAUSAL) == 0
+    q3, k3, v3 = (t.view(S, H, D).permute(1, 0, 2).float() for t in (q, k, v))
+    s16 = float(np.float16(np.float32(scale)))
+    ref = torch.bmm(q3, k3.transpose(1, 2)) * s16
+    tri = torch.ones(S, S, dtype=torch.bool, device="cuda").triu(1)
+    assert torch.all(qk[:, tri].view(torch.int16) == -1024)  # 0xFC00
+    keep = ~tri
+    rms = ref[:, keep].pow(2).mean().sqrt()
+    rel = ((qk.float() - ref).abs() / torch.maximum(ref.abs(), rms))[:, keep].max().item()
+    assert rel <= TOL, rel
+    p = torch.softmax(torch.where(tri, float("-inf"), qk.float()), dim=-1).half()
+    o = torch.zeros(S, HD, dtype=torch.float16, device="cuda")
+    so, sl, sr = (1, HD, D), (1, S, S * S), (1, HD, D)
+    assert raw_matmul("adr_matmul_f16", o, p, v, H, S, S, D, so, sl, sr) == 0
+    ref = torch.bmm(p.float(), v3).permute(1, 0, 2).reshape(S, HD)
+    rms = ref.pow(2).mean().sqrt()
+    rel = ((o.float() - ref).abs() / torch.maximum(ref.abs(), rms)).max().item()
+    assert rel <= TOL, rel

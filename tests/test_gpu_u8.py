@@ -1,0 +1,251 @@
+"""GPU parity of the u8 absmax format kernels and the u8-weight GEMV / GEMM (through the C ABI).
+
+Bars: the dequantised weight values are bit-exact against the oracle for EVERY (q, scale)
+pair, both in the stand-alone dequantise kernel and inside the fused matmul kernels (extracted
+with one-hot activations); quantise is bit-exact; matmul outputs are bit-exact where the sums
+are exactly representable and within max relative error 1e-2 of an fp32/fp64 GEMM otherwise.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import rng, randn_f16, ulp_diff_f16, max_rel_err
+from gpu_common import to_dev, to_np, nan_canon
+from adrastea_amd import GpuKernels, _ffi
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+@pytest.fixture(scope="module")
+def kern():
+    return GpuKernels()
+
+
+@pytest.fixture(scope="module")
+def ref():
+    import refgpu
+    if not refgpu.available():
+        pytest.skip("oracle/_ref code objects not built")
+    return refgpu.RefKernels()
+
+
+def u8_plan(m, p, n, bs):
+    import ctypes as C
+    buf = C.create_string_buffer(64)
+    assert _ffi.lib().adr_matmul_nt_fp16u8_plan(buf, 64, m, p, n, bs) == 0
+    return buf.value.decode()
+
+
+def test_dequantize_every_q_and_scale_bit_pattern(kern):
+    """rows = all 65536 fp16 scale patterns, cols = all 256 quantised values."""
+    q = np.tile(np.arange(256, dtype=np.uint8), (65536, 1))
+    s = np.arange(65536, dtype=np.uint16).view(np.float16).reshape(65536, 1)
+    out = torch.zeros(65536, 256, dtype=torch.float16, device="cuda")
+    kern.dequantize_absmax_uint8(out, to_dev(s), to_dev(q))
+    got = nan_canon(to_np(out).view(np.uint16))
+    want = nan_canon(oracle.dequant_table().T.copy())
+    assert np.array_equal(got, want)
+
+
+def test_dequantize_matches_reference_kernel(kern, ref):
+    g = rng(600)
+    rows, cols, bs = 64, 512, 32
+    q = g.integers(0, 256, size=(rows, cols), dtype=np.uint16).astype(np.uint8)
+    s = g.integers(0, 0x7C00, size=(rows, cols // bs), dtype=np.uint32).astype(np.uint16).view(np.float16)
+    q_t, s_t = to_dev(q), to_dev(s)
+    o_ref = torch.zeros(rows, cols, dtype=torch.float16, device="cuda")
+    ref.dequantize(o_ref, s_t, q_t)
+    torch.cuda.synchronize()
+    out = torch.zeros(rows, cols, dtype=torch.float16, device="cuda")
+    kern.dequantize_absmax_uint8(out, s_t, q_t)
+    assert np.array_equal(to_np(out).view(np.uint16), to_np(o_ref).view(np.uint16))
+    assert np.array_equal(to_np(o_ref).view(np.uint16),
+                          oracle.dequantize_absmax_u8(q, s, bs).view(np.uint16))
+
+
+def test_quantize_matches_oracle_and_reference_kernel(kern, ref):
+    g = rng(601)
+    rows, cols, bs = 48, 384, 32
+    x = randn_f16(g, (rows, cols), 0.05)
+    x[0, :32] = 0.25           # all-equal block
+    x[1, :32] = 0
+    x[1, 7] = -3.0             # single negative spike
+    x[2, :64] = np.float16(6.1e-5)  # smallest normal: subnormal scale
+    q_want, s_want = oracle.quantize_absmax_u8(x, bs)
+    x_t = to_dev(x)
+    q_t = torch.zeros(rows, cols, dtype=torch.uint8, device="cuda")
+    s_t = torch.zeros(rows, cols // bs, dtype=torch.float16, device="cuda")
+    kern.quantize_absmax_uint8(q_t, s_t, x_t)
+    assert np.array_equal(to_np(s_t).view(np.uint16), s_want.view(np.uint16))
+    assert np.array_equal(to_np(q_t), q_want)
+    q_r = torch.zeros_like(q_t)
+    s_r = torch.zeros_like(s_t)
+    ref.quantize(q_r, s_r, x_t)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_np(s_r).view(np.uint16), s_want.view(np.uint16))
+    assert np.array_equal(to_np(q_r), q_want)
+
+
+def _finite_scale_rows():
+    # scale patterns whose 256 dequantised values are all finite (|s| <= 512): an infinite
+    # weight times a zero activation would poison the row's sums.  Larger scales, inf and NaN
+    # are covered by the stand-alone dequantise test above.
+    s = np.arange(65536, dtype=np.uint16)
+    return s[(s & 0x7FFF) <= 0x6000]
+
+
+@pytest.mark.parametrize("m", [1, 4, 16])
+def test_fused_dequant_in_gemv_is_bit_exact_for_every_q_and_finite_scale(kern, m):
+    """One-hot activations pick single weights out of the matmul: out[r, c] = w[c, k_r]."""
+    scales_bits = _finite_scale_rows()
+    n, p, bs = scales_bits.size, 256, 32
+    assert u8_plan(m, p, n, bs) == "gemv_u8_mfma16_stream"
+    q = np.tile(np.arange(256, dtype=np.uint8), (n, 1))
+    s = np.repeat(scales_bits.view(np.float16).reshape(n, 1), p // bs, axis=1)
+    table = oracle.dequant_table()  # [q][scale bits]
+    q_t, s_t = to_dev(q), to_dev(s)
+    for base in range(0, 256, m):
+        ks = np.arange(base, base + m)
+        lhs = np.zeros((m, p), np.float16)
+        lhs[np.arange(m), ks] = 1.0
+        out = torch.zeros(m, n, dtype=torch.float16, device="cuda")
+        kern.matmul_nt_fp16u8(out, to_dev(lhs), q_t, s_t, bs)
+        got = to_np(out).view(np.uint16)
+        want = table[ks][:, scales_bits]
+        # -0.0 + 0.0 products: a dequantised -0 sums to +0; compare values for zeros
+        z = (want & 0x7FFF) == 0
+        assert np.array_equal(got[~z], want[~z]), base
+        assert np.all((got[z] & 0x7FFF) == 0)
+
+
+def test_fused_dequant_in_u8_gemm_is_bit_exact_for_every_q_and_finite_scale(kern):
+    scales_bits = _finite_scale_rows()
+    n, p, bs, m = scales_bits.size, 256, 32, 256
+    assert u8_plan(m, p, n, bs) == "gemm_nt_u8_mfma"
+    q = np.tile(np.arange(256, dtype=np.uint8), (n, 1))
+    s = np.repeat(scales_bits.view(np.float16).reshape(n, 1), p // bs, axis=1)
+    lhs = np.eye(m, dtype=np.float16)
+    out = torch.zeros(m, n, dtype=torch.float16, device="cuda")
+    kern.matmul_nt_fp16u8(out, to_dev(lhs), to_dev(q), to_dev(s), bs)
+    got = to_np(out).view(np.uint16)
+    want = oracle.dequant_table()[:, scales_bits]
+    z = (want & 0x7FFF) == 0
+    assert np.array_equal(got[~z], want[~z])
+    assert np.all((got[z] & 0x7FFF) == 0)
+
+
+def _u8_case(g, m, p, n, bs, exact):
+    q = g.integers(0, 256, size=(n, p), dtype=np.uint16).astype(np.uint8)
+    if exact:
+        # power-of-two scales and small dyadic activations: every product and sum is exact
+        s = np.exp2(g.integers(-8, -4, size=(n, p // bs))).astype(np.float16)
+        a = (g.integers(-8, 9, size=(m, p)) / 8.0).astype(np.float16)
+    else:
+        s = g.uniform(0.001, 0.02, size=(n, p // bs)).astype(np.float16)
+        a = randn_f16(g, (m, p))
+    return a, q, s
+
+
+@pytest.mark.parametrize("m", [1, 2, 4, 7, 16])
+@pytest.mark.parametrize("pn", [(256, 16), (512, 100), (1024, 33), (2816, 48)])
+def test_gemv_bit_exact_on_exact_inputs(kern, m, pn):
+    p, n = pn
+    g = rng(610 + m + n)
+    a, q, s = _u8_case(g, m, p, n, 32, exact=True)
+    prev = (g.integers(-8, 9, size=(m, n)) / 4.0).astype(np.float16)
+    for beta in (0.0, 0.5):
+        want = prev.copy()
+        oracle.matmul_nt_fp16u8(want, a, q, s, 32, beta=beta)
+        out = to_dev(prev)
+        kern.matmul_nt_fp16u8(out, to_dev(a), to_dev(q), to_dev(s), 32, beta=beta)
+        assert np.array_equal(to_np(out).view(np.uint16), want.view(np.uint16)), (m, p, n, beta)
+
+
+@pytest.mark.parametrize("m", [1, 4, 16, 17, 100, 300])
+def test_u8_matmul_random_matches_oracle_and_reference_kernel(kern, ref, m):
+    g = rng(620 + m)
+    p, n, bs = 512, 200, 32
+    a, q, s = _u8_case(g, m, p, n, bs, exact=False)
+    want = np.zeros((m, n), np.float16)
+    oracle.matmul_nt_fp16u8(want, a, q, s, bs, threads=8)
+    out = torch.zeros(m, n, dtype=torch.float16, device="cuda")
+    a_t, q_t, s_t = to_dev(a), to_dev(q), to_dev(s)
+    kern.matmul_nt_fp16u8(out, a_t, q_t, s_t, bs)
+    got = to_np(out)
+    w = oracle.dequantize_absmax_u8(q, s, bs).astype(np.float64)
+    ref64 = a.astype(np.float64) @ w.T
+    assert max_rel_err(got, ref64) <= 2e-3
+    assert np.max(ulp_diff_f16(got, want)) <= 1 or max_rel_err(got, want.astype(np.float64)) <= 2e-3
+    # the reference's naive u8 kernel (double-precision product, unrounded weights)
+    o_ref = torch.zeros(m, n, dtype=torch.float16, device="cuda")
+    ref.matmul_nt_fp16u8(o_ref, a_t, q_t, s_t, bs)
+    torch.cuda.synchronize()
+    assert max_rel_err(got, to_np(o_ref).astype(np.float64)) <= TOL
+    naive = np.zeros((m, n), np.float16)
+    oracle.matmul_nt_fp16u8(naive, a, q, s, bs, naive=True, threads=8)
+    assert np.max(ulp_diff_f16(naive, to_np(o_ref))) <= 1
+
+
+def test_u8_other_block_sizes_and_fallbacks(kern):
+    g = rng(630)
+    for m, p, n, bs in [(4, 512, 40, 64), (4, 384, 40, 128), (3, 96, 20, 8), (2, 48, 10, 16),
+                        (40, 320, 70, 64)]:
+        a, q, s = _u8_case(g, m, p, n, bs, exact=True)
+        want = np.zeros((m, n), np.float16)
+        oracle.matmul_nt_fp16u8(want, a, q, s, bs)
+        out = torch.zeros(m, n, dtype=torch.float16, device="cuda")
+        kern.matmul_nt_fp16u8(out, to_dev(a), to_dev(q), to_dev(s), bs)
+        assert np.array_equal(to_np(out).view(np.uint16), want.view(np.uint16)), (m, p, n, bs)
+    lib = _ffi.lib()
+    z = torch.zeros(64, dtype=torch.float16, device="cuda")
+    assert lib.adr_matmul_nt_fp16u8(None, z.data_ptr(), z.data_ptr(), z.data_ptr(), z.data_ptr(),
+                                    1, 40, 1, 32, 0.0) == -5   # p % block_size
+    assert lib.adr_matmul_nt_fp16u8(None, None, z.data_ptr(), z.data_ptr(), z.data_ptr(),
+                                    1, 32, 1, 32, 0.0) == -4
+
+
+DECODE = [(4096, 4096), (4096, 11008), (4096, 12288), (11008, 4096)]
+
+
+@pytest.mark.parametrize("kn", DECODE, ids=[f"K{k}_N{n}" for k, n in DECODE])
+@pytest.mark.parametrize("m", [1, 4, 16])
+def test_decode_shapes_full_size(kern, kn, m):
+    """BASELINE config 3 at full size against an fp32 GEMM on the (bit-exactly) dequantised
+    weights, computed on the device."""
+    p, n = kn
+    gen = torch.Generator(device="cuda").manual_seed(44)
+    q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)
+    s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
+    a = torch.randn(m, p, generator=gen, device="cuda").half()
+    assert u8_plan(m, p, n, 32) == "gemv_u8_mfma16_stream"
+    out = torch.zeros(m, n, dtype=torch.float16, device="cuda")
+    kern.matmul_nt_fp16u8(out, a, q, s, 32)
+    w = torch.zeros(n, p, dtype=torch.float16, device="cuda")
+    kern.dequantize_absmax_uint8(w, s, q)
+    ref32 = a.float() @ w.float().t()
+    rms = ref32.pow(2).mean().sqrt()
+    rel = ((out.float() - ref32).abs() / torch.maximum(ref32.abs(), rms)).max().item()
+    assert rel <= 2e-3, rel
+    # linearity in the activations: f(2a) == 2 f(a) exactly (powers of two commute with rounding)
+    out2 = torch.zeros_like(out)
+    kern.matmul_nt_fp16u8(out2, (a * 2).half(), q, s, 32)
+    assert torch.equal(out2, (out * 2).half())
+
+
+def test_prefill_u8_gemm_full_size(kern):
+    """BASELINE config 5 (u8 variant), the O projection: M=2048, K=4096, N=4096."""
+    m, p, n = 2048, 4096, 4096
+    gen = torch.Generator(device="cuda").manual_seed(45)
+    q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)
+    s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
+    a = torch.randn(m, p, generator=gen, device="cuda").half()
+    out = torch.zeros(m, n, dtype=torch.float16, device="cuda")
+    kern.matmul_nt_fp16u8(out, a, q, s, 32)
+    w = torch.zeros(n, p, dtype=torch.float16, device="cuda")
+    kern.dequantize_absmax_uint8(w, s, q)
+    ref32 = a.float() @ w.float().t()
+    rms = ref32.pow(2).mean().sqrt()
+    rel = ((out.float() - ref32).abs() / torch.maximum(ref32.abs(), rms)).max().item()
+    assert rel <= 2e-3, rel
