@@ -1,0 +1,280 @@
+#!/usr/bin/env python3
+"""Benchmark of the matmul hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
+
+A "step" is one pass over the LLaMA-7B per-layer GEMM set at prefill M=2048 in fp16
+(QKV 4096->12288, O 4096->4096, gate and up 4096->11008, down 11008->4096; 828.9 GFLOP),
+every launch going through the C ABI (adr_matmul_f16) with operands resident in HBM.
+Prints ONE JSON line.  `value` is the fp16 TFLOP/s of that step; `roofline` is the dominant
+kernel (the MFMA GEMM on the QKV shape) timed with HIP events on the launch stream;
+`cpu_baseline` is the CPU oracle (a scalar restatement of the reference kernel, OpenMP over
+rows) on a bounded sample of the same workload, timed on this machine's host cores;
+`secondary` carries the other BASELINE configurations: the u8 decode GEMV in GB/s against
+the HBM peak, the u8 prefill GEMMs, the CLIP GEMMs and the attention products.
+
+Input data is synthetic (seeded): activations ~ N(0,1), weights ~ N(0,1/sqrt(K)) in fp16;
+u8 weights uniform with fp16 scales ~ U(0.001, 0.02) per 32 weights.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_F16_TFLOPS = 2516.6   # 256 CU x 4 SIMD x 1024 flop/clk x 2.4 GHz (dense, no sparsity)
+PEAK_HBM_GBS = 8000.0      # HBM3E
+METRIC = "fp16 GEMM TFLOP/s (% MFMA peak); u8 GEMV GB/s (% HBM peak), LLaMA-7B"
+
+LAYER_SET = [  # (name, K, N) at M = 2048
+    ("qkv", 4096, 12288), ("o", 4096, 4096), ("gate", 4096, 11008), ("up", 4096, 11008),
+    ("down", 11008, 4096),
+]
+DECODE_SET = [(4096, 4096), (4096, 11008), (4096, 12288), (11008, 4096)]
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--quick", action="store_true", help="skip secondary configs and CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures the single-GPU matmul path only; run with --gpus 1 "
+              "(how the path would shard over several GPUs is described in DESIGN.md)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from adrastea_amd import _ffi
+    lib = _ffi.lib()  # raises if the HIP library is not built: there is no fallback
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    gen = torch.Generator(device=dev).manual_seed(42)
+    stream = lambda: torch.cuda.current_stream().cuda_stream  # noqa: E731
+
+    def randn_h(*shape, std=1.0):
+        return (torch.randn(*shape, generator=gen, device=dev) * std).half()
+
+    def mm(out, a, w, M, K, N):
+        rc = lib.adr_matmul_f16(stream(), out.data_ptr(), a.data_ptr(), w.data_ptr(), 1, M, K, N,
+                                1, N, 0, 1, K, 0, K, 1, 0, None, 0.0, 1.0, 0, 0, 0)
+        if rc != 0:
+            raise RuntimeError(f"adr_matmul_f16 failed: {_ffi.strerror(rc)}")
+
+    def timed(fn, iters, warm):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / iters  # seconds per call
+
+    # ---------------- primary workload: the fp16 layer GEMM set at M = 2048
+    M = 2048
+    acts = {4096: randn_h(M, 4096), 11008: randn_h(M, 11008)}
+    weights, outs = {}, {}
+    for name, K, N in LAYER_SET:
+        weights[name] = randn_h(N, K, std=K ** -0.5)
+        outs[name] = torch.zeros(M, N, dtype=torch.float16, device=dev)
+
+    def step():
+        for name, K, N in LAYER_SET:
+            mm(outs[name], acts[K], weights[name], M, K, N)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    step_flops = sum(2.0 * M * K * N for _, K, N in LAYER_SET)
+    ms_per_step = elapsed / args.steps * 1e3
+    value = step_flops / (elapsed / args.steps) / 1e12
+
+    # ---------------- roofline of the dominant kernel (HIP events on the launch stream)
+    name, K, N = LAYER_SET[0]
+    t_qkv = timed(lambda: mm(outs[name], acts[K], weights[name], M, K, N), 30, 3)
+    qkv_flops = 2.0 * M * K * N
+    roofline = {
+        "kernel": "gemm_nt_mfma_256x128x32 (qkv: M2048 K4096 N12288)",
+        "bound": "mfma", "achieved": round(qkv_flops / t_qkv / 1e12, 2),
+        "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
+        "frac": round(qkv_flops / t_qkv / 1e12 / PEAK_F16_TFLOPS, 4),
+        "launch_us": round(t_qkv * 1e6, 2), "traffic": None,
+    }
+
+    secondary = {}
+    if not args.quick:
+        per_gemm = {}
+        for name, K, N in LAYER_SET:
+            if name == "up":
+                continue
+            t = timed(lambda: mm(outs[name], acts[K], weights[name], M, K, N), 20, 2)
+            per_gemm[name] = {"M": M, "K": K, "N": N, "us": round(t * 1e6, 1),
+                              "tflops": round(2.0 * M * K * N / t / 1e12, 1),
+                              "frac_mfma_peak": round(2.0 * M * K * N / t / 1e12 / PEAK_F16_TFLOPS, 4)}
+        secondary["llama7b_prefill_fp16"] = per_gemm
+
+        # ---- u8 decode GEMV (BASELINE configs[2]): weight buffers rotate through > 256 MB so
+        # that repeats stream from HBM, not from the Infinity Cache
+        def u8_case(m, K, N, iters):
+            per = N * K + N * (K // 32) * 2
+            nbuf = max(2, int(600e6 // per) + 1)
+            qs = [torch.randint(0, 256, (N, K), generator=gen, device=dev, dtype=torch.uint8)
+                  for _ in range(nbuf)]
+            ss = [(torch.rand(N, K // 32, generator=gen, device=dev) * 0.019 + 0.001).half()
+                  for _ in range(nbuf)]
+            a = randn_h(m, K)
+            o = torch.zeros(m, N, dtype=torch.float16, device=dev)
+            i = [0]
+
+            def f():
+                j = i[0] % nbuf
+                i[0] += 1
+                rc = lib.adr_matmul_nt_fp16u8(stream(), o.data_ptr(), a.data_ptr(),
+                                              qs[j].data_ptr(), ss[j].data_ptr(), m, K, N, 32, 0.0)
+                if rc != 0:
+                    raise RuntimeError(_ffi.strerror(rc))
+            t = timed(f, iters, nbuf)
+            return t, per + m * K * 2 + m * N * 2
+
+        gemv = []
+        for K, N in DECODE_SET:
+            for m in (1, 4, 16):
+                t, byts = u8_case(m, K, N, 200)
+                gemv.append({"M": m, "K": K, "N": N, "us": round(t * 1e6, 2),
+                             "gbs": round(byts / t / 1e9, 1),
+                             "frac_hbm_peak": round(byts / t / 1e9 / PEAK_HBM_GBS, 4)})
+        secondary["u8_decode_gemv"] = gemv
+        best = max(gemv, key=lambda r: r["gbs"])
+        secondary["u8_decode_gemv_best"] = {"gbs": best["gbs"], "frac_hbm_peak": best["frac_hbm_peak"],
+                                            "shape": [best["M"], best["K"], best["N"]]}
+
+        # ---- u8 prefill GEMMs (configs[4], u8 half)
+        u8p = {}
+        for name, K, N in LAYER_SET:
+            if name == "up":
+                continue
+            q = torch.randint(0, 256, (N, K), generator=gen, device=dev, dtype=torch.uint8)
+            s = (torch.rand(N, K // 32, generator=gen, device=dev) * 0.019 + 0.001).half()
+
+            def f():
+                rc = lib.adr_matmul_nt_fp16u8(stream(), outs[name].data_ptr(), acts[K].data_ptr(),
+                                              q.data_ptr(), s.data_ptr(), M, K, N, 32, 0.0)
+                if rc != 0:
+                    raise RuntimeError(_ffi.strerror(rc))
+            t = timed(f, 10, 2)
+            u8p[name] = {"M": M, "K": K, "N": N, "us": round(t * 1e6, 1),
+                         "tflops": round(2.0 * M * K * N / t / 1e12, 1),
+                         "frac_mfma_peak": round(2.0 * M * K * N / t / 1e12 / PEAK_F16_TFLOPS, 4)}
+            del q, s
+        secondary["llama7b_prefill_u8"] = u8p
+
+        # ---- CLIP GEMMs (configs[0], configs[1])
+        clip = {}
+        for nm, m, K, N in (("text_qkv_M77", 77, 768, 2304), ("vision_mlp_up", 2056, 1024, 4096),
+                            ("vision_mlp_down", 2056, 4096, 1024)):
+            a, w = randn_h(m, K), randn_h(N, K, std=K ** -0.5)
+            o = torch.zeros(m, N, dtype=torch.float16, device=dev)
+            t = timed(lambda: mm(o, a, w, m, K, N), 50, 5)
+            byts = (m * K + N * K + m * N) * 2
+            clip[nm] = {"M": m, "K": K, "N": N, "us": round(t * 1e6, 2),
+                        "tflops": round(2.0 * m * K * N / t / 1e12, 1),
+                        "frac_mfma_peak": round(2.0 * m * K * N / t / 1e12 / PEAK_F16_TFLOPS, 4),
+                        "gbs": round(byts / t / 1e9, 1)}
+        secondary["clip_fp16"] = clip
+
+        # ---- attention products (configs[3]): HBM-bound by the [32, 2048, 2048] fp16 tensor
+        S, H, D = 2048, 32, 128
+        HD = H * D
+        q_, k_, v_ = randn_h(S, HD), randn_h(S, HD), randn_h(S, HD)
+        qk = torch.zeros(H, S, S, dtype=torch.float16, device=dev)
+
+        def f_qk():
+            rc = lib.adr_matmul_f16(stream(), qk.data_ptr(), q_.data_ptr(), k_.data_ptr(), H, S, D,
+                                    S, 1, S, S * S, 1, HD, D, HD, 1, D, None, 0.0,
+                                    1.0 / D ** 0.5, 4, 0, 0)
+            if rc != 0:
+                raise RuntimeError(_ffi.strerror(rc))
+        t = timed(f_qk, 10, 2)
+        byts = 2 * S * HD * 2 + H * S * S * 2
+        attn = {"qk_t": {"us": round(t * 1e6, 1), "tflops": round(2.0 * H * S * S * D / t / 1e12, 1),
+                         "gbs": round(byts / t / 1e9, 1),
+                         "frac_hbm_peak": round(byts / t / 1e9 / PEAK_HBM_GBS, 4)}}
+        p_ = torch.softmax(qk.float(), dim=-1).half()
+        o_ = torch.zeros(S, HD, dtype=torch.float16, device=dev)
+
+        def f_pv():
+            rc = lib.adr_matmul_f16(stream(), o_.data_ptr(), p_.data_ptr(), v_.data_ptr(), H, S, S,
+                                    D, 1, HD, D, 1, S, S * S, 1, HD, D, None, 0.0, 1.0, 0, 0, 0)
+            if rc != 0:
+                raise RuntimeError(_ffi.strerror(rc))
+        t = timed(f_pv, 5, 1)
+        attn["pv"] = {"us": round(t * 1e6, 1), "tflops": round(2.0 * H * S * S * D / t / 1e12, 1),
+                      "gbs": round(byts / t / 1e9, 1),
+                      "frac_hbm_peak": round(byts / t / 1e9 / PEAK_HBM_GBS, 4)}
+        secondary["llama7b_attention_fp16"] = attn
+
+    # ---------------- CPU baseline: the oracle on a bounded sample of the same workload
+    cpu_baseline = None
+    if not args.quick:
+        import numpy as np
+        import oracle  # checker / baseline only; never on the product path
+        cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+        rows = 128
+        name, K, N = LAYER_SET[0]
+        a_np = acts[K][:rows].cpu().numpy()
+        w_np = weights[name].cpu().numpy()
+        o_np = np.zeros(rows * N, np.float16)
+        t0 = time.perf_counter()
+        oracle.matmul_f16(o_np, a_np, w_np, 1, rows, K, N, (1, N, 0), (1, K, 0), (K, 1, 0),
+                          mode=oracle.FAITHFUL, threads=cores)
+        dt = time.perf_counter() - t0
+        cpu_baseline = {
+            "value": round(2.0 * rows * K * N / dt / 1e12, 6), "unit": "TFLOP/s", "cores": cores,
+            "kind": "port",
+            "sample": f"first {rows} of 2048 activation rows of the qkv GEMM (K4096 N12288), "
+                      f"{2.0 * rows * K * N / 1e9:.1f} GFLOP in {dt:.1f} s, reference-faithful "
+                      "scalar arithmetic (fp16 products, fp32 sum)",
+        }
+        # parity spot check of the sample against a fresh device result
+        mm(outs[name], acts[K], weights[name], M, K, N)
+        torch.cuda.synchronize()
+        got = outs[name][:rows].cpu().numpy().astype(np.float64)
+        ref = o_np.reshape(rows, N).astype(np.float64)
+        rms = np.sqrt(np.mean(ref ** 2))
+        cpu_baseline["max_rel_err_gpu_vs_cpu"] = float(
+            np.max(np.abs(got - ref) / np.maximum(np.abs(ref), rms)))
+
+    line = {
+        "metric": METRIC, "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": "llama7b_layer_gemm_set_fp16_prefill_M2048 (BASELINE configs[4], "
+                               "fp16 weights: qkv, o, gate, up, down)",
+                   "gflop_per_step": round(step_flops / 1e9, 1),
+                   "frac_mfma_peak": round(value / PEAK_F16_TFLOPS, 4)},
+        "roofline": roofline, "cpu_baseline": cpu_baseline, "secondary": secondary,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

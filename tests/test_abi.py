@@ -1,0 +1,80 @@
+"""CPU-only checks of the boundary: the built library loads, exports every declared symbol,
+validates arguments on the host, and selects kernels as documented.  No device call is made."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from adrastea_amd import _ffi, TensorLayout, MatmulOptions, MatmulStore, MatmulLoad, MatmulMask
+from adrastea_amd import kernels as K
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_header_symbols_are_all_exported():
+    text = open(os.path.join(ROOT, "include", "adrastea_kernels.h")).read()
+    declared = set(re.findall(r"\b(adr_[a-z0-9_]+)\s*\(", text))
+    assert declared == set(_ffi.SYMBOLS)
+    lib = _ffi.lib()
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert lib.adr_abi_version() >= 1
+
+
+def test_strerror_covers_codes():
+    for code in range(-6, 1):
+        assert _ffi.strerror(code)
+    assert "GeluBias" in _ffi.strerror(-3)
+
+
+def _plan(B, M, Kd, N, so, sl, sr, store=0, load=0, mask=0):
+    buf = C.create_string_buffer(64)
+    rc = _ffi.lib().adr_matmul_f16_plan(buf, 64, B, M, Kd, N, *so, *sl, *sr, store, load, mask)
+    return rc, buf.value.decode()
+
+
+def test_plan_validation_codes():
+    nt = ((1, 64, 0), (1, 64, 0), (64, 1, 0))
+    assert _plan(1, 64, 64, 64, *nt)[0] == 0
+    assert _plan(1, 64, 64, 64, *nt, store=1)[0] == _ffi.ADR_ENOTIMPL
+    assert _plan(1, 64, 64, 64, *nt, store=7)[0] == _ffi.ADR_EINVAL_ENUM
+    assert _plan(1, 64, 64, 64, *nt, load=2)[0] == _ffi.ADR_EINVAL_ENUM
+    assert _plan(1, 64, 64, 64, *nt, mask=2)[0] == _ffi.ADR_EINVAL_ENUM
+    assert _plan(1, -1, 64, 64, *nt)[0] == _ffi.ADR_EINVAL_SHAPE
+    assert _plan(0, 64, 64, 64, *nt) == (0, "none (empty)")
+
+
+def test_kernel_selection_for_the_callers_layouts():
+    # linear layers: W[N,K].permute([1,0]) (llama.rs:503-508)
+    M, Kd, N = 2048, 4096, 12288
+    out, lhs = TensorLayout.row_major([M, N]), TensorLayout.row_major([M, Kd])
+    w = TensorLayout.row_major([N, Kd]).permute([1, 0])
+    assert K.plan_matmul(out, lhs, w) == "gemm_nt_mfma_256x128x32"
+    # QK^T on the head views (llama.rs:534-550)
+    S, H, D = 2048, 32, 128
+    q = TensorLayout.row_major([S, H * D]).shape_cast([S, H, -1]).permute([1, 0, 2])
+    k = TensorLayout.row_major([S, H * D]).shape_cast([S, H, -1]).permute([1, 2, 0])
+    qk = TensorLayout.row_major([H, S, S])
+    opts = MatmulOptions.new().store(MatmulStore.Scale(1.0 / D ** 0.5)).mask(MatmulMask.CAUSAL)
+    assert K.plan_matmul(qk, q, k, opts).startswith("gemm_nt_mfma")
+    # a row-major right operand with K % 8 != 0 falls back to the general kernel
+    assert K.plan_matmul(TensorLayout.row_major([10, 12]), TensorLayout.row_major([10, 7]),
+                         TensorLayout.row_major([7, 12])) == "matmul_general"
+    # small CLIP text GEMM
+    assert K.plan_matmul(TensorLayout.row_major([77, 2304]), TensorLayout.row_major([77, 768]),
+                         TensorLayout.row_major([2304, 768]).permute([1, 0])).startswith("gemm_nt_mfma")
+
+
+def test_u8_plan():
+    def plan(m, p, n, bs):
+        buf = C.create_string_buffer(64)
+        rc = _ffi.lib().adr_matmul_nt_fp16u8_plan(buf, 64, m, p, n, bs)
+        return rc, buf.value.decode()
+    for m in (1, 4, 16):
+        assert plan(m, 4096, 4096, 32) == (0, "gemv_u8_mfma16_stream")
+        assert plan(m, 11008, 4096, 32) == (0, "gemv_u8_mfma16_stream")
+    assert plan(2048, 4096, 4096, 32) == (0, "gemm_nt_u8_mfma")
+    assert plan(4, 4096, 4096, 64)[1] == "gemm_nt_u8_mfma"
+    assert plan(4, 4100, 64, 32)[0] == _ffi.ADR_EDIVISIBILITY
+    assert plan(4, 64, 64, 0)[0] == _ffi.ADR_EINVAL_SHAPE
