@@ -62,9 +62,8 @@ struct Epilogue {
            store == ADR_STORE_QUICK_GELU_BIAS;
   }
 
-  __device__ __forceinline__ half_t apply(float acc, half_t prev, half_t bias_x) const {
-    if (store == STORE_ACC_BETA) return (half_t)(acc + beta * (float)prev);
-    half_t s16 = (half_t)acc;
+  // Operators on the already narrowed accumulator (everything but STORE_ACC_BETA).
+  __device__ __forceinline__ half_t apply_s16(half_t s16, half_t prev, half_t bias_x) const {
     switch (store) {
       default:
       case ADR_STORE_IDENTITY:
@@ -87,6 +86,11 @@ struct Epilogue {
         return (half_t)(g + beta * (float)prev);
       }
     }
+  }
+
+  __device__ __forceinline__ half_t apply(float acc, half_t prev, half_t bias_x) const {
+    if (store == STORE_ACC_BETA) return (half_t)(acc + beta * (float)prev);
+    return apply_s16((half_t)acc, prev, bias_x);
   }
 };
 

@@ -5,12 +5,28 @@
 // and the attention score product Q.K^T on the interleaved-head views of llama.rs:534-550.
 // Row strides (stride_ly, stride_rx, stride_oy) and batch strides are free.
 //
-// Structure: one workgroup per BM x BN output tile, WM x WN wavefronts, each owning a
-// (BM/WM) x (BN/WN) sub-tile as 32x32 fp32 accumulators of v_mfma_f32_32x32x16_f16.  A and B
-// K-slices of depth BK are staged global -> registers -> LDS with 128-bit accesses, double
-// buffered in LDS so that the global loads of slice t+1 are in flight while slice t feeds the
-// MFMAs; one barrier per slice.  LDS rows are XOR-swizzled at 16-byte granularity so that the
-// 128-bit fragment reads of 8 consecutive rows hit 8 different bank groups.
+// Two kernels share the tiling, the LDS layout and the epilogue:
+//
+//  gemm_nt_dma_kernel   K % 64 == 0, plain fp16 operands.  K slices of depth 64 go from global
+//                       memory straight into LDS (global_load_lds_dwordx4, no register round
+//                       trip) into 2 or 3 statically separate LDS stages, so the loads of the
+//                       next one or two slices are in flight while the current slice feeds the
+//                       MFMAs; one barrier per slice.  MFMA fragments are prefetched one k-step
+//                       ahead and interleaved with the MFMAs by scheduling-group barriers.
+//  gemm_nt_stage_kernel any K % 8 == 0, and the variants that must touch the data on the way
+//                       in: u8 weights dequantised while staging (adr_matmul_nt_fp16u8), and
+//                       the Load Scale operator.  Global -> registers -> LDS, two LDS stages.
+//
+// One workgroup owns a BM x BN output tile, WM x WN wavefronts each own a (BM/WM) x (BN/WN)
+// sub-tile as 32x32 fp32 accumulators of v_mfma_f32_32x32x16_f16.  LDS rows are XOR-swizzled
+// at 16-byte granularity over 256-byte lines (64 banks) so that the 128-bit fragment reads of
+// 16 consecutive rows are conflict-free (SQ_LDS_BANK_CONFLICT reads 0).  Accumulators are kept
+// TRANSPOSED (the weight fragment is the first MFMA operand) so that a lane owns 4 consecutive
+// output columns; the epilogue narrows them to fp16, transposes through a per-wavefront LDS
+// slot and writes whole 16-byte chunks of output rows, applying the store operator, the bias
+// and the causal mask on the way.
+#include <type_traits>
+
 #include "adr_common.hpp"
 
 namespace adr {
@@ -19,78 +35,403 @@ namespace {
 
 constexpr int XCDS = 8;  // MI355X: 8 accelerator dies, workgroup i is dispatched to die i % 8
 
+#define ADR_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+#define ADR_GLB_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
+
 // Physical byte offset of 16-byte chunk `kc` of row `row` in a [rows][CPR chunks] LDS tile.
+// 16 chunks = one 256-byte line = all 64 banks; the chunk position inside a line is XORed
+// with the line number.
 template <int CPR>
 __device__ __forceinline__ int lds_chunk_off(int row, int kc) {
   int idx = row * CPR + kc;
-  int line = idx >> 3, pos = idx & 7;  // 8 chunks = one 128-byte line = all 32 banks
-  return ((line << 3) | (pos ^ (line & 7))) << 4;
+  int line = idx >> 4, pos = idx & 15;
+  return ((line << 4) | (pos ^ (line & (CPR - 1)))) << 4;
+}
+// Inverse: which (row, kc) lives at physical chunk `phys`.
+template <int CPR>
+__device__ __forceinline__ void lds_chunk_inv(int phys, int& row, int& kc) {
+  int line = phys >> 4, pos = (phys & 15) ^ (line & (CPR - 1));
+  int idx = (line << 4) | pos;
+  row = idx / CPR;
+  kc = idx % CPR;
 }
 
-// Work decomposition shared by host and device.
 struct TileMap {
   int tiles_m, tiles_n, tiles_per_batch, total;
   int group_m;  // tile rows per L2-reuse group
 };
 
-template <int BM, int BN, int BK, int WM, int WN, int MINB, bool LOAD_SCALE, bool WQ>
-__global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_kernel(MatmulArgs a, TileMap map) {
-  constexpr int NT = WM * WN * 64;
-  constexpr int CPR = BK / 8;                // 16-byte chunks per tile row
-  constexpr int LA = BM * CPR / NT;          // chunks each thread stages for A
-  constexpr int LB = BN * CPR / NT;
-  constexpr int WTM = BM / WM, WTN = BN / WN;
-  constexpr int TM = WTM / 32, TN = WTN / 32;
-  constexpr int KK = BK / 16;
-  static_assert(BM * CPR % NT == 0 && BN * CPR % NT == 0, "staging must divide evenly");
-  static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % 16 == 0, "MFMA 32x32x16 tiling");
-
-  extern __shared__ __attribute__((aligned(128))) unsigned char smem[];
-  unsigned char* const sA = smem;                         // [2][BM][BK] halves
-  unsigned char* const sB = smem + 2 * BM * BK * 2;       // [2][BN][BK] halves
-
-  // ---- which tile: XCD-aware remap, then grouped (tile-row-major inside groups of group_m)
+// blockIdx.x -> (batch, tile_m, tile_n).  Consecutive ids land on different dies, so ids are
+// first regrouped per die; inside a batch, tiles are walked column by column within groups of
+// `group_m` tile rows so that the tiles resident on one die share A and B panels in its L2.
+__device__ __forceinline__ void map_tile(const TileMap& map, int& batch, int& tile_m,
+                                         int& tile_n) {
   int id = blockIdx.x;
-  {
-    const int per = (map.total + XCDS - 1) / XCDS;
-    const int tall = map.total % XCDS == 0 ? XCDS : map.total % XCDS;
-    const int xcd = id % XCDS, local = id / XCDS;
-    id = xcd < tall ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
-  }
-  const int batch = id / map.tiles_per_batch;
+  const int per = (map.total + XCDS - 1) / XCDS;
+  const int tall = map.total % XCDS == 0 ? XCDS : map.total % XCDS;
+  const int xcd = id % XCDS, local = id / XCDS;
+  id = xcd < tall ? xcd * per + local : tall * per + (xcd - tall) * (per - 1) + local;
+  batch = id / map.tiles_per_batch;
   int t = id - batch * map.tiles_per_batch;
   const int group_span = map.group_m * map.tiles_n;
   const int g = t / group_span;
   const int gm0 = g * map.group_m;
   const int gsz = min(map.group_m, map.tiles_m - gm0);
   t -= g * group_span;
-  const int tile_m = gm0 + t % gsz;
-  const int tile_n = t / gsz;
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  tile_m = gm0 + t % gsz;
+  tile_n = t / gsz;
+}
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave / WN, wn = wave % WN;
+__device__ __forceinline__ bool out_vectorizable(const MatmulArgs& a, const half_t* out) {
+  // 16-byte row chunks need aligned rows; STORE_ACC_BETA with beta != 0 works on the fp32
+  // accumulator and therefore stays on the element-wise path
+  if ((a.stride_oy & 7) || ((uintptr_t)out & 15)) return false;
+  if (Epilogue::needs_bias(a.store) && ((uintptr_t)a.bias & 15)) return false;
+  if (a.store == STORE_ACC_BETA && a.beta != 0.0f) return false;
+  return true;
+}
 
-  half_t* const out = a.output + (int64_t)batch * a.stride_oz;
+// One 16-byte chunk (8 consecutive columns x..x+7 of output row y) through the store operator.
+__device__ __forceinline__ void store_chunk(const MatmulArgs& a, const Epilogue& ep, half_t* out,
+                                            int y, int x, half8_t v) {
+  half_t* p = out + (int64_t)y * a.stride_oy + x;
+  const bool causal = a.mask == ADR_MASK_CAUSAL;
+  if (x + 8 <= a.n) {
+    half8_t prev = {0, 0, 0, 0, 0, 0, 0, 0}, bias = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (Epilogue::needs_prev(a.store)) prev = *(const half8_t*)p;
+    if (Epilogue::needs_bias(a.store)) bias = *(const half8_t*)(a.bias + x);
+    half8_t r;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      half_t s16 = v[e];
+      if (a.store == STORE_ACC_BETA) {
+        // beta == 0 here: acc + 0 * prev.  Non-finite garbage in the output poisons the
+        // result exactly as in the reference; a finite one leaves the accumulator.
+        float t = 0.0f * (float)prev[e];
+        r[e] = (t == t) ? s16 : (half_t)t;
+      } else {
+        r[e] = ep.apply_s16(s16, prev[e], bias[e]);
+      }
+      if (causal && x + e > y) r[e] = neg_inf_half();
+    }
+    *(half8_t*)p = r;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      if (x + e >= a.n) break;
+      half_t prev = Epilogue::needs_prev(a.store) ? p[e] : (half_t)0;
+      half_t bias = Epilogue::needs_bias(a.store) ? a.bias[x + e] : (half_t)0;
+      half_t r;
+      if (a.store == STORE_ACC_BETA) {
+        float t = 0.0f * (float)prev;
+        r = (t == t) ? v[e] : (half_t)t;
+      } else {
+        r = ep.apply_s16(v[e], prev, bias);
+      }
+      if (causal && x + e > y) r = neg_inf_half();
+      p[e] = r;
+    }
+  }
+}
 
-  // ---- fully masked tile: every x > every y (matmul.cu:182-184) -> write -inf, no math
-  if (a.mask == ADR_MASK_CAUSAL && n0 > m0 + BM - 1) {
+// Epilogue of one wavefront.  acc[i][j] is the TRANSPOSED 32x32 accumulator of row block i,
+// column block j: lane l holds output row l % 32 and, in element r, column
+// 8*(r/4) + 4*(l/32) + r%4.  (y0, x0) is the origin of the wavefront's sub-tile; `slot` is an
+// LDS region private to this wavefront of at least 32 * (TN*64 + 16) bytes.
+template <int TM, int TN>
+__device__ __forceinline__ void wave_epilogue(const MatmulArgs& a, half_t* out,
+                                              float16_t (&acc)[TM][TN], int y0, int x0,
+                                              unsigned char* slot, half_t hscale, int lane) {
+  Epilogue ep{a.bias, a.beta, hscale, a.store};
+  const int lrow = lane & 31, g = lane >> 5;
+  if (out_vectorizable(a, out)) {
+    constexpr int PITCH = TN * 64 + 16;  // bytes per staged row (TN*32 halves + pad)
+    constexpr int CPW = TN * 4;          // 16-byte chunks per staged row
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          half4_t h;
+#pragma unroll
+          for (int e = 0; e < 4; e++) h[e] = (half_t)acc[i][j][4 * q + e];
+          *(half4_t*)(slot + lrow * PITCH + (j * 32 + 8 * q + 4 * g) * 2) = h;
+        }
+#pragma unroll
+      for (int it = 0; it < TN * 2; it++) {
+        const int idx = it * 64 + lane;
+        const int row = idx / CPW, c = idx % CPW;
+        const half8_t v = *(const half8_t*)(slot + row * PITCH + c * 16);
+        const int y = y0 + i * 32 + row, x = x0 + c * 8;
+        if (y < a.m && x < a.n) store_chunk(a, ep, out, y, x, v);
+      }
+    }
+  } else {
+    const bool need_prev = Epilogue::needs_prev(a.store);
+    const bool need_bias = Epilogue::needs_bias(a.store);
+    const bool causal = a.mask == ADR_MASK_CAUSAL;
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+      const int y = y0 + i * 32 + lrow;
+      if (y >= a.m) continue;
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int x = x0 + j * 32 + 8 * (r / 4) + 4 * g + (r % 4);
+          if (x >= a.n) continue;
+          half_t* p = out + (int64_t)y * a.stride_oy + x;
+          if (causal && x > y) {
+            *p = neg_inf_half();
+          } else {
+            half_t prev = need_prev ? *p : (half_t)0;
+            half_t bias = need_bias ? a.bias[x] : (half_t)0;
+            *p = ep.apply(acc[i][j][r], prev, bias);
+          }
+        }
+    }
+  }
+}
+
+// A tile that lies entirely above the diagonal of a causal product (every x > every y,
+// matmul.cu:182-184) is -inf: written without any math.
+template <int BM, int BN, int NT>
+__device__ __forceinline__ void fill_masked_tile(const MatmulArgs& a, half_t* out, int m0, int n0,
+                                                 int tid) {
+  if (out_vectorizable(a, out)) {
+    const half_t ninf = neg_inf_half();
+    const half8_t v = {ninf, ninf, ninf, ninf, ninf, ninf, ninf, ninf};
+    for (int e = tid; e < BM * BN / 8; e += NT) {
+      const int y = m0 + e / (BN / 8), x = n0 + (e % (BN / 8)) * 8;
+      if (y >= a.m || x >= a.n) continue;
+      half_t* p = out + (int64_t)y * a.stride_oy + x;
+      if (x + 8 <= a.n) {
+        *(half8_t*)p = v;
+      } else {
+        for (int q = 0; x + q < a.n; q++) p[q] = ninf;
+      }
+    }
+  } else {
     for (int e = tid; e < BM * BN; e += NT) {
-      int y = m0 + e / BN, x = n0 + e % BN;
+      const int y = m0 + e / BN, x = n0 + e % BN;
       if (y < a.m && x < a.n) out[(int64_t)y * a.stride_oy + x] = neg_inf_half();
     }
+  }
+}
+
+// =============================================================================================
+// Direct-to-LDS kernel
+// =============================================================================================
+template <int BM, int BN, int WM, int WN, int NSTAGE, int MINB>
+__global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulArgs a,
+                                                                         TileMap map) {
+  constexpr int BK = 64, CPR = 8, KK = 4;
+  constexpr int NW = WM * WN, NT = NW * 64;
+  constexpr int IA = BM * CPR / NT, IB = BN * CPR / NT;  // DMA instructions per thread and slice
+  constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
+  constexpr int SLOT = 32 * (TN * 64 + 16);
+  static_assert(BM * CPR % NT == 0 && BN * CPR % NT == 0, "slices must split evenly over lanes");
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "MFMA 32x32x16 tiling");
+  static_assert((NW / 2) * SLOT <= BM * BK * 2, "epilogue slots must fit in two A stages");
+  static_assert(NSTAGE == 2 || NSTAGE == 3, "2 or 3 LDS stages");
+  // Separate objects per stage: the compiler's alias analysis then knows that the asynchronous
+  // LDS writes of one stage cannot touch the stage being read, and does not serialise them.
+  __shared__ __attribute__((aligned(1024))) unsigned char sA0[BM * BK * 2];
+  __shared__ __attribute__((aligned(1024))) unsigned char sA1[BM * BK * 2];
+  __shared__ __attribute__((aligned(1024))) unsigned char sA2[NSTAGE > 2 ? BM * BK * 2 : 1024];
+  __shared__ __attribute__((aligned(1024))) unsigned char sB0[BN * BK * 2];
+  __shared__ __attribute__((aligned(1024))) unsigned char sB1[BN * BK * 2];
+  __shared__ __attribute__((aligned(1024))) unsigned char sB2[NSTAGE > 2 ? BN * BK * 2 : 1024];
+
+  int batch, tile_m, tile_n;
+  map_tile(map, batch, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  half_t* const out = a.output + (int64_t)batch * a.stride_oz;
+
+  if (a.mask == ADR_MASK_CAUSAL && n0 > m0 + BM - 1) {
+    fill_masked_tile<BM, BN, NT>(a, out, m0, n0, tid);
+    return;
+  }
+
+  const half_t* const A = a.lhs + (int64_t)batch * a.stride_lz;
+  const half_t* const B = a.rhs + (int64_t)batch * a.stride_rz;
+
+  // DMA instruction i of this wavefront fills LDS chunks [(i*NW + wave)*64, +64) of a stage,
+  // lane l the l-th of them; the lane fetches whatever (row, k-chunk) the swizzle puts there.
+  // Rows beyond the matrix are clamped to the last row (their results are never stored).
+  const half_t* gA[IA];
+  const half_t* gB[IB];
+#pragma unroll
+  for (int i = 0; i < IA; i++) {
+    int row, kc;
+    lds_chunk_inv<CPR>((i * NW + wave) * 64 + lane, row, kc);
+    gA[i] = A + (int64_t)min(m0 + row, a.m - 1) * a.stride_ly + kc * 8;
+  }
+#pragma unroll
+  for (int i = 0; i < IB; i++) {
+    int row, kc;
+    lds_chunk_inv<CPR>((i * NW + wave) * 64 + lane, row, kc);
+    gB[i] = B + (int64_t)min(n0 + row, a.n - 1) * a.stride_rx + kc * 8;
+  }
+  const int KT = a.k / BK;
+  int kload = 0;  // next slice to fetch; past the end the last slice is fetched again (unused)
+  auto dma = [&](unsigned char* dA, unsigned char* dB) {
+    const int k0 = min(kload, KT - 1) * BK;
+    kload++;
+#pragma unroll
+    for (int i = 0; i < IA; i++)
+      __builtin_amdgcn_global_load_lds(ADR_GLB_PTR(gA[i] + k0),
+                                       ADR_LDS_PTR(dA + (i * NW + wave) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < IB; i++)
+      __builtin_amdgcn_global_load_lds(ADR_GLB_PTR(gB[i] + k0),
+                                       ADR_LDS_PTR(dB + (i * NW + wave) * 1024), 16, 0, 0);
+  };
+
+  float16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+  // fragment addressing: lane -> (row = lane % 32, k-group = lane / 32), 8 halves = one chunk
+  const int frow = lane & 31, fkg = lane >> 5;
+  int offA[TM][KK], offB[TN][KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; kk++) {
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+      offA[i][kk] = lds_chunk_off<CPR>(wm * WTM + i * 32 + frow, kk * 2 + fkg);
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+      offB[j][kk] = lds_chunk_off<CPR>(wn * WTN + j * 32 + frow, kk * 2 + fkg);
+  }
+
+  half8_t fa[2][TM], fb[2][TN];
+  auto load_frags = [&](int slot, const unsigned char* cA, const unsigned char* cB, int kk) {
+#pragma unroll
+    for (int i = 0; i < TM; i++) fa[slot][i] = *(const half8_t*)(cA + offA[i][kk]);
+#pragma unroll
+    for (int j = 0; j < TN; j++) fb[slot][j] = *(const half8_t*)(cB + offB[j][kk]);
+  };
+  auto mfmas = [&](int slot) {
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[slot][j], fa[slot][i], acc[i][j],
+                                                           0, 0, 0);
+  };
+  // s_waitcnt vmcnt(n) lgkmcnt(0): n outstanding DMA instructions may remain in flight
+  auto wait_dma_barrier = [&](auto n_tag) {
+    constexpr int n = decltype(n_tag)::value;
+    __builtin_amdgcn_s_waitcnt(0x0070 | (n & 0xF) | ((n >> 4) << 14));
+    __builtin_amdgcn_s_barrier();
+  };
+  constexpr int INFLIGHT = NSTAGE == 3 ? IA + IB : 0;
+  // One K slice.  cur: stage being consumed (its k-step 0 fragments already sit in fragment
+  // slot 0); nxt: the stage consumed next; (dA, dB): the stage the DMA issued here refills.
+  auto slice = [&](const unsigned char* cA, const unsigned char* cB, const unsigned char* nA,
+                   const unsigned char* nB, unsigned char* dA, unsigned char* dB) {
+    dma(dA, dB);
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++) {
+      if (kk + 1 < KK) {
+        load_frags((kk + 1) & 1, cA, cB, kk + 1);
+        mfmas(kk & 1);
+        // interleave: one LDS read behind each of the first MFMAs of this k-step
+#pragma unroll
+        for (int q = 0; q < TM + TN; q++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
+      } else {
+        mfmas(kk & 1);
+      }
+    }
+    // the next stage has landed (only the DMA issued in this slice may still be in flight)
+    // and every wavefront has left the current one
+    wait_dma_barrier(std::integral_constant<int, INFLIGHT>{});
+    load_frags(0, nA, nB, 0);
+  };
+
+  if (NSTAGE == 3) {
+    dma(sA0, sB0);
+    dma(sA1, sB1);
+    wait_dma_barrier(std::integral_constant<int, INFLIGHT>{});
+    load_frags(0, sA0, sB0, 0);
+    int kt = 0;
+    for (; kt + 3 <= KT; kt += 3) {
+      slice(sA0, sB0, sA1, sB1, sA2, sB2);
+      slice(sA1, sB1, sA2, sB2, sA0, sB0);
+      slice(sA2, sB2, sA0, sB0, sA1, sB1);
+    }
+    if (kt < KT) { slice(sA0, sB0, sA1, sB1, sA2, sB2); kt++; }
+    if (kt < KT) { slice(sA1, sB1, sA2, sB2, sA0, sB0); kt++; }
+  } else {
+    dma(sA0, sB0);
+    wait_dma_barrier(std::integral_constant<int, 0>{});
+    load_frags(0, sA0, sB0, 0);
+    int kt = 0;
+    for (; kt + 2 <= KT; kt += 2) {
+      slice(sA0, sB0, sA1, sB1, sA1, sB1);
+      slice(sA1, sB1, sA0, sB0, sA0, sB0);
+    }
+    if (kt < KT) slice(sA0, sB0, sA1, sB1, sA1, sB1);
+  }
+  // drain the trailing (redundant) DMA before the stages are reused by the epilogue
+  wait_dma_barrier(std::integral_constant<int, 0>{});
+
+  unsigned char* slot = (wave < NW / 2 ? sA0 : sA1) + (wave % (NW / 2)) * SLOT;
+  wave_epilogue<TM, TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, slot, (half_t)a.scale, lane);
+}
+
+// =============================================================================================
+// Register-staged kernel (any K % 8 == 0; Load Scale; u8 weights)
+// =============================================================================================
+template <int BM, int BN, int BK, int WM, int WN, int MINB, bool LOAD_SCALE, bool WQ>
+__global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_stage_kernel(MatmulArgs a,
+                                                                           TileMap map) {
+  constexpr int NT = WM * WN * 64;
+  constexpr int CPR = BK / 8;
+  constexpr int LA = BM * CPR / NT, LB = BN * CPR / NT;  // chunks each thread stages
+  constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32, KK = BK / 16;
+  constexpr int SLOT = 32 * (TN * 64 + 16);
+  static_assert(BM * CPR % NT == 0 && BN * CPR % NT == 0, "staging must divide evenly");
+  static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % 16 == 0, "MFMA 32x32x16 tiling");
+  static_assert(WM * WN * SLOT <= 2 * (BM + BN) * BK * 2, "epilogue slots must fit in LDS");
+
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  unsigned char* const sA = smem;                    // [2][BM][BK] halves
+  unsigned char* const sB = smem + 2 * BM * BK * 2;  // [2][BN][BK] halves
+
+  int batch, tile_m, tile_n;
+  map_tile(map, batch, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  half_t* const out = a.output + (int64_t)batch * a.stride_oz;
+
+  if (a.mask == ADR_MASK_CAUSAL && n0 > m0 + BM - 1) {
+    fill_masked_tile<BM, BN, NT>(a, out, m0, n0, tid);
     return;
   }
 
   const half_t* const A = a.lhs + (int64_t)batch * a.stride_lz;
   const half_t* const B = a.rhs + (int64_t)batch * a.stride_rz;  // fp16 right operand (!WQ)
 
-  // ---- staging assignment: chunk c = tid + i*NT -> (row, kc); out-of-range rows are clamped
-  // to the last valid row (their products are discarded at the store)
+  // staging assignment: chunk c = tid + i*NT -> (row, kc); rows beyond the matrix are clamped
+  // to the last valid row (their products are never stored)
   const half_t* gA[LA];
-  const half_t* gB[LB];       // fp16 right operand
-  const uint8_t* gQ[LB];      // u8 right operand: 8 weights per chunk ...
-  const half_t* gS[LB];       // ... and the scale row of that weight row
+  const half_t* gB[LB];   // fp16 right operand
+  const uint8_t* gQ[LB];  // u8 right operand: 8 weights per chunk ...
+  const half_t* gS[LB];   // ... and the scale row of that weight row
   int offA[LA], offB[LB], kcA[LA], kcB[LB];
 #pragma unroll
   for (int i = 0; i < LA; i++) {
@@ -134,7 +475,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_kernel(MatmulArgs a
     for (int i = 0; i < LB; i++) {
       if (WQ) {
         // a chunk of 8 weights never straddles a scale block (block_size % 8 == 0); chunks
-        // beyond K get scale 0 with mid-range weights, i.e. exact zeros
+        // beyond K get scale 0, i.e. zeros
         const bool in = full || k0 + kcB[i] < K;
         rq[i] = in ? *(const u32x2_t*)(gQ[i] + k0) : u32x2_t{0, 0};
         rs[i] = in ? gS[i][(k0 + kcB[i]) / a.block_size] : (half_t)0;
@@ -180,7 +521,6 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_kernel(MatmulArgs a
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-  // fragment addressing: lane -> (row = lane % 32, k-group = lane / 32)
   const int frow = lane & 31, fkg = lane >> 5;
 
   load_slice(0);
@@ -205,73 +545,89 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_kernel(MatmulArgs a
       for (int i = 0; i < TM; i++)
 #pragma unroll
         for (int j = 0; j < TN; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[j], fa[i], acc[i][j], 0, 0, 0);
     }
     if (kt + 1 < KT) store_slice(buf ^ 1);
     __syncthreads();
   }
 
-  // ---- epilogue: accumulator element r of a 32x32 tile is row 8*(r/4) + 4*(lane/32) + r%4,
-  // column lane % 32
-  Epilogue ep{a.bias, a.beta, hscale, a.store};
-  const bool need_prev = Epilogue::needs_prev(a.store);
-  const bool need_bias = Epilogue::needs_bias(a.store);
-  const bool causal = a.mask == ADR_MASK_CAUSAL;
-#pragma unroll
-  for (int j = 0; j < TN; j++) {
-    const int x = n0 + wn * WTN + j * 32 + frow;
-    if (x >= a.n) continue;
-    const half_t bias_x = need_bias ? a.bias[x] : (half_t)0;
-#pragma unroll
-    for (int i = 0; i < TM; i++) {
-      const int ybase = m0 + wm * WTM + i * 32 + 4 * fkg;
-#pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int y = ybase + 8 * (r / 4) + (r % 4);
-        if (y >= a.m) continue;
-        half_t* p = out + (int64_t)y * a.stride_oy + x;
-        if (causal && x > y) {
-          *p = neg_inf_half();
-        } else {
-          half_t prev = need_prev ? *p : (half_t)0;
-          *p = ep.apply(acc[i][j][r], prev, bias_x);
-        }
-      }
-    }
-  }
+  wave_epilogue<TM, TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, smem + wave * SLOT, hscale,
+                        lane);
 }
 
-struct GemmShape {
-  int bm, bn, bk, threads, lds;
-  const char* name;
-};
-
-template <int BM, int BN, int BK, int WM, int WN, int MINB>
-hipError_t launch_cfg(hipStream_t stream, const MatmulArgs& a) {
+// =============================================================================================
+// Host side: configuration choice and launch
+// =============================================================================================
+TileMap make_map(const MatmulArgs& a, int bm, int bn) {
   TileMap map;
-  map.tiles_m = (a.m + BM - 1) / BM;
-  map.tiles_n = (a.n + BN - 1) / BN;
+  map.tiles_m = (a.m + bm - 1) / bm;
+  map.tiles_n = (a.n + bn - 1) / bn;
   map.tiles_per_batch = map.tiles_m * map.tiles_n;
   const int64_t total = (int64_t)map.tiles_per_batch * a.batches;
-  if (total > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-  map.total = (int)total;
+  map.total = total > 0x7fffffffLL ? -1 : (int)total;
   map.group_m = map.tiles_m < 8 ? map.tiles_m : 8;
-  constexpr int LDS = 2 * (BM + BN) * BK * 2;
-  dim3 grid((unsigned)map.total, 1, 1), block(WM * WN * 64, 1, 1);
-  static_assert(LDS <= 64 * 1024, "larger tiles need hipFuncSetAttribute per device");
-  if (a.rhs_q)
-    hipLaunchKernelGGL((gemm_nt_kernel<BM, BN, BK, WM, WN, MINB, false, true>), grid, block, LDS,
-                       stream, a, map);
-  else if (a.load == ADR_LOAD_SCALE)
-    hipLaunchKernelGGL((gemm_nt_kernel<BM, BN, BK, WM, WN, MINB, true, false>), grid, block, LDS,
-                       stream, a, map);
-  else
-    hipLaunchKernelGGL((gemm_nt_kernel<BM, BN, BK, WM, WN, MINB, false, false>), grid, block, LDS,
-                       stream, a, map);
+  return map;
+}
+
+template <int BM, int BN, int WM, int WN, int NSTAGE, int MINB>
+hipError_t launch_dma(hipStream_t stream, const MatmulArgs& a) {
+  TileMap map = make_map(a, BM, BN);
+  if (map.total < 0) return hipErrorInvalidConfiguration;
+  hipLaunchKernelGGL((gemm_nt_dma_kernel<BM, BN, WM, WN, NSTAGE, MINB>), dim3((unsigned)map.total),
+                     dim3(WM * WN * 64), 0, stream, a, map);
   return hipGetLastError();
 }
 
-enum GemmChoice { GEMM_NONE = 0, GEMM_256x128, GEMM_128x128, GEMM_64x64 };
+template <int BM, int BN, int BK, int WM, int WN, int MINB>
+hipError_t launch_stage(hipStream_t stream, const MatmulArgs& a) {
+  TileMap map = make_map(a, BM, BN);
+  if (map.total < 0) return hipErrorInvalidConfiguration;
+  constexpr int LDS = 2 * (BM + BN) * BK * 2;
+  static_assert(LDS <= 64 * 1024, "dynamic LDS above 64 KiB needs a per-device attribute");
+  dim3 grid((unsigned)map.total), block(WM * WN * 64);
+  if (a.rhs_q)
+    hipLaunchKernelGGL((gemm_nt_stage_kernel<BM, BN, BK, WM, WN, MINB, false, true>), grid, block,
+                       LDS, stream, a, map);
+  else if (a.load == ADR_LOAD_SCALE)
+    hipLaunchKernelGGL((gemm_nt_stage_kernel<BM, BN, BK, WM, WN, MINB, true, false>), grid, block,
+                       LDS, stream, a, map);
+  else
+    hipLaunchKernelGGL((gemm_nt_stage_kernel<BM, BN, BK, WM, WN, MINB, false, false>), grid, block,
+                       LDS, stream, a, map);
+  return hipGetLastError();
+}
+
+enum GemmChoice {
+  GEMM_NONE = 0,
+  DMA_256x192, DMA_256x128, DMA_128x128, DMA_64x64,
+  STAGE_256x128, STAGE_128x128, STAGE_64x64,
+};
+
+struct Candidate {
+  GemmChoice id;
+  int bm, bn;
+  int slots;   // workgroups resident per CU
+  float eff;   // measured relative throughput of one busy CU with this tile
+};
+
+constexpr int NUM_CU = 256;
+
+// Estimated cost: rounds of resident workgroups times the work of one tile over its efficiency.
+GemmChoice pick(const MatmulArgs& a, const Candidate* c, int n) {
+  GemmChoice best = GEMM_NONE;
+  double best_cost = 0;
+  for (int i = 0; i < n; i++) {
+    const int64_t tiles = (int64_t)((a.m + c[i].bm - 1) / c[i].bm) * ((a.n + c[i].bn - 1) / c[i].bn) *
+                          a.batches;
+    const int64_t rounds = (tiles + NUM_CU * c[i].slots - 1) / (NUM_CU * c[i].slots);
+    const double cost = (double)rounds * c[i].slots * c[i].bm * c[i].bn / c[i].eff;
+    if (best == GEMM_NONE || cost < best_cost) {
+      best = c[i].id;
+      best_cost = cost;
+    }
+  }
+  return best;
+}
 
 // The MFMA family needs 16-byte aligned, K-contiguous rows on both operands.
 GemmChoice choose(const MatmulArgs& a) {
@@ -280,29 +636,43 @@ GemmChoice choose(const MatmulArgs& a) {
   if ((a.stride_ly % 8) | (a.stride_rx % 8) | (a.stride_lz % 8) | (a.stride_rz % 8)) return GEMM_NONE;
   if (a.lhs && ((uintptr_t)a.lhs % 16 != 0 || (uintptr_t)a.rhs % 16 != 0 ||
                 (uintptr_t)a.rhs_q % 8 != 0)) return GEMM_NONE;
-  const int64_t t256 = (int64_t)((a.m + 255) / 256) * ((a.n + 127) / 128) * a.batches;
-  const int64_t t128 = (int64_t)((a.m + 127) / 128) * ((a.n + 127) / 128) * a.batches;
-  if (t256 >= 200) return GEMM_256x128;
-  if (t128 >= 128) return GEMM_128x128;
-  return GEMM_64x64;
+  const bool plain = !a.rhs_q && a.load == ADR_LOAD_IDENTITY;
+  if (plain && a.k % 64 == 0) {
+    static const Candidate dma[] = {
+        {DMA_256x192, 256, 192, 1, 1.10f}, {DMA_256x128, 256, 128, 1, 1.00f},
+        {DMA_128x128, 128, 128, 2, 0.80f}, {DMA_64x64, 64, 64, 4, 0.40f}};
+    return pick(a, dma, 4);
+  }
+  static const Candidate stage[] = {{STAGE_256x128, 256, 128, 2, 1.00f},
+                                    {STAGE_128x128, 128, 128, 2, 0.85f},
+                                    {STAGE_64x64, 64, 64, 4, 0.45f}};
+  return pick(a, stage, 3);
 }
 
 }  // namespace
 
 bool mfma_gemm_supported(const MatmulArgs& a, const char** name) {
   switch (choose(a)) {
-    case GEMM_256x128: *name = "gemm_nt_mfma_256x128x32"; return true;
-    case GEMM_128x128: *name = "gemm_nt_mfma_128x128x32"; return true;
-    case GEMM_64x64: *name = "gemm_nt_mfma_64x64x64"; return true;
+    case DMA_256x192: *name = "gemm_nt_mfma_dma_256x192x64"; return true;
+    case DMA_256x128: *name = "gemm_nt_mfma_dma_256x128x64"; return true;
+    case DMA_128x128: *name = "gemm_nt_mfma_dma_128x128x64"; return true;
+    case DMA_64x64: *name = "gemm_nt_mfma_dma_64x64x64"; return true;
+    case STAGE_256x128: *name = "gemm_nt_mfma_stage_256x128x32"; return true;
+    case STAGE_128x128: *name = "gemm_nt_mfma_stage_128x128x32"; return true;
+    case STAGE_64x64: *name = "gemm_nt_mfma_stage_64x64x64"; return true;
     default: return false;
   }
 }
 
 hipError_t launch_mfma_gemm(hipStream_t stream, const MatmulArgs& a) {
   switch (choose(a)) {
-    case GEMM_256x128: return launch_cfg<256, 128, 32, 2, 2, 2>(stream, a);
-    case GEMM_128x128: return launch_cfg<128, 128, 32, 2, 2, 2>(stream, a);
-    case GEMM_64x64: return launch_cfg<64, 64, 64, 2, 2, 2>(stream, a);
+    case DMA_256x192: return launch_dma<256, 192, 4, 2, 2, 1>(stream, a);
+    case DMA_256x128: return launch_dma<256, 128, 4, 2, 3, 1>(stream, a);
+    case DMA_128x128: return launch_dma<128, 128, 2, 2, 2, 2>(stream, a);
+    case DMA_64x64: return launch_dma<64, 64, 2, 2, 3, 3>(stream, a);
+    case STAGE_256x128: return launch_stage<256, 128, 32, 2, 2, 2>(stream, a);
+    case STAGE_128x128: return launch_stage<128, 128, 32, 2, 2, 2>(stream, a);
+    case STAGE_64x64: return launch_stage<64, 64, 64, 2, 2, 2>(stream, a);
     default: return hipErrorInvalidValue;
   }
 }

@@ -50,7 +50,7 @@ def test_kernel_selection_for_the_callers_layouts():
     M, Kd, N = 2048, 4096, 12288
     out, lhs = TensorLayout.row_major([M, N]), TensorLayout.row_major([M, Kd])
     w = TensorLayout.row_major([N, Kd]).permute([1, 0])
-    assert K.plan_matmul(out, lhs, w) == "gemm_nt_mfma_256x128x32"
+    assert K.plan_matmul(out, lhs, w).startswith("gemm_nt_mfma_dma_")
     # QK^T on the head views (llama.rs:534-550)
     S, H, D = 2048, 32, 128
     q = TensorLayout.row_major([S, H * D]).shape_cast([S, H, -1]).permute([1, 0, 2])
