@@ -91,46 +91,69 @@ __device__ __forceinline__ bool out_vectorizable(const MatmulArgs& a, const half
   return true;
 }
 
+// The store operator on 8 narrowed accumulators at once; the switch is taken once per chunk.
+__device__ __forceinline__ half8_t apply_chunk(const MatmulArgs& a, const Epilogue& ep, half8_t v,
+                                               half8_t prev, half8_t bias) {
+  half8_t r = v;
+  switch (a.store) {
+    default:
+    case ADR_STORE_IDENTITY:
+      break;
+    case ADR_STORE_SCALE:
+      r = v * ep.hscale;
+      break;
+    case ADR_STORE_ADD:
+      r = v + prev;
+      break;
+    case STORE_ACC_BETA:
+      // beta == 0 on this path: acc + 0 * prev.  Non-finite garbage in the output poisons the
+      // result exactly as in the reference; a finite one leaves the accumulator.
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        float t = 0.0f * (float)prev[e];
+        r[e] = (t == t) ? v[e] : (half_t)t;
+      }
+      break;
+    case ADR_STORE_BETA_BIAS:
+    case ADR_STORE_QUICK_GELU_BIAS:
+    case ADR_STORE_BETA_GELU_BIAS:
+#pragma unroll
+      for (int e = 0; e < 8; e++) r[e] = ep.apply_s16(v[e], prev[e], bias[e]);
+      break;
+  }
+  return r;
+}
+
 // One 16-byte chunk (8 consecutive columns x..x+7 of output row y) through the store operator.
 __device__ __forceinline__ void store_chunk(const MatmulArgs& a, const Epilogue& ep, half_t* out,
                                             int y, int x, half8_t v) {
   half_t* p = out + (int64_t)y * a.stride_oy + x;
-  const bool causal = a.mask == ADR_MASK_CAUSAL;
-  if (x + 8 <= a.n) {
-    half8_t prev = {0, 0, 0, 0, 0, 0, 0, 0}, bias = {0, 0, 0, 0, 0, 0, 0, 0};
+  const bool full = x + 8 <= a.n;
+  half8_t prev = {0, 0, 0, 0, 0, 0, 0, 0}, bias = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (full) {
     if (Epilogue::needs_prev(a.store)) prev = *(const half8_t*)p;
     if (Epilogue::needs_bias(a.store)) bias = *(const half8_t*)(a.bias + x);
-    half8_t r;
-#pragma unroll
-    for (int e = 0; e < 8; e++) {
-      half_t s16 = v[e];
-      if (a.store == STORE_ACC_BETA) {
-        // beta == 0 here: acc + 0 * prev.  Non-finite garbage in the output poisons the
-        // result exactly as in the reference; a finite one leaves the accumulator.
-        float t = 0.0f * (float)prev[e];
-        r[e] = (t == t) ? s16 : (half_t)t;
-      } else {
-        r[e] = ep.apply_s16(s16, prev[e], bias[e]);
-      }
-      if (causal && x + e > y) r[e] = neg_inf_half();
-    }
-    *(half8_t*)p = r;
   } else {
 #pragma unroll
     for (int e = 0; e < 8; e++) {
-      if (x + e >= a.n) break;
-      half_t prev = Epilogue::needs_prev(a.store) ? p[e] : (half_t)0;
-      half_t bias = Epilogue::needs_bias(a.store) ? a.bias[x + e] : (half_t)0;
-      half_t r;
-      if (a.store == STORE_ACC_BETA) {
-        float t = 0.0f * (float)prev;
-        r = (t == t) ? v[e] : (half_t)t;
-      } else {
-        r = ep.apply_s16(v[e], prev, bias);
+      if (x + e < a.n) {
+        if (Epilogue::needs_prev(a.store)) prev[e] = p[e];
+        if (Epilogue::needs_bias(a.store)) bias[e] = a.bias[x + e];
       }
-      if (causal && x + e > y) r = neg_inf_half();
-      p[e] = r;
     }
+  }
+  half8_t r = apply_chunk(a, ep, v, prev, bias);
+  if (a.mask == ADR_MASK_CAUSAL && x + 7 > y) {
+#pragma unroll
+    for (int e = 0; e < 8; e++)
+      if (x + e > y) r[e] = neg_inf_half();
+  }
+  if (full) {
+    *(half8_t*)p = r;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; e++)
+      if (x + e < a.n) p[e] = r[e];
   }
 }
 
@@ -158,7 +181,7 @@ __device__ __forceinline__ void wave_epilogue(const MatmulArgs& a, half_t* out,
           for (int e = 0; e < 4; e++) h[e] = (half_t)acc[i][j][4 * q + e];
           *(half4_t*)(slot + lrow * PITCH + (j * 32 + 8 * q + 4 * g) * 2) = h;
         }
-#pragma unroll
+#pragma unroll 1
       for (int it = 0; it < TN * 2; it++) {
         const int idx = it * 64 + lane;
         const int row = idx / CPW, c = idx % CPW;
