@@ -1,18 +1,30 @@
 // u8-quantised-weight skinny GEMM / GEMV for decode (m <= 16):
 //   out[r,c] = fp16( sum_i lhs[r,i] * w[c,i] + beta * out[r,c] ),
-//   w[c,i]   = fp16( (float(q[c,i]) - 127.5f) * float(scales[c, i/block_size]) )
-// (adrastea_kernels/cpp/matmul_nt_wmma_16x128x256_fp16u8.cu:5-7, 43-83; format quantize.cu).
+//   w[c,i]   = (float(q[c,i]) - 127.5f) * float(scales[c, i/block_size])
+// (adrastea_kernels/cpp/matmul_nt_fp16u8.cu:4-24 and
+// matmul_nt_wmma_16x128x256_fp16u8.cu:5-7, 43-83; format quantize.cu:3-56).
 //
-// The problem is bound by streaming the u8 weights from HBM once.  Each workgroup owns 16
-// consecutive weight rows; its wavefronts split K in 256-element macro steps.  Per macro step
-// a lane (row r = lane % 16, group g = lane / 16) streams 64 consecutive weight bytes of its
-// row with four 128-bit loads -- four lanes cover 256 contiguous bytes of a row, whole cache
-// lines -- plus one dword holding the two fp16 scales of those 64 weights.  The weights are
-// dequantised in registers to packed fp16 and fed to v_mfma_f32_16x16x32_f16 as the A operand
-// (16 weight rows x 32 k); the activations are the B operand (32 k x 16 activation rows, rows
-// beyond m are zero).  The k slots of an MFMA may hold any 32 distinct k as long as both
-// operands agree, which is what lets a lane use contiguous bytes.  Partial sums of the
-// wavefronts are reduced through LDS.
+// The problem is bound by streaming the u8 weights from HBM once.  Two kernels:
+//
+//  gemv_u8_dot_kernel (m <= 4)   no matrix cores.  A wavefront streams whole 1 KiB segments of
+//      one weight row per load instruction (lane l: 16 bytes at l*16, perfectly coalesced),
+//      keeps its activation slices in registers for all rows of the workgroup, and evaluates
+//        sum_k x_k (q_k - 127.5) s  =  s * ( sum_k x_k (1024 + q_k)  -  1151.5 * sum_k x_k )
+//      per lane (16 weights of one scale block): the bytes are unpacked with one v_perm_b32
+//      per pair into the fp16 numbers 1024 + q (bit pattern 0x6400 | q) and fed to
+//      v_dot2_f32_f16 with fp32 accumulation; the second term is row independent and computed
+//      once.  This is the arithmetic of the reference's naive kernel (unrounded weights,
+//      matmul_nt_fp16u8.cu:17-21) in fp32.  Lane sums are reduced with DPP adds.
+//
+//  gemv_u8_kernel (m <= 16)      v_mfma_f32_16x16x32_f16 with the 16 weight rows of the
+//      workgroup as the A operand and the activations as the B operand (rows beyond m are
+//      zero).  Per 256-element macro step a lane (row r = lane % 16, group g = lane / 16)
+//      loads 4 x 16 weight bytes such that the four lanes of a row cover 64 contiguous bytes
+//      per instruction, dequantises them in registers to fp16 exactly as the stand-alone
+//      dequantise kernel does (the WMMA kernel's arithmetic) and issues two MFMAs per load.
+//      The k slots of an MFMA may hold any 32 distinct k as long as both operands agree,
+//      which is what lets a lane use 16 contiguous bytes.  Wavefronts split K; partial sums
+//      are reduced through LDS.
 #include "adr_common.hpp"
 
 namespace adr {
@@ -23,9 +35,9 @@ constexpr int MACRO_K = 256;  // k elements per macro step
 constexpr int ROWS = 16;      // weight rows per workgroup
 
 struct Stage {
-  u32x4_t w[4];   // 64 weight bytes of this lane's row
-  uint32_t sc;    // two fp16 scales (block_size 32) covering them
-  u32x4_t x[8];   // 64 activation halves of this lane's activation row
+  u32x4_t w[4];   // 4 x 16 weight bytes of this lane's row
+  u32x4_t sc;     // the eight fp16 scales (block_size 32) of the macro step
+  u32x4_t x[8];   // 4 x 16 activation halves of this lane's activation row
 };
 
 template <int NW>
@@ -40,30 +52,35 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_kernel(half_t* __restrict__ o
   const int n0 = blockIdx.x * ROWS;
   const int row = min(n0 + r, n - 1);  // tail rows are clamped; their sums are not stored
   const int nblk = p / 32;
-  const uint8_t* wrow = rhs + (int64_t)row * p + g * 64;
-  const half_t* srow = scales + (int64_t)row * nblk + g * 2;
+  // load j of a macro step takes bytes j*64 + g*16 .. +16 of the row: the four lanes of a row
+  // cover 64 contiguous bytes per instruction
+  const uint8_t* wrow = rhs + (int64_t)row * p + g * 16;
+  const half_t* srow = scales + (int64_t)row * nblk;
   const bool xvalid = r < m;
-  const half_t* xrow = lhs + (int64_t)(xvalid ? r : 0) * p + g * 64;
+  const half_t* xrow = lhs + (int64_t)(xvalid ? r : 0) * p + g * 16;
   const int steps = p / MACRO_K;
 
   auto load = [&](Stage& s, int ms) {
     const uint8_t* wp = wrow + (int64_t)ms * MACRO_K;
 #pragma unroll
-    for (int j = 0; j < 4; j++) s.w[j] = __builtin_nontemporal_load((const u32x4_t*)(wp + j * 16));
-    s.sc = *(const uint32_t*)(srow + ms * (MACRO_K / 32));
+    for (int j = 0; j < 4; j++) s.w[j] = *(const u32x4_t*)(wp + j * 64);
+    s.sc = *(const u32x4_t*)(srow + ms * (MACRO_K / 32));
     const half_t* xp = xrow + (int64_t)ms * MACRO_K;
 #pragma unroll
-    for (int j = 0; j < 8; j++)
-      s.x[j] = xvalid ? *(const u32x4_t*)(xp + j * 8) : u32x4_t{0, 0, 0, 0};
+    for (int j = 0; j < 4; j++) {
+      s.x[2 * j] = xvalid ? *(const u32x4_t*)(xp + j * 64) : u32x4_t{0, 0, 0, 0};
+      s.x[2 * j + 1] = xvalid ? *(const u32x4_t*)(xp + j * 64 + 8) : u32x4_t{0, 0, 0, 0};
+    }
   };
 
   float4_t acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
   auto compute = [&](const Stage& s) {
-    const half2_t sc = __builtin_bit_cast(half2_t, s.sc);
-    const half2_t s_lo = {sc[0], sc[0]}, s_hi = {sc[1], sc[1]};
+    const half8_t sc = __builtin_bit_cast(half8_t, s.sc);
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-      const half2_t s2 = j < 2 ? s_lo : s_hi;
+      // the lane's 16 weights of load j sit in scale block 2j (g < 2) or 2j + 1
+      const half_t sv = g < 2 ? sc[2 * j] : sc[2 * j + 1];
+      const half2_t s2 = {sv, sv};
       half8_t a0 = dequant8(s.w[j][0], s.w[j][1], s2);
       half8_t a1 = dequant8(s.w[j][2], s.w[j][3], s2);
       half8_t b0 = __builtin_bit_cast(half8_t, s.x[2 * j]);
@@ -107,6 +124,127 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_kernel(half_t* __restrict__ o
   }
 }
 
+
+typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+
+template <int CTRL, int ROWMASK>
+__device__ __forceinline__ float dpp_add(float v) {
+  int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROWMASK, 0xf, true);
+  return v + __builtin_bit_cast(float, t);
+}
+// Sum over the 64 lanes with data-parallel-primitive adds (no LDS); the total is in lane 63.
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+  v = dpp_add<0x111, 0xf>(v);  // row_shr:1
+  v = dpp_add<0x112, 0xf>(v);  // row_shr:2
+  v = dpp_add<0x114, 0xf>(v);  // row_shr:4
+  v = dpp_add<0x118, 0xf>(v);  // row_shr:8   lane 15 of each 16-lane row = row sum
+  v = dpp_add<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+  v = dpp_add<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
+// MR activation rows, NW wavefronts, RPB weight rows per workgroup, SEGW 1 KiB K segments per
+// wavefront (wavefront w owns segments w, w+NW, ...).
+template <int MR, int NW, int RPB, int SEGW>
+__global__ __launch_bounds__(NW * 64) void gemv_u8_dot_kernel(half_t* __restrict__ out,
+                                                              const half_t* __restrict__ lhs,
+                                                              const uint8_t* __restrict__ rhs,
+                                                              const half_t* __restrict__ scales,
+                                                              int m, int p, int n, int block_size,
+                                                              float beta) {
+  __shared__ float partial[NW][RPB][MR];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n0 = blockIdx.x * RPB;
+  const int nblk = p / block_size;
+  const int nseg = (p + 1023) / 1024;
+  half8_t xr[SEGW][MR][2];  // this lane's 16 activations of each owned segment and row
+  float xs[SEGW][MR];       // 1151.5 * their sum
+  bool act[SEGW];
+  int sidx[SEGW];           // scale block of the lane's 16 weights
+#pragma unroll
+  for (int j = 0; j < SEGW; j++) {
+    const int seg = wave + j * NW;
+    const int k = seg * 1024 + lane * 16;
+    act[j] = seg < nseg && k < p;
+    sidx[j] = k / block_size;
+#pragma unroll
+    for (int mm = 0; mm < MR; mm++) {
+      const bool v = act[j] && mm < m;
+      const u32x4_t z = {0, 0, 0, 0};
+      xr[j][mm][0] = __builtin_bit_cast(half8_t, v ? *(const u32x4_t*)(lhs + (int64_t)mm * p + k) : z);
+      xr[j][mm][1] = __builtin_bit_cast(half8_t, v ? *(const u32x4_t*)(lhs + (int64_t)mm * p + k + 8) : z);
+      float sum = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 8; e++) sum += (float)xr[j][mm][0][e] + (float)xr[j][mm][1][e];
+      xs[j][mm] = 1151.5f * sum;
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < RPB; r++) {
+    const int row = min(n0 + r, n - 1);  // rows beyond n are clamped; their sums are not stored
+    const uint8_t* wp = rhs + (int64_t)row * p + lane * 16;
+    const half_t* sp = scales + (int64_t)row * nblk;
+    u32x4_t w[SEGW];
+    half_t sc[SEGW];
+#pragma unroll
+    for (int j = 0; j < SEGW; j++) {
+      w[j] = act[j] ? *(const u32x4_t*)(wp + (wave + j * NW) * 1024) : u32x4_t{0, 0, 0, 0};
+      sc[j] = act[j] ? sp[sidx[j]] : (half_t)0;
+    }
+    float tot[MR];
+#pragma unroll
+    for (int mm = 0; mm < MR; mm++) tot[mm] = 0.0f;
+#pragma unroll
+    for (int j = 0; j < SEGW; j++) {
+      float pp[MR];
+#pragma unroll
+      for (int mm = 0; mm < MR; mm++) pp[mm] = -xs[j][mm];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        // bytes b0..b3 of the dword -> halves (1024+b0, 1024+b1) and (1024+b2, 1024+b3)
+        const uint32_t lo = __builtin_amdgcn_perm(0x64646464u, w[j][e], 0x07010700u);
+        const uint32_t hi = __builtin_amdgcn_perm(0x64646464u, w[j][e], 0x07030702u);
+#pragma unroll
+        for (int mm = 0; mm < MR; mm++) {
+          const half8_t x8 = xr[j][mm][e >> 1];
+          const h2_t x01 = {x8[(e & 1) * 4], x8[(e & 1) * 4 + 1]};
+          const h2_t x23 = {x8[(e & 1) * 4 + 2], x8[(e & 1) * 4 + 3]};
+          pp[mm] = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, lo), x01, pp[mm], false);
+          pp[mm] = __builtin_amdgcn_fdot2(__builtin_bit_cast(h2_t, hi), x23, pp[mm], false);
+        }
+      }
+      const float s = (float)sc[j];
+#pragma unroll
+      for (int mm = 0; mm < MR; mm++) tot[mm] += s * pp[mm];
+    }
+#pragma unroll
+    for (int mm = 0; mm < MR; mm++) {
+      const float v = wave_sum_dpp(tot[mm]);
+      if (lane == 63) partial[wave][r][mm] = v;
+    }
+  }
+  __syncthreads();
+  for (int e = tid; e < RPB * MR; e += NW * 64) {
+    const int mm = e / RPB, r = e % RPB;  // consecutive threads -> consecutive output columns
+    if (mm < m && n0 + r < n) {
+      float sum = 0.0f;
+#pragma unroll
+      for (int w2 = 0; w2 < NW; w2++) sum += partial[w2][r][mm];
+      half_t* o = out + (int64_t)mm * n + n0 + r;
+      // the previous output is read even for beta == 0, as the reference does
+      *o = (half_t)(sum + beta * (float)*o);
+    }
+  }
+}
+
+template <int MR, int NW, int RPB, int SEGW>
+hipError_t launch_dot(hipStream_t stream, half_t* out, const half_t* lhs, const uint8_t* rhs,
+                      const half_t* scales, int m, int p, int n, int block_size, float beta) {
+  hipLaunchKernelGGL((gemv_u8_dot_kernel<MR, NW, RPB, SEGW>), dim3((n + RPB - 1) / RPB),
+                     dim3(NW * 64), 0, stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
+  return hipGetLastError();
+}
+
 // Safety net for shapes / alignments the streaming kernel does not take: one thread per
 // output, dequantising each weight to fp16 exactly as above and accumulating in fp32.
 __global__ __launch_bounds__(256) void gemm_u8_naive_kernel(half_t* out, const half_t* lhs,
@@ -127,13 +265,17 @@ __global__ __launch_bounds__(256) void gemm_u8_naive_kernel(half_t* out, const h
   *o = (half_t)(sum + beta * (float)*o);
 }
 
-enum U8Choice { U8_NAIVE = 0, U8_GEMV, U8_GEMM };
+enum U8Choice { U8_NAIVE = 0, U8_DOT, U8_GEMV, U8_GEMM };
 
 U8Choice choose_u8(const void* lhs, const void* rhs, const void* scales, int m, int p, int n,
                    int block_size) {
   const bool aligned = ((uintptr_t)lhs % 16 == 0) && ((uintptr_t)rhs % 16 == 0) &&
-                       ((uintptr_t)scales % 4 == 0);
+                       ((uintptr_t)scales % 16 == 0);
   if (!aligned) return U8_NAIVE;
+  // dot-product kernel: 16 weights of a lane share one scale; at most 16 segments of 1 KiB.
+  // It wins for one or two activation rows, and for up to four on wide matrices.
+  const bool dot_ok = block_size % 16 == 0 && p % 16 == 0 && p <= 16 * 1024;
+  if (dot_ok && (m <= 2 || (m <= 4 && p <= 4096 && n >= 8192))) return U8_DOT;
   if (m <= 16 && block_size == 32 && p % MACRO_K == 0) return U8_GEMV;
   if (block_size % 8 == 0 && p % 8 == 0) return U8_GEMM;
   return U8_NAIVE;
@@ -147,6 +289,7 @@ hipError_t launch_gemm_u8_mfma(hipStream_t stream, half_t* out, const half_t* lh
 
 const char* gemm_u8_plan(int m, int p, int n, int block_size) {
   switch (choose_u8(nullptr, nullptr, nullptr, m, p, n, block_size)) {
+    case U8_DOT: return "gemv_u8_dot2_stream";
     case U8_GEMV: return "gemv_u8_mfma16_stream";
     case U8_GEMM: return "gemm_nt_u8_mfma";
     default: return "gemm_u8_naive";
@@ -156,6 +299,18 @@ const char* gemm_u8_plan(int m, int p, int n, int block_size) {
 hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, const uint8_t* rhs,
                           const half_t* scales, int m, int p, int n, int block_size, float beta) {
   switch (choose_u8(lhs, rhs, scales, m, p, n, block_size)) {
+    case U8_DOT: {
+      const bool wide = n > 6144;
+      if (p <= 4096) {  // 4 wavefronts, one segment each
+        if (m == 1) return wide ? launch_dot<1, 4, 8, 1>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta)
+                                : launch_dot<1, 4, 2, 1>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
+        if (m == 2) return launch_dot<2, 4, 4, 1>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
+        return launch_dot<4, 4, 4, 1>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
+      }
+      // up to 16 segments: 8 wavefronts, two segments each
+      if (m == 1) return launch_dot<1, 8, 4, 2>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
+      return launch_dot<2, 8, 4, 2>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
+    }
     case U8_GEMV: {
       const int blocks = (n + ROWS - 1) / ROWS;
       const int steps = p / MACRO_K;

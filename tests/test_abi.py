@@ -71,10 +71,14 @@ def test_u8_plan():
         buf = C.create_string_buffer(64)
         rc = _ffi.lib().adr_matmul_nt_fp16u8_plan(buf, 64, m, p, n, bs)
         return rc, buf.value.decode()
-    for m in (1, 4, 16):
+    for m in (1, 2):
+        assert plan(m, 4096, 4096, 32) == (0, "gemv_u8_dot2_stream")
+        assert plan(m, 11008, 4096, 32) == (0, "gemv_u8_dot2_stream")
+    for m in (4, 16):
         assert plan(m, 4096, 4096, 32) == (0, "gemv_u8_mfma16_stream")
         assert plan(m, 11008, 4096, 32) == (0, "gemv_u8_mfma16_stream")
+    assert plan(4, 4096, 12288, 32) == (0, "gemv_u8_dot2_stream")
     assert plan(2048, 4096, 4096, 32) == (0, "gemm_nt_u8_mfma")
-    assert plan(4, 4096, 4096, 64)[1] == "gemm_nt_u8_mfma"
+    assert plan(8, 4096, 4096, 64)[1] == "gemm_nt_u8_mfma"
     assert plan(4, 4100, 64, 32)[0] == _ffi.ADR_EDIVISIBILITY
     assert plan(4, 64, 64, 0)[0] == _ffi.ADR_EINVAL_SHAPE

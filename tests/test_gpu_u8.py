@@ -101,7 +101,7 @@ def test_fused_dequant_in_gemv_is_bit_exact_for_every_q_and_finite_scale(kern, m
     """One-hot activations pick single weights out of the matmul: out[r, c] = w[c, k_r]."""
     scales_bits = _finite_scale_rows()
     n, p, bs = scales_bits.size, 256, 32
-    assert u8_plan(m, p, n, bs) == "gemv_u8_mfma16_stream"
+    assert u8_plan(m, p, n, bs) in ("gemv_u8_mfma16_stream", "gemv_u8_dot2_stream")
     q = np.tile(np.arange(256, dtype=np.uint8), (n, 1))
     s = np.repeat(scales_bits.view(np.float16).reshape(n, 1), p // bs, axis=1)
     table = oracle.dequant_table()  # [q][scale bits]
@@ -219,7 +219,7 @@ def test_decode_shapes_full_size(kern, kn, m):
     q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)
     s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
     a = torch.randn(m, p, generator=gen, device="cuda").half()
-    assert u8_plan(m, p, n, 32) == "gemv_u8_mfma16_stream"
+    assert u8_plan(m, p, n, 32) in ("gemv_u8_mfma16_stream", "gemv_u8_dot2_stream")
     out = torch.zeros(m, n, dtype=torch.float16, device="cuda")
     kern.matmul_nt_fp16u8(out, a, q, s, 32)
     w = torch.zeros(n, p, dtype=torch.float16, device="cuda")
