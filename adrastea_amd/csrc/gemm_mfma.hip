@@ -246,7 +246,7 @@ __device__ __forceinline__ void fill_masked_tile(const MatmulArgs& a, half_t* ou
 // =============================================================================================
 // Direct-to-LDS kernel
 // =============================================================================================
-template <int BM, int BN, int WM, int WN, int NSTAGE, int MINB>
+template <int BM, int BN, int WM, int WN, int NSTAGE, int MINB, bool NN>
 __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulArgs a,
                                                                          TileMap map) {
   constexpr int BK = 64, CPR = 8, KK = 4;
@@ -258,6 +258,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "MFMA 32x32x16 tiling");
   static_assert((NW / 2) * SLOT <= BM * BK * 2, "epilogue slots must fit in two A stages");
   static_assert(NSTAGE == 2 || NSTAGE == 3, "2 or 3 LDS stages");
+  static_assert(!NN || BN == 128, "the N-contiguous right operand is staged as [64][128] tiles");
   // Separate objects per stage: the compiler's alias analysis then knows that the asynchronous
   // LDS writes of one stage cannot touch the stage being read, and does not serialise them.
   __shared__ __attribute__((aligned(1024))) unsigned char sA0[BM * BK * 2];
@@ -295,14 +296,25 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   }
 #pragma unroll
   for (int i = 0; i < IB; i++) {
-    int row, kc;
-    lds_chunk_inv<CPR>((i * NW + wave) * 64 + lane, row, kc);
-    gB[i] = B + (int64_t)min(n0 + row, a.n - 1) * a.stride_rx + kc * 8;
+    if (NN) {
+      // right operand stored [k][n] (n contiguous): the stage is a [64 k][128 n] tile, one DMA
+      // instruction brings 4 k-rows of 256 bytes; 16-byte chunk c of row k sits at position
+      // c ^ ((k & 3) << 2) so that the transposing fragment reads spread over all banks
+      const int krow = (i * NW + wave) * 4 + (lane >> 4);
+      const int c = (lane & 15) ^ ((krow & 3) << 2);
+      gB[i] = B + (int64_t)krow * a.stride_ry + min(n0 + c * 8, a.n - 8);
+    } else {
+      int row, kc;
+      lds_chunk_inv<CPR>((i * NW + wave) * 64 + lane, row, kc);
+      gB[i] = B + (int64_t)min(n0 + row, a.n - 1) * a.stride_rx + kc * 8;
+    }
   }
+  const int64_t b_slice = NN ? (int64_t)BK * a.stride_ry : BK;  // elements per K slice
   const int KT = a.k / BK;
   int kload = 0;  // next slice to fetch; past the end the last slice is fetched again (unused)
   auto dma = [&](unsigned char* dA, unsigned char* dB) {
-    const int k0 = min(kload, KT - 1) * BK;
+    const int ks = min(kload, KT - 1);
+    const int k0 = ks * BK;
     kload++;
 #pragma unroll
     for (int i = 0; i < IA; i++)
@@ -310,7 +322,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
                                        ADR_LDS_PTR(dA + (i * NW + wave) * 1024), 16, 0, 0);
 #pragma unroll
     for (int i = 0; i < IB; i++)
-      __builtin_amdgcn_global_load_lds(ADR_GLB_PTR(gB[i] + k0),
+      __builtin_amdgcn_global_load_lds(ADR_GLB_PTR(gB[i] + ks * b_slice),
                                        ADR_LDS_PTR(dB + (i * NW + wave) * 1024), 16, 0, 0);
   };
 
@@ -331,8 +343,21 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
     for (int i = 0; i < TM; i++)
       offA[i][kk] = lds_chunk_off<CPR>(wm * WTM + i * 32 + frow, kk * 2 + fkg);
 #pragma unroll
-    for (int j = 0; j < TN; j++)
-      offB[j][kk] = lds_chunk_off<CPR>(wn * WTN + j * 32 + frow, kk * 2 + fkg);
+    for (int j = 0; j < TN; j++) {
+      if (NN) {
+        // transposing read (ds_read_b64_tr_b16): inside each group of 16 lanes, lanes 4r..4r+3
+        // address 16 consecutive halves of k-row r and lane i receives column i of that 4 x 16
+        // block.  Group q = lane / 16 takes columns 16*(q%2).. of the 32-column block and
+        // k-rows 8*(q/2).. of the k-step, so that lane l ends up with column l % 32 and
+        // k-group l / 32, the MFMA operand layout.
+        const int q = lane >> 4, r = (lane >> 2) & 3, jj = lane & 3;
+        const int krow = kk * 16 + (q >> 1) * 8 + r;
+        const int col = wn * WTN + j * 32 + 16 * (q & 1) + 4 * jj;
+        offB[j][kk] = krow * 256 + ((((col >> 3) ^ ((krow & 3) << 2))) << 4) + (jj & 1) * 8;
+      } else {
+        offB[j][kk] = lds_chunk_off<CPR>(wn * WTN + j * 32 + frow, kk * 2 + fkg);
+      }
+    }
   }
 
   half8_t fa[2][TM], fb[2][TN];
@@ -340,7 +365,20 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
 #pragma unroll
     for (int i = 0; i < TM; i++) fa[slot][i] = *(const half8_t*)(cA + offA[i][kk]);
 #pragma unroll
-    for (int j = 0; j < TN; j++) fb[slot][j] = *(const half8_t*)(cB + offB[j][kk]);
+    for (int j = 0; j < TN; j++) {
+      if (NN) {
+        typedef short short4_t __attribute__((ext_vector_type(4)));
+        typedef __attribute__((address_space(3))) short4_t lds_short4_t;
+        const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (lds_short4_t*)ADR_LDS_PTR(cB + offB[j][kk]));
+        const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (lds_short4_t*)ADR_LDS_PTR(cB + offB[j][kk] + 4 * 256));  // k-rows + 4
+        fb[slot][j] = __builtin_shufflevector(__builtin_bit_cast(half4_t, lo),
+                                              __builtin_bit_cast(half4_t, hi), 0, 1, 2, 3, 4, 5, 6, 7);
+      } else {
+        fb[slot][j] = *(const half8_t*)(cB + offB[j][kk]);
+      }
+    }
   };
   auto mfmas = [&](int slot) {
 #pragma unroll
@@ -367,13 +405,14 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
       if (kk + 1 < KK) {
         load_frags((kk + 1) & 1, cA, cB, kk + 1);
         mfmas(kk & 1);
-        // interleave: one LDS read behind each of the first MFMAs of this k-step
+        // interleave: LDS reads behind the first MFMAs of this k-step
+        constexpr int READS = TM + (NN ? 2 * TN : TN);
+        constexpr int PER = (READS + TM * TN - 1) / (TM * TN);
 #pragma unroll
-        for (int q = 0; q < TM + TN; q++) {
+        for (int q = 0; q < TM * TN; q++) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, PER, 0);
         }
-        __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
       } else {
         mfmas(kk & 1);
       }
@@ -592,12 +631,12 @@ TileMap make_map(const MatmulArgs& a, int bm, int bn) {
   return map;
 }
 
-template <int BM, int BN, int WM, int WN, int NSTAGE, int MINB>
+template <int BM, int BN, int WM, int WN, int NSTAGE, int MINB, bool NN = false>
 hipError_t launch_dma(hipStream_t stream, const MatmulArgs& a) {
   TileMap map = make_map(a, BM, BN);
   if (map.total < 0) return hipErrorInvalidConfiguration;
-  hipLaunchKernelGGL((gemm_nt_dma_kernel<BM, BN, WM, WN, NSTAGE, MINB>), dim3((unsigned)map.total),
-                     dim3(WM * WN * 64), 0, stream, a, map);
+  hipLaunchKernelGGL((gemm_nt_dma_kernel<BM, BN, WM, WN, NSTAGE, MINB, NN>),
+                     dim3((unsigned)map.total), dim3(WM * WN * 64), 0, stream, a, map);
   return hipGetLastError();
 }
 
@@ -623,6 +662,7 @@ hipError_t launch_stage(hipStream_t stream, const MatmulArgs& a) {
 enum GemmChoice {
   GEMM_NONE = 0,
   DMA_256x192, DMA_256x128, DMA_128x128, DMA_64x64,
+  DMA_NN_256x128, DMA_NN_128x128,
   STAGE_256x128, STAGE_128x128, STAGE_64x64,
 };
 
@@ -654,6 +694,16 @@ GemmChoice pick(const MatmulArgs& a, const Candidate* c, int n) {
 
 // The MFMA family needs 16-byte aligned, K-contiguous rows on both operands.
 GemmChoice choose(const MatmulArgs& a) {
+  // "NN": both the left operand (k contiguous) and the right operand (n contiguous) are row
+  // major, e.g. P.V on the head views of llama.rs:552-554
+  if (a.stride_lx == 1 && a.stride_rx == 1 && a.stride_ry != 1 && a.stride_ox == 1 && !a.rhs_q &&
+      a.load == ADR_LOAD_IDENTITY && a.k % 64 == 0 && a.k >= 64 && a.n % 8 == 0 && a.n >= 8 &&
+      !((a.stride_ly % 8) | (a.stride_ry % 8) | (a.stride_lz % 8) | (a.stride_rz % 8)) &&
+      !(a.lhs && ((uintptr_t)a.lhs % 16 != 0 || (uintptr_t)a.rhs % 16 != 0))) {
+    static const Candidate nn[] = {{DMA_NN_256x128, 256, 128, 1, 1.00f},
+                                   {DMA_NN_128x128, 128, 128, 2, 0.80f}};
+    return pick(a, nn, 2);
+  }
   if (a.stride_lx != 1 || a.stride_ry != 1 || a.stride_ox != 1) return GEMM_NONE;
   if (a.k % 8 != 0 || a.k < 8) return GEMM_NONE;
   if ((a.stride_ly % 8) | (a.stride_rx % 8) | (a.stride_lz % 8) | (a.stride_rz % 8)) return GEMM_NONE;
@@ -680,6 +730,8 @@ bool mfma_gemm_supported(const MatmulArgs& a, const char** name) {
     case DMA_256x128: *name = "gemm_nt_mfma_dma_256x128x64"; return true;
     case DMA_128x128: *name = "gemm_nt_mfma_dma_128x128x64"; return true;
     case DMA_64x64: *name = "gemm_nt_mfma_dma_64x64x64"; return true;
+    case DMA_NN_256x128: *name = "gemm_nn_mfma_dma_256x128x64"; return true;
+    case DMA_NN_128x128: *name = "gemm_nn_mfma_dma_128x128x64"; return true;
     case STAGE_256x128: *name = "gemm_nt_mfma_stage_256x128x32"; return true;
     case STAGE_128x128: *name = "gemm_nt_mfma_stage_128x128x32"; return true;
     case STAGE_64x64: *name = "gemm_nt_mfma_stage_64x64x64"; return true;
@@ -693,6 +745,8 @@ hipError_t launch_mfma_gemm(hipStream_t stream, const MatmulArgs& a) {
     case DMA_256x128: return launch_dma<256, 128, 4, 2, 3, 1>(stream, a);
     case DMA_128x128: return launch_dma<128, 128, 2, 2, 2, 2>(stream, a);
     case DMA_64x64: return launch_dma<64, 64, 2, 2, 3, 3>(stream, a);
+    case DMA_NN_256x128: return launch_dma<256, 128, 4, 2, 3, 1, true>(stream, a);
+    case DMA_NN_128x128: return launch_dma<128, 128, 2, 2, 2, 2, true>(stream, a);
     case STAGE_256x128: return launch_stage<256, 128, 32, 2, 2, 2>(stream, a);
     case STAGE_128x128: return launch_stage<128, 128, 32, 2, 2, 2>(stream, a);
     case STAGE_64x64: return launch_stage<64, 64, 64, 2, 2, 2>(stream, a);

@@ -224,7 +224,7 @@ def test_attention_views_qk_and_pv():
     """llama.rs:534-554 with S=160, 4 heads, head_dim 64: QK^T with Scale + Causal on the
     interleaved-head views, then P.V into the strided output view."""
     g = rng(530)
-    S, H, D = 160, 4, 64
+    S, H, D = 192, 4, 64
     HD = H * D
     q, k, v = (dyadic(g, S * HD) for _ in range(3))
     scale = 1.0 / np.sqrt(D)
@@ -244,6 +244,32 @@ def test_attention_views_qk_and_pv():
     want = oracle_matmul(np.zeros(S * HD, np.float16), p, v, H, S, S, D, so, sl, sr, mode=mode)
     o_t = to_dev(np.zeros(S * HD, np.float16))
     assert raw_matmul("adr_matmul_f16", o_t, to_dev(p), to_dev(v), H, S, S, D, so, sl, sr) == 0
+    assert np.array_equal(to_np(o_t).view(np.uint16), want.view(np.uint16))
+
+
+NN_SHAPES = [(2, 100, 128, 136), (1, 300, 64, 128), (3, 257, 192, 72), (1, 64, 64, 8),
+             (2, 513, 256, 264)]
+
+
+@pytest.mark.parametrize("shape", NN_SHAPES)
+@pytest.mark.parametrize("mask", [oracle.MASK_NONE, oracle.MASK_CAUSAL])
+def test_fast_nn_row_major_right_operand(shape, mask):
+    """Right operand stored [K, N] row-major (n contiguous), as V is in P.V: goes through the
+    transposing LDS reads.  Padded row and batch strides; dyadic inputs -> bit-exact."""
+    B, M, K, N = shape
+    g = rng(535 + M + N)
+    ly, ry, oy = K + 8, N + 16, N + 8
+    lz, rz, oz = M * ly + 16, K * ry + 8, M * oy + 24
+    so, sl, sr = (1, oy, oz), (1, ly, lz), (1, ry, rz)
+    assert plan(B, M, K, N, so, sl, sr, mask=mask).startswith("gemm_nn_mfma")
+    lbuf = (g.integers(-8, 9, size=B * lz + 8) / 64.0).astype(np.float16)
+    rbuf = (g.integers(-8, 9, size=B * rz + 8) / 64.0).astype(np.float16)
+    obuf = np.full(B * oz + 8, 3.0, np.float16)
+    want = oracle_matmul(obuf, lbuf, rbuf, B, M, K, N, so, sl, sr, mode=oracle.EXACT, mask=mask,
+                         offsets=(8, 8, 8))
+    o_t = to_dev(obuf)
+    assert raw_matmul("adr_matmul_f16", o_t, to_dev(lbuf), to_dev(rbuf), B, M, K, N, so, sl, sr,
+                      mask=mask, offsets=(8, 8, 8)) == 0
     assert np.array_equal(to_np(o_t).view(np.uint16), want.view(np.uint16))
 
 
