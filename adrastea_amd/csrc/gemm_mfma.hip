@@ -711,6 +711,13 @@ GemmChoice choose(const MatmulArgs& a) {
                 (uintptr_t)a.rhs_q % 8 != 0)) return GEMM_NONE;
   const bool plain = !a.rhs_q && a.load == ADR_LOAD_IDENTITY;
   if (plain && a.k % 64 == 0) {
+    // Few K slices: the tile is dominated by its load latency and its epilogue; two resident
+    // workgroups per CU overlap those phases, which one large tile cannot.
+    if (a.k <= 256) {
+      static const Candidate shortk[] = {{DMA_128x128, 128, 128, 2, 1.00f},
+                                         {DMA_64x64, 64, 64, 4, 0.50f}};
+      return pick(a, shortk, 2);
+    }
     static const Candidate dma[] = {
         {DMA_256x192, 256, 192, 1, 1.10f}, {DMA_256x128, 256, 128, 1, 1.00f},
         {DMA_128x128, 128, 128, 2, 0.80f}, {DMA_64x64, 64, 64, 4, 0.40f}};

@@ -41,9 +41,12 @@ DECODE_SET = [(4096, 4096), (4096, 11008), (4096, 12288), (11008, 4096)]
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--quick", action="store_true", help="skip secondary configs and CPU baseline")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run only a plain 256 MiB device copy (reference point for the "
+                         "FETCH_SIZE / WRITE_SIZE counters of rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures the single-GPU matmul path only; run with --gpus 1 "
@@ -59,6 +62,14 @@ def main():
         sys.exit(2)
     dev = "cuda:0"
     torch.cuda.set_device(0)
+    if args.copy_calibration:
+        src = torch.ones(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes": 256 << 20, "launches": 5}))
+        return
     gen = torch.Generator(device=dev).manual_seed(42)
     stream = lambda: torch.cuda.current_stream().cuda_stream  # noqa: E731
 
@@ -82,6 +93,31 @@ def main():
         e1.record()
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1e-3 / iters  # seconds per call
+
+    def timed_graph(fn, calls_per_graph, replays, warm_replays=3):
+        """Kernels of a few microseconds cannot be issued fast enough from Python: record
+        `calls_per_graph` launches into a HIP graph and time its replays (HIP events on the
+        launch stream), so that the figure is the device time per launch."""
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fn()  # first call outside capture (lazy module loading)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(calls_per_graph):
+                fn()
+        for _ in range(warm_replays):
+            graph.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(replays):
+            graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / (replays * calls_per_graph)
 
     # ---------------- primary workload: the fp16 layer GEMM set at M = 2048
     M = 2048
@@ -109,10 +145,10 @@ def main():
 
     # ---------------- roofline of the dominant kernel (HIP events on the launch stream)
     name, K, N = LAYER_SET[0]
-    t_qkv = timed(lambda: mm(outs[name], acts[K], weights[name], M, K, N), 30, 3)
+    t_qkv = timed(lambda: mm(outs[name], acts[K], weights[name], M, K, N), 200, 20)
     qkv_flops = 2.0 * M * K * N
     roofline = {
-        "kernel": "gemm_nt_mfma_256x128x32 (qkv: M2048 K4096 N12288)",
+        "kernel": "gemm_nt_dma_kernel<256,192,...> (qkv: M2048 K4096 N12288)",
         "bound": "mfma", "achieved": round(qkv_flops / t_qkv / 1e12, 2),
         "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
         "frac": round(qkv_flops / t_qkv / 1e12 / PEAK_F16_TFLOPS, 4),
@@ -125,7 +161,7 @@ def main():
         for name, K, N in LAYER_SET:
             if name == "up":
                 continue
-            t = timed(lambda: mm(outs[name], acts[K], weights[name], M, K, N), 20, 2)
+            t = timed(lambda: mm(outs[name], acts[K], weights[name], M, K, N), 100, 10)
             per_gemm[name] = {"M": M, "K": K, "N": N, "us": round(t * 1e6, 1),
                               "tflops": round(2.0 * M * K * N / t / 1e12, 1),
                               "frac_mfma_peak": round(2.0 * M * K * N / t / 1e12 / PEAK_F16_TFLOPS, 4)}
@@ -151,7 +187,7 @@ def main():
                                               qs[j].data_ptr(), ss[j].data_ptr(), m, K, N, 32, 0.0)
                 if rc != 0:
                     raise RuntimeError(_ffi.strerror(rc))
-            t = timed(f, iters, nbuf)
+            t = timed_graph(f, 2 * nbuf, max(2, iters // (2 * nbuf)))
             return t, per + m * K * 2 + m * N * 2
 
         gemv = []
@@ -179,7 +215,7 @@ def main():
                                               q.data_ptr(), s.data_ptr(), M, K, N, 32, 0.0)
                 if rc != 0:
                     raise RuntimeError(_ffi.strerror(rc))
-            t = timed(f, 10, 2)
+            t = timed(f, 50, 5)
             u8p[name] = {"M": M, "K": K, "N": N, "us": round(t * 1e6, 1),
                          "tflops": round(2.0 * M * K * N / t / 1e12, 1),
                          "frac_mfma_peak": round(2.0 * M * K * N / t / 1e12 / PEAK_F16_TFLOPS, 4)}
@@ -212,7 +248,7 @@ def main():
                                     1.0 / D ** 0.5, 4, 0, 0)
             if rc != 0:
                 raise RuntimeError(_ffi.strerror(rc))
-        t = timed(f_qk, 10, 2)
+        t = timed(f_qk, 50, 5)
         byts = 2 * S * HD * 2 + H * S * S * 2
         attn = {"qk_t": {"us": round(t * 1e6, 1), "tflops": round(2.0 * H * S * S * D / t / 1e12, 1),
                          "gbs": round(byts / t / 1e9, 1),
@@ -225,7 +261,7 @@ def main():
                                     D, 1, HD, D, 1, S, S * S, 1, HD, D, None, 0.0, 1.0, 0, 0, 0)
             if rc != 0:
                 raise RuntimeError(_ffi.strerror(rc))
-        t = timed(f_pv, 5, 1)
+        t = timed(f_pv, 50, 5)
         attn["pv"] = {"us": round(t * 1e6, 1), "tflops": round(2.0 * H * S * S * D / t / 1e12, 1),
                       "gbs": round(byts / t / 1e9, 1),
                       "frac_hbm_peak": round(byts / t / 1e9 / PEAK_HBM_GBS, 4)}
