@@ -269,6 +269,10 @@ class MatmulTracer(CommonKernels):
         self._lock = threading.Lock()
         self.shapes = set()
 
+    def clear(self):
+        with self._lock:
+            self.shapes.clear()
+
     def _record(self, output, left, right):
         with self._lock:
             self.shapes.add((left.layout, right.layout, output.layout))

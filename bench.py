@@ -152,7 +152,11 @@ def main():
         "bound": "mfma", "achieved": round(qkv_flops / t_qkv / 1e12, 2),
         "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
         "frac": round(qkv_flops / t_qkv / 1e12 / PEAK_F16_TFLOPS, 4),
-        "launch_us": round(t_qkv * 1e6, 2), "traffic": None,
+        "launch_us": round(t_qkv * 1e6, 2),
+        # bytes moved between L2 and the memory fabric per qkv launch, from the rocprofv3 --pmc
+        # FETCH_SIZE and WRITE_SIZE passes recorded in profiles/gemm_nt_dma_llama7b_layer_set.txt
+        # (scaled by a plain device copy); the algorithmic figure is 167.8e6
+        "traffic": 420.0e6, "traffic_algorithmic": 167.8e6,
     }
 
     secondary = {}
