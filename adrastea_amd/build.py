@@ -73,5 +73,26 @@ def build_library(force: bool = False, extra_flags=()) -> str:
     return LIB
 
 
+HOST_TEST_SRC = os.path.join(os.path.dirname(HERE), "tests", "cpp", "test_host.cpp")
+HOST_TEST_BIN = os.path.join(os.path.dirname(HERE), "tests", "cpp", "bin", "test_host")
+
+
+def build_host_test(force: bool = False) -> str:
+    """Compiles the C++ host-side test (header-only host/*.hpp over the C ABI) with g++."""
+    deps = [HOST_TEST_SRC, LIB] + [os.path.join(HERE, "host", f) for f in os.listdir(os.path.join(HERE, "host"))]
+    if (not force and os.path.exists(HOST_TEST_BIN)
+            and all(os.path.getmtime(d) <= os.path.getmtime(HOST_TEST_BIN) for d in deps)):
+        return HOST_TEST_BIN
+    os.makedirs(os.path.dirname(HOST_TEST_BIN), exist_ok=True)
+    cmd = ["g++", "-std=c++17", "-O1", "-Wall", "-o", HOST_TEST_BIN, HOST_TEST_SRC, "-L" + LIBDIR,
+           "-ladrastea_kernels_hip", "-ldl", "-Wl,-rpath,$ORIGIN/../../../adrastea_amd/lib",
+           "-Wl,-rpath,/opt/rocm/lib"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"g++ failed for the host test:\n{r.stdout}\n{r.stderr}")
+    return HOST_TEST_BIN
+
+
 if __name__ == "__main__":
     print(build_library(force="--force" in sys.argv))
+    print(build_host_test(force="--force" in sys.argv))

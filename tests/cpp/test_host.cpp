@@ -1,0 +1,126 @@
+// C++ host-side tests.  Without arguments: CPU-only checks of the layout algebra (the reference's
+// own unit tests, adrastea_models/src/tensor.rs:583-664, restated), the lowering rules
+// (kernels.rs:821-890) and kernel selection.  With "gpu": one matmul through GpuKernels on the
+// device (HIP runtime loaded with dlopen so that this file needs no HIP headers), checked against
+// a host triple loop on integer-valued inputs.
+#include <dlfcn.h>
+
+#include <cstdio>
+#include <cstring>
+#include <vector>
+
+#include "../../adrastea_amd/host/kernels.hpp"
+
+using namespace adrastea;
+
+static int failures = 0;
+#define CHECK(c) do { if (!(c)) { printf("FAIL %s:%d %s\n", __FILE__, __LINE__, #c); failures++; } } while (0)
+template <typename F> static bool throws(F f) { try { f(); } catch (const std::exception&) { return true; } return false; }
+
+static uint16_t f2h_small_int(int v) {  // exact fp16 of an integer |v| <= 2048
+  if (v == 0) return 0;
+  uint16_t sign = v < 0 ? 0x8000 : 0; unsigned a = v < 0 ? -v : v; int e = 0;
+  while ((a >> (e + 1)) != 0) e++;
+  return sign | (uint16_t)((e + 15) << 10) | (uint16_t)(((a << (10 - e)) & 0x3ff));
+}
+static int h2i(uint16_t h) {
+  if ((h & 0x7fff) == 0) return 0;
+  int e = ((h >> 10) & 31) - 15; int m = 0x400 | (h & 0x3ff); int v = e >= 10 ? m << (e - 10) : m >> (10 - e);
+  return (h & 0x8000) ? -v : v;
+}
+
+static void cpu_tests() {
+  CHECK((TensorLayout::row_major({2, 3, 4}).strides == std::vector<size_t>{12, 4, 1}));
+  CHECK((TensorLayout::column_major({3, 4}).strides == std::vector<size_t>{1, 4}));
+  CHECK((TensorLayout::row_major({3, 3}).permute({1, 0}).strides == std::vector<size_t>{1, 3}));
+  CHECK(TensorLayout::row_major({2, 3, 4}).largest_address() == 23);
+  CHECK(throws([] { TensorLayout({2, 0}, {1, 1}); }));
+  // shape_cast (tensor.rs:599-613) and its should_panic twin (:619-625)
+  auto c = TensorLayout::row_major({4, 4}).shape_cast({-1, 8});
+  CHECK((c.dims == std::vector<size_t>{2, 8}) && (c.strides == std::vector<size_t>{8, 1}));
+  CHECK(throws([] { TensorLayout::row_major({256}).shape_cast({16, 1}); }));
+  // skip_and_take (tensor.rs:627-664)
+  auto r = TensorLayout::row_major({256}).shape_cast({16, 16});
+  auto sk = r.skip({15, 0});
+  CHECK(sk.first == 240 && sk.second.size(-2) == 1 && sk.second.size(-1) == 16);
+  auto tk = r.skip({1, 0}).second.take({1, 16});
+  CHECK(r.skip({1, 0}).first == 16 && tk.size(-2) == 1 && tk.size(-1) == 16);
+  // LLaMA-7B attention views (llama.rs:534-554)
+  const size_t S = 2048, H = 32, D = 128;
+  auto base = TensorLayout::row_major({S, H * D});
+  auto q = base.shape_cast({(long)S, (long)H, -1}).permute({1, 0, 2});
+  auto k = base.shape_cast({(long)S, (long)H, -1}).permute({1, 2, 0});
+  auto qk = TensorLayout::row_major({H, S, S});
+  auto low = lower_matmul(qk, q, k, MatmulOptions::make().store(MatmulStore::Scale(0.0883883f)).mask(MatmulMask::Causal));
+  CHECK(low.batches == 32 && low.m == 2048 && low.k == 128 && low.n == 2048);
+  CHECK(low.sl[0] == 1 && low.sl[1] == 4096 && low.sl[2] == 128);
+  CHECK(low.sr[0] == 4096 && low.sr[1] == 1 && low.sr[2] == 128);
+  CHECK(low.so[0] == 1 && low.so[1] == 2048 && low.so[2] == 2048 * 2048);
+  CHECK(low.store == 4 && low.load == 0 && low.mask == 1 && low.beta == 0.0f);
+  // lowering rules
+  auto out = TensorLayout::row_major({5, 7}), lhs = TensorLayout::row_major({5, 3});
+  auto w = TensorLayout::row_major({7, 3}).permute({1, 0});
+  auto l2 = lower_matmul(TensorLayout::row_major({4, 5, 7}), TensorLayout::row_major({4, 5, 3}), w, MatmulOptions::make());
+  CHECK(l2.batches == 4 && l2.sr[2] == 0 && l2.sl[2] == 15);
+  auto l3 = lower_matmul(out, lhs, w, MatmulOptions::make().load(MatmulLoad::Scale(0.5f)).store(MatmulStore::Scale(0.25f)));
+  CHECK(l3.scale == 0.125f && l3.store == 4 && l3.load == 1);
+  CHECK(lower_matmul(out, lhs, w, MatmulOptions::make().store(MatmulStore::BetaBias(1.0f, nullptr))).beta == 1.0f);
+  CHECK(lower_matmul(out, lhs, w, MatmulOptions::make().store(MatmulStore::Add())).beta == 0.0f);
+  CHECK(throws([&] { lower_matmul(TensorLayout::row_major({5, 8}), lhs, w, MatmulOptions::make()); }));
+  CHECK(throws([&] { lower_matmul(out, TensorLayout::row_major({5, 4}), w, MatmulOptions::make()); }));
+  // kernel selection through the library (host only)
+  GpuKernels gk;
+  auto big_o = TensorLayout::row_major({2048, 12288}), big_l = TensorLayout::row_major({2048, 4096});
+  auto big_w = TensorLayout::row_major({12288, 4096}).permute({1, 0});
+  CHECK(gk.plan(big_o, big_l, big_w, MatmulOptions::make()).rfind("gemm_nt_mfma", 0) == 0);
+  CHECK(gk.plan(TensorLayout::row_major({10, 12}), TensorLayout::row_major({10, 7}), TensorLayout::row_major({7, 12}),
+                MatmulOptions::make()) == "matmul_general");
+  CHECK(throws([&] { gk.plan(out, lhs, w, MatmulOptions::make().store(MatmulStore::GeluBias(nullptr))); }));
+}
+
+static void gpu_test() {
+  void* hip = dlopen("libamdhip64.so", RTLD_NOW);
+  if (!hip) { printf("FAIL dlopen libamdhip64.so\n"); failures++; return; }
+  auto hipMalloc = (int (*)(void**, size_t))dlsym(hip, "hipMalloc");
+  auto hipMemcpy = (int (*)(void*, const void*, size_t, int))dlsym(hip, "hipMemcpy");
+  auto hipDeviceSynchronize = (int (*)())dlsym(hip, "hipDeviceSynchronize");
+  const int M = 70, K = 64, N = 96;
+  std::vector<uint16_t> a(M * K), w(N * K), o(M * N, 0);
+  unsigned s = 7;
+  auto rnd = [&] { s = s * 1664525u + 1013904223u; return (int)((s >> 16) % 7) - 3; };
+  for (auto& v : a) v = f2h_small_int(rnd());
+  for (auto& v : w) v = f2h_small_int(rnd());
+  uint16_t *da, *dw, *dout;
+  CHECK(hipMalloc((void**)&da, a.size() * 2) == 0 && hipMalloc((void**)&dw, w.size() * 2) == 0 &&
+        hipMalloc((void**)&dout, o.size() * 2) == 0);
+  hipMemcpy(da, a.data(), a.size() * 2, 1); hipMemcpy(dw, w.data(), w.size() * 2, 1); hipMemcpy(dout, o.data(), o.size() * 2, 1);
+  GpuKernels gk;
+  MatmulTracer tr(gk);
+  TensorView<f16> ov(dout, TensorLayout::row_major({(size_t)M, (size_t)N}));
+  TensorView<const f16> lv(da, TensorLayout::row_major({(size_t)M, (size_t)K}));
+  TensorView<const f16> wv(dw, TensorLayout::row_major({(size_t)N, (size_t)K}));
+  for (int slow = 0; slow < 2; slow++) {
+    if (slow) tr.matmul_f16_slow(ov, lv, wv.permute({1, 0}), MatmulOptions::make().mask(MatmulMask::Causal));
+    else tr.matmul_f16(ov, lv, wv.permute({1, 0}), MatmulOptions::make().mask(MatmulMask::Causal));
+    CHECK(hipDeviceSynchronize() == 0);
+    hipMemcpy(o.data(), dout, o.size() * 2, 2);
+    int bad = 0;
+    for (int y = 0; y < M; y++)
+      for (int x = 0; x < N; x++) {
+        if (x > y) { bad += o[y * N + x] != 0xFC00; continue; }
+        int ref = 0;
+        for (int k = 0; k < K; k++) ref += h2i(a[y * K + k]) * h2i(w[x * K + k]);
+        bad += h2i(o[y * N + x]) != ref;
+      }
+    CHECK(bad == 0);
+  }
+  CHECK(tr.shapes().size() == 1);
+  uint16_t bias = 0;
+  CHECK(throws([&] { tr.matmul_f16(ov, lv, wv.permute({1, 0}), MatmulOptions::make().store(MatmulStore::GeluBias(&bias))); }));
+}
+
+int main(int argc, char** argv) {
+  if (argc > 1 && !strcmp(argv[1], "gpu")) gpu_test(); else cpu_tests();
+  printf(failures ? "FAILED (%d)\n" : "OK\n", failures);
+  return failures != 0;
+}

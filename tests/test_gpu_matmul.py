@@ -432,3 +432,18 @@ def test_full_size_attention_products():
     rms = ref.pow(2).mean().sqrt()
     rel = ((o.float() - ref).abs() / torch.maximum(ref.abs(), rms)).max().item()
     assert rel <= TOL, rel
+
+
+def test_matmul_f16_raw_entry_point():
+    """matmul_f16_raw (matmul.cu:515-517): the 16 common arguments, identity operators."""
+    from adrastea_amd import _ffi
+    g = rng(580)
+    B, M, K, N = 2, 40, 64, 56
+    l, r = dyadic(g, B * M * K), dyadic(g, B * K * N)
+    so, sl, sr = (1, N, M * N), (1, K, M * K), (K, 1, K * N)
+    want = oracle_matmul(np.zeros(B * M * N, np.float16), l, r, B, M, K, N, so, sl, sr)
+    o_t, l_t, r_t = to_dev(np.zeros(B * M * N, np.float16)), to_dev(l), to_dev(r)
+    rc = _ffi.lib().adr_matmul_f16_raw(torch.cuda.current_stream().cuda_stream, o_t.data_ptr(),
+                                       l_t.data_ptr(), r_t.data_ptr(), B, M, K, N, *so, *sl, *sr)
+    assert rc == 0
+    assert np.array_equal(to_np(o_t).view(np.uint16), want.view(np.uint16))

@@ -249,3 +249,35 @@ def test_prefill_u8_gemm_full_size(kern):
     rms = ref32.pow(2).mean().sqrt()
     rel = ((out.float() - ref32).abs() / torch.maximum(ref32.abs(), rms)).max().item()
     assert rel <= 2e-3, rel
+
+
+def test_descriptor_forms_on_strided_views(kern):
+    """adr_dequantize_absmax_uint8 / adr_quantize_absmax_uint8 take the reference's by-value
+    TensorGpuDescriptor (index 0 = innermost dim, kernels.rs:28-61); views with row padding."""
+    from adrastea_amd import TensorView, TensorLayout
+    from adrastea_amd.kernels import descriptor
+    g = rng(640)
+    rows, cols, bs, pad = 7, 96, 32, 40
+    x = randn_f16(g, (rows, cols), 0.05)
+    xb = torch.zeros(rows, cols + pad, dtype=torch.float16, device="cuda")
+    xb[:, :cols] = to_dev(x)
+    qb = torch.zeros(rows, cols + pad, dtype=torch.uint8, device="cuda")
+    sb = torch.zeros(rows, cols // bs + 3, dtype=torch.float16, device="cuda")
+    xv = TensorView(xb, TensorLayout((rows, cols), (cols + pad, 1)))
+    qv = TensorView(qb, TensorLayout((rows, cols), (cols + pad, 1)))
+    sv = TensorView(sb, TensorLayout((rows, cols // bs), (cols // bs + 3, 1)))
+    lib = _ffi.lib()
+    assert lib.adr_quantize_absmax_uint8(None, descriptor(qv), descriptor(sv), descriptor(xv)) == 0
+    q_want, s_want = oracle.quantize_absmax_u8(x, bs)
+    assert np.array_equal(to_np(qb)[:, :cols], q_want)
+    assert np.all(to_np(qb)[:, cols:] == 0)
+    assert np.array_equal(to_np(sb)[:, :cols // bs].view(np.uint16), s_want.view(np.uint16))
+    ob = torch.full((rows, cols + pad), 9.0, dtype=torch.float16, device="cuda")
+    ov = TensorView(ob, TensorLayout((rows, cols), (cols + pad, 1)))
+    assert lib.adr_dequantize_absmax_uint8(None, descriptor(ov), descriptor(sv), descriptor(qv)) == 0
+    want = oracle.dequantize_absmax_u8(q_want, s_want, bs)
+    assert np.array_equal(to_np(ob)[:, :cols].view(np.uint16), want.view(np.uint16))
+    assert np.all(to_np(ob)[:, cols:] == 9.0)
+    # shape errors
+    bad = TensorView(sb, TensorLayout((rows + 1, cols // bs), (cols // bs + 3, 1)))
+    assert lib.adr_dequantize_absmax_uint8(None, descriptor(ov), descriptor(bad), descriptor(qv)) == -1
