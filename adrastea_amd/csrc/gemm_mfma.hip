@@ -400,6 +400,9 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   auto slice = [&](const unsigned char* cA, const unsigned char* cB, const unsigned char* nA,
                    const unsigned char* nB, unsigned char* dA, unsigned char* dB) {
     dma(dA, dB);
+    // pin the DMA issue to the head of the slice: sunk towards the wait below, the whole
+    // global -> LDS latency would be exposed
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int kk = 0; kk < KK; kk++) {
       if (kk + 1 < KK) {
