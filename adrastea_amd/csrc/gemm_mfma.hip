@@ -458,6 +458,177 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
 }
 
 // =============================================================================================
+// u8-weight kernel: left operand by DMA, weights dequantised on their way into LDS
+// =============================================================================================
+// K % 64 == 0, block size a power of two >= 8.  The fp16 left operand goes global -> LDS by DMA
+// through three stages (two slices ahead).  The u8 weights of slice kt+2 are fetched into
+// registers (8 weights + their scale per chunk, three chunks per lane) while slice kt runs; the
+// chunks of slice kt+1 are dequantised (bit-identical to quantize.cu:53-54) and written to one
+// of two fp16 LDS stages in the same swizzled layout the DMA produces, so that every weight is
+// dequantised once per workgroup and the MFMA loop is the one of the fp16 kernel.
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a, TileMap map,
+                                                                   int block_shift) {
+  constexpr int BK = 64, CPR = 8, KK = 4;
+  constexpr int NW = WM * WN, NT = NW * 64;
+  constexpr int IA = BM * CPR / NT;   // DMA instructions per lane and slice
+  constexpr int LB = BN * CPR / NT;   // 8-weight chunks per lane and slice
+  constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
+  constexpr int SLOT = 32 * (TN * 64 + 16);
+  static_assert(BM * CPR % NT == 0 && BN * CPR % NT == 0, "slices must split evenly over lanes");
+  static_assert((NW / 2) * SLOT <= BM * BK * 2, "epilogue slots must fit in two A stages");
+  __shared__ __attribute__((aligned(1024))) unsigned char sA0[BM * BK * 2];
+  __shared__ __attribute__((aligned(1024))) unsigned char sA1[BM * BK * 2];
+  __shared__ __attribute__((aligned(1024))) unsigned char sA2[BM * BK * 2];
+  __shared__ __attribute__((aligned(1024))) unsigned char sB0[BN * BK * 2];
+  __shared__ __attribute__((aligned(1024))) unsigned char sB1[BN * BK * 2];
+
+  int batch, tile_m, tile_n;
+  map_tile(map, batch, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  half_t* const out = a.output;
+
+  const half_t* gA[IA];
+#pragma unroll
+  for (int i = 0; i < IA; i++) {
+    int row, kc;
+    lds_chunk_inv<CPR>((i * NW + wave) * 64 + lane, row, kc);
+    gA[i] = a.lhs + (int64_t)min(m0 + row, a.m - 1) * a.stride_ly + kc * 8;
+  }
+  // weight chunk c = tid + i*NT -> (row, 8-weight group kc); rows beyond N are clamped
+  const uint8_t* gQ[LB];
+  const half_t* gS[LB];
+  int offB[LB];
+#pragma unroll
+  for (int i = 0; i < LB; i++) {
+    const int c = tid + i * NT, row = c / CPR, kc = c % CPR;
+    const int brow = min(n0 + row, a.n - 1);
+    gQ[i] = a.rhs_q + (int64_t)brow * a.k + kc * 8;
+    // block of weight k0 + 8*kc: k0 is a multiple of 64 and 8*kc < 64, so the two parts of the
+    // index add up exactly for any power-of-two block size
+    gS[i] = a.scales + (int64_t)brow * (a.k >> block_shift) + ((kc * 8) >> block_shift);
+    offB[i] = lds_chunk_off<CPR>(row, kc);
+  }
+  const int KT = a.k / BK;
+  int kloadA = 0, kloadQ = 0;
+  auto dmaA = [&](unsigned char* dA) {
+    const int k0 = min(kloadA, KT - 1) * BK;
+    kloadA++;
+#pragma unroll
+    for (int i = 0; i < IA; i++)
+      __builtin_amdgcn_global_load_lds(ADR_GLB_PTR(gA[i] + k0),
+                                       ADR_LDS_PTR(dA + (i * NW + wave) * 1024), 16, 0, 0);
+  };
+  u32x2_t rq[2][LB];
+  half_t rs[2][LB];
+  auto fetchQ = [&](int set) {
+    const int ks = min(kloadQ, KT - 1);
+    kloadQ++;
+#pragma unroll
+    for (int i = 0; i < LB; i++) {
+      rq[set][i] = *(const u32x2_t*)(gQ[i] + ks * BK);
+      rs[set][i] = gS[i][(ks * BK) >> block_shift];
+    }
+  };
+  auto dequant_store = [&](int set, unsigned char* dB) {
+#pragma unroll
+    for (int i = 0; i < LB; i++) {
+      const half2_t s2 = {rs[set][i], rs[set][i]};
+      *(half8_t*)(dB + offB[i]) = dequant8(rq[set][i][0], rq[set][i][1], s2);
+    }
+  };
+
+  float16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+  const int frow = lane & 31, fkg = lane >> 5;
+  int offFA[TM][KK], offFB[TN][KK];
+#pragma unroll
+  for (int kk = 0; kk < KK; kk++) {
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+      offFA[i][kk] = lds_chunk_off<CPR>(wm * WTM + i * 32 + frow, kk * 2 + fkg);
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+      offFB[j][kk] = lds_chunk_off<CPR>(wn * WTN + j * 32 + frow, kk * 2 + fkg);
+  }
+  half8_t fa[2][TM], fb[2][TN];
+  auto load_frags = [&](int slot, const unsigned char* cA, const unsigned char* cB, int kk) {
+#pragma unroll
+    for (int i = 0; i < TM; i++) fa[slot][i] = *(const half8_t*)(cA + offFA[i][kk]);
+#pragma unroll
+    for (int j = 0; j < TN; j++) fb[slot][j] = *(const half8_t*)(cB + offFB[j][kk]);
+  };
+  auto mfmas = [&](int slot) {
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[slot][j], fa[slot][i], acc[i][j],
+                                                           0, 0, 0);
+  };
+  // Slice kt.  (cA, cB): its stages; (nA, nB): those of slice kt+1 -- nB is filled here from
+  // register set `nset`; dA: the A stage refilled with slice kt+2; `fset`: the register set
+  // that receives the weights of slice kt+2 (the one slice kt was dequantised from).
+  auto slice = [&](const unsigned char* cA, const unsigned char* cB, const unsigned char* nA,
+                   unsigned char* nB, unsigned char* dA, int fset, int nset) {
+    fetchQ(fset);
+    dmaA(dA);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++) {
+      if (kk + 1 < KK) load_frags((kk + 1) & 1, cA, cB, kk + 1);
+      if (kk == 1) dequant_store(nset, nB);
+      mfmas(kk & 1);
+    }
+    // A(kt+1) has landed: only the weight fetch and the DMA issued in this slice may still be
+    // in flight; the dequantised weights of slice kt+1 are in LDS
+    constexpr int n = 2 * LB + IA;
+    __builtin_amdgcn_s_waitcnt(0x0070 | (n & 0xF) | ((n >> 4) << 14));
+    __builtin_amdgcn_s_barrier();
+    load_frags(0, nA, nB, 0);
+  };
+
+  fetchQ(0);
+  fetchQ(1);
+  dmaA(sA0);
+  dmaA(sA1);
+  dequant_store(0, sB0);
+  {
+    constexpr int n = IA;
+    __builtin_amdgcn_s_waitcnt(0x0070 | (n & 0xF) | ((n >> 4) << 14));
+    __builtin_amdgcn_s_barrier();
+  }
+  load_frags(0, sA0, sB0, 0);
+  int kt = 0;
+  for (; kt + 6 <= KT; kt += 6) {
+    slice(sA0, sB0, sA1, sB1, sA2, 0, 1);
+    slice(sA1, sB1, sA2, sB0, sA0, 1, 0);
+    slice(sA2, sB0, sA0, sB1, sA1, 0, 1);
+    slice(sA0, sB1, sA1, sB0, sA2, 1, 0);
+    slice(sA1, sB0, sA2, sB1, sA0, 0, 1);
+    slice(sA2, sB1, sA0, sB0, sA1, 1, 0);
+  }
+  if (kt < KT) { slice(sA0, sB0, sA1, sB1, sA2, 0, 1); kt++; }
+  if (kt < KT) { slice(sA1, sB1, sA2, sB0, sA0, 1, 0); kt++; }
+  if (kt < KT) { slice(sA2, sB0, sA0, sB1, sA1, 0, 1); kt++; }
+  if (kt < KT) { slice(sA0, sB1, sA1, sB0, sA2, 1, 0); kt++; }
+  if (kt < KT) { slice(sA1, sB0, sA2, sB1, sA0, 0, 1); kt++; }
+  __builtin_amdgcn_s_waitcnt(0x0070);
+  __builtin_amdgcn_s_barrier();
+
+  unsigned char* slot = (wave < NW / 2 ? sA0 : sA1) + (wave % (NW / 2)) * SLOT;
+  wave_epilogue<TM, TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, slot, (half_t)a.scale, lane);
+}
+
+// =============================================================================================
 // Register-staged kernel (any K % 8 == 0; Load Scale; u8 weights)
 // =============================================================================================
 template <int BM, int BN, int BK, int WM, int WN, int MINB, bool LOAD_SCALE, bool WQ>
@@ -662,8 +833,18 @@ hipError_t launch_stage(hipStream_t stream, const MatmulArgs& a) {
   return hipGetLastError();
 }
 
+template <int BM, int BN, int WM, int WN>
+hipError_t launch_u8(hipStream_t stream, const MatmulArgs& a) {
+  TileMap map = make_map(a, BM, BN);
+  if (map.total < 0) return hipErrorInvalidConfiguration;
+  hipLaunchKernelGGL((gemm_nt_u8_kernel<BM, BN, WM, WN>), dim3((unsigned)map.total),
+                     dim3(WM * WN * 64), 0, stream, a, map, __builtin_ctz(a.block_size));
+  return hipGetLastError();
+}
+
 enum GemmChoice {
   GEMM_NONE = 0,
+  U8_256x192, U8_256x128,
   DMA_256x192, DMA_256x128, DMA_128x128, DMA_64x64,
   DMA_NN_256x128, DMA_NN_128x128,
   STAGE_256x128, STAGE_128x128, STAGE_64x64,
@@ -726,6 +907,11 @@ GemmChoice choose(const MatmulArgs& a) {
         {DMA_128x128, 128, 128, 2, 0.80f}, {DMA_64x64, 64, 64, 4, 0.40f}};
     return pick(a, dma, 4);
   }
+  if (a.rhs_q && a.k % 64 == 0 && a.block_size >= 8 && (a.block_size & (a.block_size - 1)) == 0 &&
+      (int64_t)a.m * a.n >= 256 * 1024) {
+    static const Candidate u8[] = {{U8_256x192, 256, 192, 1, 1.10f}, {U8_256x128, 256, 128, 1, 1.00f}};
+    return pick(a, u8, 2);
+  }
   static const Candidate stage[] = {{STAGE_256x128, 256, 128, 2, 1.00f},
                                     {STAGE_128x128, 128, 128, 2, 0.85f},
                                     {STAGE_64x64, 64, 64, 4, 0.45f}};
@@ -736,6 +922,8 @@ GemmChoice choose(const MatmulArgs& a) {
 
 bool mfma_gemm_supported(const MatmulArgs& a, const char** name) {
   switch (choose(a)) {
+    case U8_256x192: *name = "gemm_nt_u8_mfma_256x192x64"; return true;
+    case U8_256x128: *name = "gemm_nt_u8_mfma_256x128x64"; return true;
     case DMA_256x192: *name = "gemm_nt_mfma_dma_256x192x64"; return true;
     case DMA_256x128: *name = "gemm_nt_mfma_dma_256x128x64"; return true;
     case DMA_128x128: *name = "gemm_nt_mfma_dma_128x128x64"; return true;
@@ -751,6 +939,8 @@ bool mfma_gemm_supported(const MatmulArgs& a, const char** name) {
 
 hipError_t launch_mfma_gemm(hipStream_t stream, const MatmulArgs& a) {
   switch (choose(a)) {
+    case U8_256x192: return launch_u8<256, 192, 4, 2>(stream, a);
+    case U8_256x128: return launch_u8<256, 128, 4, 2>(stream, a);
     case DMA_256x192: return launch_dma<256, 192, 4, 2, 2, 1>(stream, a);
     case DMA_256x128: return launch_dma<256, 128, 4, 2, 3, 1>(stream, a);
     case DMA_128x128: return launch_dma<128, 128, 2, 2, 2, 2>(stream, a);

@@ -188,6 +188,26 @@ def test_u8_matmul_random_matches_oracle_and_reference_kernel(kern, ref, m):
     assert np.max(ulp_diff_f16(naive, to_np(o_ref))) <= 1
 
 
+@pytest.mark.parametrize("case", [(300, 64, 1000, 32), (257, 128, 1030, 8), (512, 192, 520, 16),
+                                  (260, 320, 1100, 64), (1024, 384, 300, 128), (1024, 448, 300, 64), (256, 832, 1024, 32),
+                                  (700, 768, 400, 256)],
+                         ids=lambda c: "M%d_K%d_N%d_bs%d" % c)
+def test_u8_prefill_kernel_ragged_tiles_and_k_tails_bit_exact(kern, case):
+    """The DMA + dequant-while-staging kernel (m*n >= 256 Ki, K % 64 == 0, power-of-two blocks):
+    partial tiles in M and N, every remainder of the six-slice unrolled K loop, block sizes
+    below, at and above the slice depth, and the beta path -- exact inputs, compared bit for bit."""
+    m, p, n, bs = case
+    g = rng(640 + m + p)
+    a, q, s = _u8_case(g, m, p, n, bs, exact=True)
+    for beta in (0.0, 1.0):
+        prev = (g.integers(-8, 9, size=(m, n)) / 4.0).astype(np.float16)
+        want = prev.copy()
+        oracle.matmul_nt_fp16u8(want, a, q, s, bs, beta=beta, threads=8)
+        out = to_dev(prev)
+        kern.matmul_nt_fp16u8(out, to_dev(a), to_dev(q), to_dev(s), bs, beta=beta)
+        assert np.array_equal(to_np(out).view(np.uint16), want.view(np.uint16)), (case, beta)
+
+
 def test_u8_other_block_sizes_and_fallbacks(kern):
     g = rng(630)
     for m, p, n, bs in [(4, 512, 40, 64), (4, 384, 40, 128), (3, 96, 20, 8), (2, 48, 10, 16),
