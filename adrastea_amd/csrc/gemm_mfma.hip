@@ -167,9 +167,47 @@ __device__ __forceinline__ void wave_epilogue(const MatmulArgs& a, half_t* out,
                                               unsigned char* slot, half_t hscale, int lane) {
   Epilogue ep{a.bias, a.beta, hscale, a.store};
   const int lrow = lane & 31, g = lane >> 5;
+  constexpr int PITCH = TN * 64 + 16;  // bytes per staged row (TN*32 halves + pad)
+  constexpr int CPW = TN * 4;          // 16-byte chunks per staged row
+  // Common case, straight-line: the sub-tile lies inside the matrix and (for a causal product)
+  // on or below the diagonal, the operator is Identity or Scale, rows are 16-byte aligned.
+  const bool plain_op = a.store == ADR_STORE_IDENTITY || a.store == ADR_STORE_SCALE;
+  const bool inside = y0 + TM * 32 <= a.m && x0 + TN * 32 <= a.n;
+  const bool unmasked = a.mask != ADR_MASK_CAUSAL || x0 + TN * 32 - 1 <= y0;
+  if (plain_op && inside && unmasked && !(a.stride_oy & 7) && !((uintptr_t)out & 15)) {
+    const half_t mul = a.store == ADR_STORE_SCALE ? hscale : (half_t)1.0f;
+    // store round `it` of a 32-row block: lane -> 16-byte chunk it*64 + lane of the staged block
+    int rd[TN * 2];
+    int64_t po[TN * 2];
+#pragma unroll
+    for (int it = 0; it < TN * 2; it++) {
+      const int idx = it * 64 + lane, row = idx / CPW, c = idx % CPW;
+      rd[it] = row * PITCH + c * 16;
+      po[it] = (int64_t)row * a.stride_oy + c * 8;
+    }
+    half_t* const p0 = out + (int64_t)y0 * a.stride_oy + x0;
+    const int64_t blk = (int64_t)32 * a.stride_oy;
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          half4_t h;
+#pragma unroll
+          for (int e = 0; e < 4; e++) h[e] = (half_t)acc[i][j][4 * q + e];
+          // x * 1 is exact, so one multiply serves both operators (matmul.cu Scale: fp16 product)
+          *(half4_t*)(slot + lrow * PITCH + (j * 32 + 8 * q + 4 * g) * 2) = h * mul;
+        }
+#pragma unroll
+      for (int it = 0; it < TN * 2; it++) {
+        const half8_t v = *(const half8_t*)(slot + rd[it]);
+        *(half8_t*)(p0 + i * blk + po[it]) = v;
+      }
+    }
+    return;
+  }
   if (out_vectorizable(a, out)) {
-    constexpr int PITCH = TN * 64 + 16;  // bytes per staged row (TN*32 halves + pad)
-    constexpr int CPW = TN * 4;          // 16-byte chunks per staged row
 #pragma unroll
     for (int i = 0; i < TM; i++) {
 #pragma unroll
@@ -458,6 +496,168 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
 }
 
 // =============================================================================================
+// Short-K persistent kernel (K == 64 or K == 128): QK^T-shaped products
+// =============================================================================================
+// With one or two K slices a tile is all load latency and epilogue, and the job is bound by the
+// output writes.  One workgroup per CU walks a sequence of 128x128 tiles: the whole K extent of
+// a tile's two panels sits in one of two LDS buffers.  Wavefronts 4..7 only load: they wait for
+// the DMA of tile i, meet the others at the barrier and issue the DMA of tile i+1.  Wavefronts
+// 0..3 (2 x 2, 64 x 64 each) only multiply and store: their output writes are never waited for
+// (a wavefront's memory counter covers its own loads and stores alike, which is why the two
+// roles are kept in different wavefronts), so loads, MFMAs and the writes of neighbouring tiles
+// overlap and no workgroup launch is paid per tile.
+struct ShortKMap {
+  int tiles_m, tiles_n, tiles_per_batch, total;
+};
+
+template <int CPR>  // 16-byte chunks per row: 8 (K = 64) or 16 (K = 128)
+__global__ __launch_bounds__(512, 1) void gemm_nt_shortk_kernel(MatmulArgs a, ShortKMap map) {
+  constexpr int BM = 128, BN = 128, NWC = 4, NWL = 4, NTC = NWC * 64, KK = CPR / 2;
+  constexpr int TM = 2, TN = 2;
+  constexpr int IT = BM * CPR / (NWL * 64);    // DMA instructions per loader lane and operand
+  constexpr int ROWS_PER_I = NWL * 64 / CPR;   // rows between a lane's successive instructions
+  constexpr int SLOT = 32 * (TN * 64 + 16);
+  __shared__ __attribute__((aligned(1024))) unsigned char sA0[BM * CPR * 16];
+  __shared__ __attribute__((aligned(1024))) unsigned char sA1[BM * CPR * 16];
+  __shared__ __attribute__((aligned(1024))) unsigned char sB0[BN * CPR * 16];
+  __shared__ __attribute__((aligned(1024))) unsigned char sB1[BN * CPR * 16];
+  __shared__ __attribute__((aligned(1024))) unsigned char sEpi[NWC * SLOT];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int G = gridDim.x;
+
+  // step t of this workgroup -> linear tile.  Workgroup g runs on die g % 8; the workgroups of a
+  // die take consecutive tiles (two tile rows of one batch for 32 workgroups) so that they share
+  // panels in the die's L2 and write neighbouring output rows.
+  auto tile_of = [&](int t) -> int {
+    const int g = blockIdx.x;
+    if (G % XCDS == 0) {
+      const int per = G / XCDS;
+      return (t * XCDS + g % XCDS) * per + g / XCDS;
+    }
+    return t * G + g;
+  };
+  struct Tile { int batch, m0, n0; bool valid, masked; };
+  auto decode = [&](int t) -> Tile {
+    Tile r;
+    const int L = tile_of(t);
+    r.valid = L < map.total;
+    const int Lc = r.valid ? L : 0;
+    r.batch = Lc / map.tiles_per_batch;
+    const int rem = Lc - r.batch * map.tiles_per_batch;
+    const int tm = rem / map.tiles_n;
+    r.m0 = tm * BM;
+    r.n0 = (rem - tm * map.tiles_n) * BN;
+    r.masked = a.mask == ADR_MASK_CAUSAL && r.n0 > r.m0 + BM - 1;
+    return r;
+  };
+
+  if (wave >= NWC) {
+    // ---------------------------------------------------------------- loader wavefronts
+    const int lw = wave - NWC;
+    // the lane's place in a DMA instruction does not depend on the instruction index
+    int drow, dkc;
+    lds_chunk_inv<CPR>(lw * 64 + lane, drow, dkc);
+    auto dma = [&](const Tile& t, unsigned char* dA, unsigned char* dB) {
+      const half_t* A = a.lhs + (int64_t)t.batch * a.stride_lz + dkc * 8;
+      const half_t* B = a.rhs + (int64_t)t.batch * a.stride_rz + dkc * 8;
+#pragma unroll
+      for (int i = 0; i < IT; i++) {
+        const int row = drow + i * ROWS_PER_I;
+        __builtin_amdgcn_global_load_lds(
+            ADR_GLB_PTR(A + (int64_t)min(t.m0 + row, a.m - 1) * a.stride_ly),
+            ADR_LDS_PTR(dA + (i * NWL + lw) * 1024), 16, 0, 0);
+      }
+#pragma unroll
+      for (int i = 0; i < IT; i++) {
+        const int row = drow + i * ROWS_PER_I;
+        __builtin_amdgcn_global_load_lds(
+            ADR_GLB_PTR(B + (int64_t)min(t.n0 + row, a.n - 1) * a.stride_rx),
+            ADR_LDS_PTR(dB + (i * NWL + lw) * 1024), 16, 0, 0);
+      }
+    };
+    Tile cur = decode(0);
+    if (!cur.valid) return;
+    if (!cur.masked) dma(cur, sA0, sB0);
+    for (int it = 0;; it += 2) {
+      Tile nxt = decode(it + 1);
+      __builtin_amdgcn_s_waitcnt(0x0070);  // tile `it` has landed
+      __builtin_amdgcn_s_barrier();        // ... and tile it-1 has been read by everyone
+      if (!nxt.valid) break;
+      if (!nxt.masked) dma(nxt, sA1, sB1);
+      cur = decode(it + 2);
+      __builtin_amdgcn_s_waitcnt(0x0070);
+      __builtin_amdgcn_s_barrier();
+      if (!cur.valid) break;
+      if (!cur.masked) dma(cur, sA0, sB0);
+    }
+    return;
+  }
+
+  // ------------------------------------------------------------------ compute wavefronts
+  const int wm = wave >> 1, wn = wave & 1;
+  const int frow = lane & 31, fkg = lane >> 5;
+  int offA[TM], offB[TN];  // k-step 0; k-step kk is at (off ^ (kk << 5))
+#pragma unroll
+  for (int i = 0; i < TM; i++) offA[i] = lds_chunk_off<CPR>(wm * 64 + i * 32 + frow, fkg);
+#pragma unroll
+  for (int j = 0; j < TN; j++) offB[j] = lds_chunk_off<CPR>(wn * 64 + j * 32 + frow, fkg);
+  unsigned char* const slot = sEpi + wave * SLOT;
+  const half_t hscale = (half_t)a.scale;
+
+  auto compute_store = [&](const Tile& t, const unsigned char* cA, const unsigned char* cB) {
+    float16_t acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+    half8_t fa[2][TM], fb[2][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++) fa[0][i] = *(const half8_t*)(cA + offA[i]);
+#pragma unroll
+    for (int j = 0; j < TN; j++) fb[0][j] = *(const half8_t*)(cB + offB[j]);
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++) {
+      if (kk + 1 < KK) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+          fa[(kk + 1) & 1][i] = *(const half8_t*)(cA + (offA[i] ^ ((kk + 1) << 5)));
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+          fb[(kk + 1) & 1][j] = *(const half8_t*)(cB + (offB[j] ^ ((kk + 1) << 5)));
+      }
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[kk & 1][j], fa[kk & 1][i],
+                                                             acc[i][j], 0, 0, 0);
+    }
+    half_t* const out = a.output + (int64_t)t.batch * a.stride_oz;
+    wave_epilogue<TM, TN>(a, out, acc, t.m0 + wm * 64, t.n0 + wn * 64, slot, hscale, lane);
+  };
+  auto step = [&](const Tile& cur, const unsigned char* cA, const unsigned char* cB) {
+    __builtin_amdgcn_s_barrier();
+    if (cur.masked) {
+      fill_masked_tile<BM, BN, NTC>(a, a.output + (int64_t)cur.batch * a.stride_oz, cur.m0,
+                                    cur.n0, tid);
+    } else {
+      compute_store(cur, cA, cB);
+    }
+  };
+  for (int it = 0;; it += 2) {
+    Tile cur = decode(it);
+    if (!cur.valid) break;
+    step(cur, sA0, sB0);
+    cur = decode(it + 1);
+    if (!cur.valid) break;
+    step(cur, sA1, sB1);
+  }
+}
+
+// =============================================================================================
 // u8-weight kernel: left operand by DMA, weights dequantised on their way into LDS
 // =============================================================================================
 // K % 64 == 0, block size a power of two >= 8.  The fp16 left operand goes global -> LDS by DMA
@@ -587,6 +787,19 @@ __global__ __launch_bounds__(WM* WN * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a
       if (kk + 1 < KK) load_frags((kk + 1) & 1, cA, cB, kk + 1);
       if (kk == 1) dequant_store(nset, nB);
       mfmas(kk & 1);
+      if (kk + 1 < KK) {
+        // fragment reads behind the first MFMAs of the k-step; the dequantisation (VALU and
+        // LDS writes) of k-step 1 fills the gaps between the remaining ones
+#pragma unroll
+        for (int q = 0; q < TM * TN; q++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          if (kk == 1) {
+            __builtin_amdgcn_sched_group_barrier(0x002, 2 * LB * 8 / (TM * TN) + 1, 0);
+            if (q % 2 == 1) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+          }
+        }
+      }
     }
     // A(kt+1) has landed: only the weight fetch and the DMA issued in this slice may still be
     // in flight; the dequantised weights of slice kt+1 are in LDS
@@ -842,8 +1055,25 @@ hipError_t launch_u8(hipStream_t stream, const MatmulArgs& a) {
   return hipGetLastError();
 }
 
+constexpr int NUM_CU = 256;
+
+template <int CPR>
+hipError_t launch_shortk(hipStream_t stream, const MatmulArgs& a) {
+  ShortKMap map;
+  map.tiles_m = (a.m + 127) / 128;
+  map.tiles_n = (a.n + 127) / 128;
+  map.tiles_per_batch = map.tiles_m * map.tiles_n;
+  const int64_t total = (int64_t)map.tiles_per_batch * a.batches;
+  if (total > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+  map.total = (int)total;
+  const unsigned grid = total < NUM_CU ? (unsigned)total : NUM_CU;
+  hipLaunchKernelGGL((gemm_nt_shortk_kernel<CPR>), dim3(grid), dim3(512), 0, stream, a, map);
+  return hipGetLastError();
+}
+
 enum GemmChoice {
   GEMM_NONE = 0,
+  SHORTK_64, SHORTK_128,
   U8_256x192, U8_256x128,
   DMA_256x192, DMA_256x128, DMA_128x128, DMA_64x64,
   DMA_NN_256x128, DMA_NN_128x128,
@@ -856,8 +1086,6 @@ struct Candidate {
   int slots;   // workgroups resident per CU
   float eff;   // measured relative throughput of one busy CU with this tile
 };
-
-constexpr int NUM_CU = 256;
 
 // Estimated cost: rounds of resident workgroups times the work of one tile over its efficiency.
 GemmChoice pick(const MatmulArgs& a, const Candidate* c, int n) {
@@ -897,6 +1125,9 @@ GemmChoice choose(const MatmulArgs& a) {
   if (plain && a.k % 64 == 0) {
     // Few K slices: the tile is dominated by its load latency and its epilogue; two resident
     // workgroups per CU overlap those phases, which one large tile cannot.
+    if ((a.k == 64 || a.k == 128) &&
+        (int64_t)((a.m + 127) / 128) * ((a.n + 127) / 128) * a.batches >= 2 * NUM_CU)
+      return a.k == 64 ? SHORTK_64 : SHORTK_128;
     if (a.k <= 256) {
       static const Candidate shortk[] = {{DMA_128x128, 128, 128, 2, 1.00f},
                                          {DMA_64x64, 64, 64, 4, 0.50f}};
@@ -922,6 +1153,8 @@ GemmChoice choose(const MatmulArgs& a) {
 
 bool mfma_gemm_supported(const MatmulArgs& a, const char** name) {
   switch (choose(a)) {
+    case SHORTK_64: *name = "gemm_nt_mfma_persistent_128x128_k64"; return true;
+    case SHORTK_128: *name = "gemm_nt_mfma_persistent_128x128_k128"; return true;
     case U8_256x192: *name = "gemm_nt_u8_mfma_256x192x64"; return true;
     case U8_256x128: *name = "gemm_nt_u8_mfma_256x128x64"; return true;
     case DMA_256x192: *name = "gemm_nt_mfma_dma_256x192x64"; return true;
@@ -939,6 +1172,8 @@ bool mfma_gemm_supported(const MatmulArgs& a, const char** name) {
 
 hipError_t launch_mfma_gemm(hipStream_t stream, const MatmulArgs& a) {
   switch (choose(a)) {
+    case SHORTK_64: return launch_shortk<8>(stream, a);
+    case SHORTK_128: return launch_shortk<16>(stream, a);
     case U8_256x192: return launch_u8<256, 192, 4, 2>(stream, a);
     case U8_256x128: return launch_u8<256, 128, 4, 2>(stream, a);
     case DMA_256x192: return launch_dma<256, 192, 4, 2, 2, 1>(stream, a);

@@ -247,6 +247,57 @@ def test_attention_views_qk_and_pv():
     assert np.array_equal(to_np(o_t).view(np.uint16), want.view(np.uint16))
 
 
+SHORTK = [
+    # (B, M, K, N): at least 512 tiles of 128x128 so that the persistent kernel is selected
+    (9, 1000, 128, 1000),    # ragged tiles in M and N, 64 tiles per batch
+    (40, 500, 64, 450),      # K = 64 variant, 16 tiles per batch
+    (3, 1700, 128, 1800),    # more tiles than workgroups per batch, odd tile counts
+]
+
+
+@pytest.mark.parametrize("shape", SHORTK, ids=lambda c: "B%d_M%d_K%d_N%d" % c)
+@pytest.mark.parametrize("mask", [oracle.MASK_NONE, oracle.MASK_CAUSAL])
+def test_persistent_short_k_kernel_head_views(shape, mask):
+    """QK^T-shaped products (K = head size) on interleaved head views as in llama.rs:534-545:
+    every workgroup walks several tiles, including ragged, diagonal and fully masked ones."""
+    B, M, K, N = shape
+    g = rng(900 + B + M + mask)
+    HD = B * K
+    # heads interleaved in the rows of [S, H*D] buffers; output [H, M, N] with padded rows
+    NP = N + 8
+    so, sl, sr = (1, NP, M * NP), (1, HD, K), (HD, 1, K)
+    assert plan(B, M, K, N, so, sl, sr, store=oracle.STORE_SCALE, mask=mask).startswith(
+        "gemm_nt_mfma_persistent")
+    l, r = dyadic(g, M * HD), dyadic(g, N * HD)
+    prev = randn_f16(g, B * M * NP)
+    kw = dict(store=oracle.STORE_SCALE, scale=0.125, mask=mask)
+    want = oracle_matmul(prev, l, r, B, M, K, N, so, sl, sr, mode=oracle.EXACT, **kw)
+    o_t = to_dev(prev)
+    assert raw_matmul("adr_matmul_f16", o_t, to_dev(l), to_dev(r), B, M, K, N, so, sl, sr, **kw) == 0
+    assert np.array_equal(to_np(o_t).view(np.uint16), want.view(np.uint16))
+
+
+@pytest.mark.parametrize("store", [oracle.STORE_ADD] + STORES_F32)
+def test_persistent_short_k_kernel_epilogues(store):
+    g = rng(950 + store)
+    B, M, K, N = 20, 640, 128, 650
+    so, sl, sr = (1, N, M * N), (1, K, M * K), (K, 1, K * N)
+    assert plan(B, M, K, N, so, sl, sr, store=store).startswith("gemm_nt_mfma_persistent")
+    l = (g.integers(-16, 17, size=B * M * K) / 16.0).astype(np.float16)
+    r = (g.integers(-16, 17, size=B * K * N) / 16.0).astype(np.float16)
+    prev, bias = randn_f16(g, B * M * N), randn_f16(g, N)
+    kw = dict(beta=0.7, scale=0.2, store=store, mask=oracle.MASK_CAUSAL)
+    want = oracle_matmul(prev, l, r, B, M, K, N, so, sl, sr, bias=bias, mode=oracle.EXACT, **kw)
+    o_t = to_dev(prev)
+    assert raw_matmul("adr_matmul_f16", o_t, to_dev(l), to_dev(r), B, M, K, N, so, sl, sr,
+                      bias_t=to_dev(bias), **kw) == 0
+    got = to_np(o_t)
+    if store in STORES_EXACT:
+        assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    else:
+        assert np.max(ulp_diff_f16(got, want)) <= 2
+
+
 NN_SHAPES = [(2, 100, 128, 136), (1, 300, 64, 128), (3, 257, 192, 72), (1, 64, 64, 8),
              (2, 513, 256, 264)]
 
