@@ -499,97 +499,118 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
 // Short-K persistent kernel (K == 64 or K == 128): QK^T-shaped products
 // =============================================================================================
 // With one or two K slices a tile is all load latency and epilogue, and the job is bound by the
-// output writes.  One workgroup per CU walks a sequence of 128x128 tiles: the whole K extent of
-// a tile's two panels sits in one of two LDS buffers.  Wavefronts 4..7 only load: they wait for
-// the DMA of tile i, meet the others at the barrier and issue the DMA of tile i+1.  Wavefronts
-// 0..3 (2 x 2, 64 x 64 each) only multiply and store: their output writes are never waited for
-// (a wavefront's memory counter covers its own loads and stores alike, which is why the two
-// roles are kept in different wavefronts), so loads, MFMAs and the writes of neighbouring tiles
-// overlap and no workgroup launch is paid per tile.
+// output writes.  One workgroup per CU walks segments of tile rows (128 x 128 tiles): the left
+// panel of the segment stays in LDS, the right panels stream through a ring of three buffers.
+// Wavefronts 4..7 only load: they keep the DMA two tiles ahead, wait for the panel of tile j and
+// meet the others at a barrier.  Wavefronts 0..3 (2 x 2, 64 x 64 each) only multiply and store:
+// their output writes are never waited for (a wavefront's memory counter covers its own loads
+// and stores alike, which is why the two roles live in different wavefronts), so loads, MFMAs
+// and the writes of neighbouring tiles overlap and no workgroup launch is paid per tile.
 struct ShortKMap {
-  int tiles_m, tiles_n, tiles_per_batch, total;
+  int tiles_m, tiles_n, rows;   // rows = batches * tiles_m
+  int seg, segs_per_row, units; // a unit is `seg` consecutive tiles of one tile row
 };
 
 template <int CPR>  // 16-byte chunks per row: 8 (K = 64) or 16 (K = 128)
 __global__ __launch_bounds__(512, 1) void gemm_nt_shortk_kernel(MatmulArgs a, ShortKMap map) {
-  constexpr int BM = 128, BN = 128, NWC = 4, NWL = 4, NTC = NWC * 64, KK = CPR / 2;
-  constexpr int TM = 2, TN = 2;
-  constexpr int IT = BM * CPR / (NWL * 64);    // DMA instructions per loader lane and operand
+  constexpr int BM = 128, BN = 128, NWC = 4, NWL = 4, KK = CPR / 2;
+  constexpr int TM = 2, TN = 2, RING = 3;
+  constexpr int IT = BM * CPR / (NWL * 64);    // DMA instructions per loader lane and panel
   constexpr int ROWS_PER_I = NWL * 64 / CPR;   // rows between a lane's successive instructions
+  constexpr int PANEL = BM * CPR * 16;         // bytes of one 128-row panel
   constexpr int SLOT = 32 * (TN * 64 + 16);
-  __shared__ __attribute__((aligned(1024))) unsigned char sA0[BM * CPR * 16];
-  __shared__ __attribute__((aligned(1024))) unsigned char sA1[BM * CPR * 16];
-  __shared__ __attribute__((aligned(1024))) unsigned char sB0[BN * CPR * 16];
-  __shared__ __attribute__((aligned(1024))) unsigned char sB1[BN * CPR * 16];
+  __shared__ __attribute__((aligned(1024))) unsigned char sA[PANEL];
+  __shared__ __attribute__((aligned(1024))) unsigned char sB[RING * PANEL];
   __shared__ __attribute__((aligned(1024))) unsigned char sEpi[NWC * SLOT];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int G = gridDim.x;
+  // Workgroup g runs on die g % 8: the workgroups of a die take neighbouring units (they share
+  // right panels in the die's L2).  Odd rounds walk the workgroups backwards, which pairs long
+  // and short rows of a causal product.
+  const int gl = G % XCDS == 0 ? (blockIdx.x % XCDS) * (G / XCDS) + blockIdx.x / XCDS : blockIdx.x;
 
-  // step t of this workgroup -> linear tile.  Workgroup g runs on die g % 8; the workgroups of a
-  // die take consecutive tiles (two tile rows of one batch for 32 workgroups) so that they share
-  // panels in the die's L2 and write neighbouring output rows.
-  auto tile_of = [&](int t) -> int {
-    const int g = blockIdx.x;
-    if (G % XCDS == 0) {
-      const int per = G / XCDS;
-      return (t * XCDS + g % XCDS) * per + g / XCDS;
-    }
-    return t * G + g;
+  // Cursor over the unmasked tiles of this workgroup's units, in processing order.
+  struct Cursor {
+    int t, unit, batch, m0, n, n_end, n_vis_end;  // tiles [n, n_vis_end) computed, [.., n_end) filled
+    bool valid;
   };
-  struct Tile { int batch, m0, n0; bool valid, masked; };
-  auto decode = [&](int t) -> Tile {
-    Tile r;
-    const int L = tile_of(t);
-    r.valid = L < map.total;
-    const int Lc = r.valid ? L : 0;
-    r.batch = Lc / map.tiles_per_batch;
-    const int rem = Lc - r.batch * map.tiles_per_batch;
-    const int tm = rem / map.tiles_n;
-    r.m0 = tm * BM;
-    r.n0 = (rem - tm * map.tiles_n) * BN;
-    r.masked = a.mask == ADR_MASK_CAUSAL && r.n0 > r.m0 + BM - 1;
-    return r;
+  auto load_unit = [&](Cursor& c) {
+    for (;; c.t++) {
+      c.unit = c.t * G + ((c.t & 1) ? G - 1 - gl : gl);
+      if (c.unit >= map.units) { c.valid = false; return; }
+      const int row = c.unit / map.segs_per_row, sg = c.unit - row * map.segs_per_row;
+      c.batch = row / map.tiles_m;
+      c.m0 = (row - c.batch * map.tiles_m) * BM;
+      c.n = sg * map.seg;
+      c.n_end = min(c.n + map.seg, map.tiles_n);
+      // tiles with n0 > m0 + BM - 1 of a causal product are all -inf
+      const int vis = a.mask == ADR_MASK_CAUSAL ? (c.m0 + BM - 1) / BN + 1 : map.tiles_n;
+      c.n_vis_end = min(c.n_end, vis);
+      c.valid = true;
+      return;
+    }
   };
 
   if (wave >= NWC) {
     // ---------------------------------------------------------------- loader wavefronts
     const int lw = wave - NWC;
-    // the lane's place in a DMA instruction does not depend on the instruction index
-    int drow, dkc;
+    int drow, dkc;  // the lane's place in a DMA instruction does not depend on the instruction
     lds_chunk_inv<CPR>(lw * 64 + lane, drow, dkc);
-    auto dma = [&](const Tile& t, unsigned char* dA, unsigned char* dB) {
-      const half_t* A = a.lhs + (int64_t)t.batch * a.stride_lz + dkc * 8;
-      const half_t* B = a.rhs + (int64_t)t.batch * a.stride_rz + dkc * 8;
+    auto panel = [&](const half_t* base, int64_t row_stride, int r0, int rmax, unsigned char* dst) {
 #pragma unroll
       for (int i = 0; i < IT; i++) {
         const int row = drow + i * ROWS_PER_I;
         __builtin_amdgcn_global_load_lds(
-            ADR_GLB_PTR(A + (int64_t)min(t.m0 + row, a.m - 1) * a.stride_ly),
-            ADR_LDS_PTR(dA + (i * NWL + lw) * 1024), 16, 0, 0);
-      }
-#pragma unroll
-      for (int i = 0; i < IT; i++) {
-        const int row = drow + i * ROWS_PER_I;
-        __builtin_amdgcn_global_load_lds(
-            ADR_GLB_PTR(B + (int64_t)min(t.n0 + row, a.n - 1) * a.stride_rx),
-            ADR_LDS_PTR(dB + (i * NWL + lw) * 1024), 16, 0, 0);
+            ADR_GLB_PTR(base + (int64_t)min(r0 + row, rmax) * row_stride + dkc * 8),
+            ADR_LDS_PTR(dst + (i * NWL + lw) * 1024), 16, 0, 0);
       }
     };
-    Tile cur = decode(0);
-    if (!cur.valid) return;
-    if (!cur.masked) dma(cur, sA0, sB0);
-    for (int it = 0;; it += 2) {
-      Tile nxt = decode(it + 1);
-      __builtin_amdgcn_s_waitcnt(0x0070);  // tile `it` has landed
-      __builtin_amdgcn_s_barrier();        // ... and tile it-1 has been read by everyone
-      if (!nxt.valid) break;
-      if (!nxt.masked) dma(nxt, sA1, sB1);
-      cur = decode(it + 2);
-      __builtin_amdgcn_s_waitcnt(0x0070);
-      __builtin_amdgcn_s_barrier();
-      if (!cur.valid) break;
-      if (!cur.masked) dma(cur, sA0, sB0);
+    auto issueA = [&](const Cursor& c) {
+      panel(a.lhs + (int64_t)c.batch * a.stride_lz, a.stride_ly, c.m0, a.m - 1, sA);
+    };
+    auto issueB = [&](const Cursor& c, int slot) {
+      panel(a.rhs + (int64_t)c.batch * a.stride_rz, a.stride_rx, c.n * BN, a.n - 1,
+            sB + slot * PANEL);
+    };
+    // advance to the next tile that is computed (skipping units without one)
+    auto next_item = [&](Cursor& c) {
+      c.n++;
+      while (c.valid && c.n >= c.n_vis_end) { c.t++; load_unit(c); }
+    };
+    Cursor w;  // tile being waited for
+    w.t = 0;
+    load_unit(w);
+    while (w.valid && w.n >= w.n_vis_end) { w.t++; load_unit(w); }
+    if (!w.valid) return;
+    Cursor is = w;  // next tile to issue
+    int issued = 0;
+    issueA(w);
+    for (int k = 0; k < RING - 1 && is.valid; k++) {
+      issueB(is, issued % RING);
+      issued++;
+      next_item(is);
+    }
+    for (int j = 0; w.valid; j++) {
+      // the panel of tile j has landed; at most the one of tile j+1 is still in flight
+      if (issued - j - 1 >= 1)
+        __builtin_amdgcn_s_waitcnt(0x0070 | (IT & 0xF) | ((IT >> 4) << 14));
+      else
+        __builtin_amdgcn_s_waitcnt(0x0070);
+      __builtin_amdgcn_s_barrier();  // tile j: data ready; tile j-1 has been read by everyone
+      if (is.valid) {
+        issueB(is, issued % RING);
+        issued++;
+        next_item(is);
+      }
+      Cursor nx = w;
+      next_item(nx);
+      if (nx.valid && nx.unit != w.unit) {
+        __builtin_amdgcn_s_barrier();  // tile j has been multiplied: the left panel is free
+        issueA(nx);
+        __builtin_amdgcn_s_waitcnt(0x0070);
+      }
+      w = nx;
     }
     return;
   }
@@ -605,7 +626,7 @@ __global__ __launch_bounds__(512, 1) void gemm_nt_shortk_kernel(MatmulArgs a, Sh
   unsigned char* const slot = sEpi + wave * SLOT;
   const half_t hscale = (half_t)a.scale;
 
-  auto compute_store = [&](const Tile& t, const unsigned char* cA, const unsigned char* cB) {
+  auto compute_store = [&](int batch, int m0, int n0, const unsigned char* cB) {
     float16_t acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; i++)
@@ -615,7 +636,7 @@ __global__ __launch_bounds__(512, 1) void gemm_nt_shortk_kernel(MatmulArgs a, Sh
         for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
     half8_t fa[2][TM], fb[2][TN];
 #pragma unroll
-    for (int i = 0; i < TM; i++) fa[0][i] = *(const half8_t*)(cA + offA[i]);
+    for (int i = 0; i < TM; i++) fa[0][i] = *(const half8_t*)(sA + offA[i]);
 #pragma unroll
     for (int j = 0; j < TN; j++) fb[0][j] = *(const half8_t*)(cB + offB[j]);
 #pragma unroll
@@ -623,7 +644,7 @@ __global__ __launch_bounds__(512, 1) void gemm_nt_shortk_kernel(MatmulArgs a, Sh
       if (kk + 1 < KK) {
 #pragma unroll
         for (int i = 0; i < TM; i++)
-          fa[(kk + 1) & 1][i] = *(const half8_t*)(cA + (offA[i] ^ ((kk + 1) << 5)));
+          fa[(kk + 1) & 1][i] = *(const half8_t*)(sA + (offA[i] ^ ((kk + 1) << 5)));
 #pragma unroll
         for (int j = 0; j < TN; j++)
           fb[(kk + 1) & 1][j] = *(const half8_t*)(cB + (offB[j] ^ ((kk + 1) << 5)));
@@ -635,25 +656,34 @@ __global__ __launch_bounds__(512, 1) void gemm_nt_shortk_kernel(MatmulArgs a, Sh
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[kk & 1][j], fa[kk & 1][i],
                                                              acc[i][j], 0, 0, 0);
     }
-    half_t* const out = a.output + (int64_t)t.batch * a.stride_oz;
-    wave_epilogue<TM, TN>(a, out, acc, t.m0 + wm * 64, t.n0 + wn * 64, slot, hscale, lane);
+    half_t* const out = a.output + (int64_t)batch * a.stride_oz;
+    wave_epilogue<TM, TN>(a, out, acc, m0 + wm * 64, n0 + wn * 64, slot, hscale, lane);
   };
-  auto step = [&](const Tile& cur, const unsigned char* cA, const unsigned char* cB) {
-    __builtin_amdgcn_s_barrier();
-    if (cur.masked) {
-      fill_masked_tile<BM, BN, NTC>(a, a.output + (int64_t)cur.batch * a.stride_oz, cur.m0,
-                                    cur.n0, tid);
-    } else {
-      compute_store(cur, cA, cB);
+
+  Cursor c;
+  c.t = 0;
+  load_unit(c);
+  int j = 0;
+  while (c.valid) {
+    const int first = c.n;  // first tile of the unit
+    if (c.n < c.n_vis_end) {
+      for (; c.n < c.n_vis_end; c.n++, j++) {
+        __builtin_amdgcn_s_barrier();  // tile j: panels ready
+        compute_store(c.batch, c.m0, c.n * BN, sB + (j % RING) * PANEL);
+      }
+      // was this the last computed tile before a change of unit?  Then the loaders wait for
+      // the left panel to be released.
+      Cursor nx = c;
+      nx.n = nx.n_vis_end;
+      do { nx.t++; load_unit(nx); } while (nx.valid && nx.n >= nx.n_vis_end);
+      if (nx.valid) __builtin_amdgcn_s_barrier();
     }
-  };
-  for (int it = 0;; it += 2) {
-    Tile cur = decode(it);
-    if (!cur.valid) break;
-    step(cur, sA0, sB0);
-    cur = decode(it + 1);
-    if (!cur.valid) break;
-    step(cur, sA1, sB1);
+    // fully masked tiles of this unit
+    for (int n = max(first, c.n_vis_end); n < c.n_end; n++)
+      fill_masked_tile<BM, BN, NWC * 64>(a, a.output + (int64_t)c.batch * a.stride_oz, c.m0,
+                                         n * BN, tid);
+    c.t++;
+    load_unit(c);
   }
 }
 
@@ -1062,11 +1092,16 @@ hipError_t launch_shortk(hipStream_t stream, const MatmulArgs& a) {
   ShortKMap map;
   map.tiles_m = (a.m + 127) / 128;
   map.tiles_n = (a.n + 127) / 128;
-  map.tiles_per_batch = map.tiles_m * map.tiles_n;
-  const int64_t total = (int64_t)map.tiles_per_batch * a.batches;
-  if (total > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-  map.total = (int)total;
-  const unsigned grid = total < NUM_CU ? (unsigned)total : NUM_CU;
+  const int64_t rows = (int64_t)map.tiles_m * a.batches;
+  if (rows * map.tiles_n > 0x3fffffffLL) return hipErrorInvalidConfiguration;
+  map.rows = (int)rows;
+  // split tile rows into segments until there are at least two units per workgroup
+  map.seg = map.tiles_n;
+  while (rows * ((map.tiles_n + map.seg - 1) / map.seg) < 2 * NUM_CU && map.seg > 4)
+    map.seg = (map.seg + 1) / 2;
+  map.segs_per_row = (map.tiles_n + map.seg - 1) / map.seg;
+  map.units = map.rows * map.segs_per_row;
+  const unsigned grid = map.units < NUM_CU ? (unsigned)map.units : NUM_CU;
   hipLaunchKernelGGL((gemm_nt_shortk_kernel<CPR>), dim3(grid), dim3(512), 0, stream, a, map);
   return hipGetLastError();
 }
