@@ -295,7 +295,8 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   static_assert(BM * CPR % NT == 0 && BN * CPR % NT == 0, "slices must split evenly over lanes");
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "MFMA 32x32x16 tiling");
   static_assert((NW / 2) * SLOT <= BM * BK * 2, "epilogue slots must fit in two A stages");
-  static_assert(NSTAGE == 2 || NSTAGE == 3, "2 or 3 LDS stages");
+  static_assert(NSTAGE == 2 || NSTAGE == 3 || NSTAGE == 5,
+                "2 or 3 LDS stages, or 5: three stages of the left and two of the right operand");
   static_assert(!NN || BN == 128, "the N-contiguous right operand is staged as [64][128] tiles");
   // Separate objects per stage: the compiler's alias analysis then knows that the asynchronous
   // LDS writes of one stage cannot touch the stage being read, and does not serialise them.
@@ -304,7 +305,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   __shared__ __attribute__((aligned(1024))) unsigned char sA2[NSTAGE > 2 ? BM * BK * 2 : 1024];
   __shared__ __attribute__((aligned(1024))) unsigned char sB0[BN * BK * 2];
   __shared__ __attribute__((aligned(1024))) unsigned char sB1[BN * BK * 2];
-  __shared__ __attribute__((aligned(1024))) unsigned char sB2[NSTAGE > 2 ? BN * BK * 2 : 1024];
+  __shared__ __attribute__((aligned(1024))) unsigned char sB2[NSTAGE == 3 ? BN * BK * 2 : 1024];
 
   int batch, tile_m, tile_n;
   map_tile(map, batch, tile_m, tile_n);
@@ -350,18 +351,23 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   const int64_t b_slice = NN ? (int64_t)BK * a.stride_ry : BK;  // elements per K slice
   const int KT = a.k / BK;
   int kload = 0;  // next slice to fetch; past the end the last slice is fetched again (unused)
-  auto dma = [&](unsigned char* dA, unsigned char* dB) {
-    const int ks = min(kload, KT - 1);
-    const int k0 = ks * BK;
-    kload++;
+  auto dmaA = [&](int ks, unsigned char* dA) {
 #pragma unroll
     for (int i = 0; i < IA; i++)
-      __builtin_amdgcn_global_load_lds(ADR_GLB_PTR(gA[i] + k0),
+      __builtin_amdgcn_global_load_lds(ADR_GLB_PTR(gA[i] + ks * BK),
                                        ADR_LDS_PTR(dA + (i * NW + wave) * 1024), 16, 0, 0);
+  };
+  auto dmaB = [&](int ks, unsigned char* dB) {
 #pragma unroll
     for (int i = 0; i < IB; i++)
       __builtin_amdgcn_global_load_lds(ADR_GLB_PTR(gB[i] + ks * b_slice),
                                        ADR_LDS_PTR(dB + (i * NW + wave) * 1024), 16, 0, 0);
+  };
+  auto dma = [&](unsigned char* dA, unsigned char* dB) {
+    const int ks = min(kload, KT - 1);
+    kload++;
+    dmaA(ks, dA);
+    dmaB(ks, dB);
   };
 
   float16_t acc[TM][TN];
@@ -464,7 +470,56 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
     load_frags(0, nA, nB, 0);
   };
 
-  if (NSTAGE == 3) {
+  if (NSTAGE == 5) {
+    // Three stages of the left and two of the right operand (what fits beside a 256 x 192
+    // tile): slice kt reads A stage kt % 3 and B stage kt % 2; at its head the DMA of B(kt+1)
+    // and then of A(kt+2) is issued, spread one instruction per MFMA over the first k-steps,
+    // and at its end everything but A(kt+2) has to have landed.  The DMA engine of the CU
+    // (about 45 bytes per clock) then never idles between the barrier and the next burst.
+    int kA = 0, kB = 0;
+    auto slice5 = [&](const unsigned char* cA, const unsigned char* cB, const unsigned char* nA,
+                      const unsigned char* nB, unsigned char* dA, unsigned char* dB) {
+      dmaB(min(kB++, KT - 1), dB);
+      dmaA(min(kA++, KT - 1), dA);
+#pragma unroll
+      for (int kk = 0; kk < KK; kk++) {
+        if (kk + 1 < KK) {
+          load_frags((kk + 1) & 1, cA, cB, kk + 1);
+          mfmas(kk & 1);
+#pragma unroll
+          for (int q = 0; q < TM * TN; q++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (kk < 2) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+          }
+        } else {
+          mfmas(kk & 1);
+        }
+      }
+      wait_dma_barrier(std::integral_constant<int, IA>{});
+      load_frags(0, nA, nB, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    dmaA(min(kA++, KT - 1), sA0);
+    dmaB(min(kB++, KT - 1), sB0);
+    dmaA(min(kA++, KT - 1), sA1);
+    wait_dma_barrier(std::integral_constant<int, IA>{});
+    load_frags(0, sA0, sB0, 0);
+    int kt = 0;
+    for (; kt + 6 <= KT; kt += 6) {
+      slice5(sA0, sB0, sA1, sB1, sA2, sB1);
+      slice5(sA1, sB1, sA2, sB0, sA0, sB0);
+      slice5(sA2, sB0, sA0, sB1, sA1, sB1);
+      slice5(sA0, sB1, sA1, sB0, sA2, sB0);
+      slice5(sA1, sB0, sA2, sB1, sA0, sB1);
+      slice5(sA2, sB1, sA0, sB0, sA1, sB0);
+    }
+    if (kt < KT) { slice5(sA0, sB0, sA1, sB1, sA2, sB1); kt++; }
+    if (kt < KT) { slice5(sA1, sB1, sA2, sB0, sA0, sB0); kt++; }
+    if (kt < KT) { slice5(sA2, sB0, sA0, sB1, sA1, sB1); kt++; }
+    if (kt < KT) { slice5(sA0, sB1, sA1, sB0, sA2, sB0); kt++; }
+    if (kt < KT) { slice5(sA1, sB0, sA2, sB1, sA0, sB1); kt++; }
+  } else if (NSTAGE == 3) {
     dma(sA0, sB0);
     dma(sA1, sB1);
     wait_dma_barrier(std::integral_constant<int, INFLIGHT>{});
@@ -1211,7 +1266,7 @@ hipError_t launch_mfma_gemm(hipStream_t stream, const MatmulArgs& a) {
     case SHORTK_128: return launch_shortk<16>(stream, a);
     case U8_256x192: return launch_u8<256, 192, 4, 2>(stream, a);
     case U8_256x128: return launch_u8<256, 128, 4, 2>(stream, a);
-    case DMA_256x192: return launch_dma<256, 192, 4, 2, 2, 1>(stream, a);
+    case DMA_256x192: return launch_dma<256, 192, 4, 2, 5, 1>(stream, a);
     case DMA_256x128: return launch_dma<256, 128, 4, 2, 3, 1>(stream, a);
     case DMA_128x128: return launch_dma<128, 128, 2, 2, 2, 2>(stream, a);
     case DMA_64x64: return launch_dma<64, 64, 2, 2, 3, 3>(stream, a);
