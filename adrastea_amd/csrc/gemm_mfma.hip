@@ -443,10 +443,10 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   // slot 0); nxt: the stage consumed next; (dA, dB): the stage the DMA issued here refills.
   auto slice = [&](const unsigned char* cA, const unsigned char* cB, const unsigned char* nA,
                    const unsigned char* nB, unsigned char* dA, unsigned char* dB) {
+    // the DMA is issued in the first k-steps, one instruction per MFMA: sunk towards the wait
+    // below, the whole global -> LDS latency would be exposed; issued as one burst, it would
+    // hold up the MFMAs behind it
     dma(dA, dB);
-    // pin the DMA issue to the head of the slice: sunk towards the wait below, the whole
-    // global -> LDS latency would be exposed
-    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int kk = 0; kk < KK; kk++) {
       if (kk + 1 < KK) {
@@ -459,6 +459,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
         for (int q = 0; q < TM * TN; q++) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x100, PER, 0);
+          if (kk * TM * TN + q < IA + IB) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
         }
       } else {
         mfmas(kk & 1);
@@ -468,6 +469,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
     // and every wavefront has left the current one
     wait_dma_barrier(std::integral_constant<int, INFLIGHT>{});
     load_frags(0, nA, nB, 0);
+    __builtin_amdgcn_sched_barrier(0);
   };
 
   if (NSTAGE == 5) {
