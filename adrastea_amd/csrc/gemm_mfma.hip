@@ -764,6 +764,7 @@ __global__ __launch_bounds__(WM* WN * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a
   constexpr int SLOT = 32 * (TN * 64 + 16);
   static_assert(BM * CPR % NT == 0 && BN * CPR % NT == 0, "slices must split evenly over lanes");
   static_assert((NW / 2) * SLOT <= BM * BK * 2, "epilogue slots must fit in two A stages");
+  static_assert(LB < KK, "one chunk per k-step, none in the last");
   __shared__ __attribute__((aligned(1024))) unsigned char sA0[BM * BK * 2];
   __shared__ __attribute__((aligned(1024))) unsigned char sA1[BM * BK * 2];
   __shared__ __attribute__((aligned(1024))) unsigned char sA2[BM * BK * 2];
@@ -819,12 +820,13 @@ __global__ __launch_bounds__(WM* WN * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a
       rs[set][i] = gS[i][(ks * BK) >> block_shift];
     }
   };
+  auto dequant_store1 = [&](int set, unsigned char* dB, int i) {
+    const half2_t s2 = {rs[set][i], rs[set][i]};
+    *(half8_t*)(dB + offB[i]) = dequant8(rq[set][i][0], rq[set][i][1], s2);
+  };
   auto dequant_store = [&](int set, unsigned char* dB) {
 #pragma unroll
-    for (int i = 0; i < LB; i++) {
-      const half2_t s2 = {rs[set][i], rs[set][i]};
-      *(half8_t*)(dB + offB[i]) = dequant8(rq[set][i][0], rq[set][i][1], s2);
-    }
+    for (int i = 0; i < LB; i++) dequant_store1(set, dB, i);
   };
 
   float16_t acc[TM][TN];
@@ -872,18 +874,18 @@ __global__ __launch_bounds__(WM* WN * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a
 #pragma unroll
     for (int kk = 0; kk < KK; kk++) {
       if (kk + 1 < KK) load_frags((kk + 1) & 1, cA, cB, kk + 1);
-      if (kk == 1) dequant_store(nset, nB);
+      // one 8-weight chunk is dequantised per k-step: its VALU work and its LDS write fill the
+      // gaps between the MFMAs of that step
+      if (kk < LB) dequant_store1(nset, nB, kk);
       mfmas(kk & 1);
       if (kk + 1 < KK) {
-        // fragment reads behind the first MFMAs of the k-step; the dequantisation (VALU and
-        // LDS writes) of k-step 1 fills the gaps between the remaining ones
 #pragma unroll
         for (int q = 0; q < TM * TN; q++) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-          if (kk == 1) {
-            __builtin_amdgcn_sched_group_barrier(0x002, 2 * LB * 8 / (TM * TN) + 1, 0);
-            if (q % 2 == 1) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+          if (kk < LB) {
+            __builtin_amdgcn_sched_group_barrier(0x002, 20 / (TM * TN) + 1, 0);
+            if (q == TM * TN - 1) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
           }
         }
       }
@@ -1167,7 +1169,7 @@ enum GemmChoice {
   GEMM_NONE = 0,
   SHORTK_64, SHORTK_128,
   U8_256x192, U8_256x128,
-  DMA_256x192, DMA_256x128, DMA_128x128, DMA_64x64,
+  DMA_256x192, DMA_256x128, DMA_128x128, DMA_128x64, DMA_64x64,
   DMA_NN_256x128, DMA_NN_128x128,
   STAGE_256x128, STAGE_128x128, STAGE_64x64,
 };
@@ -1179,15 +1181,17 @@ struct Candidate {
   float eff;   // measured relative throughput of one busy CU with this tile
 };
 
-// Estimated cost: rounds of resident workgroups times the work of one tile over its efficiency.
+// Estimated cost: the tiles of the busiest CU times the work of one tile over the efficiency of
+// a CU running this tile shape.  (With few long tiles the transfer rate into one CU's LDS, not
+// the matrix pipe, bounds a tile: spreading the same work over all CUs with smaller tiles wins.)
 GemmChoice pick(const MatmulArgs& a, const Candidate* c, int n) {
   GemmChoice best = GEMM_NONE;
   double best_cost = 0;
   for (int i = 0; i < n; i++) {
     const int64_t tiles = (int64_t)((a.m + c[i].bm - 1) / c[i].bm) * ((a.n + c[i].bn - 1) / c[i].bn) *
                           a.batches;
-    const int64_t rounds = (tiles + NUM_CU * c[i].slots - 1) / (NUM_CU * c[i].slots);
-    const double cost = (double)rounds * c[i].slots * c[i].bm * c[i].bn / c[i].eff;
+    const int64_t per_cu = (tiles + NUM_CU - 1) / NUM_CU;
+    const double cost = (double)per_cu * c[i].bm * c[i].bn / c[i].eff;
     if (best == GEMM_NONE || cost < best_cost) {
       best = c[i].id;
       best_cost = cost;
@@ -1227,8 +1231,9 @@ GemmChoice choose(const MatmulArgs& a) {
     }
     static const Candidate dma[] = {
         {DMA_256x192, 256, 192, 1, 1.10f}, {DMA_256x128, 256, 128, 1, 1.00f},
-        {DMA_128x128, 128, 128, 2, 0.80f}, {DMA_64x64, 64, 64, 4, 0.40f}};
-    return pick(a, dma, 4);
+        {DMA_128x128, 128, 128, 2, 0.80f}, {DMA_128x64, 128, 64, 2, 0.60f},
+        {DMA_64x64, 64, 64, 4, 0.40f}};
+    return pick(a, dma, 5);
   }
   if (a.rhs_q && a.k % 64 == 0 && a.block_size >= 8 && (a.block_size & (a.block_size - 1)) == 0 &&
       (int64_t)a.m * a.n >= 256 * 1024) {
@@ -1252,6 +1257,7 @@ bool mfma_gemm_supported(const MatmulArgs& a, const char** name) {
     case DMA_256x192: *name = "gemm_nt_mfma_dma_256x192x64"; return true;
     case DMA_256x128: *name = "gemm_nt_mfma_dma_256x128x64"; return true;
     case DMA_128x128: *name = "gemm_nt_mfma_dma_128x128x64"; return true;
+    case DMA_128x64: *name = "gemm_nt_mfma_dma_128x64x64"; return true;
     case DMA_64x64: *name = "gemm_nt_mfma_dma_64x64x64"; return true;
     case DMA_NN_256x128: *name = "gemm_nn_mfma_dma_256x128x64"; return true;
     case DMA_NN_128x128: *name = "gemm_nn_mfma_dma_128x128x64"; return true;
@@ -1270,7 +1276,8 @@ hipError_t launch_mfma_gemm(hipStream_t stream, const MatmulArgs& a) {
     case U8_256x128: return launch_u8<256, 128, 4, 2>(stream, a);
     case DMA_256x192: return launch_dma<256, 192, 4, 2, 5, 1>(stream, a);
     case DMA_256x128: return launch_dma<256, 128, 4, 2, 3, 1>(stream, a);
-    case DMA_128x128: return launch_dma<128, 128, 2, 2, 2, 2>(stream, a);
+    case DMA_128x128: return launch_dma<128, 128, 2, 2, 3, 1>(stream, a);
+    case DMA_128x64: return launch_dma<128, 64, 2, 2, 3, 2>(stream, a);
     case DMA_64x64: return launch_dma<64, 64, 2, 2, 3, 3>(stream, a);
     case DMA_NN_256x128: return launch_dma<256, 128, 4, 2, 3, 1, true>(stream, a);
     case DMA_NN_128x128: return launch_dma<128, 128, 2, 2, 2, 2, true>(stream, a);
