@@ -146,6 +146,8 @@ SHAPES = [
     (1, 515, 136, 1100),
     (3, 129, 96, 257),
     (1, 2056, 256, 1024),   # config-2-like M tail with the large tile
+    (1, 1000, 320, 2040),   # 128x64 tiles (256 of them), ragged in M and N
+    (1, 2056, 320, 1024),   # 128x128 tiles, three stages, K tail of the 3-slice loop
 ]
 
 
