@@ -125,6 +125,95 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_kernel(half_t* __restrict__ o
 }
 
 
+// Variant for wide matrices: a workgroup covers RG groups of 16 weight rows, and a wavefront keeps
+// the activation fragments of its macro step in registers while it walks the RG groups, so the
+// activations are fetched once per 16*RG weight rows instead of once per 16.
+struct WStage {
+  u32x4_t w[4];  // 4 x 16 weight bytes of this lane's row
+  u32x4_t sc;    // the eight fp16 scales (block_size 32) of the macro step
+};
+
+template <int NW, int RG>
+__global__ __launch_bounds__(NW * 64) void gemv_u8_wide_kernel(half_t* __restrict__ out,
+                                                               const half_t* __restrict__ lhs,
+                                                               const uint8_t* __restrict__ rhs,
+                                                               const half_t* __restrict__ scales,
+                                                               int m, int p, int n, float beta) {
+  __shared__ float partial[NW][RG][ROWS * 16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * (ROWS * RG);
+  const int nblk = p / 32;
+  const bool xvalid = r < m;
+  const half_t* xrow = lhs + (int64_t)(xvalid ? r : 0) * p + g * 16;
+  const int steps = p / MACRO_K;
+  const uint8_t* wrow[RG];
+  const half_t* srow[RG];
+#pragma unroll
+  for (int q = 0; q < RG; q++) {
+    const int row = min(n0 + q * ROWS + r, n - 1);  // tail rows are clamped, never stored
+    wrow[q] = rhs + (int64_t)row * p + g * 16;
+    srow[q] = scales + (int64_t)row * nblk;
+  }
+  auto load_w = [&](WStage& s, int q, int ms) {
+    const uint8_t* wp = wrow[q] + (int64_t)ms * MACRO_K;
+#pragma unroll
+    for (int j = 0; j < 4; j++) s.w[j] = *(const u32x4_t*)(wp + j * 64);
+    s.sc = *(const u32x4_t*)(srow[q] + ms * (MACRO_K / 32));
+  };
+  auto load_x = [&](u32x4_t (&x)[8], int ms) {
+    const half_t* xp = xrow + (int64_t)ms * MACRO_K;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      x[2 * j] = xvalid ? *(const u32x4_t*)(xp + j * 64) : u32x4_t{0, 0, 0, 0};
+      x[2 * j + 1] = xvalid ? *(const u32x4_t*)(xp + j * 64 + 8) : u32x4_t{0, 0, 0, 0};
+    }
+  };
+  float4_t acc[RG][2];
+#pragma unroll
+  for (int q = 0; q < RG; q++) acc[q][0] = acc[q][1] = float4_t{0, 0, 0, 0};
+  auto compute = [&](const WStage& s, const u32x4_t (&x)[8], float4_t (&a)[2]) {
+    const half8_t sc = __builtin_bit_cast(half8_t, s.sc);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const half_t sv = g < 2 ? sc[2 * j] : sc[2 * j + 1];
+      const half2_t s2 = {sv, sv};
+      half8_t a0 = dequant8(s.w[j][0], s.w[j][1], s2);
+      half8_t a1 = dequant8(s.w[j][2], s.w[j][3], s2);
+      a[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, __builtin_bit_cast(half8_t, x[2 * j]), a[0], 0, 0, 0);
+      a[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, __builtin_bit_cast(half8_t, x[2 * j + 1]), a[1], 0, 0, 0);
+    }
+  };
+
+  // all weight loads of a macro step are issued before its first use
+  for (int ms = wave; ms < steps; ms += NW) {
+    u32x4_t x[8];
+    WStage s[RG];
+    load_x(x, ms);
+#pragma unroll
+    for (int q = 0; q < RG; q++) load_w(s[q], q, ms);
+#pragma unroll
+    for (int q = 0; q < RG; q++) compute(s[q], x, acc[q]);
+  }
+
+#pragma unroll
+  for (int q = 0; q < RG; q++)
+#pragma unroll
+    for (int i = 0; i < 4; i++) partial[wave][q][(4 * g + i) * 16 + r] = acc[q][0][i] + acc[q][1][i];
+  __syncthreads();
+  for (int e = tid; e < RG * ROWS * 16; e += NW * 64) {
+    const int mm = e / (RG * ROWS), nn = e % (RG * ROWS);  // consecutive threads -> consecutive columns
+    if (mm < m && n0 + nn < n) {
+      float sum = 0.0f;
+#pragma unroll
+      for (int w = 0; w < NW; w++) sum += partial[w][nn / ROWS][(nn % ROWS) * 16 + mm];
+      half_t* o = out + (int64_t)mm * n + n0 + nn;
+      // the previous output is read even for beta == 0, as the reference does
+      *o = (half_t)(sum + beta * (float)*o);
+    }
+  }
+}
+
 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
 
 template <int CTRL, int ROWMASK>
@@ -273,9 +362,10 @@ U8Choice choose_u8(const void* lhs, const void* rhs, const void* scales, int m, 
                        ((uintptr_t)scales % 16 == 0);
   if (!aligned) return U8_NAIVE;
   // dot-product kernel: 16 weights of a lane share one scale; at most 16 segments of 1 KiB.
-  // It wins for one or two activation rows, and for up to four on wide matrices.
+  // It wins for one or two activation rows; from three on its VALU work (dot products and lane
+  // reductions per activation row) costs more than the MFMA kernels' less coalesced loads.
   const bool dot_ok = block_size % 16 == 0 && p % 16 == 0 && p <= 16 * 1024;
-  if (dot_ok && (m <= 2 || (m <= 4 && p <= 4096 && n >= 8192))) return U8_DOT;
+  if (dot_ok && m <= 2) return U8_DOT;
   if (m <= 16 && block_size == 32 && p % MACRO_K == 0) return U8_GEMV;
   if (block_size % 8 == 0 && p % 8 == 0) return U8_GEMM;
   return U8_NAIVE;
@@ -290,7 +380,7 @@ hipError_t launch_gemm_u8_mfma(hipStream_t stream, half_t* out, const half_t* lh
 const char* gemm_u8_plan(int m, int p, int n, int block_size) {
   switch (choose_u8(nullptr, nullptr, nullptr, m, p, n, block_size)) {
     case U8_DOT: return "gemv_u8_dot2_stream";
-    case U8_GEMV: return "gemv_u8_mfma16_stream";
+    case U8_GEMV: return n >= 8192 ? "gemv_u8_mfma16_wide" : "gemv_u8_mfma16_stream";
     case U8_GEMM: return "gemm_nt_u8_mfma";
     default: return "gemm_u8_naive";
   }
@@ -315,6 +405,12 @@ hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, co
       const int blocks = (n + ROWS - 1) / ROWS;
       const int steps = p / MACRO_K;
       // enough wavefronts per workgroup to keep every macro step of a small problem in flight
+      // wide matrices: 48 weight rows per workgroup share one fetch of the activations
+      if (n >= 8192) {
+        hipLaunchKernelGGL((gemv_u8_wide_kernel<8, 3>), dim3((n + 3 * ROWS - 1) / (3 * ROWS)),
+                           dim3(512), 0, stream, out, lhs, rhs, scales, m, p, n, beta);
+        return hipGetLastError();
+      }
       if (steps >= 16 && blocks <= 1024)
         hipLaunchKernelGGL(gemv_u8_kernel<8>, dim3(blocks), dim3(512), 0, stream, out, lhs, rhs,
                            scales, m, p, n, beta);

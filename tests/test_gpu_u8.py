@@ -97,11 +97,14 @@ def _finite_scale_rows():
 
 
 @pytest.mark.parametrize("m", [1, 4, 16])
-def test_fused_dequant_in_gemv_is_bit_exact_for_every_q_and_finite_scale(kern, m):
-    """One-hot activations pick single weights out of the matmul: out[r, c] = w[c, k_r]."""
-    scales_bits = _finite_scale_rows()
+@pytest.mark.parametrize("every", [1, 8], ids=["all_scales", "every_8th_scale"])
+def test_fused_dequant_in_gemv_is_bit_exact_for_every_q_and_finite_scale(kern, m, every):
+    """One-hot activations pick single weights out of the matmul: out[r, c] = w[c, k_r].
+    All finite scales make a wide matrix (48-row workgroups), every 8th a narrow one."""
+    scales_bits = _finite_scale_rows()[::every]
     n, p, bs = scales_bits.size, 256, 32
-    assert u8_plan(m, p, n, bs) in ("gemv_u8_mfma16_stream", "gemv_u8_dot2_stream")
+    assert u8_plan(m, p, n, bs) == ("gemv_u8_dot2_stream" if m <= 2 else
+                                    "gemv_u8_mfma16_wide" if n >= 8192 else "gemv_u8_mfma16_stream")
     q = np.tile(np.arange(256, dtype=np.uint8), (n, 1))
     s = np.repeat(scales_bits.view(np.float16).reshape(n, 1), p // bs, axis=1)
     table = oracle.dequant_table()  # [q][scale bits]
@@ -158,6 +161,23 @@ def test_gemv_bit_exact_on_exact_inputs(kern, m, pn):
     for beta in (0.0, 0.5):
         want = prev.copy()
         oracle.matmul_nt_fp16u8(want, a, q, s, 32, beta=beta)
+        out = to_dev(prev)
+        kern.matmul_nt_fp16u8(out, to_dev(a), to_dev(q), to_dev(s), 32, beta=beta)
+        assert np.array_equal(to_np(out).view(np.uint16), want.view(np.uint16)), (m, p, n, beta)
+
+
+@pytest.mark.parametrize("m", [3, 7, 16])
+@pytest.mark.parametrize("pn", [(256, 8192), (768, 8200), (1024, 8251)])
+def test_wide_gemv_bit_exact_on_exact_inputs(kern, m, pn):
+    """The 48-rows-per-workgroup variant (n >= 8192): ragged last workgroup, beta path."""
+    p, n = pn
+    g = rng(660 + m + p)
+    assert u8_plan(m, p, n, 32) == "gemv_u8_mfma16_wide"
+    a, q, s = _u8_case(g, m, p, n, 32, exact=True)
+    for beta in (0.0, 1.0):
+        prev = (g.integers(-8, 9, size=(m, n)) / 4.0).astype(np.float16)
+        want = prev.copy()
+        oracle.matmul_nt_fp16u8(want, a, q, s, 32, beta=beta, threads=8)
         out = to_dev(prev)
         kern.matmul_nt_fp16u8(out, to_dev(a), to_dev(q), to_dev(s), 32, beta=beta)
         assert np.array_equal(to_np(out).view(np.uint16), want.view(np.uint16)), (m, p, n, beta)
@@ -239,7 +259,8 @@ def test_decode_shapes_full_size(kern, kn, m):
     q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)
     s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
     a = torch.randn(m, p, generator=gen, device="cuda").half()
-    assert u8_plan(m, p, n, 32) in ("gemv_u8_mfma16_stream", "gemv_u8_dot2_stream")
+    assert u8_plan(m, p, n, 32) in ("gemv_u8_mfma16_stream", "gemv_u8_mfma16_wide",
+                                    "gemv_u8_dot2_stream")
     out = torch.zeros(m, n, dtype=torch.float16, device="cuda")
     kern.matmul_nt_fp16u8(out, a, q, s, 32)
     w = torch.zeros(n, p, dtype=torch.float16, device="cuda")
