@@ -44,6 +44,8 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--quick", action="store_true", help="skip secondary configs and CPU baseline")
+    ap.add_argument("--decode-only", action="store_true",
+                    help="run only the u8 decode GEMV configurations (for profiling that kernel)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain 256 MiB device copy (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters of rocprofv3 --pmc)")
@@ -119,6 +121,43 @@ def main():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1e-3 / (replays * calls_per_graph)
 
+    # ---- u8 decode GEMV (BASELINE configs[2]): weight buffers rotate through > 256 MB so
+    # that repeats stream from HBM, not from the Infinity Cache
+    def u8_case(m, K, N, iters):
+        per = N * K + N * (K // 32) * 2
+        nbuf = max(2, int(600e6 // per) + 1)
+        qs = [torch.randint(0, 256, (N, K), generator=gen, device=dev, dtype=torch.uint8)
+              for _ in range(nbuf)]
+        ss = [(torch.rand(N, K // 32, generator=gen, device=dev) * 0.019 + 0.001).half()
+              for _ in range(nbuf)]
+        a = randn_h(m, K)
+        o = torch.zeros(m, N, dtype=torch.float16, device=dev)
+        i = [0]
+
+        def f():
+            j = i[0] % nbuf
+            i[0] += 1
+            rc = lib.adr_matmul_nt_fp16u8(stream(), o.data_ptr(), a.data_ptr(),
+                                          qs[j].data_ptr(), ss[j].data_ptr(), m, K, N, 32, 0.0)
+            if rc != 0:
+                raise RuntimeError(_ffi.strerror(rc))
+        t = timed_graph(f, 2 * nbuf, max(2, iters // (2 * nbuf)))
+        return t, per + m * K * 2 + m * N * 2
+
+    def decode_set():
+        gemv = []
+        for K, N in DECODE_SET:
+            for m in (1, 4, 16):
+                t, byts = u8_case(m, K, N, 200)
+                gemv.append({"M": m, "K": K, "N": N, "us": round(t * 1e6, 2),
+                             "gbs": round(byts / t / 1e9, 1),
+                             "frac_hbm_peak": round(byts / t / 1e9 / PEAK_HBM_GBS, 4)})
+        return gemv
+
+    if args.decode_only:
+        print(json.dumps({"u8_decode_gemv": decode_set()}))
+        return
+
     # ---------------- primary workload: the fp16 layer GEMM set at M = 2048
     M = 2048
     acts = {4096: randn_h(M, 4096), 11008: randn_h(M, 11008)}
@@ -171,36 +210,7 @@ def main():
                               "frac_mfma_peak": round(2.0 * M * K * N / t / 1e12 / PEAK_F16_TFLOPS, 4)}
         secondary["llama7b_prefill_fp16"] = per_gemm
 
-        # ---- u8 decode GEMV (BASELINE configs[2]): weight buffers rotate through > 256 MB so
-        # that repeats stream from HBM, not from the Infinity Cache
-        def u8_case(m, K, N, iters):
-            per = N * K + N * (K // 32) * 2
-            nbuf = max(2, int(600e6 // per) + 1)
-            qs = [torch.randint(0, 256, (N, K), generator=gen, device=dev, dtype=torch.uint8)
-                  for _ in range(nbuf)]
-            ss = [(torch.rand(N, K // 32, generator=gen, device=dev) * 0.019 + 0.001).half()
-                  for _ in range(nbuf)]
-            a = randn_h(m, K)
-            o = torch.zeros(m, N, dtype=torch.float16, device=dev)
-            i = [0]
-
-            def f():
-                j = i[0] % nbuf
-                i[0] += 1
-                rc = lib.adr_matmul_nt_fp16u8(stream(), o.data_ptr(), a.data_ptr(),
-                                              qs[j].data_ptr(), ss[j].data_ptr(), m, K, N, 32, 0.0)
-                if rc != 0:
-                    raise RuntimeError(_ffi.strerror(rc))
-            t = timed_graph(f, 2 * nbuf, max(2, iters // (2 * nbuf)))
-            return t, per + m * K * 2 + m * N * 2
-
-        gemv = []
-        for K, N in DECODE_SET:
-            for m in (1, 4, 16):
-                t, byts = u8_case(m, K, N, 200)
-                gemv.append({"M": m, "K": K, "N": N, "us": round(t * 1e6, 2),
-                             "gbs": round(byts / t / 1e9, 1),
-                             "frac_hbm_peak": round(byts / t / 1e9 / PEAK_HBM_GBS, 4)})
+        gemv = decode_set()
         secondary["u8_decode_gemv"] = gemv
         best = max(gemv, key=lambda r: r["gbs"])
         secondary["u8_decode_gemv_best"] = {"gbs": best["gbs"], "frac_hbm_peak": best["frac_hbm_peak"],
