@@ -149,7 +149,7 @@ __device__ __forceinline__ void store_chunk(const MatmulArgs& a, const Epilogue&
       if (x + e > y) r[e] = neg_inf_half();
   }
   if (full) {
-    *(half8_t*)p = r;
+    __builtin_nontemporal_store(r, (half8_t*)p);
   } else {
 #pragma unroll
     for (int e = 0; e < 8; e++)
@@ -202,7 +202,9 @@ __device__ __forceinline__ void wave_epilogue(const MatmulArgs& a, half_t* out,
 #pragma unroll
       for (int it = 0; it < TN * 2; it++) {
         const half8_t v = *(const half8_t*)(slot + rd[it]);
-        *(half8_t*)(p0 + i * blk + po[it]) = v;
+        // streaming store: the output is not read again by this launch and should not evict
+        // operand panels from L2
+        __builtin_nontemporal_store(v, (half8_t*)(p0 + i * blk + po[it]));
       }
     }
     return;
@@ -268,7 +270,7 @@ __device__ __forceinline__ void fill_masked_tile(const MatmulArgs& a, half_t* ou
       if (y >= a.m || x >= a.n) continue;
       half_t* p = out + (int64_t)y * a.stride_oy + x;
       if (x + 8 <= a.n) {
-        *(half8_t*)p = v;
+        __builtin_nontemporal_store(v, (half8_t*)p);
       } else {
         for (int q = 0; x + q < a.n; q++) p[q] = ninf;
       }
@@ -557,28 +559,34 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
 // =============================================================================================
 // With one or two K slices a tile is all load latency and epilogue, and the job is bound by the
 // output writes.  One workgroup per CU walks segments of tile rows (128 x 128 tiles): the left
-// panel of the segment stays in LDS, the right panels stream through a ring of three buffers.
-// Wavefronts 4..7 only load: they keep the DMA two tiles ahead, wait for the panel of tile j and
-// meet the others at a barrier.  Wavefronts 0..3 (2 x 2, 64 x 64 each) only multiply and store:
-// their output writes are never waited for (a wavefront's memory counter covers its own loads
-// and stores alike, which is why the two roles live in different wavefronts), so loads, MFMAs
-// and the writes of neighbouring tiles overlap and no workgroup launch is paid per tile.
+// panel of the segment stays in LDS, the right panels stream through a ring of three buffers,
+// and the wavefronts have three roles:
+//   0..3  multiply: MFMAs of tile j (2 x 2, 64 x 64 each), then the narrowed result goes into a
+//         128 x 128 fp16 staging tile in LDS;
+//   4..7  write: read tile j-1 from the staging tile as whole 256-byte rows, apply the store
+//         operator, issue the global stores.  Output writes stall the wavefront that issues
+//         them (the job is write bound), so they come from wavefronts that feed nothing else;
+//   8..11 load: keep the DMA two tiles ahead and wait for it.  A wavefront's memory counter
+//         covers its loads and stores alike, which is why loading and writing are not combined.
+// Two barriers per tile: X(j) (panel j landed, staging tile j-1 complete) and Y(j) (tile j
+// multiplied, staging tile j-1 read): between X(j) and Y(j) the MFMAs of tile j overlap the writes
+// of tile j-1.
 struct ShortKMap {
   int tiles_m, tiles_n, rows;   // rows = batches * tiles_m
   int seg, segs_per_row, units; // a unit is `seg` consecutive tiles of one tile row
 };
 
 template <int CPR>  // 16-byte chunks per row: 8 (K = 64) or 16 (K = 128)
-__global__ __launch_bounds__(512, 1) void gemm_nt_shortk_kernel(MatmulArgs a, ShortKMap map) {
-  constexpr int BM = 128, BN = 128, NWC = 4, NWL = 4, KK = CPR / 2;
+__global__ __launch_bounds__(1024, 1) void gemm_nt_shortk_kernel(MatmulArgs a, ShortKMap map) {
+  constexpr int BM = 128, BN = 128, NWL = 4, KK = CPR / 2;
   constexpr int TM = 2, TN = 2, RING = 3;
   constexpr int IT = BM * CPR / (NWL * 64);    // DMA instructions per loader lane and panel
   constexpr int ROWS_PER_I = NWL * 64 / CPR;   // rows between a lane's successive instructions
   constexpr int PANEL = BM * CPR * 16;         // bytes of one 128-row panel
-  constexpr int SLOT = 32 * (TN * 64 + 16);
   __shared__ __attribute__((aligned(1024))) unsigned char sA[PANEL];
   __shared__ __attribute__((aligned(1024))) unsigned char sB[RING * PANEL];
-  __shared__ __attribute__((aligned(1024))) unsigned char sEpi[NWC * SLOT];
+  // staging tile: row r = 256 bytes, 16-byte chunk c at position c ^ (r & 15)
+  __shared__ __attribute__((aligned(1024))) unsigned char sC[BM * BN * 2];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int G = gridDim.x;
@@ -587,31 +595,38 @@ __global__ __launch_bounds__(512, 1) void gemm_nt_shortk_kernel(MatmulArgs a, Sh
   // and short rows of a causal product.
   const int gl = G % XCDS == 0 ? (blockIdx.x % XCDS) * (G / XCDS) + blockIdx.x / XCDS : blockIdx.x;
 
-  // Cursor over the unmasked tiles of this workgroup's units, in processing order.
+  // Cursor over this workgroup's units and the tiles in them, in processing order.
   struct Cursor {
     int t, unit, batch, m0, n, n_end, n_vis_end;  // tiles [n, n_vis_end) computed, [.., n_end) filled
     bool valid;
   };
   auto load_unit = [&](Cursor& c) {
-    for (;; c.t++) {
-      c.unit = c.t * G + ((c.t & 1) ? G - 1 - gl : gl);
-      if (c.unit >= map.units) { c.valid = false; return; }
-      const int row = c.unit / map.segs_per_row, sg = c.unit - row * map.segs_per_row;
-      c.batch = row / map.tiles_m;
-      c.m0 = (row - c.batch * map.tiles_m) * BM;
-      c.n = sg * map.seg;
-      c.n_end = min(c.n + map.seg, map.tiles_n);
-      // tiles with n0 > m0 + BM - 1 of a causal product are all -inf
-      const int vis = a.mask == ADR_MASK_CAUSAL ? (c.m0 + BM - 1) / BN + 1 : map.tiles_n;
-      c.n_vis_end = min(c.n_end, vis);
-      c.valid = true;
-      return;
-    }
+    c.unit = c.t * G + ((c.t & 1) ? G - 1 - gl : gl);
+    if (c.unit >= map.units) { c.valid = false; return; }
+    const int row = c.unit / map.segs_per_row, sg = c.unit - row * map.segs_per_row;
+    c.batch = row / map.tiles_m;
+    c.m0 = (row - c.batch * map.tiles_m) * BM;
+    c.n = sg * map.seg;
+    c.n_end = min(c.n + map.seg, map.tiles_n);
+    // tiles with n0 > m0 + BM - 1 of a causal product are all -inf
+    const int vis = a.mask == ADR_MASK_CAUSAL ? (c.m0 + BM - 1) / BN + 1 : map.tiles_n;
+    c.n_vis_end = min(c.n_end, vis);
+    c.valid = true;
+  };
+  // first / next tile that is computed (units without one are skipped)
+  auto first_item = [&](Cursor& c) {
+    c.t = 0;
+    load_unit(c);
+    while (c.valid && c.n >= c.n_vis_end) { c.t++; load_unit(c); }
+  };
+  auto next_item = [&](Cursor& c) {
+    c.n++;
+    while (c.valid && c.n >= c.n_vis_end) { c.t++; load_unit(c); }
   };
 
-  if (wave >= NWC) {
+  if (wave >= 12) {
     // ---------------------------------------------------------------- loader wavefronts
-    const int lw = wave - NWC;
+    const int lw = wave - 12;
     int drow, dkc;  // the lane's place in a DMA instruction does not depend on the instruction
     lds_chunk_inv<CPR>(lw * 64 + lane, drow, dkc);
     auto panel = [&](const half_t* base, int64_t row_stride, int r0, int rmax, unsigned char* dst) {
@@ -630,49 +645,126 @@ __global__ __launch_bounds__(512, 1) void gemm_nt_shortk_kernel(MatmulArgs a, Sh
       panel(a.rhs + (int64_t)c.batch * a.stride_rz, a.stride_rx, c.n * BN, a.n - 1,
             sB + slot * PANEL);
     };
-    // advance to the next tile that is computed (skipping units without one)
-    auto next_item = [&](Cursor& c) {
-      c.n++;
-      while (c.valid && c.n >= c.n_vis_end) { c.t++; load_unit(c); }
-    };
     Cursor w;  // tile being waited for
-    w.t = 0;
-    load_unit(w);
-    while (w.valid && w.n >= w.n_vis_end) { w.t++; load_unit(w); }
-    if (!w.valid) return;
-    Cursor is = w;  // next tile to issue
-    int issued = 0;
-    issueA(w);
-    for (int k = 0; k < RING - 1 && is.valid; k++) {
-      issueB(is, issued % RING);
-      issued++;
-      next_item(is);
-    }
-    for (int j = 0; w.valid; j++) {
-      // the panel of tile j has landed; at most the one of tile j+1 is still in flight
-      if (issued - j - 1 >= 1)
-        __builtin_amdgcn_s_waitcnt(0x0070 | (IT & 0xF) | ((IT >> 4) << 14));
-      else
-        __builtin_amdgcn_s_waitcnt(0x0070);
-      __builtin_amdgcn_s_barrier();  // tile j: data ready; tile j-1 has been read by everyone
-      if (is.valid) {
+    first_item(w);
+    if (w.valid) {
+      Cursor is = w;  // next tile to issue
+      int issued = 0;
+      bool a_young = false;  // a left panel was issued after the youngest right panel
+      issueA(w);
+      for (int k = 0; k < RING - 1 && is.valid; k++) {
         issueB(is, issued % RING);
         issued++;
         next_item(is);
       }
-      Cursor nx = w;
-      next_item(nx);
-      if (nx.valid && nx.unit != w.unit) {
-        __builtin_amdgcn_s_barrier();  // tile j has been multiplied: the left panel is free
-        issueA(nx);
-        __builtin_amdgcn_s_waitcnt(0x0070);
+      for (int j = 0; w.valid; j++) {
+        // the panel of tile j has landed; at most the one of tile j+1 is still in flight
+        if (issued - j - 1 >= 1 && !a_young)
+          __builtin_amdgcn_s_waitcnt(0x0070 | (IT & 0xF) | ((IT >> 4) << 14));
+        else
+          __builtin_amdgcn_s_waitcnt(0x0070);
+        a_young = false;
+        __builtin_amdgcn_s_barrier();  // X(j)
+        if (is.valid) {
+          issueB(is, issued % RING);  // into the buffer of tile j-1, read before Y(j-1)
+          issued++;
+          next_item(is);
+        }
+        __builtin_amdgcn_s_barrier();  // Y(j): tile j has been multiplied, the left panel is free
+        Cursor nx = w;
+        next_item(nx);
+        if (nx.valid && nx.unit != w.unit) {
+          issueA(nx);
+          a_young = true;
+        }
+        w = nx;
       }
-      w = nx;
     }
+    __builtin_amdgcn_s_barrier();  // Z: last staging tile complete
     return;
   }
 
-  // ------------------------------------------------------------------ compute wavefronts
+  if (wave >= 4) {
+    // ---------------------------------------------------------------- writer wavefronts
+    const int sw = wave - 4;                       // rows sw*16 .. +15 of a tile
+    const int rrow = lane >> 4, rc = lane & 15;    // read round it: row it*4 + rrow, chunk rc
+    const half_t hscale = (half_t)a.scale;
+    Epilogue ep{a.bias, a.beta, hscale, a.store};
+    const bool vec = out_vectorizable(a, a.output) && !(a.stride_oz & 7);
+    const bool plain = vec && (a.store == ADR_STORE_IDENTITY || a.store == ADR_STORE_SCALE);
+    const half_t mul = a.store == ADR_STORE_SCALE ? hscale : (half_t)1.0f;
+    auto write_tile = [&](int batch, int m0, int n0) {
+      half8_t v[4];
+#pragma unroll
+      for (int it = 0; it < 4; it++) {
+        const int row = sw * 16 + it * 4 + rrow;
+        v[it] = *(const half8_t*)(sC + row * 256 + ((rc ^ (row & 15)) << 4));
+      }
+      half_t* const out = a.output + (int64_t)batch * a.stride_oz;
+      const int y0 = m0 + sw * 16 + rrow, x = n0 + rc * 8;
+      const bool inside = m0 + sw * 16 + 16 <= a.m && n0 + BN <= a.n;
+      const bool unmasked = a.mask != ADR_MASK_CAUSAL || n0 + BN - 1 <= m0 + sw * 16;
+      if (plain && inside && unmasked) {
+        // x * 1 is exact: one multiply serves Identity and Scale (fp16 product, matmul.cu)
+        half_t* const p = out + (int64_t)y0 * a.stride_oy + x;
+#pragma unroll
+        for (int it = 0; it < 4; it++)
+          __builtin_nontemporal_store(v[it] * mul, (half8_t*)(p + (int64_t)(it * 4) * a.stride_oy));
+      } else if (vec) {
+#pragma unroll 1
+        for (int it = 0; it < 4; it++) {
+          const int y = y0 + it * 4;
+          if (y < a.m && x < a.n) store_chunk(a, ep, out, y, x, v[it]);
+        }
+      } else {
+        const bool need_prev = Epilogue::needs_prev(a.store);
+        const bool need_bias = Epilogue::needs_bias(a.store);
+#pragma unroll 1
+        for (int it = 0; it < 4; it++) {
+          const int y = y0 + it * 4;
+          if (y >= a.m) continue;
+#pragma unroll
+          for (int e = 0; e < 8; e++) {
+            if (x + e >= a.n) continue;
+            half_t* p = out + (int64_t)y * a.stride_oy + x + e;
+            if (a.mask == ADR_MASK_CAUSAL && x + e > y) {
+              *p = neg_inf_half();
+            } else {
+              const half_t prev = need_prev ? *p : (half_t)0;
+              const half_t bias = need_bias ? a.bias[x + e] : (half_t)0;
+              *p = ep.apply_s16(v[it][e], prev, bias);
+            }
+          }
+        }
+      }
+    };
+    Cursor c;
+    c.t = 0;
+    load_unit(c);
+    bool have_prev = false;
+    int pb = 0, pm = 0, pn = 0;
+    while (c.valid) {
+      const int first = c.n;
+      for (; c.n < c.n_vis_end; c.n++) {
+        __builtin_amdgcn_s_barrier();  // X(j): staging tile j-1 complete
+        if (have_prev) write_tile(pb, pm, pn);
+        __builtin_amdgcn_s_barrier();  // Y(j): staging tile j-1 read
+        have_prev = true;
+        pb = c.batch; pm = c.m0; pn = c.n * BN;
+      }
+      // fully masked tiles of this unit
+      for (int n = max(first, c.n_vis_end); n < c.n_end; n++)
+        fill_masked_tile<BM, BN, 512>(a, a.output + (int64_t)c.batch * a.stride_oz, c.m0, n * BN,
+                                      tid - 256);
+      c.t++;
+      load_unit(c);
+    }
+    __builtin_amdgcn_s_barrier();  // Z
+    if (have_prev) write_tile(pb, pm, pn);
+    return;
+  }
+
+  // ------------------------------------------------------------------ multiplying wavefronts
   const int wm = wave >> 1, wn = wave & 1;
   const int frow = lane & 31, fkg = lane >> 5;
   int offA[TM], offB[TN];  // k-step 0; k-step kk is at (off ^ (kk << 5))
@@ -680,22 +772,25 @@ __global__ __launch_bounds__(512, 1) void gemm_nt_shortk_kernel(MatmulArgs a, Sh
   for (int i = 0; i < TM; i++) offA[i] = lds_chunk_off<CPR>(wm * 64 + i * 32 + frow, fkg);
 #pragma unroll
   for (int j = 0; j < TN; j++) offB[j] = lds_chunk_off<CPR>(wn * 64 + j * 32 + frow, fkg);
-  unsigned char* const slot = sEpi + wave * SLOT;
-  const half_t hscale = (half_t)a.scale;
 
-  auto compute_store = [&](int batch, int m0, int n0, const unsigned char* cB) {
+  Cursor c;
+  first_item(c);
+  for (int j = 0; c.valid; j++) {
+    const unsigned char* cB = sB + (j % RING) * PANEL;
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // the staging tile of tile j-1 is written (lgkmcnt 0)
+    __builtin_amdgcn_s_barrier();        // X(j): panels of tile j ready
     float16_t acc[TM][TN];
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
-      for (int j = 0; j < TN; j++)
+      for (int jj = 0; jj < TN; jj++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+        for (int r = 0; r < 16; r++) acc[i][jj][r] = 0.0f;
     half8_t fa[2][TM], fb[2][TN];
 #pragma unroll
     for (int i = 0; i < TM; i++) fa[0][i] = *(const half8_t*)(sA + offA[i]);
 #pragma unroll
-    for (int j = 0; j < TN; j++) fb[0][j] = *(const half8_t*)(cB + offB[j]);
+    for (int jj = 0; jj < TN; jj++) fb[0][jj] = *(const half8_t*)(cB + offB[jj]);
 #pragma unroll
     for (int kk = 0; kk < KK; kk++) {
       if (kk + 1 < KK) {
@@ -703,45 +798,39 @@ __global__ __launch_bounds__(512, 1) void gemm_nt_shortk_kernel(MatmulArgs a, Sh
         for (int i = 0; i < TM; i++)
           fa[(kk + 1) & 1][i] = *(const half8_t*)(sA + (offA[i] ^ ((kk + 1) << 5)));
 #pragma unroll
-        for (int j = 0; j < TN; j++)
-          fb[(kk + 1) & 1][j] = *(const half8_t*)(cB + (offB[j] ^ ((kk + 1) << 5)));
+        for (int jj = 0; jj < TN; jj++)
+          fb[(kk + 1) & 1][jj] = *(const half8_t*)(cB + (offB[jj] ^ ((kk + 1) << 5)));
       }
 #pragma unroll
       for (int i = 0; i < TM; i++)
 #pragma unroll
-        for (int j = 0; j < TN; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[kk & 1][j], fa[kk & 1][i],
-                                                             acc[i][j], 0, 0, 0);
+        for (int jj = 0; jj < TN; jj++)
+          acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[kk & 1][jj], fa[kk & 1][i],
+                                                              acc[i][jj], 0, 0, 0);
     }
-    half_t* const out = a.output + (int64_t)batch * a.stride_oz;
-    wave_epilogue<TM, TN>(a, out, acc, m0 + wm * 64, n0 + wn * 64, slot, hscale, lane);
-  };
-
-  Cursor c;
-  c.t = 0;
-  load_unit(c);
-  int j = 0;
-  while (c.valid) {
-    const int first = c.n;  // first tile of the unit
-    if (c.n < c.n_vis_end) {
-      for (; c.n < c.n_vis_end; c.n++, j++) {
-        __builtin_amdgcn_s_barrier();  // tile j: panels ready
-        compute_store(c.batch, c.m0, c.n * BN, sB + (j % RING) * PANEL);
-      }
-      // was this the last computed tile before a change of unit?  Then the loaders wait for
-      // the left panel to be released.
-      Cursor nx = c;
-      nx.n = nx.n_vis_end;
-      do { nx.t++; load_unit(nx); } while (nx.valid && nx.n >= nx.n_vis_end);
-      if (nx.valid) __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // the panels have been read
+    __builtin_amdgcn_s_barrier();        // Y(j): the staging tile has been read
+    // narrow and write the wavefront's 64 x 64 block: lane (row l % 32, half l / 32) of block
+    // (i, jj) holds columns 8q + 4*(l/32) .. +3 in elements 4q .. 4q+3
+    const int lrow = lane & 31, g = lane >> 5;
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+      const int row = wm * 64 + i * 32 + lrow;
+#pragma unroll
+      for (int jj = 0; jj < TN; jj++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+          half4_t h;
+#pragma unroll
+          for (int e = 0; e < 4; e++) h[e] = (half_t)acc[i][jj][4 * q + e];
+          const int cc = wn * 8 + jj * 4 + q;
+          *(half4_t*)(sC + row * 256 + ((cc ^ (row & 15)) << 4) + g * 8) = h;
+        }
     }
-    // fully masked tiles of this unit
-    for (int n = max(first, c.n_vis_end); n < c.n_end; n++)
-      fill_masked_tile<BM, BN, NWC * 64>(a, a.output + (int64_t)c.batch * a.stride_oz, c.m0,
-                                         n * BN, tid);
-    c.t++;
-    load_unit(c);
+    next_item(c);
   }
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  __builtin_amdgcn_s_barrier();  // Z: last staging tile complete
 }
 
 // =============================================================================================
@@ -1161,7 +1250,7 @@ hipError_t launch_shortk(hipStream_t stream, const MatmulArgs& a) {
   map.segs_per_row = (map.tiles_n + map.seg - 1) / map.seg;
   map.units = map.rows * map.segs_per_row;
   const unsigned grid = map.units < NUM_CU ? (unsigned)map.units : NUM_CU;
-  hipLaunchKernelGGL((gemm_nt_shortk_kernel<CPR>), dim3(grid), dim3(512), 0, stream, a, map);
+  hipLaunchKernelGGL((gemm_nt_shortk_kernel<CPR>), dim3(grid), dim3(1024), 0, stream, a, map);
   return hipGetLastError();
 }
 
@@ -1221,7 +1310,7 @@ GemmChoice choose(const MatmulArgs& a) {
   if (plain && a.k % 64 == 0) {
     // Few K slices: the tile is dominated by its load latency and its epilogue; two resident
     // workgroups per CU overlap those phases, which one large tile cannot.
-    if ((a.k == 64 || a.k == 128) &&
+    if ((a.k == 64 || a.k == 128) && !(a.store == STORE_ACC_BETA && a.beta != 0.0f) &&
         (int64_t)((a.m + 127) / 128) * ((a.n + 127) / 128) * a.batches >= 2 * NUM_CU)
       return a.k == 64 ? SHORTK_64 : SHORTK_128;
     if (a.k <= 256) {
