@@ -277,7 +277,9 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_dot_kernel(half_t* __restrict
     half_t sc[SEGW];
 #pragma unroll
     for (int j = 0; j < SEGW; j++) {
-      w[j] = act[j] ? *(const u32x4_t*)(wp + (wave + j * NW) * 1024) : u32x4_t{0, 0, 0, 0};
+      // streaming load: a weight byte is read once per launch
+      w[j] = act[j] ? __builtin_nontemporal_load((const u32x4_t*)(wp + (wave + j * NW) * 1024))
+                    : u32x4_t{0, 0, 0, 0};
       sc[j] = act[j] ? sp[sidx[j]] : (half_t)0;
     }
     float tot[MR];
