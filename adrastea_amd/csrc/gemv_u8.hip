@@ -57,7 +57,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_kernel(half_t* __restrict__ o
   const uint8_t* wrow = rhs + (int64_t)row * p + g * 16;
   const half_t* srow = scales + (int64_t)row * nblk;
   const bool xvalid = r < m;
-  const half_t* xrow = lhs + (int64_t)(xvalid ? r : 0) * p + g * 16;
+  const half_t* xrow = lhs + (int64_t)min(r, m - 1) * p + g * 16;
   const int steps = p / MACRO_K;
 
   auto load = [&](Stage& s, int ms) {
@@ -68,8 +68,11 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_kernel(half_t* __restrict__ o
     const half_t* xp = xrow + (int64_t)ms * MACRO_K;
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-      s.x[2 * j] = xvalid ? *(const u32x4_t*)(xp + j * 64) : u32x4_t{0, 0, 0, 0};
-      s.x[2 * j + 1] = xvalid ? *(const u32x4_t*)(xp + j * 64 + 8) : u32x4_t{0, 0, 0, 0};
+      // (lanes beyond m load row m-1 again -- same addresses as its own lanes, no extra
+      // traffic -- and are zeroed: a load under a branch would be waited for at the join)
+      const u32x4_t x0 = *(const u32x4_t*)(xp + j * 64), x1 = *(const u32x4_t*)(xp + j * 64 + 8);
+      s.x[2 * j] = xvalid ? x0 : u32x4_t{0, 0, 0, 0};
+      s.x[2 * j + 1] = xvalid ? x1 : u32x4_t{0, 0, 0, 0};
     }
   };
 
@@ -145,7 +148,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_wide_kernel(half_t* __restric
   const int n0 = blockIdx.x * (ROWS * RG);
   const int nblk = p / 32;
   const bool xvalid = r < m;
-  const half_t* xrow = lhs + (int64_t)(xvalid ? r : 0) * p + g * 16;
+  const half_t* xrow = lhs + (int64_t)min(r, m - 1) * p + g * 16;
   const int steps = p / MACRO_K;
   const uint8_t* wrow[RG];
   const half_t* srow[RG];
@@ -165,6 +168,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_wide_kernel(half_t* __restric
     const half_t* xp = xrow + (int64_t)ms * MACRO_K;
 #pragma unroll
     for (int j = 0; j < 4; j++) {
+      // (under the lane mask on purpose: measured faster here than unconditional loads of a
+      // clamped row, which is what the 16-row kernel does)
       x[2 * j] = xvalid ? *(const u32x4_t*)(xp + j * 64) : u32x4_t{0, 0, 0, 0};
       x[2 * j + 1] = xvalid ? *(const u32x4_t*)(xp + j * 64 + 8) : u32x4_t{0, 0, 0, 0};
     }
@@ -268,20 +273,30 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_dot_kernel(half_t* __restrict
       xs[j][mm] = 1151.5f * sum;
     }
   }
+  // every weight load of the workgroup is issued before the first one is used
+  u32x4_t wall[RPB][SEGW];
+  half_t scall[RPB][SEGW];
 #pragma unroll
   for (int r = 0; r < RPB; r++) {
     const int row = min(n0 + r, n - 1);  // rows beyond n are clamped; their sums are not stored
     const uint8_t* wp = rhs + (int64_t)row * p + lane * 16;
     const half_t* sp = scales + (int64_t)row * nblk;
-    u32x4_t w[SEGW];
-    half_t sc[SEGW];
 #pragma unroll
     for (int j = 0; j < SEGW; j++) {
       // streaming load: a weight byte is read once per launch
-      w[j] = act[j] ? __builtin_nontemporal_load((const u32x4_t*)(wp + (wave + j * NW) * 1024))
-                    : u32x4_t{0, 0, 0, 0};
-      sc[j] = act[j] ? sp[sidx[j]] : (half_t)0;
+      // (unconditional loads from a clamped address: a load under a branch would be waited
+      // for at the join, one memory latency per row; the activations of an inactive segment
+      // are zero, its scale is replaced by zero)
+      wall[r][j] = __builtin_nontemporal_load(
+          (const u32x4_t*)(wp + (act[j] ? (wave + j * NW) * 1024 : -lane * 16)));
+      const half_t sv = sp[act[j] ? sidx[j] : 0];
+      scall[r][j] = act[j] ? sv : (half_t)0;
     }
+  }
+#pragma unroll
+  for (int r = 0; r < RPB; r++) {
+    const u32x4_t (&w)[SEGW] = wall[r];
+    const half_t (&sc)[SEGW] = scall[r];
     float tot[MR];
 #pragma unroll
     for (int mm = 0; mm < MR; mm++) tot[mm] = 0.0f;
@@ -394,7 +409,7 @@ hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, co
     case U8_DOT: {
       const bool wide = n > 6144;
       if (p <= 4096) {  // 4 wavefronts, one segment each
-        if (m == 1) return wide ? launch_dot<1, 4, 8, 1>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta)
+        if (m == 1) return wide ? launch_dot<1, 4, 4, 1>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta)
                                 : launch_dot<1, 4, 2, 1>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
         if (m == 2) return launch_dot<2, 4, 4, 1>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
         return launch_dot<4, 4, 4, 1>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
