@@ -255,25 +255,24 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_dot_kernel(half_t* __restrict
   float xs[SEGW][MR];       // 1151.5 * their sum
   bool act[SEGW];
   int sidx[SEGW];           // scale block of the lane's 16 weights
+  // All loads of the workgroup are issued up front and unconditionally (a load under a branch
+  // would be waited for at the join): inactive segments and rows beyond m read a clamped address
+  // and are zeroed afterwards.
+  u32x4_t xraw[SEGW][MR][2];
 #pragma unroll
   for (int j = 0; j < SEGW; j++) {
     const int seg = wave + j * NW;
     const int k = seg * 1024 + lane * 16;
     act[j] = seg < nseg && k < p;
     sidx[j] = k / block_size;
+    const int kc = act[j] ? k : 0;
 #pragma unroll
     for (int mm = 0; mm < MR; mm++) {
-      const bool v = act[j] && mm < m;
-      const u32x4_t z = {0, 0, 0, 0};
-      xr[j][mm][0] = __builtin_bit_cast(half8_t, v ? *(const u32x4_t*)(lhs + (int64_t)mm * p + k) : z);
-      xr[j][mm][1] = __builtin_bit_cast(half8_t, v ? *(const u32x4_t*)(lhs + (int64_t)mm * p + k + 8) : z);
-      float sum = 0.0f;
-#pragma unroll
-      for (int e = 0; e < 8; e++) sum += (float)xr[j][mm][0][e] + (float)xr[j][mm][1][e];
-      xs[j][mm] = 1151.5f * sum;
+      const half_t* xp = lhs + (int64_t)min(mm, m - 1) * p + kc;
+      xraw[j][mm][0] = *(const u32x4_t*)xp;
+      xraw[j][mm][1] = *(const u32x4_t*)(xp + 8);
     }
   }
-  // every weight load of the workgroup is issued before the first one is used
   u32x4_t wall[RPB][SEGW];
   half_t scall[RPB][SEGW];
 #pragma unroll
@@ -284,13 +283,24 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_dot_kernel(half_t* __restrict
 #pragma unroll
     for (int j = 0; j < SEGW; j++) {
       // streaming load: a weight byte is read once per launch
-      // (unconditional loads from a clamped address: a load under a branch would be waited
-      // for at the join, one memory latency per row; the activations of an inactive segment
-      // are zero, its scale is replaced by zero)
       wall[r][j] = __builtin_nontemporal_load(
           (const u32x4_t*)(wp + (act[j] ? (wave + j * NW) * 1024 : -lane * 16)));
       const half_t sv = sp[act[j] ? sidx[j] : 0];
       scall[r][j] = act[j] ? sv : (half_t)0;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < SEGW; j++) {
+#pragma unroll
+    for (int mm = 0; mm < MR; mm++) {
+      const bool v = act[j] && mm < m;
+      const u32x4_t z = {0, 0, 0, 0};
+      xr[j][mm][0] = __builtin_bit_cast(half8_t, v ? xraw[j][mm][0] : z);
+      xr[j][mm][1] = __builtin_bit_cast(half8_t, v ? xraw[j][mm][1] : z);
+      float sum = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 8; e++) sum += (float)xr[j][mm][0][e] + (float)xr[j][mm][1][e];
+      xs[j][mm] = 1151.5f * sum;
     }
   }
 #pragma unroll
