@@ -76,6 +76,39 @@ __global__ __launch_bounds__(256) void quantize_kernel(adr_tensor_desc out, adr_
   }
 }
 
+// Contiguous rows, block sizes 8 * 2^k <= 512: a lane takes 8 consecutive values (one 16-byte
+// load, one 8-byte store), the bs/8 lanes of a block find the absmax with xor shuffles.  Same
+// arithmetic, operation for operation, as quantize_kernel.
+__global__ __launch_bounds__(256) void quantize_vec_kernel(adr_tensor_desc out, adr_tensor_desc scales,
+                                                           adr_tensor_desc in, int block_size) {
+  const uint32_t row = blockIdx.x;
+  const uint32_t cols = in.shape[0];
+  const uint32_t c = (blockIdx.y * 256 + threadIdx.x) * 8;
+  const bool live = c < cols;  // cols % block_size == 0, so a block is all live or all dead
+  const half_t* x = (const half_t*)in.ptr + (size_t)row * in.strides[1];
+  uint8_t* q = (uint8_t*)out.ptr + (size_t)row * out.strides[1];
+  half8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (live) v = *(const half8_t*)(x + c);
+  float absmax = 0.0f;
+#pragma unroll
+  for (int e = 0; e < 8; e++) absmax = fmaxf(absmax, fabsf((float)v[e]));
+  const int lanes = block_size / 8;
+  for (int off = 1; off < lanes; off <<= 1) absmax = fmaxf(absmax, __shfl_xor(absmax, off, 64));
+  if (!live) return;
+  const half_t hs = (half_t)(absmax / 127.5f);  // quantize.cu:33
+  if ((c % block_size) == 0)
+    ((half_t*)scales.ptr)[(size_t)row * scales.strides[1] + (size_t)(c / block_size) * scales.strides[0]] = hs;
+  const float fs = (float)hs;
+  uint32_t w[2] = {0, 0};
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    float r = roundf(127.5f + (float)v[e] / fs);  // quantize.cu:41-42
+    uint32_t b = (r != r) ? 0u : (uint32_t)fminf(fmaxf(r, 0.0f), 255.0f);
+    w[e >> 2] |= b << (8 * (e & 3));
+  }
+  *(u32x2_t*)(q + c) = u32x2_t{w[0], w[1]};
+}
+
 hipError_t launch_dequantize(hipStream_t stream, adr_tensor_desc out, adr_tensor_desc scales,
                              adr_tensor_desc in) {
   const uint32_t cols = out.shape[0], rows = out.shape[1];
@@ -92,6 +125,16 @@ hipError_t launch_quantize(hipStream_t stream, adr_tensor_desc out, adr_tensor_d
   const uint32_t cols = out.shape[0], rows = out.shape[1];
   const int blocks_per_row = scales.shape[0];
   const int block_size = cols / blocks_per_row;
+  const int lanes = block_size / 8;
+  const bool vec = block_size % 8 == 0 && lanes <= 64 && (lanes & (lanes - 1)) == 0 &&
+                   in.strides[0] == 1 && out.strides[0] == 1 && in.strides[1] % 8 == 0 &&
+                   out.strides[1] % 8 == 0 && (uintptr_t)in.ptr % 16 == 0 &&
+                   (uintptr_t)out.ptr % 8 == 0 && (cols + 2047) / 2048 <= 65535;
+  if (vec) {
+    hipLaunchKernelGGL(quantize_vec_kernel, dim3(rows, (cols + 2047) / 2048, 1), dim3(256, 1, 1), 0,
+                       stream, out, scales, in, block_size);
+    return hipGetLastError();
+  }
   if ((blocks_per_row + 3) / 4 > 65535) return hipErrorInvalidConfiguration;
   hipLaunchKernelGGL(quantize_kernel, dim3(rows, (blocks_per_row + 3) / 4, 1), dim3(256, 1, 1), 0,
                      stream, out, scales, in, block_size, blocks_per_row);

@@ -88,6 +88,26 @@ def test_quantize_matches_oracle_and_reference_kernel(kern, ref):
     assert np.array_equal(to_np(q_r), q_want)
 
 
+@pytest.mark.parametrize("bs", [8, 16, 24, 32, 64, 96, 256, 512, 1024])
+def test_quantize_block_sizes_vector_and_scalar_paths(kern, bs):
+    """Block sizes 8 * 2^k <= 512 take the vectorised kernel, the others the one-wavefront-per-
+    block kernel; both must agree with the oracle bit for bit, including all-zero blocks (scale 0:
+    the value/0 quotients are NaN or infinite and map to 0 or saturate), and a ragged column
+    count (cols not a multiple of the 2048 columns a workgroup covers)."""
+    g = rng(670 + bs)
+    rows, cols = 37, bs * 9
+    x = randn_f16(g, (rows, cols), 0.3)
+    x[3, :bs] = 0                      # all-zero block
+    x[4, bs:2 * bs] = np.float16(65504.0)
+    x[5, 0] = np.float16(-65504.0)
+    q_want, s_want = oracle.quantize_absmax_u8(x, bs)
+    q_t = torch.zeros(rows, cols, dtype=torch.uint8, device="cuda")
+    s_t = torch.zeros(rows, cols // bs, dtype=torch.float16, device="cuda")
+    kern.quantize_absmax_uint8(q_t, s_t, to_dev(x))
+    assert np.array_equal(to_np(s_t).view(np.uint16), s_want.view(np.uint16))
+    assert np.array_equal(to_np(q_t), q_want)
+
+
 def _finite_scale_rows():
     # scale patterns whose 256 dequantised values are all finite (|s| <= 512): an infinite
     # weight times a zero activation would poison the row's sums.  Larger scales, inf and NaN
