@@ -213,4 +213,13 @@ int adr_quantize_absmax_u8(adr_stream_t stream, uint8_t* q, uint16_t* scales,
                                    desc2d(input, rows, cols));
 }
 
+int adr_softmax_rows(adr_stream_t stream, uint16_t* output, const uint16_t* input, int32_t heads,
+                     int32_t h, int32_t w, float temp) {
+  if (heads < 0 || h < 0 || w < 0) return ADR_EINVAL_SHAPE;
+  if (heads == 0 || h == 0 || w == 0) return ADR_OK;
+  if (!output || !input) return ADR_ENULL;
+  return (int)launch_softmax_rows((hipStream_t)stream, (half_t*)output, (const half_t*)input,
+                                  (int64_t)heads * h, w, temp);
+}
+
 }  // extern "C"

@@ -91,6 +91,7 @@ struct CommonKernels {
                           const TensorView<const f16>& right, const MatmulOptions& options) = 0;
   virtual void matmul_f16_slow(TensorView<f16>& output, const TensorView<const f16>& left,
                                const TensorView<const f16>& right, const MatmulOptions& options) = 0;
+  virtual void softmax_rows_inplace(TensorView<f16>& output, float temperature) = 0;
 };
 
 class GpuKernels : public CommonKernels {
@@ -100,6 +101,14 @@ class GpuKernels : public CommonKernels {
                   const MatmulOptions& opt) override { run(adr_matmul_f16, "matmul_f16", o, l, r, opt); }
   void matmul_f16_slow(TensorView<f16>& o, const TensorView<const f16>& l, const TensorView<const f16>& r,
                        const MatmulOptions& opt) override { run(adr_matmul_f16_slow, "matmul_f16_slow", o, l, r, opt); }
+  // kernels.rs:892-915: rows = size(-2), heads = size(-3) (1 for rank 2), width = size(-1); like
+  // the reference's kernel, the view is taken to be contiguous.
+  void softmax_rows_inplace(TensorView<f16>& o, float temperature) override {
+    if (!(o.layout == TensorLayout::row_major(o.layout.dims))) throw std::logic_error("softmax_rows: contiguous view");
+    const int32_t heads = o.layout.dims.size() > 2 ? (int32_t)o.size(-3) : 1;
+    int rc = adr_softmax_rows(stream_, o.ptr, o.ptr, heads, (int32_t)o.size(-2), (int32_t)o.size(-1), temperature);
+    if (rc) throw AdrasteaError(rc, "softmax_rows_inplace");
+  }
   std::string plan(const TensorLayout& o, const TensorLayout& l, const TensorLayout& r, const MatmulOptions& opt) const {
     LoweredMatmul w = lower_matmul(o, l, r, opt);
     char name[64];
@@ -131,6 +140,7 @@ class MatmulTracer : public CommonKernels {
                   const MatmulOptions& opt) override { rec(o, l, r); inner_.matmul_f16(o, l, r, opt); }
   void matmul_f16_slow(TensorView<f16>& o, const TensorView<const f16>& l, const TensorView<const f16>& r,
                        const MatmulOptions& opt) override { rec(o, l, r); inner_.matmul_f16_slow(o, l, r, opt); }
+  void softmax_rows_inplace(TensorView<f16>& o, float t) override { inner_.softmax_rows_inplace(o, t); }
 
  private:
   void rec(const TensorView<f16>& o, const TensorView<const f16>& l, const TensorView<const f16>& r) {

@@ -165,6 +165,9 @@ class CommonKernels:
                         options: MatmulOptions) -> None:
         raise NotImplementedError
 
+    def softmax_rows_inplace(self, output: TensorView, temperature: float) -> None:
+        raise NotImplementedError
+
 
 def _current_stream() -> int:
     import torch
@@ -195,6 +198,17 @@ class GpuKernels(CommonKernels):
     def matmul_f16_slow(self, output, left, right, options=MatmulOptions()):
         self._matmul(self._lib.adr_matmul_f16_slow, "matmul_f16_slow", output, left, right,
                      options)
+
+    def softmax_rows_inplace(self, output, temperature: float = 1.0):
+        """kernels.rs:892-915: rows = size(-2), heads = size(-3) (1 for rank 2), width size(-1);
+        like the reference's kernel, the tensor is taken to be contiguous."""
+        lay = output.layout
+        assert lay == TensorLayout.row_major(list(lay.dims)), "softmax_rows needs a contiguous view"
+        heads = lay.size(-3) if len(lay.dims) > 2 else 1
+        rc = self._lib.adr_softmax_rows(_current_stream(), output.data_ptr(), output.data_ptr(),
+                                        heads, lay.size(-2), lay.size(-1), float(temperature))
+        if rc != 0:
+            raise AdrasteaError(rc, "softmax_rows_inplace")
 
     # -- contiguous NT forms (device signatures only in the reference) --
     def matmul_nt_f16(self, output, lhs, rhs, beta: float = 0.0):
@@ -284,3 +298,6 @@ class MatmulTracer(CommonKernels):
     def matmul_f16_slow(self, output, left, right, options=MatmulOptions()):
         self._record(output, left, right)
         self.inner.matmul_f16_slow(output, left, right, options)
+
+    def softmax_rows_inplace(self, output, temperature: float = 1.0):
+        self.inner.softmax_rows_inplace(output, temperature)   # forwarded (kernels.rs:334-338)

@@ -267,6 +267,17 @@ def main():
         attn = {"qk_t": {"us": round(t * 1e6, 1), "tflops": round(2.0 * H * S * S * D / t / 1e12, 1),
                          "gbs": round(byts / t / 1e9, 1),
                          "frac_hbm_peak": round(byts / t / 1e9 / PEAK_HBM_GBS, 4)}}
+        # softmax_rows in place on the scores (read + write of the [32, 2048, 2048] tensor)
+        def f_sm():
+            rc = lib.adr_softmax_rows(stream(), qk.data_ptr(), qk.data_ptr(), H, S, S, 1.0)
+            if rc != 0:
+                raise RuntimeError(_ffi.strerror(rc))
+        f_qk()
+        t = timed(f_sm, 30, 3)
+        sm_bytes = 2 * H * S * S * 2
+        attn["softmax_rows"] = {"us": round(t * 1e6, 1), "gbs": round(sm_bytes / t / 1e9, 1),
+                                "frac_hbm_peak": round(sm_bytes / t / 1e9 / PEAK_HBM_GBS, 4)}
+        f_qk()
         p_ = torch.softmax(qk.float(), dim=-1).half()
         o_ = torch.zeros(S, HD, dtype=torch.float16, device=dev)
 

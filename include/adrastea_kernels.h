@@ -147,6 +147,18 @@ int adr_quantize_absmax_uint8(adr_stream_t stream, adr_tensor_desc output,
                               adr_tensor_desc scales, adr_tensor_desc input);
 
 /*
+ * Row-wise softmax with temperature, the step between QK^T and P.V
+ * (device: adrastea_kernels/cpp/normalize.cu:147-220 `softmax_rows(output, input, h, w, temp)` on
+ * a (heads, h) grid; host: CommonKernels::softmax_rows_inplace, adrastea_models/src/kernels.rs:214,
+ * 892-915, which passes output twice).  `input` and `output` are contiguous [heads, h, w] fp16
+ * tensors and may be the same buffer:
+ *   out[i] = fp16( expf(in[i]/temp - max) / sum_j expf(in[j]/temp - max) )   over each row of w.
+ * The reference's third and fourth arguments (h, w) are kept; `heads` replaces its grid.y.
+ */
+int adr_softmax_rows(adr_stream_t stream, uint16_t* output, const uint16_t* input, int32_t heads,
+                     int32_t h, int32_t w, float temp);
+
+/*
  * Diagnostics (no counterpart in the reference).
  *
  * adr_matmul_f16_plan: writes the name of the kernel adr_matmul_f16 would launch for these

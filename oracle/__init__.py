@@ -70,6 +70,7 @@ def lib():
         L.adr_o_dequantize_absmax_u8.argtypes = [u16p, u8p, u16p, C.c_int, C.c_int, C.c_int]
         L.adr_o_quantize_absmax_u8.argtypes = [u8p, u16p, u16p, C.c_int, C.c_int, C.c_int]
         L.adr_o_dequant_table.argtypes = [u16p]
+        L.adr_o_softmax_rows.argtypes = [u16p, u16p, C.c_int64, C.c_int, C.c_float, C.c_int]
         _lib = L
     return _lib
 
@@ -154,6 +155,18 @@ def quantize_absmax_u8(x, block_size):
     lib().adr_o_quantize_absmax_u8(_p8(q), _p16(scales.view(np.uint16)), _p16(x.view(np.uint16)),
                                    rows, cols, block_size)
     return q, scales
+
+
+def softmax_rows(x, temp=1.0, mode=0):
+    """normalize.cu:147-220 over the last axis of a contiguous fp16 array.  mode 0: the
+    reference's fp32 arithmetic and reduction order; mode 1: float64, one final rounding."""
+    x = np.ascontiguousarray(x)
+    assert x.dtype == np.float16
+    w = x.shape[-1]
+    out = np.empty_like(x)
+    lib().adr_o_softmax_rows(_p16(out.reshape(-1).view(np.uint16)),
+                             _p16(x.reshape(-1).view(np.uint16)), x.size // w, w, float(temp), mode)
+    return out
 
 
 def dequant_table():

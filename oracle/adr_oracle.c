@@ -326,3 +326,56 @@ void adr_o_dequant_table(uint16_t* out) {
   for (int q = 0; q < 256; q++)
     for (int s = 0; s < 65536; s++) out[(int64_t)q * 65536 + s] = dequant_one((uint8_t)q, (uint16_t)s);
 }
+
+/* ---- softmax_rows (normalize.cu:147-220) ------------------------------------------------ */
+
+/* xor-butterfly over `n` values (n a power of two), as __shfl_xor_sync with offsets n/2 .. 1
+ * leaves it in lane 0; op 0 = fmaxf, 1 = + */
+static float xor_tree(float* v, int n, int op) {
+  float tmp[32];
+  for (int off = n / 2; off > 0; off /= 2) {
+    for (int i = 0; i < n; i++) {
+      float o = v[i ^ off];
+      tmp[i] = op ? v[i] + o : fmaxf(v[i], o);
+    }
+    memcpy(v, tmp, sizeof(float) * n);
+  }
+  return v[0];
+}
+
+void adr_o_softmax_rows(uint16_t* output, const uint16_t* input, int64_t rows, int w, float temp,
+                        int mode) {
+  for (int64_t r = 0; r < rows; r++) {
+    const uint16_t* in = input + r * w;
+    uint16_t* out = output + r * w;
+    if (mode == 1) {
+      double mx = -INFINITY, sum = 0.0;
+      for (int i = 0; i < w; i++) mx = fmax(mx, (double)adr_o_h2f(in[i]) / (double)temp);
+      for (int i = 0; i < w; i++) sum += exp((double)adr_o_h2f(in[i]) / (double)temp - mx);
+      for (int i = 0; i < w; i++)
+        out[i] = adr_o_d2h(exp((double)adr_o_h2f(in[i]) / (double)temp - mx) / sum);
+      continue;
+    }
+    /* :160-163 per-thread maxima, thread t takes i = t, t + 256, ... */
+    float part[256], grp[8];
+    for (int t = 0; t < 256; t++) {
+      float m = -INFINITY;
+      for (int i = t; i < w; i += 256) m = fmaxf(m, adr_o_h2f(in[i]) / temp);
+      part[t] = m;
+    }
+    /* :166-184 32-lane trees, then the 8 leaders */
+    for (int g = 0; g < 8; g++) grp[g] = xor_tree(part + 32 * g, 32, 0);
+    const float mx = xor_tree(grp, 8, 0);
+    /* :186-191 */
+    for (int t = 0; t < 256; t++) {
+      float sacc = 0.0f;
+      for (int i = t; i < w; i += 256) sacc += expf(adr_o_h2f(in[i]) / temp - mx);
+      part[t] = sacc;
+    }
+    /* :193-211 */
+    for (int g = 0; g < 8; g++) grp[g] = xor_tree(part + 32 * g, 32, 1);
+    const float sum = xor_tree(grp, 8, 1);
+    /* :213-216 */
+    for (int i = 0; i < w; i++) out[i] = adr_o_f2h(expf(adr_o_h2f(in[i]) / temp - mx) / sum);
+  }
+}

@@ -90,6 +90,13 @@ void adr_o_dequantize_absmax_u8(uint16_t* output, const uint8_t* q, const uint16
 void adr_o_quantize_absmax_u8(uint8_t* q, uint16_t* scales, const uint16_t* input, int rows,
                               int cols, int block_size);
 
+/* normalize.cu:147-220 softmax_rows on a contiguous [rows, w] fp16 tensor (rows = heads * h).
+ * mode 0: the reference's arithmetic and reduction order in fp32 (256 threads striding the row,
+ * xor trees over 32-lane groups, then over the 8 group results); mode 1: float64 throughout,
+ * one rounding to fp16 at the end. */
+void adr_o_softmax_rows(uint16_t* output, const uint16_t* input, int64_t rows, int w, float temp,
+                        int mode);
+
 /* exhaustive dequant table: out[q * 65536 + s] = dequant(q, scale bits s) */
 void adr_o_dequant_table(uint16_t* out);
 

@@ -21,6 +21,10 @@ def available():
                for f in ("matmul.co", "quantize.co", "matmul_nt_fp16u8.co"))
 
 
+def has(name):
+    return os.path.exists(os.path.join(REF_DIR, name))
+
+
 class TensorDesc(C.Structure):
     _fields_ = [("ptr", C.c_void_p), ("dims", C.c_uint32), ("shape", C.c_uint32 * 7),
                 ("strides", C.c_uint32 * 7)]
@@ -113,3 +117,10 @@ class RefKernels:
         f = self._fn("quantize.co", QUANTIZE_SYM)
         args = [desc2d(q), desc2d(scales), desc2d(x)]
         self._launch(f, (scales.shape[1], x.shape[0], 1), (32, 1, 1), 0, args)
+
+    def softmax_rows(self, out, inp, heads, h, w, temp=1.0):
+        """normalize.cu:147-220 with the launch of kernels.rs:892-915 ((h, heads) x 256)."""
+        f = self._fn("normalize.co", b"softmax_rows")
+        args = [C.c_void_p(out.data_ptr()), C.c_void_p(inp.data_ptr()), C.c_int(h), C.c_int(w),
+                C.c_float(temp)]
+        self._launch(f, (h, heads, 1), (256, 1, 1), 0, args)
