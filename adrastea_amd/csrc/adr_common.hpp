@@ -136,6 +136,8 @@ hipError_t launch_dequantize(hipStream_t stream, adr_tensor_desc out, adr_tensor
                              adr_tensor_desc in);
 hipError_t launch_quantize(hipStream_t stream, adr_tensor_desc out, adr_tensor_desc scales,
                            adr_tensor_desc in);
+hipError_t launch_error_stats(hipStream_t stream, float* out, const void* lhs, const void* rhs,
+                              int64_t length, int64_t sl, int64_t sr, bool f32);
 hipError_t launch_softmax_rows(hipStream_t stream, half_t* out, const half_t* in, int64_t rows,
                                int w, float temp);
 

@@ -222,4 +222,25 @@ int adr_softmax_rows(adr_stream_t stream, uint16_t* output, const uint16_t* inpu
                                   (int64_t)heads * h, w, temp);
 }
 
+static int error_stats_common(adr_stream_t stream, adr_tensor_desc output, adr_tensor_desc lhs,
+                              adr_tensor_desc rhs, bool f32) {
+  if (output.dims != 1 || lhs.dims != 1 || rhs.dims != 1) return ADR_EINVAL_SHAPE;
+  if (output.shape[0] < 3 || output.strides[0] != 1 || lhs.shape[0] != rhs.shape[0])
+    return ADR_EINVAL_SHAPE;
+  if (lhs.shape[0] == 0) return ADR_OK;
+  if (!output.ptr || !lhs.ptr || !rhs.ptr) return ADR_ENULL;
+  return (int)launch_error_stats((hipStream_t)stream, (float*)output.ptr, lhs.ptr, rhs.ptr,
+                                 lhs.shape[0], lhs.strides[0], rhs.strides[0], f32);
+}
+
+int adr_error_stats_f16(adr_stream_t stream, adr_tensor_desc output, adr_tensor_desc lhs,
+                        adr_tensor_desc rhs) {
+  return error_stats_common(stream, output, lhs, rhs, false);
+}
+
+int adr_error_stats_f32(adr_stream_t stream, adr_tensor_desc output, adr_tensor_desc lhs,
+                        adr_tensor_desc rhs) {
+  return error_stats_common(stream, output, lhs, rhs, true);
+}
+
 }  // extern "C"

@@ -92,7 +92,24 @@ struct CommonKernels {
   virtual void matmul_f16_slow(TensorView<f16>& output, const TensorView<const f16>& left,
                                const TensorView<const f16>& right, const MatmulOptions& options) = 0;
   virtual void softmax_rows_inplace(TensorView<f16>& output, float temperature) = 0;
+  virtual void error_stats_f16(TensorView<float>& output, const TensorView<const f16>& lhs,
+                               const TensorView<const f16>& rhs) = 0;
+  virtual void error_stats_f32(TensorView<float>& output, const TensorView<const float>& lhs,
+                               const TensorView<const float>& rhs) = 0;
 };
+
+// TensorGpuDescriptor::from (kernels.rs:38-55): dims and strides reversed, innermost first.
+template <typename T>
+inline adr_tensor_desc descriptor(const TensorView<T>& v) {
+  adr_tensor_desc d{};
+  d.ptr = (void*)v.ptr;
+  d.dims = (uint32_t)v.layout.dims.size();
+  for (size_t i = 0; i < v.layout.dims.size(); i++) {
+    d.shape[i] = (uint32_t)v.layout.dims[v.layout.dims.size() - 1 - i];
+    d.strides[i] = (uint32_t)v.layout.strides[v.layout.dims.size() - 1 - i];
+  }
+  return d;
+}
 
 class GpuKernels : public CommonKernels {
  public:
@@ -108,6 +125,19 @@ class GpuKernels : public CommonKernels {
     const int32_t heads = o.layout.dims.size() > 2 ? (int32_t)o.size(-3) : 1;
     int rc = adr_softmax_rows(stream_, o.ptr, o.ptr, heads, (int32_t)o.size(-2), (int32_t)o.size(-1), temperature);
     if (rc) throw AdrasteaError(rc, "softmax_rows_inplace");
+  }
+  // kernels.rs:717-751: both operands flattened with shape_cast(&[-1]); equal lengths
+  void error_stats_f16(TensorView<float>& out, const TensorView<const f16>& l, const TensorView<const f16>& r) override {
+    auto lf = l.shape_cast({-1}), rf = r.shape_cast({-1});
+    if (lf.size(-1) != rf.size(-1)) throw std::logic_error("error_stats: length mismatch");
+    int rc = adr_error_stats_f16(stream_, descriptor(out), descriptor(lf), descriptor(rf));
+    if (rc) throw AdrasteaError(rc, "error_stats_f16");
+  }
+  void error_stats_f32(TensorView<float>& out, const TensorView<const float>& l, const TensorView<const float>& r) override {
+    auto lf = l.shape_cast({-1}), rf = r.shape_cast({-1});
+    if (lf.size(-1) != rf.size(-1)) throw std::logic_error("error_stats: length mismatch");
+    int rc = adr_error_stats_f32(stream_, descriptor(out), descriptor(lf), descriptor(rf));
+    if (rc) throw AdrasteaError(rc, "error_stats_f32");
   }
   std::string plan(const TensorLayout& o, const TensorLayout& l, const TensorLayout& r, const MatmulOptions& opt) const {
     LoweredMatmul w = lower_matmul(o, l, r, opt);
@@ -141,6 +171,8 @@ class MatmulTracer : public CommonKernels {
   void matmul_f16_slow(TensorView<f16>& o, const TensorView<const f16>& l, const TensorView<const f16>& r,
                        const MatmulOptions& opt) override { rec(o, l, r); inner_.matmul_f16_slow(o, l, r, opt); }
   void softmax_rows_inplace(TensorView<f16>& o, float t) override { inner_.softmax_rows_inplace(o, t); }
+  void error_stats_f16(TensorView<float>& out, const TensorView<const f16>& l, const TensorView<const f16>& r) override { inner_.error_stats_f16(out, l, r); }
+  void error_stats_f32(TensorView<float>& out, const TensorView<const float>& l, const TensorView<const float>& r) override { inner_.error_stats_f32(out, l, r); }
 
  private:
   void rec(const TensorView<f16>& o, const TensorView<const f16>& l, const TensorView<const f16>& r) {

@@ -210,6 +210,20 @@ class GpuKernels(CommonKernels):
         if rc != 0:
             raise AdrasteaError(rc, "softmax_rows_inplace")
 
+    def _error_stats(self, fn, what, output, lhs, rhs):
+        # kernels.rs:717-751: both operands flattened with shape_cast(&[-1]); equal lengths
+        lhs, rhs = lhs.shape_cast([-1]), rhs.shape_cast([-1])
+        assert lhs.size(-1) == rhs.size(-1)
+        rc = fn(_current_stream(), descriptor(output), descriptor(lhs), descriptor(rhs))
+        if rc != 0:
+            raise AdrasteaError(rc, what)
+
+    def error_stats_f16(self, output, lhs, rhs):
+        self._error_stats(self._lib.adr_error_stats_f16, "error_stats_f16", output, lhs, rhs)
+
+    def error_stats_f32(self, output, lhs, rhs):
+        self._error_stats(self._lib.adr_error_stats_f32, "error_stats_f32", output, lhs, rhs)
+
     # -- contiguous NT forms (device signatures only in the reference) --
     def matmul_nt_f16(self, output, lhs, rhs, beta: float = 0.0):
         m, p = lhs.shape
@@ -301,3 +315,9 @@ class MatmulTracer(CommonKernels):
 
     def softmax_rows_inplace(self, output, temperature: float = 1.0):
         self.inner.softmax_rows_inplace(output, temperature)   # forwarded (kernels.rs:334-338)
+
+    def error_stats_f16(self, output, lhs, rhs):
+        self.inner.error_stats_f16(output, lhs, rhs)            # forwarded (kernels.rs:349-358)
+
+    def error_stats_f32(self, output, lhs, rhs):
+        self.inner.error_stats_f32(output, lhs, rhs)

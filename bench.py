@@ -290,6 +290,23 @@ def main():
         attn["pv"] = {"us": round(t * 1e6, 1), "tflops": round(2.0 * H * S * S * D / t / 1e12, 1),
                       "gbs": round(byts / t / 1e9, 1),
                       "frac_hbm_peak": round(byts / t / 1e9 / PEAK_HBM_GBS, 4)}
+        # error_stats_f16 of two [32, 2048, 2048] tensors (reads 2 x 268 MB, the on-device check)
+        stat = torch.zeros(3, dtype=torch.float32, device=dev)
+
+        def desc1(t):
+            d = _ffi.TensorDesc()
+            d.ptr, d.dims = t.data_ptr(), 1
+            d.shape[0], d.strides[0] = t.numel(), 1
+            return d
+        d_out, d_l, d_r = desc1(stat), desc1(qk), desc1(p_)
+
+        def f_es():
+            rc = lib.adr_error_stats_f16(stream(), d_out, d_l, d_r)
+            if rc != 0:
+                raise RuntimeError(_ffi.strerror(rc))
+        t = timed(f_es, 30, 3)
+        attn["error_stats_f16"] = {"us": round(t * 1e6, 1), "gbs": round(sm_bytes / t / 1e9, 1),
+                                   "frac_hbm_peak": round(sm_bytes / t / 1e9 / PEAK_HBM_GBS, 4)}
         secondary["llama7b_attention_fp16"] = attn
 
     # ---------------- CPU baseline: the oracle on a bounded sample of the same workload

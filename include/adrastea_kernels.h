@@ -159,6 +159,22 @@ int adr_softmax_rows(adr_stream_t stream, uint16_t* output, const uint16_t* inpu
                      int32_t h, int32_t w, float temp);
 
 /*
+ * Error statistics of two tensors, the reference's on-device parity check
+ * (device: adrastea_kernels/cpp/error_stats.cu:13-75 `error_stats_f16/_f32(output, lhs, rhs)` with
+ * by-value descriptors; host: CommonKernels::error_stats_f16/_f32, adrastea_models/src/kernels.rs:
+ * 223-228, 717-751, which flatten both operands with shape_cast(&[-1])).  1-d descriptors; `output`
+ * is an fp32 vector of at least 3 values that the CALLER zeroes:
+ *   output[0] += mean squared error, output[1] = max(output[1], max abs error),
+ *   output[2] += mean absolute error,
+ * over the first 128 * floor(length / 128) elements with the means divided by `length`, exactly as
+ * the reference's 128-block walk does (its last length % 128 elements are not visited).
+ */
+int adr_error_stats_f16(adr_stream_t stream, adr_tensor_desc output, adr_tensor_desc lhs,
+                        adr_tensor_desc rhs);
+int adr_error_stats_f32(adr_stream_t stream, adr_tensor_desc output, adr_tensor_desc lhs,
+                        adr_tensor_desc rhs);
+
+/*
  * Diagnostics (no counterpart in the reference).
  *
  * adr_matmul_f16_plan: writes the name of the kernel adr_matmul_f16 would launch for these

@@ -70,6 +70,7 @@ def lib():
         L.adr_o_dequantize_absmax_u8.argtypes = [u16p, u8p, u16p, C.c_int, C.c_int, C.c_int]
         L.adr_o_quantize_absmax_u8.argtypes = [u8p, u16p, u16p, C.c_int, C.c_int, C.c_int]
         L.adr_o_dequant_table.argtypes = [u16p]
+        L.adr_o_error_stats.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
         L.adr_o_softmax_rows.argtypes = [u16p, u16p, C.c_int64, C.c_int, C.c_float, C.c_int]
         _lib = L
     return _lib
@@ -166,6 +167,16 @@ def softmax_rows(x, temp=1.0, mode=0):
     out = np.empty_like(x)
     lib().adr_o_softmax_rows(_p16(out.reshape(-1).view(np.uint16)),
                              _p16(x.reshape(-1).view(np.uint16)), x.size // w, w, float(temp), mode)
+    return out
+
+
+def error_stats(lhs, rhs):
+    """error_stats.cu:13-75 on flat fp16 or fp32 arrays: (mse, max abs, mean abs) as float32."""
+    lhs, rhs = np.ascontiguousarray(lhs).reshape(-1), np.ascontiguousarray(rhs).reshape(-1)
+    assert lhs.dtype == rhs.dtype and lhs.dtype in (np.float16, np.float32) and lhs.size == rhs.size
+    out = np.zeros(3, np.float32)
+    lib().adr_o_error_stats(out.ctypes.data_as(C.POINTER(C.c_float)), lhs.ctypes.data_as(C.c_void_p),
+                            rhs.ctypes.data_as(C.c_void_p), lhs.size, int(lhs.dtype == np.float32))
     return out
 
 

@@ -379,3 +379,21 @@ void adr_o_softmax_rows(uint16_t* output, const uint16_t* input, int64_t rows, i
     for (int i = 0; i < w; i++) out[i] = adr_o_f2h(expf(adr_o_h2f(in[i]) / temp - mx) / sum);
   }
 }
+
+/* ---- error_stats (error_stats.cu:13-75) ---------------------------------------------------- */
+void adr_o_error_stats(float* out, const void* lhs, const void* rhs, int64_t length, int is_f32) {
+  const int64_t counted = (length / 128) * 128; /* :27-30 */
+  double sum_sq = 0.0, sum = 0.0;
+  float mx = 0.0f;
+  for (int64_t i = 0; i < counted; i++) {
+    const float a = is_f32 ? ((const float*)lhs)[i] : adr_o_h2f(((const uint16_t*)lhs)[i]);
+    const float b = is_f32 ? ((const float*)rhs)[i] : adr_o_h2f(((const uint16_t*)rhs)[i]);
+    const float d = a - b; /* :32 */
+    sum_sq += (double)(d * d);
+    sum += (double)fabsf(d);
+    mx = fmaxf(mx, fabsf(d));
+  }
+  out[0] = (float)(sum_sq / (double)length);
+  out[1] = mx;
+  out[2] = (float)(sum / (double)length);
+}

@@ -97,6 +97,12 @@ void adr_o_quantize_absmax_u8(uint8_t* q, uint16_t* scales, const uint16_t* inpu
 void adr_o_softmax_rows(uint16_t* output, const uint16_t* input, int64_t rows, int w, float temp,
                         int mode);
 
+/* error_stats.cu:13-75 on flat arrays: out[0] = sum d^2 / length, out[1] = max |d|,
+ * out[2] = sum |d| / length over the first 128 * (length / 128) elements (the reference's 128
+ * blocks of length / 128), d = float(lhs) - float(rhs) in fp32; sums carried in float64 here.
+ * is_f32 selects fp32 inputs (else fp16 bit patterns). */
+void adr_o_error_stats(float* out, const void* lhs, const void* rhs, int64_t length, int is_f32);
+
 /* exhaustive dequant table: out[q * 65536 + s] = dequant(q, scale bits s) */
 void adr_o_dequant_table(uint16_t* out);
 

@@ -115,6 +115,39 @@ static void gpu_test() {
     CHECK(bad == 0);
   }
   CHECK(tr.shapes().size() == 1);
+  // softmax_rows_inplace on the [M, N] result viewed as one head: rows of a causal product sum
+  // to 1 and the masked entries become 0; error_stats of a tensor with itself is all zero
+  tr.softmax_rows_inplace(ov, 1.0f);
+  CHECK(hipDeviceSynchronize() == 0);
+  hipMemcpy(o.data(), dout, o.size() * 2, 2);
+  {
+    int bad = 0;
+    for (int y = 0; y < M; y++) {
+      double sum = 0;
+      for (int x = 0; x < N; x++) {
+        const uint16_t h = o[y * N + x];
+        if (x > y) { bad += h != 0; continue; }
+        const int e = (h >> 10) & 31, m = h & 0x3ff;
+        sum += e ? (double)(0x400 | m) / 1024.0 * (e >= 15 ? (double)(1 << (e - 15)) : 1.0 / (double)(1 << (15 - e)))
+                 : (double)m / 1024.0 / 16384.0;
+      }
+      bad += !(sum > 0.99 && sum < 1.01);
+    }
+    CHECK(bad == 0);
+  }
+  {
+    float* dstat;
+    CHECK(hipMalloc((void**)&dstat, 12) == 0);
+    float z[3] = {0, 0, 0};
+    hipMemcpy(dstat, z, 12, 1);
+    TensorView<float> sv(dstat, TensorLayout::row_major({3}));
+    TensorView<const f16> cv(dout, TensorLayout::row_major({(size_t)M, (size_t)N}));
+    tr.error_stats_f16(sv, cv, cv);
+    CHECK(hipDeviceSynchronize() == 0);
+    float st[3] = {1, 1, 1};
+    hipMemcpy(st, dstat, 12, 2);
+    CHECK(st[0] == 0.0f && st[1] == 0.0f && st[2] == 0.0f);
+  }
   uint16_t bias = 0;
   CHECK(throws([&] { tr.matmul_f16(ov, lv, wv.permute({1, 0}), MatmulOptions::make().store(MatmulStore::GeluBias(&bias))); }));
 }

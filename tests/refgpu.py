@@ -124,3 +124,16 @@ class RefKernels:
         args = [C.c_void_p(out.data_ptr()), C.c_void_p(inp.data_ptr()), C.c_int(h), C.c_int(w),
                 C.c_float(temp)]
         self._launch(f, (h, heads, 1), (256, 1, 1), 0, args)
+
+    def error_stats(self, out, lhs, rhs):
+        """error_stats.cu:64-75 with the launch of kernels.rs:736-751 (128 blocks x 1024)."""
+        import torch
+        name = b"error_stats_f32" if lhs.dtype == torch.float32 else b"error_stats_f16"
+        f = self._fn("error_stats.co", name)
+
+        def d1(t):
+            d = TensorDesc()
+            d.ptr, d.dims = t.data_ptr(), 1
+            d.shape[0], d.strides[0] = t.numel(), 1
+            return d
+        self._launch(f, (128, 1, 1), (1024, 1, 1), 0, [d1(out), d1(lhs), d1(rhs)])
