@@ -35,12 +35,23 @@ __global__ __launch_bounds__(256) void error_stats_kernel(float* out, const T* l
   };
   if (vec) {
     const int64_t nv = counted / VEC;
-    for (int64_t i = tid; i < nv; i += nthreads) {
+    int64_t i = tid;
+    for (; i + nthreads < nv; i += 2 * nthreads) {  // four loads in flight per lane
+      const vec_t a0 = __builtin_nontemporal_load((const vec_t*)(lhs + i * VEC));
+      const vec_t b0 = __builtin_nontemporal_load((const vec_t*)(rhs + i * VEC));
+      const vec_t a1 = __builtin_nontemporal_load((const vec_t*)(lhs + (i + nthreads) * VEC));
+      const vec_t b1 = __builtin_nontemporal_load((const vec_t*)(rhs + (i + nthreads) * VEC));
+#pragma unroll
+      for (int e = 0; e < VEC; e++) take((float)a0[e], (float)b0[e]);
+#pragma unroll
+      for (int e = 0; e < VEC; e++) take((float)a1[e], (float)b1[e]);
+    }
+    for (; i < nv; i += nthreads) {
       const vec_t a = *(const vec_t*)(lhs + i * VEC), b = *(const vec_t*)(rhs + i * VEC);
 #pragma unroll
       for (int e = 0; e < VEC; e++) take((float)a[e], (float)b[e]);
     }
-    for (int64_t i = nv * VEC + tid; i < counted; i += nthreads) take((float)lhs[i], (float)rhs[i]);
+    for (int64_t j = nv * VEC + tid; j < counted; j += nthreads) take((float)lhs[j], (float)rhs[j]);
   } else {
     for (int64_t i = tid; i < counted; i += nthreads) take((float)lhs[i * sl], (float)rhs[i * sr]);
   }
@@ -70,7 +81,7 @@ hipError_t launch_t(hipStream_t stream, float* out, const T* lhs, const T* rhs, 
   const int64_t counted = (length / 128) * 128;  // error_stats.cu:27-30: 128 blocks of length/128
   const bool vec = sl == 1 && sr == 1 && ((uintptr_t)lhs % 16) == 0 && ((uintptr_t)rhs % 16) == 0;
   int64_t blocks = (counted / (16 / (int64_t)sizeof(T)) + 255) / 256;
-  if (blocks > 2048) blocks = 2048;
+  if (blocks > 1024) blocks = 1024;  // every workgroup ends in three same-address atomics
   if (blocks < 1) blocks = 1;
   hipLaunchKernelGGL(error_stats_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, out, lhs,
                      rhs, counted, length, sl, sr, vec);
