@@ -37,6 +37,11 @@ def lib():
         raise RuntimeError(
             f"{LIB_PATH} is missing: build it with `python -m adrastea_amd.build` "
             "(hipcc, gfx950); adrastea_amd has no CPU or PyTorch fallback")
+    # The host mirror keeps device memory in torch tensors, and torch ships a HIP runtime of its
+    # own: load that one first, so that this library's libamdhip64 dependency resolves to the
+    # runtime torch has initialised.  Loaded in the other order, the process holds two runtimes
+    # and the library's launches fail with hipErrorNoDevice.
+    import torch  # noqa: F401
     L = C.CDLL(LIB_PATH)
     vp, i32, u32, f32 = C.c_void_p, C.c_int32, C.c_uint32, C.c_float
     mm = [vp, vp, vp, vp] + [i32] * 13 + [vp, f32, f32, u32, u32, u32]

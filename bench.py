@@ -46,6 +46,8 @@ def main():
     ap.add_argument("--quick", action="store_true", help="skip secondary configs and CPU baseline")
     ap.add_argument("--decode-only", action="store_true",
                     help="run only the u8 decode GEMV configurations (for profiling that kernel)")
+    ap.add_argument("--attention-only", action="store_true",
+                    help="run only the attention configuration (QK^T, softmax_rows, P.V, error_stats)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain 256 MiB device copy (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters of rocprofv3 --pmc)")
@@ -154,6 +156,70 @@ def main():
                              "frac_hbm_peak": round(byts / t / 1e9 / PEAK_HBM_GBS, 4)})
         return gemv
 
+    def attention_set():
+        # ---- attention products (configs[3]): HBM-bound by the [32, 2048, 2048] fp16 tensor
+        S, H, D = 2048, 32, 128
+        HD = H * D
+        q_, k_, v_ = randn_h(S, HD), randn_h(S, HD), randn_h(S, HD)
+        qk = torch.zeros(H, S, S, dtype=torch.float16, device=dev)
+
+        def f_qk():
+            rc = lib.adr_matmul_f16(stream(), qk.data_ptr(), q_.data_ptr(), k_.data_ptr(), H, S, D,
+                                    S, 1, S, S * S, 1, HD, D, HD, 1, D, None, 0.0,
+                                    1.0 / D ** 0.5, 4, 0, 0)
+            if rc != 0:
+                raise RuntimeError(_ffi.strerror(rc))
+        t = timed(f_qk, 50, 5)
+        byts = 2 * S * HD * 2 + H * S * S * 2
+        attn = {"qk_t": {"us": round(t * 1e6, 1), "tflops": round(2.0 * H * S * S * D / t / 1e12, 1),
+                         "gbs": round(byts / t / 1e9, 1),
+                         "frac_hbm_peak": round(byts / t / 1e9 / PEAK_HBM_GBS, 4)}}
+        # softmax_rows in place on the scores (read + write of the [32, 2048, 2048] tensor)
+        def f_sm():
+            rc = lib.adr_softmax_rows(stream(), qk.data_ptr(), qk.data_ptr(), H, S, S, 1.0)
+            if rc != 0:
+                raise RuntimeError(_ffi.strerror(rc))
+        f_qk()
+        t = timed(f_sm, 30, 3)
+        sm_bytes = 2 * H * S * S * 2
+        attn["softmax_rows"] = {"us": round(t * 1e6, 1), "gbs": round(sm_bytes / t / 1e9, 1),
+                                "frac_hbm_peak": round(sm_bytes / t / 1e9 / PEAK_HBM_GBS, 4)}
+        f_qk()
+        p_ = torch.softmax(qk.float(), dim=-1).half()
+        o_ = torch.zeros(S, HD, dtype=torch.float16, device=dev)
+
+        def f_pv():
+            rc = lib.adr_matmul_f16(stream(), o_.data_ptr(), p_.data_ptr(), v_.data_ptr(), H, S, S,
+                                    D, 1, HD, D, 1, S, S * S, 1, HD, D, None, 0.0, 1.0, 0, 0, 0)
+            if rc != 0:
+                raise RuntimeError(_ffi.strerror(rc))
+        t = timed(f_pv, 50, 5)
+        attn["pv"] = {"us": round(t * 1e6, 1), "tflops": round(2.0 * H * S * S * D / t / 1e12, 1),
+                      "gbs": round(byts / t / 1e9, 1),
+                      "frac_hbm_peak": round(byts / t / 1e9 / PEAK_HBM_GBS, 4)}
+        # error_stats_f16 of two [32, 2048, 2048] tensors (reads 2 x 268 MB, the on-device check)
+        stat = torch.zeros(3, dtype=torch.float32, device=dev)
+
+        def desc1(t):
+            d = _ffi.TensorDesc()
+            d.ptr, d.dims = t.data_ptr(), 1
+            d.shape[0], d.strides[0] = t.numel(), 1
+            return d
+        d_out, d_l, d_r = desc1(stat), desc1(qk), desc1(p_)
+
+        def f_es():
+            rc = lib.adr_error_stats_f16(stream(), d_out, d_l, d_r)
+            if rc != 0:
+                raise RuntimeError(_ffi.strerror(rc))
+        t = timed(f_es, 30, 3)
+        attn["error_stats_f16"] = {"us": round(t * 1e6, 1), "gbs": round(sm_bytes / t / 1e9, 1),
+                                   "frac_hbm_peak": round(sm_bytes / t / 1e9 / PEAK_HBM_GBS, 4)}
+        return attn
+
+    if args.attention_only:
+        print(json.dumps({"llama7b_attention_fp16": attention_set()}))
+        return
+
     if args.decode_only:
         print(json.dumps({"u8_decode_gemv": decode_set()}))
         return
@@ -250,63 +316,7 @@ def main():
                         "gbs": round(byts / t / 1e9, 1)}
         secondary["clip_fp16"] = clip
 
-        # ---- attention products (configs[3]): HBM-bound by the [32, 2048, 2048] fp16 tensor
-        S, H, D = 2048, 32, 128
-        HD = H * D
-        q_, k_, v_ = randn_h(S, HD), randn_h(S, HD), randn_h(S, HD)
-        qk = torch.zeros(H, S, S, dtype=torch.float16, device=dev)
-
-        def f_qk():
-            rc = lib.adr_matmul_f16(stream(), qk.data_ptr(), q_.data_ptr(), k_.data_ptr(), H, S, D,
-                                    S, 1, S, S * S, 1, HD, D, HD, 1, D, None, 0.0,
-                                    1.0 / D ** 0.5, 4, 0, 0)
-            if rc != 0:
-                raise RuntimeError(_ffi.strerror(rc))
-        t = timed(f_qk, 50, 5)
-        byts = 2 * S * HD * 2 + H * S * S * 2
-        attn = {"qk_t": {"us": round(t * 1e6, 1), "tflops": round(2.0 * H * S * S * D / t / 1e12, 1),
-                         "gbs": round(byts / t / 1e9, 1),
-                         "frac_hbm_peak": round(byts / t / 1e9 / PEAK_HBM_GBS, 4)}}
-        # softmax_rows in place on the scores (read + write of the [32, 2048, 2048] tensor)
-        def f_sm():
-            rc = lib.adr_softmax_rows(stream(), qk.data_ptr(), qk.data_ptr(), H, S, S, 1.0)
-            if rc != 0:
-                raise RuntimeError(_ffi.strerror(rc))
-        f_qk()
-        t = timed(f_sm, 30, 3)
-        sm_bytes = 2 * H * S * S * 2
-        attn["softmax_rows"] = {"us": round(t * 1e6, 1), "gbs": round(sm_bytes / t / 1e9, 1),
-                                "frac_hbm_peak": round(sm_bytes / t / 1e9 / PEAK_HBM_GBS, 4)}
-        f_qk()
-        p_ = torch.softmax(qk.float(), dim=-1).half()
-        o_ = torch.zeros(S, HD, dtype=torch.float16, device=dev)
-
-        def f_pv():
-            rc = lib.adr_matmul_f16(stream(), o_.data_ptr(), p_.data_ptr(), v_.data_ptr(), H, S, S,
-                                    D, 1, HD, D, 1, S, S * S, 1, HD, D, None, 0.0, 1.0, 0, 0, 0)
-            if rc != 0:
-                raise RuntimeError(_ffi.strerror(rc))
-        t = timed(f_pv, 50, 5)
-        attn["pv"] = {"us": round(t * 1e6, 1), "tflops": round(2.0 * H * S * S * D / t / 1e12, 1),
-                      "gbs": round(byts / t / 1e9, 1),
-                      "frac_hbm_peak": round(byts / t / 1e9 / PEAK_HBM_GBS, 4)}
-        # error_stats_f16 of two [32, 2048, 2048] tensors (reads 2 x 268 MB, the on-device check)
-        stat = torch.zeros(3, dtype=torch.float32, device=dev)
-
-        def desc1(t):
-            d = _ffi.TensorDesc()
-            d.ptr, d.dims = t.data_ptr(), 1
-            d.shape[0], d.strides[0] = t.numel(), 1
-            return d
-        d_out, d_l, d_r = desc1(stat), desc1(qk), desc1(p_)
-
-        def f_es():
-            rc = lib.adr_error_stats_f16(stream(), d_out, d_l, d_r)
-            if rc != 0:
-                raise RuntimeError(_ffi.strerror(rc))
-        t = timed(f_es, 30, 3)
-        attn["error_stats_f16"] = {"us": round(t * 1e6, 1), "gbs": round(sm_bytes / t / 1e9, 1),
-                                   "frac_hbm_peak": round(sm_bytes / t / 1e9 / PEAK_HBM_GBS, 4)}
+        attn = attention_set()
         secondary["llama7b_attention_fp16"] = attn
 
     # ---------------- CPU baseline: the oracle on a bounded sample of the same workload
