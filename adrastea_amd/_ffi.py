@@ -12,11 +12,13 @@ SYMBOLS = (
     "adr_matmul_f16", "adr_matmul_f16_slow", "adr_matmul_f16_raw", "adr_matmul_nt_f16",
     "adr_matmul_nt_fp16u8", "adr_dequantize_absmax_u8", "adr_quantize_absmax_u8",
     "adr_dequantize_absmax_uint8", "adr_quantize_absmax_uint8", "adr_matmul_f16_plan",
-    "adr_matmul_nt_fp16u8_plan", "adr_softmax_rows", "adr_error_stats_f16", "adr_error_stats_f32", "adr_strerror", "adr_abi_version",
+    "adr_matmul_nt_fp16u8_plan", "adr_softmax_rows", "adr_error_stats_f16", "adr_error_stats_f32", "adr_attention_f16",
+    "adr_strerror", "adr_abi_version",
 )
 
 ADR_OK, ADR_EINVAL_SHAPE, ADR_EINVAL_ENUM, ADR_ENOTIMPL, ADR_ENULL, ADR_EDIVISIBILITY = (
     0, -1, -2, -3, -4, -5)
+ADR_EUNSUPPORTED_DEVICE, ADR_EUNSUPPORTED_LAYOUT = -6, -7
 
 
 class TensorDesc(C.Structure):
@@ -59,6 +61,7 @@ def lib():
     L.adr_softmax_rows.argtypes = [vp, vp, vp, i32, i32, i32, f32]
     L.adr_error_stats_f16.argtypes = [vp, TensorDesc, TensorDesc, TensorDesc]
     L.adr_error_stats_f32.argtypes = [vp, TensorDesc, TensorDesc, TensorDesc]
+    L.adr_attention_f16.argtypes = [vp, vp, vp, vp, vp] + [i32] * 16 + [f32, f32, u32]
     L.adr_strerror.argtypes = [C.c_int]
     L.adr_strerror.restype = C.c_char_p
     L.adr_abi_version.restype = C.c_int

@@ -138,6 +138,10 @@ hipError_t launch_quantize(hipStream_t stream, adr_tensor_desc out, adr_tensor_d
                            adr_tensor_desc in);
 hipError_t launch_error_stats(hipStream_t stream, float* out, const void* lhs, const void* rhs,
                               int64_t length, int64_t sl, int64_t sr, bool f32);
+hipError_t launch_attention(hipStream_t stream, half_t* out, const half_t* q, const half_t* k,
+                            const half_t* v, int heads, int m, int n, int d, int so_y, int so_z,
+                            int sq_y, int sq_z, int sk_y, int sk_z, int sv_y, int sv_z, float scale,
+                            float temp, uint32_t mask);
 hipError_t launch_softmax_rows(hipStream_t stream, half_t* out, const half_t* in, int64_t rows,
                                int w, float temp);
 

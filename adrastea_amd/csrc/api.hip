@@ -88,6 +88,9 @@ const char* adr_strerror(int code) {
     case ADR_ENULL: return "null tensor pointer or missing bias";
     case ADR_EDIVISIBILITY: return "size not divisible by block_size / unsupported block_size";
     case ADR_EUNSUPPORTED_DEVICE: return "current device is not gfx950";
+    case ADR_EUNSUPPORTED_LAYOUT:
+      return "fused attention covers head dimension 64 or 128, unit x strides, y/z strides that "
+             "are multiples of 8 and 16-byte aligned pointers";
     default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown error";
   }
 }
@@ -220,6 +223,35 @@ int adr_softmax_rows(adr_stream_t stream, uint16_t* output, const uint16_t* inpu
   if (!output || !input) return ADR_ENULL;
   return (int)launch_softmax_rows((hipStream_t)stream, (half_t*)output, (const half_t*)input,
                                   (int64_t)heads * h, w, temp);
+}
+
+int adr_attention_f16(adr_stream_t stream, uint16_t* output, const uint16_t* query,
+                      const uint16_t* key, const uint16_t* value, int32_t heads, int32_t m,
+                      int32_t n, int32_t d, int32_t stride_ox, int32_t stride_oy,
+                      int32_t stride_oz, int32_t stride_qx, int32_t stride_qy, int32_t stride_qz,
+                      int32_t stride_kx, int32_t stride_ky, int32_t stride_kz, int32_t stride_vx,
+                      int32_t stride_vy, int32_t stride_vz, float scale, float temp,
+                      uint32_t mask) {
+  if (heads < 0 || m < 0 || n < 0 || d < 0) return ADR_EINVAL_SHAPE;
+  if (mask > ADR_MASK_CAUSAL) return ADR_EINVAL_ENUM;
+  if (heads == 0 || m == 0 || d == 0) return ADR_OK;
+  if (n == 0) return ADR_EINVAL_SHAPE;
+  if (!output || !query || !key || !value) return ADR_ENULL;
+  if (d != 64 && d != 128) return ADR_EUNSUPPORTED_LAYOUT;
+  if (stride_ox != 1 || stride_qx != 1 || stride_kx != 1 || stride_vx != 1)
+    return ADR_EUNSUPPORTED_LAYOUT;
+  const int32_t st[8] = {stride_oy, stride_oz, stride_qy, stride_qz,
+                         stride_ky, stride_kz, stride_vy, stride_vz};
+  for (int i = 0; i < 8; i++)
+    if (st[i] < 0 || st[i] % 8 != 0) return ADR_EUNSUPPORTED_LAYOUT;
+  if (((uintptr_t)output | (uintptr_t)query | (uintptr_t)key | (uintptr_t)value) % 16 != 0)
+    return ADR_EUNSUPPORTED_LAYOUT;
+  if (!(scale > 0.0f) || !(temp > 0.0f)) return ADR_EUNSUPPORTED_LAYOUT;
+  // largest element offsets stay within int64 trivially; rows are addressed with 64-bit products
+  return (int)launch_attention((hipStream_t)stream, (half_t*)output, (const half_t*)query,
+                               (const half_t*)key, (const half_t*)value, heads, m, n, d,
+                               stride_oy, stride_oz, stride_qy, stride_qz, stride_ky, stride_kz,
+                               stride_vy, stride_vz, scale, temp, mask);
 }
 
 static int error_stats_common(adr_stream_t stream, adr_tensor_desc output, adr_tensor_desc lhs,

@@ -92,6 +92,12 @@ struct CommonKernels {
   virtual void matmul_f16_slow(TensorView<f16>& output, const TensorView<const f16>& left,
                                const TensorView<const f16>& right, const MatmulOptions& options) = 0;
   virtual void softmax_rows_inplace(TensorView<f16>& output, float temperature) = 0;
+  // Not in the reference's trait: the three calls of llama.rs:541-554 (QK^T with Scale and the
+  // mask, softmax_rows_inplace, P.V) as one launch.  query/output: [heads, m, d] views, key/value:
+  // [heads, n, d] views (rank 2 = one head).
+  virtual void attention_f16(TensorView<f16>& output, const TensorView<const f16>& query,
+                             const TensorView<const f16>& key, const TensorView<const f16>& value,
+                             float scale, float temperature, MatmulMask mask) = 0;
   virtual void error_stats_f16(TensorView<float>& output, const TensorView<const f16>& lhs,
                                const TensorView<const f16>& rhs) = 0;
   virtual void error_stats_f32(TensorView<float>& output, const TensorView<const float>& lhs,
@@ -125,6 +131,27 @@ class GpuKernels : public CommonKernels {
     const int32_t heads = o.layout.dims.size() > 2 ? (int32_t)o.size(-3) : 1;
     int rc = adr_softmax_rows(stream_, o.ptr, o.ptr, heads, (int32_t)o.size(-2), (int32_t)o.size(-1), temperature);
     if (rc) throw AdrasteaError(rc, "softmax_rows_inplace");
+  }
+  void attention_f16(TensorView<f16>& o, const TensorView<const f16>& q, const TensorView<const f16>& k,
+                     const TensorView<const f16>& v, float scale, float temperature, MatmulMask mask) override {
+    const size_t rank = q.layout.dims.size();
+    if ((rank != 2 && rank != 3) || o.layout.dims.size() != rank || k.layout.dims.size() != rank ||
+        v.layout.dims.size() != rank)
+      throw std::logic_error("attention_f16: rank 2 or 3 views");
+    const int32_t heads = rank == 3 ? (int32_t)q.size(-3) : 1;
+    const int32_t m = (int32_t)q.size(-2), d = (int32_t)q.size(-1), n = (int32_t)k.size(-2);
+    if ((int32_t)k.size(-1) != d || (int32_t)v.size(-1) != d || (int32_t)v.size(-2) != n ||
+        (int32_t)o.size(-2) != m || (int32_t)o.size(-1) != d ||
+        (rank == 3 && ((int32_t)o.size(-3) != heads || (int32_t)k.size(-3) != heads || (int32_t)v.size(-3) != heads)))
+      throw std::logic_error("attention_f16: shape mismatch");
+    auto z = [&](const TensorLayout& l) { return rank == 3 ? (int32_t)l.stride(-3) : 0; };
+    int rc = adr_attention_f16(stream_, o.ptr, q.ptr, k.ptr, v.ptr, heads, m, n, d,
+                               (int32_t)o.layout.stride(-1), (int32_t)o.layout.stride(-2), z(o.layout),
+                               (int32_t)q.layout.stride(-1), (int32_t)q.layout.stride(-2), z(q.layout),
+                               (int32_t)k.layout.stride(-1), (int32_t)k.layout.stride(-2), z(k.layout),
+                               (int32_t)v.layout.stride(-1), (int32_t)v.layout.stride(-2), z(v.layout),
+                               scale, temperature, (uint32_t)mask);
+    if (rc) throw AdrasteaError(rc, "attention_f16");
   }
   // kernels.rs:717-751: both operands flattened with shape_cast(&[-1]); equal lengths
   void error_stats_f16(TensorView<float>& out, const TensorView<const f16>& l, const TensorView<const f16>& r) override {
@@ -171,6 +198,10 @@ class MatmulTracer : public CommonKernels {
   void matmul_f16_slow(TensorView<f16>& o, const TensorView<const f16>& l, const TensorView<const f16>& r,
                        const MatmulOptions& opt) override { rec(o, l, r); inner_.matmul_f16_slow(o, l, r, opt); }
   void softmax_rows_inplace(TensorView<f16>& o, float t) override { inner_.softmax_rows_inplace(o, t); }
+  void attention_f16(TensorView<f16>& o, const TensorView<const f16>& q, const TensorView<const f16>& k,
+                     const TensorView<const f16>& v, float scale, float t, MatmulMask mask) override {
+    inner_.attention_f16(o, q, k, v, scale, t, mask);
+  }
   void error_stats_f16(TensorView<float>& out, const TensorView<const f16>& l, const TensorView<const f16>& r) override { inner_.error_stats_f16(out, l, r); }
   void error_stats_f32(TensorView<float>& out, const TensorView<const float>& l, const TensorView<const float>& r) override { inner_.error_stats_f32(out, l, r); }
 

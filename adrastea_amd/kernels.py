@@ -210,6 +210,32 @@ class GpuKernels(CommonKernels):
         if rc != 0:
             raise AdrasteaError(rc, "softmax_rows_inplace")
 
+    def attention_f16(self, output, query, key, value, scale: float, temperature: float = 1.0,
+                      mask: int = MatmulMask.NONE):
+        """The three calls of llama.rs:541-554 (QK^T with Scale and the mask, softmax_rows_inplace,
+        P.V) as one launch that keeps the scores out of memory.  `query`/`output` are
+        [heads, m, d] views, `key`/`value` [heads, n, d] views (rank 2 = one head).  Raises
+        AdrasteaError with code ADR_EUNSUPPORTED_LAYOUT for head dimensions or strides the fused
+        kernel does not cover; the three-call sequence remains available for those."""
+        lo, lq, lk, lv = output.layout, query.layout, key.layout, value.layout
+        rank = len(lq.dims)
+        assert rank in (2, 3) and all(len(l.dims) == rank for l in (lo, lk, lv))
+        heads = lq.size(-3) if rank == 3 else 1
+        m, d, n = lq.size(-2), lq.size(-1), lk.size(-2)
+        assert lk.size(-1) == d and lv.size(-1) == d and lv.size(-2) == n
+        assert lo.size(-2) == m and lo.size(-1) == d
+        if rank == 3:
+            assert lo.size(-3) == heads and lk.size(-3) == heads and lv.size(-3) == heads
+
+        def xyz(l):
+            return l.stride(-1), l.stride(-2), (l.stride(-3) if rank == 3 else 0)
+        rc = self._lib.adr_attention_f16(_current_stream(), output.data_ptr(), query.data_ptr(),
+                                         key.data_ptr(), value.data_ptr(), heads, m, n, d,
+                                         *xyz(lo), *xyz(lq), *xyz(lk), *xyz(lv), float(scale),
+                                         float(temperature), int(mask))
+        if rc != 0:
+            raise AdrasteaError(rc, "attention_f16")
+
     def _error_stats(self, fn, what, output, lhs, rhs):
         # kernels.rs:717-751: both operands flattened with shape_cast(&[-1]); equal lengths
         lhs, rhs = lhs.shape_cast([-1]), rhs.shape_cast([-1])
@@ -315,6 +341,10 @@ class MatmulTracer(CommonKernels):
 
     def softmax_rows_inplace(self, output, temperature: float = 1.0):
         self.inner.softmax_rows_inplace(output, temperature)   # forwarded (kernels.rs:334-338)
+
+    def attention_f16(self, output, query, key, value, scale, temperature=1.0,
+                      mask=MatmulMask.NONE):
+        self.inner.attention_f16(output, query, key, value, scale, temperature, mask)
 
     def error_stats_f16(self, output, lhs, rhs):
         self.inner.error_stats_f16(output, lhs, rhs)            # forwarded (kernels.rs:349-358)

@@ -214,6 +214,20 @@ def main():
         t = timed(f_es, 30, 3)
         attn["error_stats_f16"] = {"us": round(t * 1e6, 1), "gbs": round(sm_bytes / t / 1e9, 1),
                                    "frac_hbm_peak": round(sm_bytes / t / 1e9 / PEAK_HBM_GBS, 4)}
+        # the three products and the softmax above as one launch (adr_attention_f16); the causal
+        # form is what the LLaMA layer runs, and skips the masked half of the score tiles
+        o_ = torch.zeros(S, HD, dtype=torch.float16, device=dev)
+        for name, msk in (("fused_attention", 0), ("fused_attention_causal", 1)):
+            def f_at():
+                rc = lib.adr_attention_f16(stream(), o_.data_ptr(), q_.data_ptr(), k_.data_ptr(),
+                                           v_.data_ptr(), H, S, S, D, 1, HD, D, 1, HD, D, 1, HD, D,
+                                           1, HD, D, 1.0 / D ** 0.5, 1.0, msk)
+                if rc != 0:
+                    raise RuntimeError(_ffi.strerror(rc))
+            t = timed(f_at, 30, 3)
+            fl = 4.0 * H * S * S * D * (0.5 if msk else 1.0)
+            attn[name] = {"us": round(t * 1e6, 1), "tflops": round(fl / t / 1e12, 1),
+                          "frac_mfma_peak": round(fl / t / 1e12 / PEAK_F16_TFLOPS, 4)}
         return attn
 
     if args.attention_only:

@@ -34,7 +34,9 @@ enum {
                               (matmul.cu:450-491 -> NYI trap); rejected here instead */
   ADR_ENULL = -4,          /* null tensor pointer, or a bias operator without a bias */
   ADR_EDIVISIBILITY = -5,  /* u8 kernels: p % block_size != 0 or block_size not supported */
-  ADR_EUNSUPPORTED_DEVICE = -6 /* the current device is not gfx950 */
+  ADR_EUNSUPPORTED_DEVICE = -6, /* the current device is not gfx950 */
+  ADR_EUNSUPPORTED_LAYOUT = -7  /* adr_attention_f16: head dimension, stride or alignment that the
+                                   fused kernel does not cover; use the three-call sequence */
 };
 
 /* adrastea_models/src/kernels.rs:81-135, adrastea_kernels/cpp/matmul.cu:26-36 */
@@ -173,6 +175,30 @@ int adr_error_stats_f16(adr_stream_t stream, adr_tensor_desc output, adr_tensor_
                         adr_tensor_desc rhs);
 int adr_error_stats_f32(adr_stream_t stream, adr_tensor_desc output, adr_tensor_desc lhs,
                         adr_tensor_desc rhs);
+
+/*
+ * Fused attention of one layer (no single counterpart in the reference: it stands for the three
+ * calls at adrastea_models/src/llama.rs:541-554 -- matmul_f16 with MatmulStore::Scale and
+ * MatmulMask::Causal into a [heads, m, n] tensor, softmax_rows_inplace, matmul_f16 with the value
+ * view -- and their twins at clip.rs:372-388 and whisper.rs:424-436):
+ *   out[h, y, :] = sum_x softmax_x( mask(scale * <query[h, y, :], key[h, x, :]>) / temp ) * value[h, x, :]
+ * `query` and `output` are [heads, m, d] views, `key` and `value` [heads, n, d] views (key NOT
+ * transposed: llama.rs:537's k_view is this view with its last two axes swapped); strides are in
+ * elements with x = dim -1, y = dim -2, z = dim -3, as in adr_matmul_f16.  mask = ADR_MASK_CAUSAL
+ * removes x > y exactly as matmul.cu:182-184 does.  The scores never reach memory and stay in
+ * fp32, so results equal the three-call sequence up to the fp16 rounding that sequence applies to
+ * scores and probabilities in between.
+ * Covered: d = 64 or 128, every x stride 1, y and z strides multiples of 8, 16-byte aligned
+ * pointers, scale > 0, temp > 0; anything else returns ADR_EUNSUPPORTED_LAYOUT and launches
+ * nothing.  n = 0 with m > 0 is ADR_EINVAL_SHAPE (a softmax over no elements).
+ */
+int adr_attention_f16(adr_stream_t stream, uint16_t* output, const uint16_t* query,
+                      const uint16_t* key, const uint16_t* value, int32_t heads, int32_t m,
+                      int32_t n, int32_t d, int32_t stride_ox, int32_t stride_oy,
+                      int32_t stride_oz, int32_t stride_qx, int32_t stride_qy, int32_t stride_qz,
+                      int32_t stride_kx, int32_t stride_ky, int32_t stride_kz, int32_t stride_vx,
+                      int32_t stride_vy, int32_t stride_vz, float scale, float temp,
+                      uint32_t mask);
 
 /*
  * Diagnostics (no counterpart in the reference).

@@ -180,6 +180,35 @@ def error_stats(lhs, rhs):
     return out
 
 
+def attention_f16(q, k, v, scale, temp=1.0, mask=MASK_NONE, exact=False, threads=1):
+    """The attention of one layer as the reference composes it (llama.rs:541-554): scores =
+    matmul_f16(q, k^T) with MatmulStore::Scale and the mask, rounded to fp16; softmax_rows in
+    place, rounded to fp16; matmul_f16 with v.  q: [heads, m, d], k and v: [heads, n, d], all
+    contiguous fp16; returns [heads, m, d] fp16.  exact=True: the same function in float64 with
+    one final rounding (what a path that keeps the scores unrounded is measured against)."""
+    q, k, v = (np.ascontiguousarray(t) for t in (q, k, v))
+    heads, m, d = q.shape
+    n = k.shape[1]
+    assert k.shape == (heads, n, d) and v.shape == (heads, n, d)
+    if exact:
+        s = np.einsum("hyd,hxd->hyx", q.astype(np.float64), k.astype(np.float64))
+        s = s * np.float64(np.float16(scale))
+        if mask == MASK_CAUSAL:
+            s = np.where(np.arange(n)[None, None, :] > np.arange(m)[None, :, None], -np.inf, s)
+        s = s / temp
+        e = np.exp(s - s.max(axis=-1, keepdims=True))
+        p = e / e.sum(axis=-1, keepdims=True)
+        return np.einsum("hyx,hxd->hyd", p, v.astype(np.float64)).astype(np.float16)
+    scores = np.zeros(heads * m * n, np.float16)
+    matmul_f16(scores, q, k, heads, m, d, n, (1, n, m * n), (1, d, m * d), (d, 1, n * d),
+               scale=scale, store=STORE_SCALE, mask=mask, threads=threads)
+    probs = softmax_rows(scores.reshape(heads, m, n), temp, 0)
+    out = np.zeros(heads * m * d, np.float16)
+    matmul_f16(out, probs, v, heads, m, n, d, (1, d, m * d), (1, n, m * n), (1, d, n * d),
+               threads=threads)
+    return out.reshape(heads, m, d)
+
+
 def dequant_table():
     out = np.empty(256 * 65536, np.uint16)
     lib().adr_o_dequant_table(_p16(out))

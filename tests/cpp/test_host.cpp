@@ -29,6 +29,13 @@ static int h2i(uint16_t h) {
   return (h & 0x8000) ? -v : v;
 }
 
+static double h2d(uint16_t h) {  // any finite fp16 value
+  const int e = (h >> 10) & 31, m = h & 0x3ff;
+  const double mag = e ? (double)(0x400 | m) / 1024.0 * (e >= 15 ? (double)(1 << (e - 15)) : 1.0 / (double)(1 << (15 - e)))
+                       : (double)m / 1024.0 / 16384.0;
+  return (h & 0x8000) ? -mag : mag;
+}
+
 static void cpu_tests() {
   CHECK((TensorLayout::row_major({2, 3, 4}).strides == std::vector<size_t>{12, 4, 1}));
   CHECK((TensorLayout::column_major({3, 4}).strides == std::vector<size_t>{1, 4}));
@@ -147,6 +154,35 @@ static void gpu_test() {
     float st[3] = {1, 1, 1};
     hipMemcpy(st, dstat, 12, 2);
     CHECK(st[0] == 0.0f && st[1] == 0.0f && st[2] == 0.0f);
+  }
+  {
+    // attention_f16 with zero queries: every score is equal, the output is the mean of the value
+    // rows, exact here (64 keys, small-integer values); M x K reused as [1 head, M, K], K = d
+    static_assert(K == 64 || K == 128, "head dimension of the fused kernel");
+    const int NK = 64;
+    std::vector<uint16_t> zq((size_t)M * K, 0), vv((size_t)NK * K), oo((size_t)M * K, 0);
+    for (int x = 0; x < NK; x++)
+      for (int c = 0; c < K; c++) vv[(size_t)x * K + c] = f2h_small_int((x * 7 + c * 3) % 17 - 8);
+    uint16_t *dq, *dv, *dk, *dat;
+    CHECK(hipMalloc((void**)&dq, zq.size() * 2) == 0 && hipMalloc((void**)&dv, vv.size() * 2) == 0 &&
+          hipMalloc((void**)&dk, vv.size() * 2) == 0 && hipMalloc((void**)&dat, oo.size() * 2) == 0);
+    hipMemcpy(dq, zq.data(), zq.size() * 2, 1); hipMemcpy(dv, vv.data(), vv.size() * 2, 1);
+    hipMemcpy(dk, vv.data(), vv.size() * 2, 1);
+    TensorView<f16> av(dat, TensorLayout::row_major({(size_t)M, (size_t)K}));
+    TensorView<const f16> qv(dq, TensorLayout::row_major({(size_t)M, (size_t)K}));
+    TensorView<const f16> kv(dk, TensorLayout::row_major({(size_t)NK, (size_t)K}));
+    TensorView<const f16> vv_(dv, TensorLayout::row_major({(size_t)NK, (size_t)K}));
+    tr.attention_f16(av, qv, kv, vv_, 0.125f, 1.0f, MatmulMask::None);
+    CHECK(hipDeviceSynchronize() == 0);
+    hipMemcpy(oo.data(), dat, oo.size() * 2, 2);
+    int bad = 0;
+    for (int c = 0; c < K; c++) {
+      int sum = 0;
+      for (int x = 0; x < NK; x++) sum += h2i(vv[(size_t)x * K + c]);
+      for (int y = 0; y < M; y++) bad += h2d(oo[(size_t)y * K + c]) != (double)sum / NK;
+    }
+    CHECK(bad == 0);
+    CHECK(throws([&] { tr.attention_f16(av, qv, kv.permute({1, 0}), vv_, 0.125f, 1.0f, MatmulMask::None); }));
   }
   uint16_t bias = 0;
   CHECK(throws([&] { tr.matmul_f16(ov, lv, wv.permute({1, 0}), MatmulOptions::make().store(MatmulStore::GeluBias(&bias))); }));
