@@ -57,6 +57,30 @@ __device__ __forceinline__ int v_swz(int row) {
   return CPR == 16 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2);
 }
 
+// Reductions over the lane pair (l, l ^ 32): v_permlane32_swap exchanges the upper half of one
+// register with the lower half of the other, so with the same value in both its two results
+// hold the pair's two values in every lane, without a trip through LDS.  The second result
+// passes through an empty asm statement: without it the compiler folds a floating-point
+// operation on the two results as if they were the same register.
+__device__ __forceinline__ void pair_values(float v, float& x, float& y) {
+  const uint32_t b = __builtin_bit_cast(uint32_t, v);
+  const auto r = __builtin_amdgcn_permlane32_swap(b, b, false, false);
+  uint32_t r0 = r[0], r1 = r[1];
+  asm volatile("" : "+v"(r1));
+  x = __builtin_bit_cast(float, r0);
+  y = __builtin_bit_cast(float, r1);
+}
+__device__ __forceinline__ float pair_max(float v) {
+  float x, y;
+  pair_values(v, x, y);
+  return fmaxf(x, y);
+}
+__device__ __forceinline__ float pair_sum(float v) {
+  float x, y;
+  pair_values(v, x, y);
+  return x + y;
+}
+
 template <int HD>
 __global__ __launch_bounds__(256, 2) void attention_fwd_kernel(AttnArgs a) {
   constexpr int BM = 128, BN = 64, CPR = HD / 8;
@@ -170,39 +194,46 @@ __global__ __launch_bounds__(256, 2) void attention_fwd_kernel(AttnArgs a) {
       }
     }
     const bool edge = (causal && kv0 + BN - 1 > q0w) || kv0 + BN > a.n;
-    const int qi = q0w + frow;
+    if (edge) {
+      const int qi = q0w + frow;
+#pragma unroll
+      for (int kt = 0; kt < 2; kt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int kv = kv0 + 32 * kt + 8 * (r >> 2) + 4 * g + (r & 3);
+          if (kv >= a.n || (causal && kv > qi)) s[kt][r] = -INFINITY;
+        }
+    }
     float mx = -1.0e30f;
 #pragma unroll
     for (int kt = 0; kt < 2; kt++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        float x = s[kt][r] * a.c;
-        if (edge) {
-          const int kv = kv0 + 32 * kt + 8 * (r >> 2) + 4 * g + (r & 3);
-          if (kv >= a.n || (causal && kv > qi)) x = -INFINITY;
-        }
-        s[kt][r] = x;
-        mx = fmaxf(mx, x);
-      }
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m_run, mx);
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-    m_run = m_new;
+      for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[kt][r]);
+    mx = pair_max(mx) * a.c;  // the row's maximum in log2 units (c > 0)
+    // The exponent reference m_run follows the row maximum lazily: it moves only when some row
+    // of the wavefront outgrew it by more than 2^8 (probabilities up to 256 are as exact in fp16
+    // as those below 1), which after the first tiles is rare; the accumulator is rescaled only then.
+    if (__builtin_amdgcn_ballot_w64(mx > m_run + 8.0f) != 0) {
+      const float m_new = fmaxf(m_run, mx);
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      m_run = m_new;
+      l_run *= alpha;
+#pragma unroll
+      for (int dt = 0; dt < DT; dt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[dt][r] *= alpha;
+    }
     float sum = 0.0f;
     half8_t pf[2][2];
 #pragma unroll
     for (int kt = 0; kt < 2; kt++)
 #pragma unroll
       for (int r = 0; r < 16; r++) {
-        const float p = __builtin_amdgcn_exp2f(s[kt][r] - m_new);
+        const float p = __builtin_amdgcn_exp2f(fmaf(s[kt][r], a.c, -m_run));
         sum += p;
         pf[kt][r >> 3][r & 7] = (half_t)p;
       }
-    l_run = l_run * alpha + sum;
-#pragma unroll
-    for (int dt = 0; dt < DT; dt++)
-#pragma unroll
-      for (int r = 0; r < 16; r++) o[dt][r] *= alpha;
+    l_run += sum;
     // O^T += V^T P^T: k-step (kt, t) covers keys 32kt + 16t + {4g + j, 8 + 4g + j}
     typedef short short4_t __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) short4_t lds_short4_t;
@@ -239,7 +270,7 @@ __global__ __launch_bounds__(256, 2) void attention_fwd_kernel(AttnArgs a) {
   }
 
   // out[q][32dt + 8i + 4g + j] = o[dt][4i + j] / l
-  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  const float l_tot = pair_sum(l_run);
   const float inv = 1.0f / l_tot;
   const int qi = q0w + frow;
   if (qi < a.m) {
