@@ -98,14 +98,24 @@ __global__ __launch_bounds__(256, 2) void attention_fwd_kernel(AttnArgs a) {
   const int frow = lane & 31, g = lane >> 5;
   const bool causal = a.mask == ADR_MASK_CAUSAL;
 
-  // Workgroup -> (head, query block).  Consecutive workgroup ids go to different dies, so the
-  // id is first unfolded into a per-die sequence that keeps a head's query blocks (which share
-  // K and V) on one die; under the causal mask the blocks with most tiles come first.
-  const int total = a.heads * a.qblocks;
-  int vid = blockIdx.x;
-  if (total % 8 == 0) vid = (blockIdx.x & 7) * (total >> 3) + (blockIdx.x >> 3);
-  const int head = vid / a.qblocks;
-  const int qb = a.qblocks - 1 - vid % a.qblocks;
+  // Workgroup -> (head, query block).  Consecutive workgroup ids go to different dies; die x takes
+  // the heads [x * heads/8, (x+1) * heads/8), so that the query blocks of a head (which share K
+  // and V) meet in one L2.  Under the causal mask block b has 2b + 2 key tiles.  A die's own
+  // sequence runs through the upper half of the blocks downwards, then through the lower half
+  // upwards: with 32 heads and 16 blocks all 64 workgroups of a die are resident at once, the
+  // i-th and the (i+32)-th share a compute unit, and this order gives every unit a block b and
+  // its complement 15 - b of the same head; with more work than fits, the heavy blocks start first.
+  int head, qb;
+  if (a.heads % 8 == 0 && a.qblocks % 2 == 0) {
+    const int hx = a.heads >> 3, half = hx * (a.qblocks >> 1);
+    const int x = blockIdx.x & 7, sq = blockIdx.x >> 3;
+    const int j = sq < half ? sq : sq - half;
+    head = x * hx + j % hx;
+    qb = sq < half ? a.qblocks - 1 - j / hx : j / hx;
+  } else {
+    head = blockIdx.x / a.qblocks;
+    qb = a.qblocks - 1 - blockIdx.x % a.qblocks;
+  }
   const int q0 = qb * BM, q0w = q0 + wave * 32;
 
   const half_t* const Q = a.q + (int64_t)head * a.sq_z;
