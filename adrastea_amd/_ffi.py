@@ -12,7 +12,7 @@ SYMBOLS = (
     "adr_matmul_f16", "adr_matmul_f16_slow", "adr_matmul_f16_raw", "adr_matmul_nt_f16",
     "adr_matmul_nt_fp16u8", "adr_dequantize_absmax_u8", "adr_quantize_absmax_u8",
     "adr_dequantize_absmax_uint8", "adr_quantize_absmax_uint8", "adr_matmul_f16_plan",
-    "adr_matmul_nt_fp16u8_plan", "adr_softmax_rows", "adr_error_stats_f16", "adr_error_stats_f32", "adr_attention_f16",
+    "adr_matmul_nt_fp16u8_plan", "adr_softmax_rows", "adr_error_stats_f16", "adr_error_stats_f32", "adr_attention_f16", "adr_embed_uint8",
     "adr_strerror", "adr_abi_version",
 )
 
@@ -62,6 +62,7 @@ def lib():
     L.adr_error_stats_f16.argtypes = [vp, TensorDesc, TensorDesc, TensorDesc]
     L.adr_error_stats_f32.argtypes = [vp, TensorDesc, TensorDesc, TensorDesc]
     L.adr_attention_f16.argtypes = [vp, vp, vp, vp, vp] + [i32] * 16 + [f32, f32, u32]
+    L.adr_embed_uint8.argtypes = [vp, i32, i32, vp, vp, vp, vp, i32]
     L.adr_strerror.argtypes = [C.c_int]
     L.adr_strerror.restype = C.c_char_p
     L.adr_abi_version.restype = C.c_int

@@ -136,6 +136,9 @@ hipError_t launch_dequantize(hipStream_t stream, adr_tensor_desc out, adr_tensor
                              adr_tensor_desc in);
 hipError_t launch_quantize(hipStream_t stream, adr_tensor_desc out, adr_tensor_desc scales,
                            adr_tensor_desc in);
+hipError_t launch_embed_u8(hipStream_t stream, int n_dim, int n_ids, const int16_t* in_ids,
+                           half_t* out, const uint8_t* table, const half_t* scales,
+                           int block_size);
 hipError_t launch_error_stats(hipStream_t stream, float* out, const void* lhs, const void* rhs,
                               int64_t length, int64_t sl, int64_t sr, bool f32);
 hipError_t launch_attention(hipStream_t stream, half_t* out, const half_t* q, const half_t* k,

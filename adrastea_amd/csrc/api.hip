@@ -216,6 +216,17 @@ int adr_quantize_absmax_u8(adr_stream_t stream, uint8_t* q, uint16_t* scales,
                                    desc2d(input, rows, cols));
 }
 
+int adr_embed_uint8(adr_stream_t stream, int32_t n_dim, int32_t n_ids, const int16_t* in_ids,
+                    uint16_t* out_embeddings, const uint8_t* embeddings_table,
+                    const uint16_t* scales, int32_t block_size) {
+  if (n_dim < 0 || n_ids < 0 || block_size <= 0) return ADR_EINVAL_SHAPE;
+  if (n_dim % block_size != 0) return ADR_EDIVISIBILITY;
+  if (n_dim == 0 || n_ids == 0) return ADR_OK;
+  if (!in_ids || !out_embeddings || !embeddings_table || !scales) return ADR_ENULL;
+  return (int)launch_embed_u8((hipStream_t)stream, n_dim, n_ids, in_ids, (half_t*)out_embeddings,
+                              embeddings_table, (const half_t*)scales, block_size);
+}
+
 int adr_softmax_rows(adr_stream_t stream, uint16_t* output, const uint16_t* input, int32_t heads,
                      int32_t h, int32_t w, float temp) {
   if (heads < 0 || h < 0 || w < 0) return ADR_EINVAL_SHAPE;

@@ -109,6 +109,37 @@ __global__ __launch_bounds__(256) void quantize_vec_kernel(adr_tensor_desc out, 
   *(u32x2_t*)(q + c) = u32x2_t{w[0], w[1]};
 }
 
+// Embedding lookup in a u8-quantised table (adrastea_kernels/cpp/embed_uint8.cu:3-19):
+//   out[t, i] = fp16( (float(table[id_t, i]) - 127.5f) * float(scales[id_t, i / block_size]) )
+// with id_t = in_ids[t] (16-bit ids, as in the reference).  A gather of n_ids rows: one
+// workgroup column per id, eight weights per lane (8-byte load, one scale, 16-byte store).
+__global__ __launch_bounds__(256) void embed_u8_vec_kernel(int n_dim, const int16_t* in_ids,
+                                                           half_t* out, const uint8_t* table,
+                                                           const half_t* scales, int block_size) {
+  const int t = blockIdx.x;
+  const int i = (blockIdx.y * 256 + threadIdx.x) * 8;
+  if (i >= n_dim) return;
+  const int64_t id = in_ids[t];
+  const u32x2_t w = *(const u32x2_t*)(table + id * n_dim + i);
+  const half_t sv = scales[id * (n_dim / block_size) + i / block_size];
+  half8_t r;
+#pragma unroll
+  for (int j = 0; j < 8; j++) r[j] = dequant_one((uint8_t)((j < 4 ? w[0] : w[1]) >> (8 * (j & 3))), sv);
+  *(half8_t*)(out + (int64_t)t * n_dim + i) = r;
+}
+
+__global__ __launch_bounds__(256) void embed_u8_kernel(int n_dim, const int16_t* in_ids,
+                                                       half_t* out, const uint8_t* table,
+                                                       const half_t* scales, int block_size) {
+  const int t = blockIdx.x;
+  const int64_t id = in_ids[t];
+  const int block_count = n_dim / block_size;
+  for (int i = blockIdx.y * 256 + threadIdx.x; i < n_dim; i += gridDim.y * 256) {
+    const float sv = (float)scales[id * block_count + i / block_size];
+    out[(int64_t)t * n_dim + i] = (half_t)(((float)table[id * n_dim + i] - 127.5f) * sv);
+  }
+}
+
 hipError_t launch_dequantize(hipStream_t stream, adr_tensor_desc out, adr_tensor_desc scales,
                              adr_tensor_desc in) {
   const uint32_t cols = out.shape[0], rows = out.shape[1];
@@ -138,6 +169,23 @@ hipError_t launch_quantize(hipStream_t stream, adr_tensor_desc out, adr_tensor_d
   if ((blocks_per_row + 3) / 4 > 65535) return hipErrorInvalidConfiguration;
   hipLaunchKernelGGL(quantize_kernel, dim3(rows, (blocks_per_row + 3) / 4, 1), dim3(256, 1, 1), 0,
                      stream, out, scales, in, block_size, blocks_per_row);
+  return hipGetLastError();
+}
+
+hipError_t launch_embed_u8(hipStream_t stream, int n_dim, int n_ids, const int16_t* in_ids,
+                           half_t* out, const uint8_t* table, const half_t* scales,
+                           int block_size) {
+  const bool vec = n_dim % 8 == 0 && block_size % 8 == 0 && (uintptr_t)table % 8 == 0 &&
+                   (uintptr_t)out % 16 == 0;
+  if (vec) {
+    hipLaunchKernelGGL(embed_u8_vec_kernel, dim3(n_ids, (n_dim + 2047) / 2048, 1), dim3(256), 0,
+                       stream, n_dim, in_ids, out, table, scales, block_size);
+  } else {
+    int gy = (n_dim + 255) / 256;
+    if (gy > 64) gy = 64;
+    hipLaunchKernelGGL(embed_u8_kernel, dim3(n_ids, gy, 1), dim3(256), 0, stream, n_dim, in_ids,
+                       out, table, scales, block_size);
+  }
   return hipGetLastError();
 }
 

@@ -290,6 +290,21 @@ class GpuKernels(CommonKernels):
         if rc != 0:
             raise AdrasteaError(rc, "quantize_absmax_uint8")
 
+    def embed_uint8(self, output, ids, table, scales, block_size: int):
+        """embed_uint8.cu:3-19: output[t] = dequantised row ids[t] of the u8 table; `ids` is an
+        int16 tensor, as the reference's kernel takes them."""
+        import torch
+        assert ids.dtype == torch.int16 and table.dtype == torch.uint8
+        n_ids, n_dim = ids.numel(), table.shape[1]
+        assert tuple(output.shape) == (n_ids, n_dim)
+        assert tuple(scales.shape) == (table.shape[0], n_dim // block_size)
+        assert all(t.is_contiguous() for t in (output, ids, table, scales))
+        rc = self._lib.adr_embed_uint8(_current_stream(), n_dim, n_ids, ids.data_ptr(),
+                                       output.data_ptr(), table.data_ptr(), scales.data_ptr(),
+                                       block_size)
+        if rc != 0:
+            raise AdrasteaError(rc, "embed_uint8")
+
 
 def descriptor(view: TensorView) -> _ffi.TensorDesc:
     """TensorGpuDescriptor::from (kernels.rs:38-55): dims and strides reversed, innermost first."""

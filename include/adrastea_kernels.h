@@ -149,6 +149,19 @@ int adr_quantize_absmax_uint8(adr_stream_t stream, adr_tensor_desc output,
                               adr_tensor_desc scales, adr_tensor_desc input);
 
 /*
+ * Embedding lookup in a u8-quantised table (device: adrastea_kernels/cpp/embed_uint8.cu:3-19
+ * `embed_uint8(n_dim, n_ids, in_ids, out_embeddings, embeddings_table, scales, block_size)`; the
+ * reference compiles it but has no host call yet, so the device signature is the interface):
+ *   out[t, i] = fp16( (float(table[id_t, i]) - 127.5f) * float(scales[id_t, i / block_size]) ),
+ * id_t = in_ids[t], 16-bit ids as in the reference; `table` is [vocab, n_dim] u8 and `scales`
+ * [vocab, n_dim / block_size] fp16, the format of adr_quantize_absmax_u8.  Ids are not range
+ * checked (the kernel has no vocabulary size, as in the reference).
+ */
+int adr_embed_uint8(adr_stream_t stream, int32_t n_dim, int32_t n_ids, const int16_t* in_ids,
+                    uint16_t* out_embeddings, const uint8_t* embeddings_table,
+                    const uint16_t* scales, int32_t block_size);
+
+/*
  * Row-wise softmax with temperature, the step between QK^T and P.V
  * (device: adrastea_kernels/cpp/normalize.cu:147-220 `softmax_rows(output, input, h, w, temp)` on
  * a (heads, h) grid; host: CommonKernels::softmax_rows_inplace, adrastea_models/src/kernels.rs:214,

@@ -70,6 +70,9 @@ def lib():
         L.adr_o_dequantize_absmax_u8.argtypes = [u16p, u8p, u16p, C.c_int, C.c_int, C.c_int]
         L.adr_o_quantize_absmax_u8.argtypes = [u8p, u16p, u16p, C.c_int, C.c_int, C.c_int]
         L.adr_o_dequant_table.argtypes = [u16p]
+        L.adr_o_embed_uint8.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p,
+                                        C.c_void_p, C.c_int]
+        L.adr_o_embed_uint8.restype = None
         L.adr_o_error_stats.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
         L.adr_o_softmax_rows.argtypes = [u16p, u16p, C.c_int64, C.c_int, C.c_float, C.c_int]
         _lib = L
@@ -207,6 +210,18 @@ def attention_f16(q, k, v, scale, temp=1.0, mask=MASK_NONE, exact=False, threads
     matmul_f16(out, probs, v, heads, m, n, d, (1, d, m * d), (1, n, m * n), (1, d, n * d),
                threads=threads)
     return out.reshape(heads, m, d)
+
+
+def embed_uint8(ids, table, scales, block_size):
+    """embed_uint8.cu:3-19: rows ids[t] of the u8 table, dequantised; ids int16."""
+    ids, table, scales = (np.ascontiguousarray(a) for a in (ids, table, scales))
+    assert ids.dtype == np.int16 and table.dtype == np.uint8 and scales.dtype == np.float16
+    n_dim = table.shape[1]
+    out = np.empty((ids.size, n_dim), np.float16)
+    lib().adr_o_embed_uint8(n_dim, ids.size, ids.ctypes.data_as(C.c_void_p),
+                            out.ctypes.data_as(C.c_void_p), table.ctypes.data_as(C.c_void_p),
+                            scales.ctypes.data_as(C.c_void_p), block_size)
+    return out
 
 
 def dequant_table():

@@ -290,6 +290,17 @@ void adr_o_dequantize_absmax_u8(uint16_t* output, const uint8_t* q, const uint16
           dequant_one(q[(int64_t)r * cols + i], scales[(int64_t)r * block_count + i / block_size]);
 }
 
+void adr_o_embed_uint8(int n_dim, int n_ids, const int16_t* in_ids, uint16_t* out,
+                       const uint8_t* table, const uint16_t* scales, int block_size) {
+  int block_count = n_dim / block_size; /* embed_uint8.cu:11 */
+  for (int t = 0; t < n_ids; t++) {
+    int id = in_ids[t]; /* :13 */
+    for (int i = 0; i < n_dim; i++) /* :14-17 */
+      out[(int64_t)t * n_dim + i] =
+          dequant_one(table[(int64_t)id * n_dim + i], scales[(int64_t)id * block_count + i / block_size]);
+  }
+}
+
 void adr_o_quantize_absmax_u8(uint8_t* q, uint16_t* scales, const uint16_t* input, int rows,
                               int cols, int block_size) {
   int block_count = cols / block_size;

@@ -87,6 +87,9 @@ void adr_o_matmul_nt_fp16u8(uint16_t* output, const uint16_t* lhs, const uint8_t
 void adr_o_dequantize_absmax_u8(uint16_t* output, const uint8_t* q, const uint16_t* scales,
                                 int rows, int cols, int block_size);
 /* quantize.cu:3-44 */
+/* embed_uint8.cu:3-19: out[t, i] = dequant(table[ids[t], i], scales[ids[t], i / block_size]). */
+void adr_o_embed_uint8(int n_dim, int n_ids, const int16_t* in_ids, uint16_t* out,
+                       const uint8_t* table, const uint16_t* scales, int block_size);
 void adr_o_quantize_absmax_u8(uint8_t* q, uint16_t* scales, const uint16_t* input, int rows,
                               int cols, int block_size);
 

@@ -118,6 +118,15 @@ class RefKernels:
         args = [desc2d(q), desc2d(scales), desc2d(x)]
         self._launch(f, (scales.shape[1], x.shape[0], 1), (32, 1, 1), 0, args)
 
+    def embed_uint8(self, out, ids, table, scales, block_size):
+        """embed_uint8.cu:3-19, one thread per id (256-thread blocks)."""
+        f = self._fn("embed_uint8.co", b"embed_uint8")
+        n_ids, n_dim = ids.numel(), table.shape[1]
+        args = [C.c_int(n_dim), C.c_int(n_ids), C.c_void_p(ids.data_ptr()),
+                C.c_void_p(out.data_ptr()), C.c_void_p(table.data_ptr()),
+                C.c_void_p(scales.data_ptr()), C.c_int(block_size)]
+        self._launch(f, ((n_ids + 255) // 256, 1, 1), (256, 1, 1), 0, args)
+
     def softmax_rows(self, out, inp, heads, h, w, temp=1.0):
         """normalize.cu:147-220 with the launch of kernels.rs:892-915 ((h, heads) x 256)."""
         f = self._fn("normalize.co", b"softmax_rows")
