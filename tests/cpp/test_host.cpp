@@ -6,10 +6,15 @@
 #include <dlfcn.h>
 
 #include <cstdio>
+#include <algorithm>
+#include <cmath>
+#include <cstdlib>
 #include <cstring>
+#include <string>
 #include <vector>
 
 #include "../../adrastea_amd/host/kernels.hpp"
+#include "../../adrastea_amd/host/pickle.hpp"
 
 using namespace adrastea;
 
@@ -188,7 +193,82 @@ static void gpu_test() {
   CHECK(throws([&] { tr.matmul_f16(ov, lv, wv.permute({1, 0}), MatmulOptions::make().store(MatmulStore::GeluBias(&bias))); }));
 }
 
+// One line per tensor: name dtype rank shape.. stride.. begin end fnv1a64(bytes).  The Python
+// test compares these with what torch's own loader returns for the same file.
+static void dump_tensor(const std::string& name, const PickledModel& m, const PickledTensor& t) {
+  static const char* names[] = {"i8", "i64", "f16", "f32", "f64"};
+  uint64_t h = 1469598103934665603ull;
+  for (size_t i = t.begin; i < t.end; i++) h = (h ^ m.mapping.data()[i]) * 1099511628211ull;
+  printf("%s %s %zu", name.c_str(), names[(int)t.dtype], t.shape.size());
+  for (size_t d : t.shape) printf(" %zu", d);
+  for (size_t d : t.stride) printf(" %zu", d);
+  printf(" %zu %zu %016llx\n", t.begin, t.end, (unsigned long long)h);
+}
+
+static int pickle_dump(int argc, char** argv) {
+  try {
+    if (!strcmp(argv[1], "pickle")) {
+      auto m = PickledModel::load_file(argv[2], argc > 3 ? argv[3] : nullptr);
+      for (auto& kv : m->tensors) dump_tensor(kv.first, *m, kv.second);
+    } else {
+      auto m = ShardedModel::load_huggingface(argv[2]);
+      printf("shards %zu\n", m->shard_count());
+      for (int i = 3; i < argc; i++) {
+        auto f = m->find(argv[i]);
+        dump_tensor(argv[i], *f.first, *f.second);
+      }
+    }
+  } catch (const std::exception& e) {
+    printf("ERROR %s\n", e.what());
+    return 2;
+  }
+  return 0;
+}
+
+// Checkpoint -> device -> u8: uploads one fp16 [N, K] tensor of the file, quantises it with
+// adr_quantize_absmax_u8 and dequantises it again; prints the largest |x - dq(q(x))| / scale.
+static int pickle_quantize(const char* path, const char* name, int block_size) {
+  void* hip = dlopen("libamdhip64.so", RTLD_NOW | RTLD_GLOBAL);
+  if (!hip) { printf("ERROR no hip runtime\n"); return 2; }
+  auto hipMalloc = (int (*)(void**, size_t))dlsym(hip, "hipMalloc");
+  auto hipMemcpy = (int (*)(void*, const void*, size_t, int))dlsym(hip, "hipMemcpy");
+  auto hipDeviceSynchronize = (int (*)())dlsym(hip, "hipDeviceSynchronize");
+  try {
+    auto m = PickledModel::load_file(path);
+    const PickledTensor& t = m->tensor(name);
+    if (t.dtype != TensorDataType::F16 || t.shape.size() != 2 || t.stride[1] != 1 || t.stride[0] != t.shape[1])
+      throw std::runtime_error("expected a contiguous fp16 matrix");
+    const int rows = (int)t.shape[0], cols = (int)t.shape[1];
+    const size_t n = (size_t)rows * cols;
+    uint16_t *dx, *ds, *dy;
+    uint8_t* dq;
+    if (hipMalloc((void**)&dx, n * 2) || hipMalloc((void**)&dy, n * 2) || hipMalloc((void**)&dq, n) ||
+        hipMalloc((void**)&ds, n / block_size * 2))
+      throw std::runtime_error("hipMalloc failed");
+    hipMemcpy(dx, m->bytes(t), n * 2, 1);  // the copy of load_tensor (pickle.rs:331-335)
+    int rc = adr_quantize_absmax_u8(nullptr, dq, ds, dx, rows, cols, block_size);
+    if (!rc) rc = adr_dequantize_absmax_u8(nullptr, dy, dq, ds, rows, cols, block_size);
+    if (rc || hipDeviceSynchronize()) throw std::runtime_error("launch failed");
+    std::vector<uint16_t> y(n), sc(n / block_size);
+    hipMemcpy(y.data(), dy, n * 2, 2);
+    hipMemcpy(sc.data(), ds, sc.size() * 2, 2);
+    const uint16_t* x = (const uint16_t*)m->bytes(t);
+    double worst = 0;
+    for (size_t i = 0; i < n; i++) {
+      const double s = h2d(sc[i / block_size]);
+      if (s > 0) worst = std::max(worst, std::fabs(h2d(x[i]) - h2d(y[i])) / s);
+    }
+    printf("rows %d cols %d worst_error_in_scales %.4f\n", rows, cols, worst);
+  } catch (const std::exception& e) {
+    printf("ERROR %s\n", e.what());
+    return 2;
+  }
+  return 0;
+}
+
 int main(int argc, char** argv) {
+  if (argc > 2 && (!strcmp(argv[1], "pickle") || !strcmp(argv[1], "sharded"))) return pickle_dump(argc, argv);
+  if (argc > 4 && !strcmp(argv[1], "quantize")) return pickle_quantize(argv[2], argv[3], atoi(argv[4]));
   if (argc > 1 && !strcmp(argv[1], "gpu")) gpu_test(); else cpu_tests();
   printf(failures ? "FAILED (%d)\n" : "OK\n", failures);
   return failures != 0;

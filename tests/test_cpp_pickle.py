@@ -1,0 +1,199 @@
+"""The C++ checkpoint reader (adrastea_amd/host/pickle.hpp, mirror of adrastea_models/src/
+pickle.rs:33-338) against torch's own loader on checkpoints written here with torch.save:
+names, dtypes, shapes, strides and the exact bytes of every tensor, the `_metadata` skip, the
+nested-dict path, shared storages with offsets, non-contiguous strides, a Hugging Face style
+sharded directory, and the error cases the reference names."""
+import json
+import os
+import subprocess
+
+import pytest
+import torch
+
+from adrastea_amd import build
+
+DT = {torch.float16: ("f16", 2), torch.float32: ("f32", 4), torch.int64: ("i64", 8)}
+
+
+def fnv1a64(b: bytes) -> int:
+    h = 1469598103934665603
+    for x in b:
+        h = ((h ^ x) * 1099511628211) & 0xFFFFFFFFFFFFFFFF
+    return h
+
+
+def run(*args):
+    r = subprocess.run([build.build_host_test(), *args], capture_output=True, text=True, timeout=60)
+    return r.returncode, r.stdout
+
+
+def expected_line(name, t):
+    """What the reader must report for tensor t, derived from torch's view of it: the bytes of
+    its storage from the storage offset to the last addressed element (pickle.rs:155-168)."""
+    code, el = DT[t.dtype]
+    largest = sum((d - 1) * s for d, s in zip(t.shape, t.stride()))
+    raw = bytes(t.untyped_storage())
+    lo = t.storage_offset() * el
+    data = raw[lo:lo + (largest + 1) * el]
+    dims = " ".join(str(d) for d in t.shape)
+    strides = " ".join(str(s) for s in t.stride())
+    return f"{name} {code} {t.dim()} {dims} {strides}", len(data), f"{fnv1a64(data):016x}"
+
+
+def check(stdout, tensors):
+    lines = [l for l in stdout.strip().splitlines() if l]
+    assert len(lines) == len(tensors)
+    for line, name in zip(lines, sorted(tensors)):        # the reference's BTreeMap order
+        head, length, digest = expected_line(name, tensors[name])
+        parts = line.split()
+        assert " ".join(parts[:-3]) == head, line
+        assert int(parts[-2]) - int(parts[-3]) == length, line
+        assert parts[-1] == digest, line
+
+
+def make_state():
+    g = torch.Generator().manual_seed(3)
+    base = torch.randn(6, 10, generator=g).half()
+    return {
+        "tok_embeddings.weight": torch.randn(12, 8, generator=g).half(),
+        "layers.0.attention.wq.weight": torch.randn(8, 8, generator=g),
+        "transposed": torch.randn(5, 7, generator=g).half().t(),         # strides (1, 7)
+        "view_with_offset": base[2:5, 3:9],                               # offset 23, strides (10, 1)
+        "same_storage_other_view": base[0],
+        "steps": torch.arange(4, dtype=torch.int64),
+        "vector": torch.randn(33, generator=g).half(),
+    }
+
+
+def test_reader_matches_torch_loader(tmp_path):
+    state = make_state()
+    path = str(tmp_path / "consolidated.00.pth")
+    torch.save(state, path)
+    rc, out = run("pickle", path)
+    assert rc == 0, out
+    back = torch.load(path, weights_only=True)
+    check(out, back)
+    for k in state:                                       # and torch read back what was written
+        assert torch.equal(state[k], back[k])
+
+
+def test_state_dict_with_metadata_and_nested_path(tmp_path):
+    lin = torch.nn.Linear(5, 3).half()
+    sd = lin.state_dict()                                  # an OrderedDict carrying _metadata
+    path = str(tmp_path / "model.pt")
+    torch.save({"model": sd, "epoch": 3, "lr": 0.25, "tag": "x"}, path)
+    rc, out = run("pickle", path, "model")
+    assert rc == 0, out
+    check(out, torch.load(path, weights_only=True)["model"])
+    rc, out = run("pickle", path, "missing")
+    assert rc == 2 and "key not found" in out
+    rc, out = run("pickle", path)                          # the top level holds non-tensors
+    assert rc == 2 and "is not a tensor" in out
+
+
+def test_sharded_huggingface_directory(tmp_path):
+    g = torch.Generator().manual_seed(5)
+    a = {"model.embed.weight": torch.randn(9, 4, generator=g).half(),
+         "model.layers.0.w": torch.randn(4, 4, generator=g).half()}
+    b = {"model.layers.1.w": torch.randn(4, 4, generator=g).half(),
+         "lm_head.weight": torch.randn(9, 4, generator=g).half()}
+    torch.save(a, str(tmp_path / "pytorch_model-00001-of-00002.bin"))
+    torch.save(b, str(tmp_path / "pytorch_model-00002-of-00002.bin"))
+    index = {"metadata": {"total_size": 1}, "weight_map": {
+        **{k: "pytorch_model-00001-of-00002.bin" for k in a},
+        **{k: "pytorch_model-00002-of-00002.bin" for k in b}}}
+    (tmp_path / "pytorch_model.bin.index.json").write_text(json.dumps(index, indent=2))
+    names = sorted({**a, **b})
+    rc, out = run("sharded", str(tmp_path), *names)
+    assert rc == 0, out
+    lines = out.strip().splitlines()
+    assert lines[0] == "shards 2"
+    check("\n".join(lines[1:]), {**a, **b})
+    rc, out = run("sharded", str(tmp_path), "nope")
+    assert rc == 2 and "not found" in out
+
+
+def test_rejects_what_the_reference_rejects(tmp_path):
+    # compressed members (pickle.rs:240-242)
+    import zipfile
+    p = str(tmp_path / "compressed.pt")
+    with zipfile.ZipFile(p, "w", zipfile.ZIP_DEFLATED) as z:
+        z.writestr("archive/data.pkl", b"\x80\x02}q\x00." * 50)
+    rc, out = run("pickle", p)
+    assert rc == 2 and "compressed" in out
+    # unsupported dtype (pickle.rs:147-152)
+    p = str(tmp_path / "bf16.pt")
+    torch.save({"w": torch.zeros(2, 2, dtype=torch.bfloat16)}, p)
+    rc, out = run("pickle", p)
+    assert rc == 2 and "unsupported dtype" in out
+    # not an archive at all, and an archive without data.pkl
+    p = str(tmp_path / "junk.pt")
+    open(p, "wb").write(b"not a zip" * 10)
+    rc, out = run("pickle", p)
+    assert rc == 2 and "ERROR" in out
+    p = str(tmp_path / "empty.zip")
+    with zipfile.ZipFile(p, "w") as z:
+        z.writestr("other.txt", b"hello")
+    rc, out = run("pickle", p)
+    assert rc == 2 and "data.pkl not found" in out
+
+
+@pytest.mark.gpu
+def test_checkpoint_to_u8_on_the_device(tmp_path):
+    """zip/pickle -> [N, K] fp16 on the device -> adr_quantize_absmax_u8 -> (u8, scales), then
+    dequantised again: every weight within half a quantisation step of the file's value, plus
+    the fp16 rounding of the dequantised number (at most 127.5 scales large: 127.5 * 2^-11 / 2)."""
+    assert os.path.exists(build.HOST_TEST_BIN)
+    g = torch.Generator().manual_seed(9)
+    path = str(tmp_path / "layer.pth")
+    torch.save({"w": (torch.randn(256, 1024, generator=g) * 0.05).half()}, path)
+    r = subprocess.run([build.HOST_TEST_BIN, "quantize", path, "w", "32"], capture_output=True,
+                       text=True, timeout=120)
+    assert r.returncode == 0, r.stdout + r.stderr
+    fields = r.stdout.split()
+    assert fields[:4] == ["rows", "256", "cols", "1024"]
+    assert float(fields[-1]) <= 0.5 + 127.5 * 2.0 ** -12 + 1e-3
+
+
+def test_zip64_records(tmp_path):
+    """Archives beyond 4 GiB carry their sizes and offsets in zip64 records.  A small archive is
+    rewritten here with EVERY size and offset moved into those records (legal for any size), so
+    the reader's zip64 branch is exercised without a 4 GiB file."""
+    import struct
+    import zipfile
+    state = {"w": torch.arange(24, dtype=torch.float32).reshape(4, 6).half(),
+             "b": torch.arange(5, dtype=torch.int64)}
+    src = str(tmp_path / "small.pt")
+    torch.save(state, src)
+    with zipfile.ZipFile(src) as z:
+        members = [(i.filename, z.read(i.filename)) for i in z.infolist()]
+    blob, central = b"", b""
+    for name, data in members:
+        nb = name.encode()
+        off = len(blob)
+        # local header: sizes 0xFFFFFFFF + zip64 extra (uncompressed, compressed)
+        extra = struct.pack("<HHQQ", 1, 16, len(data), len(data))
+        blob += struct.pack("<IHHHHHIIIHH", 0x04034b50, 45, 0, 0, 0, 0, zipfile.crc32(data),
+                            0xFFFFFFFF, 0xFFFFFFFF, len(nb), len(extra)) + nb + extra + data
+        cextra = struct.pack("<HHQQQ", 1, 24, len(data), len(data), off)
+        central += struct.pack("<IHHHHHHIIIHHHHHII", 0x02014b50, 45, 45, 0, 0, 0, 0,
+                               zipfile.crc32(data), 0xFFFFFFFF, 0xFFFFFFFF, len(nb), len(cextra),
+                               0, 0, 0, 0, 0xFFFFFFFF) + nb + cextra
+    cd_off = len(blob)
+    rec_off = cd_off + len(central)
+    rec = struct.pack("<IQHHIIQQQQ", 0x06064b50, 44, 45, 45, 0, 0, len(members), len(members),
+                      len(central), cd_off)
+    loc = struct.pack("<IIQI", 0x07064b50, 0, rec_off, 1)
+    eocd = struct.pack("<IHHHHIIH", 0x06054b50, 0, 0, 0xFFFF, 0xFFFF, 0xFFFFFFFF, 0xFFFFFFFF, 0)
+    dst = str(tmp_path / "zip64.pt")
+    open(dst, "wb").write(blob + central + rec + loc + eocd)
+    with zipfile.ZipFile(dst) as z:                        # Python's reader accepts it too
+        assert z.testzip() is None
+    rc, out = run("pickle", dst)
+    assert rc == 0, out
+    lines = out.strip().splitlines()
+    ref_rc, ref_out = run("pickle", src)
+    # same tensors and bytes as the plain archive (file offsets differ)
+    strip = lambda ls: [" ".join(l.split()[:-3]) + " " + l.split()[-1] for l in ls]
+    assert ref_rc == 0 and strip(lines) == strip(ref_out.strip().splitlines())
+    check(out, state)
