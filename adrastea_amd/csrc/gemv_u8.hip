@@ -424,6 +424,10 @@ hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, co
         if (m == 2) return launch_dot<2, 4, 4, 1>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
         return launch_dot<4, 4, 4, 1>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
       }
+      // up to 12 segments: 4 wavefronts, three segments each (K = 11008 has 11: one idle slot
+      // instead of five with 8 x 2)
+      if (m == 1 && p <= 12 * 1024)
+        return launch_dot<1, 4, 4, 3>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
       // up to 16 segments: 8 wavefronts, two segments each
       if (m == 1) return launch_dot<1, 8, 4, 2>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
       return launch_dot<2, 8, 4, 2>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
