@@ -136,7 +136,7 @@ struct WStage {
   u32x4_t sc;    // the eight fp16 scales (block_size 32) of the macro step
 };
 
-template <int NW, int RG>
+template <int NW, int RG, bool UPFRONT>
 __global__ __launch_bounds__(NW * 64) void gemv_u8_wide_kernel(half_t* __restrict__ out,
                                                                const half_t* __restrict__ lhs,
                                                                const uint8_t* __restrict__ rhs,
@@ -190,15 +190,34 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_wide_kernel(half_t* __restric
     }
   };
 
-  // all weight loads of a macro step are issued before its first use
-  for (int ms = wave; ms < steps; ms += NW) {
-    u32x4_t x[8];
-    WStage s[RG];
-    load_x(x, ms);
+  if (UPFRONT) {
+    // exactly two macro steps per wavefront (K = 512 * NW): everything the wavefront reads is
+    // issued before the first multiply (the fence keeps the compiler from sinking the second
+    // step's loads below the first step's arithmetic, which would expose their latency again)
+    u32x4_t xa[8], xb[8];
+    WStage sa[RG], sb[RG];
+    load_x(xa, wave);
 #pragma unroll
-    for (int q = 0; q < RG; q++) load_w(s[q], q, ms);
+    for (int q = 0; q < RG; q++) load_w(sa[q], q, wave);
+    load_x(xb, wave + NW);
 #pragma unroll
-    for (int q = 0; q < RG; q++) compute(s[q], x, acc[q]);
+    for (int q = 0; q < RG; q++) load_w(sb[q], q, wave + NW);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int q = 0; q < RG; q++) compute(sa[q], xa, acc[q]);
+#pragma unroll
+    for (int q = 0; q < RG; q++) compute(sb[q], xb, acc[q]);
+  } else {
+    // all weight loads of a macro step are issued before its first use
+    for (int ms = wave; ms < steps; ms += NW) {
+      u32x4_t x[8];
+      WStage s[RG];
+      load_x(x, ms);
+#pragma unroll
+      for (int q = 0; q < RG; q++) load_w(s[q], q, ms);
+#pragma unroll
+      for (int q = 0; q < RG; q++) compute(s[q], x, acc[q]);
+    }
   }
 
 #pragma unroll
@@ -438,8 +457,12 @@ hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, co
       // enough wavefronts per workgroup to keep every macro step of a small problem in flight
       // wide matrices: 48 weight rows per workgroup share one fetch of the activations
       if (n >= 8192) {
-        hipLaunchKernelGGL((gemv_u8_wide_kernel<8, 3>), dim3((n + 3 * ROWS - 1) / (3 * ROWS)),
-                           dim3(512), 0, stream, out, lhs, rhs, scales, m, p, n, beta);
+        if (steps == 16)
+          hipLaunchKernelGGL((gemv_u8_wide_kernel<8, 3, true>), dim3((n + 3 * ROWS - 1) / (3 * ROWS)),
+                             dim3(512), 0, stream, out, lhs, rhs, scales, m, p, n, beta);
+        else
+          hipLaunchKernelGGL((gemv_u8_wide_kernel<8, 3, false>), dim3((n + 3 * ROWS - 1) / (3 * ROWS)),
+                             dim3(512), 0, stream, out, lhs, rhs, scales, m, p, n, beta);
         return hipGetLastError();
       }
       if (steps >= 16 && blocks <= 1024)
