@@ -238,6 +238,130 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_wide_kernel(half_t* __restric
   }
 }
 
+// Wide matrices, K = 4096: the weights come in by global -> LDS DMA, four whole 256-byte row
+// pieces per instruction (the register path touches sixteen rows with 64 bytes each per
+// instruction, which moves the same bytes about a quarter slower).  A wavefront owns two macro
+// steps x RG row groups = 2 RG tiles of 4 KiB ([16 rows][16 chunks of 16 bytes], chunk c of row r
+// at position c ^ r so that fragment reads spread over all banks) and streams them through a
+// private ring of RING tiles: nothing but its own vmcnt orders the DMA against its reads.
+// Activations and scales are loaded into registers before the first DMA, so the count of
+// outstanding loads at any later point is a multiple of the four DMA instructions of a tile.
+#define ADR_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+#define ADR_GLB_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
+
+template <int NW, int RG, int RING>
+__global__ __launch_bounds__(NW * 64) void gemv_u8_ring_kernel(half_t* __restrict__ out,
+                                                               const half_t* __restrict__ lhs,
+                                                               const uint8_t* __restrict__ rhs,
+                                                               const half_t* __restrict__ scales,
+                                                               int m, int p, int n, float beta) {
+  constexpr int TILE = ROWS * MACRO_K;  // 4096 bytes
+  constexpr int UNITS = 2 * RG;         // tiles per wavefront: macro steps wave, wave + NW
+  static_assert(RING <= UNITS && NW * RG * 256 * 4 <= NW * RING * TILE, "partials reuse the ring");
+  __shared__ __attribute__((aligned(1024))) unsigned char ring[NW * RING * TILE];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * (ROWS * RG);
+  const int nblk = p / 32;
+  const bool xvalid = r < m;
+  const half_t* xrow = lhs + (int64_t)min(r, m - 1) * p + g * 16;
+  unsigned char* const mine = ring + wave * RING * TILE;
+
+  // registers first: activations of both macro steps, scales of all tiles
+  u32x4_t x[2][8], sc[2][RG];
+#pragma unroll
+  for (int h = 0; h < 2; h++) {
+    const int ms = wave + h * NW;
+    const half_t* xp = xrow + (int64_t)ms * MACRO_K;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      // lanes beyond m read row m-1 again (the same addresses as its own lanes) and are zeroed
+      // when used: a load under a lane mask would be waited for where the lanes rejoin
+      x[h][2 * j] = *(const u32x4_t*)(xp + j * 64);
+      x[h][2 * j + 1] = *(const u32x4_t*)(xp + j * 64 + 8);
+    }
+#pragma unroll
+    for (int q = 0; q < RG; q++)
+      sc[h][q] = *(const u32x4_t*)(scales + (int64_t)min(n0 + q * ROWS + r, n - 1) * nblk +
+                                   ms * (MACRO_K / 32));
+  }
+  // DMA instruction i of a tile fills its chunks [64 i, 64 i + 64): rows 4i .. 4i+3
+  auto issue = [&](int u) {  // tile u = (macro step half u / RG, row group u % RG)
+    const int h = u / RG, q = u % RG;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int row = 4 * i + (lane >> 4), kc = (lane & 15) ^ row;
+      const uint8_t* src = rhs + (int64_t)min(n0 + q * ROWS + row, n - 1) * p +
+                           (int64_t)(wave + h * NW) * MACRO_K + kc * 16;
+      __builtin_amdgcn_global_load_lds(ADR_GLB_PTR(src),
+                                       ADR_LDS_PTR(mine + (u % RING) * TILE + i * 1024), 16, 0, 0);
+    }
+  };
+  int roff[4];  // fragment read j of the lane: logical chunk 4j + g of row r
+#pragma unroll
+  for (int j = 0; j < 4; j++) roff[j] = r * 256 + (((4 * j + g) ^ r) << 4);
+
+  float4_t acc[RG][2];
+#pragma unroll
+  for (int q = 0; q < RG; q++) acc[q][0] = acc[q][1] = float4_t{0, 0, 0, 0};
+#pragma unroll
+  for (int u = 0; u < RING; u++) issue(u);
+#pragma unroll
+  for (int u = 0; u < UNITS; u++) {
+    // tiles u+1 .. min(u+RING-1, UNITS-1) may still be in flight: four DMA instructions each
+    constexpr int Z = 0;
+    const int later = (u + RING - 1 < UNITS ? RING - 1 : UNITS - 1 - u) * 4 + Z;
+    if (later == 8) __builtin_amdgcn_s_waitcnt(0x0F70 | 8);
+    else if (later == 4) __builtin_amdgcn_s_waitcnt(0x0F70 | 4);
+    else if (later == 12) __builtin_amdgcn_s_waitcnt(0x0F70 | 12);
+    else __builtin_amdgcn_s_waitcnt(0x0F70 | 0);
+    const int h = u / RG, q = u % RG;
+    const unsigned char* tile = mine + (u % RING) * TILE;
+    const half8_t s8 = __builtin_bit_cast(half8_t, sc[h][q]);
+    const u32x4_t z = {0, 0, 0, 0};
+    u32x4_t w[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) w[j] = *(const u32x4_t*)(tile + roff[j]);
+    // the tile is in registers before its slot is refilled
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    __builtin_amdgcn_sched_barrier(0);
+    if (u + RING < UNITS) issue(u + RING);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const half_t sv = g < 2 ? s8[2 * j] : s8[2 * j + 1];
+      const half2_t s2 = {sv, sv};
+      const half8_t a0 = dequant8(w[j][0], w[j][1], s2), a1 = dequant8(w[j][2], w[j][3], s2);
+      const half8_t b0 = __builtin_bit_cast(half8_t, xvalid ? x[h][2 * j] : z);
+      const half8_t b1 = __builtin_bit_cast(half8_t, xvalid ? x[h][2 * j + 1] : z);
+      acc[q][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, b0, acc[q][0], 0, 0, 0);
+      acc[q][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, b1, acc[q][1], 0, 0, 0);
+    }
+  }
+
+  // the ring is dead: its memory takes the per-wavefront partial sums [NW][RG][256]
+  __syncthreads();
+  float* partial = (float*)ring;
+#pragma unroll
+  for (int q = 0; q < RG; q++)
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      partial[(wave * RG + q) * 256 + (4 * g + i) * 16 + r] = acc[q][0][i] + acc[q][1][i];
+  __syncthreads();
+  for (int e = tid; e < RG * ROWS * 16; e += NW * 64) {
+    const int mm = e / (RG * ROWS), nn = e % (RG * ROWS);  // consecutive threads -> consecutive columns
+    if (mm < m && n0 + nn < n) {
+      float sum = 0.0f;
+#pragma unroll
+      for (int w2 = 0; w2 < NW; w2++)
+        sum += partial[(w2 * RG + nn / ROWS) * 256 + (nn % ROWS) * 16 + mm];
+      half_t* o = out + (int64_t)mm * n + n0 + nn;
+      // the previous output is read even for beta == 0, as the reference does
+      *o = (half_t)(sum + beta * (float)*o);
+    }
+  }
+}
+
 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
 
 template <int CTRL, int ROWMASK>
@@ -426,7 +550,9 @@ hipError_t launch_gemm_u8_mfma(hipStream_t stream, half_t* out, const half_t* lh
 const char* gemm_u8_plan(int m, int p, int n, int block_size) {
   switch (choose_u8(nullptr, nullptr, nullptr, m, p, n, block_size)) {
     case U8_DOT: return "gemv_u8_dot2_stream";
-    case U8_GEMV: return n >= 8192 ? "gemv_u8_mfma16_wide" : "gemv_u8_mfma16_stream";
+    case U8_GEMV:
+      return n < 8192 ? "gemv_u8_mfma16_stream"
+                      : p == 16 * MACRO_K ? "gemv_u8_mfma16_wide_dma" : "gemv_u8_mfma16_wide";
     case U8_GEMM: return "gemm_nt_u8_mfma";
     default: return "gemm_u8_naive";
   }
@@ -458,7 +584,7 @@ hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, co
       // wide matrices: 48 weight rows per workgroup share one fetch of the activations
       if (n >= 8192) {
         if (steps == 16)
-          hipLaunchKernelGGL((gemv_u8_wide_kernel<8, 3, true>), dim3((n + 3 * ROWS - 1) / (3 * ROWS)),
+          hipLaunchKernelGGL((gemv_u8_ring_kernel<8, 3, 3>), dim3((n + 3 * ROWS - 1) / (3 * ROWS)),
                              dim3(512), 0, stream, out, lhs, rhs, scales, m, p, n, beta);
         else
           hipLaunchKernelGGL((gemv_u8_wide_kernel<8, 3, false>), dim3((n + 3 * ROWS - 1) / (3 * ROWS)),

@@ -186,6 +186,23 @@ def test_gemv_bit_exact_on_exact_inputs(kern, m, pn):
         assert np.array_equal(to_np(out).view(np.uint16), want.view(np.uint16)), (m, p, n, beta)
 
 
+@pytest.mark.parametrize("m", [3, 16])
+def test_wide_dma_gemv_bit_exact_on_exact_inputs(kern, m):
+    """K = 4096 on a wide matrix: the weights stream through the per-wavefront LDS ring; ragged
+    last workgroup (8251 = 171 * 48 + 43 rows), beta path."""
+    p, n = 4096, 8251
+    g = rng(990 + m)
+    assert u8_plan(m, p, n, 32) == "gemv_u8_mfma16_wide_dma"
+    a, q, s = _u8_case(g, m, p, n, 32, exact=True)
+    for beta in (0.0, 1.0):
+        prev = (g.integers(-8, 9, size=(m, n)) / 4.0).astype(np.float16)
+        want = prev.copy()
+        oracle.matmul_nt_fp16u8(want, a, q, s, 32, beta=beta, threads=8)
+        out = to_dev(prev)
+        kern.matmul_nt_fp16u8(out, to_dev(a), to_dev(q), to_dev(s), 32, beta=beta)
+        assert np.array_equal(to_np(out).view(np.uint16), want.view(np.uint16)), (m, beta)
+
+
 @pytest.mark.parametrize("m", [3, 7, 16])
 @pytest.mark.parametrize("pn", [(256, 8192), (768, 8200), (1024, 8251)])
 def test_wide_gemv_bit_exact_on_exact_inputs(kern, m, pn):
@@ -280,7 +297,7 @@ def test_decode_shapes_full_size(kern, kn, m):
     s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
     a = torch.randn(m, p, generator=gen, device="cuda").half()
     assert u8_plan(m, p, n, 32) in ("gemv_u8_mfma16_stream", "gemv_u8_mfma16_wide",
-                                    "gemv_u8_dot2_stream")
+                                    "gemv_u8_mfma16_wide_dma", "gemv_u8_dot2_stream")
     out = torch.zeros(m, n, dtype=torch.float16, device="cuda")
     kern.matmul_nt_fp16u8(out, a, q, s, 32)
     w = torch.zeros(n, p, dtype=torch.float16, device="cuda")
