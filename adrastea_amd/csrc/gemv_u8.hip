@@ -551,8 +551,8 @@ const char* gemm_u8_plan(int m, int p, int n, int block_size) {
   switch (choose_u8(nullptr, nullptr, nullptr, m, p, n, block_size)) {
     case U8_DOT: return "gemv_u8_dot2_stream";
     case U8_GEMV:
-      return n < 8192 ? "gemv_u8_mfma16_stream"
-                      : p == 16 * MACRO_K ? "gemv_u8_mfma16_wide_dma" : "gemv_u8_mfma16_wide";
+      if (p == 16 * MACRO_K) return n < 8192 ? "gemv_u8_mfma16_dma" : "gemv_u8_mfma16_wide_dma";
+      return n < 8192 ? "gemv_u8_mfma16_stream" : "gemv_u8_mfma16_wide";
     case U8_GEMM: return "gemm_nt_u8_mfma";
     default: return "gemm_u8_naive";
   }
@@ -589,6 +589,11 @@ hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, co
         else
           hipLaunchKernelGGL((gemv_u8_wide_kernel<8, 3, false>), dim3((n + 3 * ROWS - 1) / (3 * ROWS)),
                              dim3(512), 0, stream, out, lhs, rhs, scales, m, p, n, beta);
+        return hipGetLastError();
+      }
+      if (steps == 16) {
+        hipLaunchKernelGGL((gemv_u8_ring_kernel<8, 1, 2>), dim3(blocks), dim3(512), 0, stream, out,
+                           lhs, rhs, scales, m, p, n, beta);
         return hipGetLastError();
       }
       if (steps >= 16 && blocks <= 1024)

@@ -172,7 +172,7 @@ def _u8_case(g, m, p, n, bs, exact):
 
 
 @pytest.mark.parametrize("m", [1, 2, 4, 7, 16])
-@pytest.mark.parametrize("pn", [(256, 16), (512, 100), (1024, 33), (2816, 48)])
+@pytest.mark.parametrize("pn", [(256, 16), (512, 100), (1024, 33), (2816, 48), (4096, 52)])
 def test_gemv_bit_exact_on_exact_inputs(kern, m, pn):
     p, n = pn
     g = rng(610 + m + n)
@@ -297,7 +297,7 @@ def test_decode_shapes_full_size(kern, kn, m):
     s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
     a = torch.randn(m, p, generator=gen, device="cuda").half()
     assert u8_plan(m, p, n, 32) in ("gemv_u8_mfma16_stream", "gemv_u8_mfma16_wide",
-                                    "gemv_u8_mfma16_wide_dma", "gemv_u8_dot2_stream")
+                                    "gemv_u8_mfma16_wide_dma", "gemv_u8_mfma16_dma", "gemv_u8_dot2_stream")
     out = torch.zeros(m, n, dtype=torch.float16, device="cuda")
     kern.matmul_nt_fp16u8(out, a, q, s, 32)
     w = torch.zeros(n, p, dtype=torch.float16, device="cuda")
