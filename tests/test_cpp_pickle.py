@@ -142,7 +142,9 @@ def test_rejects_what_the_reference_rejects(tmp_path):
 def test_checkpoint_to_u8_on_the_device(tmp_path):
     """zip/pickle -> [N, K] fp16 on the device -> adr_quantize_absmax_u8 -> (u8, scales), then
     dequantised again: every weight within half a quantisation step of the file's value, plus
-    the fp16 rounding of the dequantised number (at most 127.5 scales large: 127.5 * 2^-11 / 2)."""
+    the two fp16 roundings of the format: of the scale (absmax / scale may exceed 127.5 by
+    127.5 * 2^-11 before it is clamped) and of the dequantised number (half an fp16 step at up
+    to 127.5 scales: 127.5 * 2^-11 again)."""
     assert os.path.exists(build.HOST_TEST_BIN)
     g = torch.Generator().manual_seed(9)
     path = str(tmp_path / "layer.pth")
@@ -152,7 +154,7 @@ def test_checkpoint_to_u8_on_the_device(tmp_path):
     assert r.returncode == 0, r.stdout + r.stderr
     fields = r.stdout.split()
     assert fields[:4] == ["rows", "256", "cols", "1024"]
-    assert float(fields[-1]) <= 0.5 + 127.5 * 2.0 ** -12 + 1e-3
+    assert float(fields[-1]) <= 0.5 + 2 * 127.5 * 2.0 ** -11 + 1e-3
 
 
 def test_zip64_records(tmp_path):
