@@ -362,6 +362,123 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_ring_kernel(half_t* __restric
   }
 }
 
+// Other K (multiples of 256), sixteen weight rows per workgroup: the same private ring, walked
+// ROUNDS times.  Wavefront w owns macro steps w, w + NW, ...; every ring slot holds one macro step:
+// its 4 KiB weight tile in LDS and its activations and scales in registers.  A slot is refilled
+// right after it has been multiplied, and every refill issues the same 13 memory instructions
+// whether or not the wavefront has a macro step left (the surplus ones read one 16-byte line and
+// are multiplied with zero scales), so the wait before a slot's use is "all but the 13 (RING - 1)
+// youngest" and no load sits under a branch.
+template <int NW, int RING, int ROUNDS>
+__global__ __launch_bounds__(NW * 64) void gemv_u8_ring_loop_kernel(half_t* __restrict__ out,
+                                                                    const half_t* __restrict__ lhs,
+                                                                    const uint8_t* __restrict__ rhs,
+                                                                    const half_t* __restrict__ scales,
+                                                                    int m, int p, int n, float beta) {
+  constexpr int TILE = ROWS * MACRO_K;
+  constexpr int PER = 8 + 1 + 4;  // activation loads, scale load, DMA instructions per slot
+  __shared__ __attribute__((aligned(1024))) unsigned char ring[NW * RING * TILE];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * ROWS;
+  const int nblk = p / 32;
+  const bool xvalid = r < m;
+  const int steps = p / MACRO_K;
+  const half_t* xrow = lhs + (int64_t)min(r, m - 1) * p + g * 16;
+  const half_t* srow = scales + (int64_t)min(n0 + r, n - 1) * nblk;
+  unsigned char* const mine = ring + wave * RING * TILE;
+  // DMA instruction i of a tile fills its chunks [64 i, 64 i + 64): rows 4i .. 4i+3
+  const uint8_t* wsrc[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) {
+    const int row = 4 * i + (lane >> 4), kc = (lane & 15) ^ row;
+    wsrc[i] = rhs + (int64_t)min(n0 + row, n - 1) * p + kc * 16;
+  }
+  int roff[4];  // fragment read j of the lane: logical chunk 4j + g of row r
+#pragma unroll
+  for (int j = 0; j < 4; j++) roff[j] = r * 256 + (((4 * j + g) ^ r) << 4);
+
+  u32x4_t x[RING][8];
+  u32x4_t sc[RING];
+  auto issue = [&](int slot, int ms) {
+    const bool live = ms < steps;  // wave-uniform
+    const int64_t koff = live ? (int64_t)ms * MACRO_K : 0;
+    const half_t* xp = xrow + koff;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      // lanes beyond m read row m-1 again (the same addresses as its own lanes) and are zeroed
+      // when used: a load under a lane mask would be waited for where the lanes rejoin
+      x[slot][2 * j] = *(const u32x4_t*)(xp + j * 64);
+      x[slot][2 * j + 1] = *(const u32x4_t*)(xp + j * 64 + 8);
+    }
+    sc[slot] = *(const u32x4_t*)(srow + (live ? ms * (MACRO_K / 32) : 0));
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      // a surplus slot fetches one 16-byte line (all lanes the same address)
+      const uint8_t* src = live ? wsrc[i] + koff : rhs;
+      __builtin_amdgcn_global_load_lds(ADR_GLB_PTR(src),
+                                       ADR_LDS_PTR(mine + slot * TILE + i * 1024), 16, 0, 0);
+    }
+  };
+  float4_t acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
+#pragma unroll
+  for (int i = 0; i < RING; i++) issue(i, wave + i * NW);
+  // ROUNDS = ceil(ceil(steps / NW) / RING), the same for every wavefront; unrolled, because the
+  // compiler drains all loads at the head of a run-time loop that carries loads in registers
+#pragma unroll
+  for (int rd = 0; rd < ROUNDS; rd++) {
+#pragma unroll
+    for (int i = 0; i < RING; i++) {
+      // slots issued after this one: RING - 1, fewer at the very end
+      const int later = PER * (rd + 1 < ROUNDS ? RING - 1 : RING - 1 - i);
+      static_assert(RING == 3, "the three wait immediates below");
+      if (later == 2 * PER) __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * PER) & 0xF) | (((2 * PER) >> 4) << 14));
+      else if (later == PER) __builtin_amdgcn_s_waitcnt(0x0F70 | (PER & 0xF) | ((PER >> 4) << 14));
+      else __builtin_amdgcn_s_waitcnt(0x0F70);
+      const unsigned char* tile = mine + i * TILE;
+      u32x4_t w[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++) w[j] = *(const u32x4_t*)(tile + roff[j]);
+      // zero scales for a surplus slot: it adds nothing (selected here, not where the scales
+      // are loaded: a use right behind the load would wait for it and everything before it)
+      const u32x4_t z = {0, 0, 0, 0};
+      const bool live = wave + (rd * RING + i) * NW < steps;
+      const half8_t s8 = __builtin_bit_cast(half8_t, live ? sc[i] : z);
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const half_t sv = g < 2 ? s8[2 * j] : s8[2 * j + 1];
+        const half2_t s2 = {sv, sv};
+        const half8_t a0 = dequant8(w[j][0], w[j][1], s2), a1 = dequant8(w[j][2], w[j][3], s2);
+        const half8_t b0 = __builtin_bit_cast(half8_t, xvalid ? x[i][2 * j] : z);
+        const half8_t b1 = __builtin_bit_cast(half8_t, xvalid ? x[i][2 * j + 1] : z);
+        acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, b0, acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, b1, acc1, 0, 0, 0);
+      }
+      // the slot's tile and registers have been consumed: refill it
+      __builtin_amdgcn_sched_barrier(0);
+      if (rd + 1 < ROUNDS) issue(i, wave + ((rd + 1) * RING + i) * NW);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
+  __syncthreads();
+  float* partial = (float*)ring;  // [NW][256]
+#pragma unroll
+  for (int i = 0; i < 4; i++) partial[wave * 256 + (4 * g + i) * 16 + r] = acc0[i] + acc1[i];
+  __syncthreads();
+  for (int e = tid; e < ROWS * 16; e += NW * 64) {
+    const int mm = e / ROWS, nn = e % ROWS;  // consecutive threads -> consecutive output columns
+    if (mm < m && n0 + nn < n) {
+      float sum = 0.0f;
+#pragma unroll
+      for (int w2 = 0; w2 < NW; w2++) sum += partial[w2 * 256 + nn * 16 + mm];
+      half_t* o = out + (int64_t)mm * n + n0 + nn;
+      // the previous output is read even for beta == 0, as the reference does
+      *o = (half_t)(sum + beta * (float)*o);
+    }
+  }
+}
+
 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
 
 template <int CTRL, int ROWMASK>
@@ -552,6 +669,7 @@ const char* gemm_u8_plan(int m, int p, int n, int block_size) {
     case U8_DOT: return "gemv_u8_dot2_stream";
     case U8_GEMV:
       if (p == 16 * MACRO_K) return n < 8192 ? "gemv_u8_mfma16_dma" : "gemv_u8_mfma16_wide_dma";
+      if (n < 8192 && p > 16 * MACRO_K && p <= 72 * MACRO_K) return "gemv_u8_mfma16_dma";
       return n < 8192 ? "gemv_u8_mfma16_stream" : "gemv_u8_mfma16_wide";
     case U8_GEMM: return "gemm_nt_u8_mfma";
     default: return "gemm_u8_naive";
@@ -595,6 +713,19 @@ hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, co
         hipLaunchKernelGGL((gemv_u8_ring_kernel<8, 1, 2>), dim3(blocks), dim3(512), 0, stream, out,
                            lhs, rhs, scales, m, p, n, beta);
         return hipGetLastError();
+      }
+      if (steps > 16) {
+        const int rounds = ((steps + 7) / 8 + 2) / 3;
+        if (rounds == 1)
+          hipLaunchKernelGGL((gemv_u8_ring_loop_kernel<8, 3, 1>), dim3(blocks), dim3(512), 0, stream,
+                             out, lhs, rhs, scales, m, p, n, beta);
+        else if (rounds == 2)
+          hipLaunchKernelGGL((gemv_u8_ring_loop_kernel<8, 3, 2>), dim3(blocks), dim3(512), 0, stream,
+                             out, lhs, rhs, scales, m, p, n, beta);
+        else if (rounds == 3)
+          hipLaunchKernelGGL((gemv_u8_ring_loop_kernel<8, 3, 3>), dim3(blocks), dim3(512), 0, stream,
+                             out, lhs, rhs, scales, m, p, n, beta);
+        if (rounds <= 3) return hipGetLastError();
       }
       if (steps >= 16 && blocks <= 1024)
         hipLaunchKernelGGL(gemv_u8_kernel<8>, dim3(blocks), dim3(512), 0, stream, out, lhs, rhs,

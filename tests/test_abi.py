@@ -76,7 +76,7 @@ def test_u8_plan():
         assert plan(m, 11008, 4096, 32) == (0, "gemv_u8_dot2_stream")
     for m in (4, 16):
         assert plan(m, 4096, 4096, 32) == (0, "gemv_u8_mfma16_dma")
-        assert plan(m, 11008, 4096, 32) == (0, "gemv_u8_mfma16_stream")
+        assert plan(m, 11008, 4096, 32) == (0, "gemv_u8_mfma16_dma")
     assert plan(2, 4096, 12288, 32) == (0, "gemv_u8_dot2_stream")
     assert plan(4, 4096, 12288, 32) == (0, "gemv_u8_mfma16_wide_dma")
     assert plan(4, 2048, 12288, 32) == (0, "gemv_u8_mfma16_wide")

@@ -172,7 +172,8 @@ def _u8_case(g, m, p, n, bs, exact):
 
 
 @pytest.mark.parametrize("m", [1, 2, 4, 7, 16])
-@pytest.mark.parametrize("pn", [(256, 16), (512, 100), (1024, 33), (2816, 48), (4096, 52)])
+@pytest.mark.parametrize("pn", [(256, 16), (512, 100), (1024, 33), (2816, 48), (4096, 52),
+                                (5120, 40), (11008, 24)])
 def test_gemv_bit_exact_on_exact_inputs(kern, m, pn):
     p, n = pn
     g = rng(610 + m + n)
