@@ -10,7 +10,7 @@ Prints ONE JSON line.  `value` is the fp16 TFLOP/s of that step; `roofline` is t
 kernel (the MFMA GEMM on the QKV shape) timed with HIP events on the launch stream;
 `cpu_baseline` is the CPU oracle (a scalar restatement of the reference kernel, OpenMP over
 rows) on a bounded sample of the same workload, timed on this machine's host cores;
-`secondary` carries the other BASELINE configurations: the u8 decode GEMV in GB/s against
+`secondary` carries the other benchmark configurations: the u8 decode GEMV in GB/s against
 the HBM peak, the u8 prefill GEMMs, the CLIP GEMMs and the attention products.
 
 Input data is synthetic (seeded): activations ~ N(0,1), weights ~ N(0,1/sqrt(K)) in fp16;
@@ -54,7 +54,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures the single-GPU matmul path only; run with --gpus 1 "
-              "(how the path would shard over several GPUs is described in DESIGN.md)",
+              "(every GPU box of this build has one GPU; no collectives are part of it)",
               file=sys.stderr)
         sys.exit(2)
 
@@ -123,7 +123,7 @@ def main():
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) * 1e-3 / (replays * calls_per_graph)
 
-    # ---- u8 decode GEMV (BASELINE configs[2]): weight buffers rotate through > 256 MB so
+    # ---- u8 decode GEMV (benchmark configs[2]): weight buffers rotate through > 256 MB so
     # that repeats stream from HBM, not from the Infinity Cache
     def u8_case(m, K, N, iters):
         per = N * K + N * (K // 32) * 2
@@ -369,7 +369,7 @@ def main():
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "data": "synthetic",
-        "config": {"workload": "llama7b_layer_gemm_set_fp16_prefill_M2048 (BASELINE configs[4], "
+        "config": {"workload": "llama7b_layer_gemm_set_fp16_prefill_M2048 (configs[4] of the benchmark definition, "
                                "fp16 weights: qkv, o, gate, up, down)",
                    "gflop_per_step": round(step_flops / 1e9, 1),
                    "frac_mfma_peak": round(value / PEAK_F16_TFLOPS, 4)},

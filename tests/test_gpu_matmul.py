@@ -138,7 +138,7 @@ def test_reference_tiled_kernel_agrees_with_its_naive_kernel(ref):
 
 SHAPES = [
     # (B, M, K, N): tails in every dimension, every tile configuration
-    (1, 77, 768, 2304),     # BASELINE config 1 (CLIP text QKV)
+    (1, 77, 768, 2304),     # benchmark config 1 (CLIP text QKV)
     (1, 64, 64, 64),
     (1, 1, 8, 1),
     (1, 33, 72, 130),
@@ -419,7 +419,7 @@ def test_gpukernels_interface_and_errors():
     assert np.all(to_np(o_t) == 0)
 
 
-# ------------------------------------------------------------------ BASELINE sizes: properties
+# ------------------------------------------------------------------ benchmark sizes: properties
 
 FULL = [
     # name, B, M, K, N  (fp16 NT weights)
@@ -434,7 +434,7 @@ FULL = [
 
 @pytest.mark.parametrize("case", FULL, ids=[c[0] for c in FULL])
 def test_full_size_gemm_against_fp32_gemm_and_slow_kernel(case):
-    """At BASELINE sizes: max relative error <= 1e-2 against an fp32 GEMM of the same fp16
+    """At benchmark sizes: max relative error <= 1e-2 against an fp32 GEMM of the same fp16
     inputs (torch, on the device, as the independent fp32 reference), and agreement with the
     step-for-step slow kernel on a band of rows."""
     _, B, M, K, N = case
@@ -457,7 +457,7 @@ def test_full_size_gemm_against_fp32_gemm_and_slow_kernel(case):
 
 
 def test_full_size_attention_products():
-    """BASELINE config 4: 32 heads, head_dim 128, seq 2048.  QK^T scaled by 1/sqrt(128) with the
+    """benchmark config 4: 32 heads, head_dim 128, seq 2048.  QK^T scaled by 1/sqrt(128) with the
     causal mask; P.V with softmaxed scores.  Checked per head against an fp32 batched GEMM."""
     S, H, D = 2048, 32, 128
     HD = H * D

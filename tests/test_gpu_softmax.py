@@ -79,7 +79,7 @@ def test_softmax_closed_forms_and_errors(kern):
 
 
 def test_softmax_full_size_attention_scores(kern):
-    """BASELINE config 4 size: [32, 2048, 2048] causal scores in place; rows sum to 1, masked
+    """benchmark config 4 size: [32, 2048, 2048] causal scores in place; rows sum to 1, masked
     entries are 0, and a band of rows equals the oracle."""
     H, S = 32, 2048
     gen = torch.Generator(device="cuda").manual_seed(46)

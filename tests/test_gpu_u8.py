@@ -290,7 +290,7 @@ DECODE = [(4096, 4096), (4096, 11008), (4096, 12288), (11008, 4096)]
 @pytest.mark.parametrize("kn", DECODE, ids=[f"K{k}_N{n}" for k, n in DECODE])
 @pytest.mark.parametrize("m", [1, 4, 16])
 def test_decode_shapes_full_size(kern, kn, m):
-    """BASELINE config 3 at full size against an fp32 GEMM on the (bit-exactly) dequantised
+    """benchmark config 3 at full size against an fp32 GEMM on the (bit-exactly) dequantised
     weights, computed on the device."""
     p, n = kn
     gen = torch.Generator(device="cuda").manual_seed(44)
@@ -314,7 +314,7 @@ def test_decode_shapes_full_size(kern, kn, m):
 
 
 def test_prefill_u8_gemm_full_size(kern):
-    """BASELINE config 5 (u8 variant), the O projection: M=2048, K=4096, N=4096."""
+    """benchmark config 5 (u8 variant), the O projection: M=2048, K=4096, N=4096."""
     m, p, n = 2048, 4096, 4096
     gen = torch.Generator(device="cuda").manual_seed(45)
     q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)
