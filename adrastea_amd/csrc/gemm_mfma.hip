@@ -161,6 +161,103 @@ __device__ __forceinline__ void store_chunk(const MatmulArgs& a, const Epilogue&
 // column block j: lane l holds output row l % 32 and, in element r, column
 // 8*(r/4) + 4*(l/32) + r%4.  (y0, x0) is the origin of the wavefront's sub-tile; `slot` is an
 // LDS region private to this wavefront of at least 32 * (TN*64 + 16) bytes.
+// The straight-line epilogue applies: the sub-tile's columns lie inside the matrix (rows may run
+// past the last one: those are read from the last row and not stored), it is on or below the
+// diagonal of a causal product, rows are 16-byte aligned.
+template <int TM, int TN>
+__device__ __forceinline__ bool epilogue_is_straight(const MatmulArgs& a, const half_t* out, int y0,
+                                                     int x0) {
+  const bool inside = y0 < a.m && x0 + TN * 32 <= a.n;
+  const bool unmasked = a.mask != ADR_MASK_CAUSAL || x0 + TN * 32 - 1 <= y0;
+  return inside && unmasked && out_vectorizable(a, out);
+}
+
+// The straight-line epilogue for ONE store operator (OP is a compile-time constant: every
+// operator gets its own compact instruction stream; with the operator switch inside the chunk
+// loop the code of all of them, exp and tanh included, sat between any two stores, and the
+// operators that are not Identity paid for it in instruction fetch).
+template <int TM, int TN, uint32_t OP>
+__device__ __forceinline__ void straight_epilogue(const MatmulArgs& a, half_t* out,
+                                                  float16_t (&acc)[TM][TN], int y0, int x0,
+                                                  unsigned char* slot, half_t hscale, int lane) {
+  constexpr bool plain_op = OP == ADR_STORE_IDENTITY || OP == ADR_STORE_SCALE;
+  constexpr bool np = OP == ADR_STORE_ADD || OP == ADR_STORE_BETA_BIAS ||
+                      OP == ADR_STORE_BETA_GELU_BIAS || OP == STORE_ACC_BETA;
+  constexpr bool nb = OP == ADR_STORE_BETA_BIAS || OP == ADR_STORE_BETA_GELU_BIAS ||
+                      OP == ADR_STORE_QUICK_GELU_BIAS;
+  const Epilogue ep{a.bias, a.beta, hscale, OP};
+  const int lrow = lane & 31, g = lane >> 5;
+  constexpr int PITCH = TN * 64 + 16;  // bytes per staged row (TN*32 halves + pad)
+  constexpr int CPW = TN * 4;          // 16-byte chunks per staged row
+  const half_t mul = OP == ADR_STORE_SCALE ? hscale : (half_t)1.0f;
+  // store round `it` of a 32-row block: lane -> 16-byte chunk it*64 + lane of the staged block
+  int rd[TN * 2], srow[TN * 2], scol[TN * 2];
+#pragma unroll
+  for (int it = 0; it < TN * 2; it++) {
+    const int idx = it * 64 + lane, row = idx / CPW, c = idx % CPW;
+    rd[it] = row * PITCH + c * 16;
+    srow[it] = row;
+    scol[it] = c * 8;
+  }
+  half8_t bias[TN * 2];
+  if (nb) {
+#pragma unroll
+    for (int it = 0; it < TN * 2; it++) bias[it] = *(const half8_t*)(a.bias + x0 + scol[it]);
+  }
+  half_t* const p0 = out + (int64_t)y0 * a.stride_oy + x0;
+  const int last = a.m - y0 - 1;  // last row of the matrix, relative to the sub-tile
+  // rows past the matrix are clamped for loads (so that no load sits under a lane mask) and
+  // skipped for stores
+  auto at = [&](int i, int it) {
+    return p0 + (int64_t)min(i * 32 + srow[it], last) * a.stride_oy + scol[it];
+  };
+  // all of the sub-tile's previous output in one burst: with one workgroup per compute unit
+  // nothing else hides this latency
+  half8_t prev[TM][TN * 2];
+  if (np) {
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int it = 0; it < TN * 2; it++) prev[i][it] = *(const half8_t*)at(i, it);
+  }
+#pragma unroll
+  for (int i = 0; i < TM; i++) {
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        half4_t h;
+#pragma unroll
+        for (int e = 0; e < 4; e++) h[e] = (half_t)acc[i][j][4 * q + e];
+        // x * 1 is exact, so one multiply serves Identity and Scale (matmul.cu Scale: fp16
+        // product); the other operators take the narrowed sum as it is
+        *(half4_t*)(slot + lrow * PITCH + (j * 32 + 8 * q + 4 * g) * 2) = plain_op ? h * mul : h;
+      }
+#pragma unroll
+    for (int it = 0; it < TN * 2; it++) {
+      half8_t v = *(const half8_t*)(slot + rd[it]);
+      if (OP == ADR_STORE_ADD) {
+        v = v + prev[i][it];
+      } else if (OP == STORE_ACC_BETA) {
+        // beta == 0 on this path: acc + 0 * prev.  Non-finite garbage in the output poisons the
+        // result exactly as in the reference; a finite one leaves the accumulator.
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+          const float t = 0.0f * (float)prev[i][it][e];
+          v[e] = (t == t) ? v[e] : (half_t)t;
+        }
+      } else if (!plain_op) {
+#pragma unroll
+        for (int e = 0; e < 8; e++)
+          v[e] = ep.apply_s16(v[e], np ? prev[i][it][e] : (half_t)0, bias[it][e]);
+      }
+      // streaming store: the output is not read again by this launch and should not evict
+      // operand panels from L2
+      if (i * 32 + srow[it] <= last) __builtin_nontemporal_store(v, (half8_t*)at(i, it));
+    }
+  }
+}
+
 template <int TM, int TN>
 __device__ __forceinline__ void wave_epilogue(const MatmulArgs& a, half_t* out,
                                               float16_t (&acc)[TM][TN], int y0, int x0,
@@ -169,45 +266,25 @@ __device__ __forceinline__ void wave_epilogue(const MatmulArgs& a, half_t* out,
   const int lrow = lane & 31, g = lane >> 5;
   constexpr int PITCH = TN * 64 + 16;  // bytes per staged row (TN*32 halves + pad)
   constexpr int CPW = TN * 4;          // 16-byte chunks per staged row
-  // Common case, straight-line: the sub-tile lies inside the matrix and (for a causal product)
-  // on or below the diagonal, the operator is Identity or Scale, rows are 16-byte aligned.
-  const bool plain_op = a.store == ADR_STORE_IDENTITY || a.store == ADR_STORE_SCALE;
-  const bool inside = y0 + TM * 32 <= a.m && x0 + TN * 32 <= a.n;
-  const bool unmasked = a.mask != ADR_MASK_CAUSAL || x0 + TN * 32 - 1 <= y0;
-  if (plain_op && inside && unmasked && !(a.stride_oy & 7) && !((uintptr_t)out & 15)) {
-    const half_t mul = a.store == ADR_STORE_SCALE ? hscale : (half_t)1.0f;
-    // store round `it` of a 32-row block: lane -> 16-byte chunk it*64 + lane of the staged block
-    int rd[TN * 2];
-    int64_t po[TN * 2];
-#pragma unroll
-    for (int it = 0; it < TN * 2; it++) {
-      const int idx = it * 64 + lane, row = idx / CPW, c = idx % CPW;
-      rd[it] = row * PITCH + c * 16;
-      po[it] = (int64_t)row * a.stride_oy + c * 8;
+  // Common case, straight-line: the sub-tile's columns lie inside the matrix, it is (for a
+  // causal product) on or below the diagonal, rows are 16-byte aligned.
+  if (epilogue_is_straight<TM, TN>(a, out, y0, x0)) {
+    switch (a.store) {
+      case ADR_STORE_SCALE:
+        return straight_epilogue<TM, TN, ADR_STORE_SCALE>(a, out, acc, y0, x0, slot, hscale, lane);
+      case ADR_STORE_ADD:
+        return straight_epilogue<TM, TN, ADR_STORE_ADD>(a, out, acc, y0, x0, slot, hscale, lane);
+      case ADR_STORE_BETA_BIAS:
+        return straight_epilogue<TM, TN, ADR_STORE_BETA_BIAS>(a, out, acc, y0, x0, slot, hscale, lane);
+      case ADR_STORE_QUICK_GELU_BIAS:
+        return straight_epilogue<TM, TN, ADR_STORE_QUICK_GELU_BIAS>(a, out, acc, y0, x0, slot, hscale, lane);
+      case ADR_STORE_BETA_GELU_BIAS:
+        return straight_epilogue<TM, TN, ADR_STORE_BETA_GELU_BIAS>(a, out, acc, y0, x0, slot, hscale, lane);
+      case STORE_ACC_BETA:
+        return straight_epilogue<TM, TN, STORE_ACC_BETA>(a, out, acc, y0, x0, slot, hscale, lane);
+      default:
+        return straight_epilogue<TM, TN, ADR_STORE_IDENTITY>(a, out, acc, y0, x0, slot, hscale, lane);
     }
-    half_t* const p0 = out + (int64_t)y0 * a.stride_oy + x0;
-    const int64_t blk = (int64_t)32 * a.stride_oy;
-#pragma unroll
-    for (int i = 0; i < TM; i++) {
-#pragma unroll
-      for (int j = 0; j < TN; j++)
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-          half4_t h;
-#pragma unroll
-          for (int e = 0; e < 4; e++) h[e] = (half_t)acc[i][j][4 * q + e];
-          // x * 1 is exact, so one multiply serves both operators (matmul.cu Scale: fp16 product)
-          *(half4_t*)(slot + lrow * PITCH + (j * 32 + 8 * q + 4 * g) * 2) = h * mul;
-        }
-#pragma unroll
-      for (int it = 0; it < TN * 2; it++) {
-        const half8_t v = *(const half8_t*)(slot + rd[it]);
-        // streaming store: the output is not read again by this launch and should not evict
-        // operand panels from L2
-        __builtin_nontemporal_store(v, (half8_t*)(p0 + i * blk + po[it]));
-      }
-    }
-    return;
   }
   if (out_vectorizable(a, out)) {
 #pragma unroll
