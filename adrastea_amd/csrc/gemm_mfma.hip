@@ -375,16 +375,16 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "MFMA 32x32x16 tiling");
   static_assert((NW / 2) * SLOT <= BM * BK * 2, "epilogue slots must fit in two A stages");
   static_assert(NSTAGE == 2 || NSTAGE == 3 || NSTAGE == 5,
-                "2 or 3 LDS stages, or 5: three stages of the left and two of the right operand");
+                "2 or 3 LDS stages, or 5: two stages of the left and three of the right operand");
   static_assert(!NN || BN == 128, "the N-contiguous right operand is staged as [64][128] tiles");
   // Separate objects per stage: the compiler's alias analysis then knows that the asynchronous
   // LDS writes of one stage cannot touch the stage being read, and does not serialise them.
   __shared__ __attribute__((aligned(1024))) unsigned char sA0[BM * BK * 2];
   __shared__ __attribute__((aligned(1024))) unsigned char sA1[BM * BK * 2];
-  __shared__ __attribute__((aligned(1024))) unsigned char sA2[NSTAGE > 2 ? BM * BK * 2 : 1024];
+  __shared__ __attribute__((aligned(1024))) unsigned char sA2[NSTAGE == 3 ? BM * BK * 2 : 1024];
   __shared__ __attribute__((aligned(1024))) unsigned char sB0[BN * BK * 2];
   __shared__ __attribute__((aligned(1024))) unsigned char sB1[BN * BK * 2];
-  __shared__ __attribute__((aligned(1024))) unsigned char sB2[NSTAGE == 3 ? BN * BK * 2 : 1024];
+  __shared__ __attribute__((aligned(1024))) unsigned char sB2[NSTAGE >= 3 ? BN * BK * 2 : 1024];
 
   int batch, tile_m, tile_n;
   map_tile(map, batch, tile_m, tile_n);
@@ -552,16 +552,16 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   };
 
   if (NSTAGE == 5) {
-    // Three stages of the left and two of the right operand (what fits beside a 256 x 192
-    // tile): slice kt reads A stage kt % 3 and B stage kt % 2; at its head the DMA of B(kt+1)
-    // and then of A(kt+2) is issued, spread one instruction per MFMA over the first k-steps,
-    // and at its end everything but A(kt+2) has to have landed.  The DMA engine of the CU
-    // (about 45 bytes per clock) then never idles between the barrier and the next burst.
+    // Two stages of the left and three of the right operand: slice kt reads A stage kt % 2 and
+    // B stage kt % 3; at its head the DMA of A(kt+1) and then of B(kt+2) is issued, and at its
+    // end everything but B(kt+2) has to have landed.  The right operand (weights that no cache
+    // holds between launches of a model) gets two slices to arrive, the left one (activations
+    // just written, resident in L2) one.
     int kA = 0, kB = 0;
     auto slice5 = [&](const unsigned char* cA, const unsigned char* cB, const unsigned char* nA,
                       const unsigned char* nB, unsigned char* dA, unsigned char* dB) {
-      dmaB(min(kB++, KT - 1), dB);
       dmaA(min(kA++, KT - 1), dA);
+      dmaB(min(kB++, KT - 1), dB);
 #pragma unroll
       for (int kk = 0; kk < KK; kk++) {
         if (kk + 1 < KK) {
@@ -577,29 +577,29 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
           mfmas(kk & 1);
         }
       }
-      wait_dma_barrier(std::integral_constant<int, IA>{});
+      wait_dma_barrier(std::integral_constant<int, IB>{});
       load_frags(0, nA, nB, 0);
       __builtin_amdgcn_sched_barrier(0);
     };
-    dmaA(min(kA++, KT - 1), sA0);
     dmaB(min(kB++, KT - 1), sB0);
-    dmaA(min(kA++, KT - 1), sA1);
-    wait_dma_barrier(std::integral_constant<int, IA>{});
+    dmaA(min(kA++, KT - 1), sA0);
+    dmaB(min(kB++, KT - 1), sB1);
+    wait_dma_barrier(std::integral_constant<int, IB>{});
     load_frags(0, sA0, sB0, 0);
     int kt = 0;
     for (; kt + 6 <= KT; kt += 6) {
-      slice5(sA0, sB0, sA1, sB1, sA2, sB1);
-      slice5(sA1, sB1, sA2, sB0, sA0, sB0);
-      slice5(sA2, sB0, sA0, sB1, sA1, sB1);
-      slice5(sA0, sB1, sA1, sB0, sA2, sB0);
-      slice5(sA1, sB0, sA2, sB1, sA0, sB1);
-      slice5(sA2, sB1, sA0, sB0, sA1, sB0);
+      slice5(sA0, sB0, sA1, sB1, sA1, sB2);
+      slice5(sA1, sB1, sA0, sB2, sA0, sB0);
+      slice5(sA0, sB2, sA1, sB0, sA1, sB1);
+      slice5(sA1, sB0, sA0, sB1, sA0, sB2);
+      slice5(sA0, sB1, sA1, sB2, sA1, sB0);
+      slice5(sA1, sB2, sA0, sB0, sA0, sB1);
     }
-    if (kt < KT) { slice5(sA0, sB0, sA1, sB1, sA2, sB1); kt++; }
-    if (kt < KT) { slice5(sA1, sB1, sA2, sB0, sA0, sB0); kt++; }
-    if (kt < KT) { slice5(sA2, sB0, sA0, sB1, sA1, sB1); kt++; }
-    if (kt < KT) { slice5(sA0, sB1, sA1, sB0, sA2, sB0); kt++; }
-    if (kt < KT) { slice5(sA1, sB0, sA2, sB1, sA0, sB1); kt++; }
+    if (kt < KT) { slice5(sA0, sB0, sA1, sB1, sA1, sB2); kt++; }
+    if (kt < KT) { slice5(sA1, sB1, sA0, sB2, sA0, sB0); kt++; }
+    if (kt < KT) { slice5(sA0, sB2, sA1, sB0, sA1, sB1); kt++; }
+    if (kt < KT) { slice5(sA1, sB0, sA0, sB1, sA0, sB2); kt++; }
+    if (kt < KT) { slice5(sA0, sB1, sA1, sB2, sA1, sB0); kt++; }
   } else if (NSTAGE == 3) {
     dma(sA0, sB0);
     dma(sA1, sB1);
@@ -1440,7 +1440,7 @@ hipError_t launch_mfma_gemm(hipStream_t stream, const MatmulArgs& a) {
     case SHORTK_128: return launch_shortk<16>(stream, a);
     case U8_256x192: return launch_u8<256, 192, 4, 2>(stream, a);
     case U8_256x128: return launch_u8<256, 128, 4, 2>(stream, a);
-    case DMA_256x192: return launch_dma<256, 192, 4, 2, 5, 1>(stream, a);
+        case DMA_256x192: return launch_dma<256, 192, 4, 2, 5, 1>(stream, a);
     case DMA_256x128: return launch_dma<256, 128, 4, 2, 3, 1>(stream, a);
     case DMA_128x128: return launch_dma<128, 128, 2, 2, 3, 1>(stream, a);
     case DMA_128x64: return launch_dma<128, 64, 2, 2, 3, 2>(stream, a);
