@@ -1440,7 +1440,7 @@ hipError_t launch_mfma_gemm(hipStream_t stream, const MatmulArgs& a) {
     case SHORTK_128: return launch_shortk<16>(stream, a);
     case U8_256x192: return launch_u8<256, 192, 4, 2>(stream, a);
     case U8_256x128: return launch_u8<256, 128, 4, 2>(stream, a);
-        case DMA_256x192: return launch_dma<256, 192, 4, 2, 5, 1>(stream, a);
+    case DMA_256x192: return launch_dma<256, 192, 4, 2, 5, 1>(stream, a);
     case DMA_256x128: return launch_dma<256, 128, 4, 2, 3, 1>(stream, a);
     case DMA_128x128: return launch_dma<128, 128, 2, 2, 3, 1>(stream, a);
     case DMA_128x64: return launch_dma<128, 64, 2, 2, 3, 2>(stream, a);

@@ -456,6 +456,23 @@ def test_full_size_gemm_against_fp32_gemm_and_slow_kernel(case):
     assert rel <= TOL, rel
 
 
+@pytest.mark.parametrize("K", [320, 384, 448, 512, 576, 640])
+def test_large_tile_kernel_every_k_tail_exact(K):
+    """The 256 x 192 kernel rotates two left and three right LDS stages with a period of six
+    slices: every remainder of that loop, on inputs whose fp32 sums are exact, must give the
+    correctly rounded product bit for bit (ragged last tile row and column included)."""
+    M, N = 2000, 12200
+    so, sl, sr = nt_strides(M, K, N)
+    assert plan(1, M, K, N, so, sl, sr) == "gemm_nt_mfma_dma_256x192x64"
+    gen = torch.Generator(device="cuda").manual_seed(K)
+    a = (torch.randint(-8, 9, (M, K), generator=gen, device="cuda").float() / 64).half()
+    w = (torch.randint(-8, 9, (N, K), generator=gen, device="cuda").float() / 64).half()
+    out = torch.full((M, N), 9.0, dtype=torch.float16, device="cuda")
+    assert raw_matmul("adr_matmul_f16", out, a, w, 1, M, K, N, so, sl, sr) == 0
+    want = (a.double() @ w.double().t()).half()
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+
+
 def test_full_size_attention_products():
     """benchmark config 4: 32 heads, head_dim 128, seq 2048.  QK^T scaled by 1/sqrt(128) with the
     causal mask; P.V with softmaxed scores.  Checked per head against an fp32 batched GEMM."""
