@@ -7,7 +7,7 @@
 // length % 128 elements do not enter the statistics while the means still divide by `length`;
 // that is kept.  Differences are formed in fp32 from the stored values, as there.
 // Bound by reading both tensors once: 16-byte loads on contiguous views, shuffle reductions,
-// one atomic triple per workgroup.
+// one atomic triple per workgroup of 1024 threads.
 #include "adr_common.hpp"
 
 namespace adr {
@@ -19,14 +19,20 @@ __device__ __forceinline__ void atomic_max_nonneg(float* addr, float v) {
   atomicMax((int*)addr, __builtin_bit_cast(int, v));
 }
 
+// Every workgroup ends in three atomics on the same three addresses, and the workgroups finish
+// together: the atomics queue up behind each other at the end of the launch (1024 workgroups:
+// 27 us of a 105 us launch).  Hence few, large workgroups -- one per CU, 16 wavefronts each.
+constexpr int ES_NT = 1024;
+constexpr int ES_MAX_BLOCKS = 256;
+
 template <typename T>
-__global__ __launch_bounds__(256) void error_stats_kernel(float* out, const T* lhs, const T* rhs,
+__global__ __launch_bounds__(ES_NT) void error_stats_kernel(float* out, const T* lhs, const T* rhs,
                                                           int64_t counted, int64_t length,
                                                           int64_t sl, int64_t sr, bool vec) {
   constexpr int VEC = 16 / sizeof(T);
   typedef T vec_t __attribute__((ext_vector_type(VEC)));
   float sum_sq = 0.0f, mx = 0.0f, sum = 0.0f;
-  const int64_t tid = (int64_t)blockIdx.x * 256 + threadIdx.x, nthreads = (int64_t)gridDim.x * 256;
+  const int64_t tid = (int64_t)blockIdx.x * ES_NT + threadIdx.x, nthreads = (int64_t)gridDim.x * ES_NT;
   auto take = [&](float a, float b) {
     const float d = a - b;
     sum_sq += d * d;
@@ -61,14 +67,18 @@ __global__ __launch_bounds__(256) void error_stats_kernel(float* out, const T* l
     mx = fmaxf(mx, __shfl_xor(mx, off, 64));
     sum += __shfl_xor(sum, off, 64);
   }
-  __shared__ float red[3][4];
+  constexpr int NW = ES_NT / 64;
+  __shared__ float red[3][NW];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   if (lane == 0) { red[0][wave] = sum_sq; red[1][wave] = mx; red[2][wave] = sum; }
   __syncthreads();
   if (threadIdx.x == 0) {
-    sum_sq = (red[0][0] + red[0][1]) + (red[0][2] + red[0][3]);
-    mx = fmaxf(fmaxf(red[1][0], red[1][1]), fmaxf(red[1][2], red[1][3]));
-    sum = (red[2][0] + red[2][1]) + (red[2][2] + red[2][3]);
+    sum_sq = 0.0f; mx = 0.0f; sum = 0.0f;
+    for (int w = 0; w < NW; w++) {
+      sum_sq += red[0][w];
+      mx = fmaxf(mx, red[1][w]);
+      sum += red[2][w];
+    }
     atomicAdd(out + 0, sum_sq / (float)length);  // error_stats.cu:59-61
     atomic_max_nonneg(out + 1, mx);
     atomicAdd(out + 2, sum / (float)length);
@@ -80,10 +90,10 @@ hipError_t launch_t(hipStream_t stream, float* out, const T* lhs, const T* rhs, 
                     int64_t sl, int64_t sr) {
   const int64_t counted = (length / 128) * 128;  // error_stats.cu:27-30: 128 blocks of length/128
   const bool vec = sl == 1 && sr == 1 && ((uintptr_t)lhs % 16) == 0 && ((uintptr_t)rhs % 16) == 0;
-  int64_t blocks = (counted / (16 / (int64_t)sizeof(T)) + 255) / 256;
-  if (blocks > 1024) blocks = 1024;  // every workgroup ends in three same-address atomics
+  int64_t blocks = (counted / (16 / (int64_t)sizeof(T)) + ES_NT - 1) / ES_NT;
+  if (blocks > ES_MAX_BLOCKS) blocks = ES_MAX_BLOCKS;
   if (blocks < 1) blocks = 1;
-  hipLaunchKernelGGL(error_stats_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, stream, out, lhs,
+  hipLaunchKernelGGL(error_stats_kernel<T>, dim3((unsigned)blocks), dim3(ES_NT), 0, stream, out, lhs,
                      rhs, counted, length, sl, sr, vec);
   return hipGetLastError();
 }
