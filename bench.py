@@ -214,6 +214,19 @@ def main():
         t = timed(f_es, 30, 3)
         attn["error_stats_f16"] = {"us": round(t * 1e6, 1), "gbs": round(sm_bytes / t / 1e9, 1),
                                    "frac_hbm_peak": round(sm_bytes / t / 1e9 / PEAK_HBM_GBS, 4)}
+        # QK^T -> softmax_rows in place -> P.V back to back, as a model runs them: each launch
+        # then finds its input in HBM, not in the cache its own previous run left behind
+        def f_seq():
+            f_qk()
+            f_sm()
+            rc = lib.adr_matmul_f16(stream(), o_.data_ptr(), qk.data_ptr(), v_.data_ptr(), H, S, S,
+                                    D, 1, HD, D, 1, S, S * S, 1, HD, D, None, 0.0, 1.0, 0, 0, 0)
+            if rc != 0:
+                raise RuntimeError(_ffi.strerror(rc))
+        t = timed(f_seq, 30, 3)
+        seq_bytes = 2 * byts + sm_bytes
+        attn["qk_softmax_pv_sequence"] = {"us": round(t * 1e6, 1), "gbs": round(seq_bytes / t / 1e9, 1),
+                                          "frac_hbm_peak": round(seq_bytes / t / 1e9 / PEAK_HBM_GBS, 4)}
         # the three products and the softmax above as one launch (adr_attention_f16); the causal
         # form is what the LLaMA layer runs, and skips the masked half of the score tiles
         o_ = torch.zeros(S, HD, dtype=torch.float16, device=dev)
