@@ -74,6 +74,30 @@ def build_library(force: bool = False, extra_flags=()) -> str:
     return LIB
 
 
+# Code objects for an unmodified host of the reference: module name -> source.  Each exports the
+# device symbols that host looks up in its module of that name, with the same kernel arguments.
+LEGACY_DIR = os.path.join(LIBDIR, "legacy")
+LEGACY_MODULES = {"matmul.co": "legacy_matmul.hip", "error_stats.co": "legacy_error_stats.hip"}
+
+
+def build_legacy_modules(force: bool = False) -> list:
+    """hipcc --genco of the legacy-symbol code objects into lib/legacy/."""
+    os.makedirs(LEGACY_DIR, exist_ok=True)
+    outs = []
+    for name, src in LEGACY_MODULES.items():
+        out = os.path.join(LEGACY_DIR, name)
+        outs.append(out)
+        if (not force and os.path.exists(out)
+                and all(os.path.getmtime(f) <= os.path.getmtime(out) for f in _deps())):
+            continue
+        flags = [f for f in CXXFLAGS if f != "-fPIC"]
+        cmd = [HIPCC, "--genco", *flags, os.path.join(CSRC, src), "-o", out]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"hipcc --genco failed for {src}:\n{r.stdout}\n{r.stderr}")
+    return outs
+
+
 HOST_TEST_SRC = os.path.join(os.path.dirname(HERE), "tests", "cpp", "test_host.cpp")
 HOST_TEST_BIN = os.path.join(os.path.dirname(HERE), "tests", "cpp", "bin", "test_host")
 
@@ -96,4 +120,5 @@ def build_host_test(force: bool = False) -> str:
 
 if __name__ == "__main__":
     print(build_library(force="--force" in sys.argv))
+    print(build_legacy_modules(force="--force" in sys.argv))
     print(build_host_test(force="--force" in sys.argv))

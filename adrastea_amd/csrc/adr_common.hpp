@@ -96,6 +96,40 @@ struct Epilogue {
 
 __device__ __forceinline__ half_t neg_inf_half() { return bits_to_half(0xFC00u); }
 
+// One output element of the general strided/batched matmul, with the arithmetic of the
+// reference's naive kernel (adrastea_kernels/cpp/matmul.cu:195-222) step for step: operands
+// optionally scaled in fp16, the product formed in fp16, widened, and summed sequentially in
+// fp32; then the mask and the store operator.  The caller guarantees y < m, x < n.
+__device__ __forceinline__ void matmul_one_output(const MatmulArgs& a, int b, int y, int x) {
+  half_t* out = a.output + (int64_t)b * a.stride_oz + (int64_t)y * a.stride_oy +
+                (int64_t)x * a.stride_ox;
+  if (a.mask == ADR_MASK_CAUSAL && x > y) {  // matmul.cu:210-213
+    *out = neg_inf_half();
+    return;
+  }
+  const half_t* l = a.lhs + (int64_t)b * a.stride_lz + (int64_t)y * a.stride_ly;
+  const half_t* r = a.rhs + (int64_t)b * a.stride_rz + (int64_t)x * a.stride_rx;
+  const half_t hscale = (half_t)a.scale;
+  float sum = 0.0f;
+  if (a.load == ADR_LOAD_SCALE) {
+    for (int i = 0; i < a.k; i++) {
+      half_t lv = l[(int64_t)i * a.stride_lx] * hscale;
+      half_t rv = r[(int64_t)i * a.stride_ry] * hscale;
+      half_t p = lv * rv;
+      sum += (float)p;
+    }
+  } else {
+    for (int i = 0; i < a.k; i++) {
+      half_t p = l[(int64_t)i * a.stride_lx] * r[(int64_t)i * a.stride_ry];
+      sum += (float)p;
+    }
+  }
+  Epilogue ep{a.bias, a.beta, hscale, a.store};
+  half_t prev = Epilogue::needs_prev(a.store) ? *out : (half_t)0;
+  half_t bias_x = Epilogue::needs_bias(a.store) ? a.bias[x] : (half_t)0;
+  *out = ep.apply(sum, prev, bias_x);
+}
+
 // Four u8 weights (one dword) -> four fp16 values (q - 127.5) * s with ONE rounding each, the
 // reference's dequantisation (adrastea_kernels/cpp/quantize.cu:53-54) bit for bit:
 // 0x6000 | (q << 1) is the fp16 number 512 + q (the step at 512 is 0.5); subtracting 639.5

@@ -136,7 +136,7 @@ struct WStage {
   u32x4_t sc;    // the eight fp16 scales (block_size 32) of the macro step
 };
 
-template <int NW, int RG, bool UPFRONT>
+template <int NW, int RG>
 __global__ __launch_bounds__(NW * 64) void gemv_u8_wide_kernel(half_t* __restrict__ out,
                                                                const half_t* __restrict__ lhs,
                                                                const uint8_t* __restrict__ rhs,
@@ -190,34 +190,15 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_wide_kernel(half_t* __restric
     }
   };
 
-  if (UPFRONT) {
-    // exactly two macro steps per wavefront (K = 512 * NW): everything the wavefront reads is
-    // issued before the first multiply (the fence keeps the compiler from sinking the second
-    // step's loads below the first step's arithmetic, which would expose their latency again)
-    u32x4_t xa[8], xb[8];
-    WStage sa[RG], sb[RG];
-    load_x(xa, wave);
+  // all weight loads of a macro step are issued before its first use
+  for (int ms = wave; ms < steps; ms += NW) {
+    u32x4_t x[8];
+    WStage s[RG];
+    load_x(x, ms);
 #pragma unroll
-    for (int q = 0; q < RG; q++) load_w(sa[q], q, wave);
-    load_x(xb, wave + NW);
+    for (int q = 0; q < RG; q++) load_w(s[q], q, ms);
 #pragma unroll
-    for (int q = 0; q < RG; q++) load_w(sb[q], q, wave + NW);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int q = 0; q < RG; q++) compute(sa[q], xa, acc[q]);
-#pragma unroll
-    for (int q = 0; q < RG; q++) compute(sb[q], xb, acc[q]);
-  } else {
-    // all weight loads of a macro step are issued before its first use
-    for (int ms = wave; ms < steps; ms += NW) {
-      u32x4_t x[8];
-      WStage s[RG];
-      load_x(x, ms);
-#pragma unroll
-      for (int q = 0; q < RG; q++) load_w(s[q], q, ms);
-#pragma unroll
-      for (int q = 0; q < RG; q++) compute(s[q], x, acc[q]);
-    }
+    for (int q = 0; q < RG; q++) compute(s[q], x, acc[q]);
   }
 
 #pragma unroll
@@ -705,7 +686,7 @@ hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, co
           hipLaunchKernelGGL((gemv_u8_ring_kernel<8, 3, 3>), dim3((n + 3 * ROWS - 1) / (3 * ROWS)),
                              dim3(512), 0, stream, out, lhs, rhs, scales, m, p, n, beta);
         else
-          hipLaunchKernelGGL((gemv_u8_wide_kernel<8, 3, false>), dim3((n + 3 * ROWS - 1) / (3 * ROWS)),
+          hipLaunchKernelGGL((gemv_u8_wide_kernel<8, 3>), dim3((n + 3 * ROWS - 1) / (3 * ROWS)),
                              dim3(512), 0, stream, out, lhs, rhs, scales, m, p, n, beta);
         return hipGetLastError();
       }

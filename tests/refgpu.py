@@ -40,8 +40,11 @@ def desc2d(t):
 
 
 class RefKernels:
-    def __init__(self):
+    def __init__(self, directory=REF_DIR):
+        """`directory` holds the code objects: the reference's own by default; the package's
+        lib/legacy/ directory holds this build's modules with the same symbols and arguments."""
         import torch
+        self.dir = directory
         torch.cuda.init()
         torch.zeros(1, device="cuda")  # make sure the primary context exists
         self.hip = C.CDLL("libamdhip64.so")
@@ -57,7 +60,7 @@ class RefKernels:
         if key not in self.fns:
             if module not in self.mods:
                 m = C.c_void_p()
-                rc = self.hip.hipModuleLoad(C.byref(m), os.path.join(REF_DIR, module).encode())
+                rc = self.hip.hipModuleLoad(C.byref(m), os.path.join(self.dir, module).encode())
                 assert rc == 0, f"hipModuleLoad({module}) = {rc}"
                 self.mods[module] = m
             f = C.c_void_p()
@@ -88,6 +91,13 @@ class RefKernels:
         f = self._fn("matmul.co", b"matmul_f16")
         args = self._matmul_args(out_ptr, l_ptr, r_ptr, B, M, K, N, so, sl, sr, bias_ptr, beta,
                                  scale, store, load, mask)
+        self._launch(f, ((N + 15) // 16, (M + 15) // 16, B), (16, 16, 1), 0, args)
+
+    def matmul_f16_raw(self, out_ptr, l_ptr, r_ptr, B, M, K, N, so, sl, sr):
+        """The identity-operator form (matmul.cu:515-517), launched like the naive kernel."""
+        f = self._fn("matmul.co", b"matmul_f16_raw")
+        args = self._matmul_args(out_ptr, l_ptr, r_ptr, B, M, K, N, so, sl, sr, None, 0.0, 1.0,
+                                 0, 0, 0)[:16]
         self._launch(f, ((N + 15) // 16, (M + 15) // 16, B), (16, 16, 1), 0, args)
 
     def matmul_f16_fast(self, out_ptr, l_ptr, r_ptr, B, M, K, N, so, sl, sr, bias_ptr=None,
