@@ -6,7 +6,7 @@
 //
 // The problem is bound by streaming the u8 weights from HBM once.  Two kernels:
 //
-//  gemv_u8_dot_kernel (m <= 4)   no matrix cores.  A wavefront streams whole 1 KiB segments of
+//  gemv_u8_dot_kernel (m <= 2)   no matrix cores.  A wavefront streams whole 1 KiB segments of
 //      one weight row per load instruction (lane l: 16 bytes at l*16, perfectly coalesced),
 //      keeps its activation slices in registers for all rows of the workgroup, and evaluates
 //        sum_k x_k (q_k - 127.5) s  =  s * ( sum_k x_k (1024 + q_k)  -  1151.5 * sum_k x_k )
@@ -665,8 +665,7 @@ hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, co
       if (p <= 4096) {  // 4 wavefronts, one segment each
         if (m == 1) return wide ? launch_dot<1, 4, 4, 1>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta)
                                 : launch_dot<1, 4, 2, 1>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
-        if (m == 2) return launch_dot<2, 4, 4, 1>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
-        return launch_dot<4, 4, 4, 1>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
+        return launch_dot<2, 4, 4, 1>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
       }
       // up to 12 segments: 4 wavefronts, three segments each (K = 11008 has 11: one idle slot
       // instead of five with 8 x 2)
