@@ -1350,7 +1350,7 @@ struct Candidate {
 // Estimated cost: the tiles of the busiest CU times the work of one tile over the efficiency of
 // a CU running this tile shape.  (With few long tiles the transfer rate into one CU's LDS, not
 // the matrix pipe, bounds a tile: spreading the same work over all CUs with smaller tiles wins.)
-GemmChoice pick(const MatmulArgs& a, const Candidate* c, int n) {
+GemmChoice pick(const MatmulArgs& a, const Candidate* c, int n, double* cost_out = nullptr) {
   GemmChoice best = GEMM_NONE;
   double best_cost = 0;
   for (int i = 0; i < n; i++) {
@@ -1363,8 +1363,14 @@ GemmChoice pick(const MatmulArgs& a, const Candidate* c, int n) {
       best_cost = cost;
     }
   }
+  if (cost_out) *cost_out = best_cost;
   return best;
 }
+
+const Candidate DMA_TILES[] = {
+    {DMA_256x192, 256, 192, 1, 1.10f}, {DMA_256x128, 256, 128, 1, 1.00f},
+    {DMA_128x128, 128, 128, 2, 0.80f}, {DMA_128x64, 128, 64, 2, 0.60f},
+    {DMA_64x64, 64, 64, 4, 0.40f}};
 
 // The MFMA family needs 16-byte aligned, K-contiguous rows on both operands.
 GemmChoice choose(const MatmulArgs& a) {
@@ -1395,11 +1401,7 @@ GemmChoice choose(const MatmulArgs& a) {
                                          {DMA_64x64, 64, 64, 4, 0.50f}};
       return pick(a, shortk, 2);
     }
-    static const Candidate dma[] = {
-        {DMA_256x192, 256, 192, 1, 1.10f}, {DMA_256x128, 256, 128, 1, 1.00f},
-        {DMA_128x128, 128, 128, 2, 0.80f}, {DMA_128x64, 128, 64, 2, 0.60f},
-        {DMA_64x64, 64, 64, 4, 0.40f}};
-    return pick(a, dma, 5);
+    return pick(a, DMA_TILES, 5);
   }
   if (a.rhs_q && a.k % 64 == 0 && a.block_size >= 8 && (a.block_size & (a.block_size - 1)) == 0 &&
       (int64_t)a.m * a.n >= 256 * 1024) {
@@ -1414,8 +1416,8 @@ GemmChoice choose(const MatmulArgs& a) {
 
 }  // namespace
 
-bool mfma_gemm_supported(const MatmulArgs& a, const char** name) {
-  switch (choose(a)) {
+static bool choice_name(GemmChoice c, const char** name) {
+  switch (c) {
     case SHORTK_64: *name = "gemm_nt_mfma_persistent_128x128_k64"; return true;
     case SHORTK_128: *name = "gemm_nt_mfma_persistent_128x128_k128"; return true;
     case U8_256x192: *name = "gemm_nt_u8_mfma_256x192x64"; return true;
@@ -1434,8 +1436,8 @@ bool mfma_gemm_supported(const MatmulArgs& a, const char** name) {
   }
 }
 
-hipError_t launch_mfma_gemm(hipStream_t stream, const MatmulArgs& a) {
-  switch (choose(a)) {
+static hipError_t launch_choice(hipStream_t stream, const MatmulArgs& a, GemmChoice c) {
+  switch (c) {
     case SHORTK_64: return launch_shortk<8>(stream, a);
     case SHORTK_128: return launch_shortk<16>(stream, a);
     case U8_256x192: return launch_u8<256, 192, 4, 2>(stream, a);
@@ -1452,6 +1454,53 @@ hipError_t launch_mfma_gemm(hipStream_t stream, const MatmulArgs& a) {
     case STAGE_64x64: return launch_stage<64, 64, 64, 2, 2, 2>(stream, a);
     default: return hipErrorInvalidValue;
   }
+}
+
+// A few rows past a multiple of the tile height (M = 2056 = 8 x 257 image tokens) would add a
+// whole row of tiles that do almost no useful work and break an otherwise even split over the
+// CUs (2048 x 4096 is exactly one 256 x 128 tile per CU).  Such products are issued as two
+// launches: the rows up to the last multiple of 128, and the remaining rows as a small problem
+// of their own.  Rows are independent in every store operator; the causal mask compares absolute
+// row numbers and is therefore left alone.
+static bool split_m_tail(const MatmulArgs& a, MatmulArgs& head, MatmulArgs& tail) {
+  const int t = a.m % 128;
+  if (a.mask != ADR_MASK_NONE || a.rhs_q || a.m < 1024 || t == 0 || t > 32) return false;
+  head = a;
+  head.m = a.m - t;
+  tail = a;
+  tail.m = t;
+  // (the plan query passes no pointers)
+  tail.lhs = a.lhs ? a.lhs + (int64_t)head.m * a.stride_ly : nullptr;
+  tail.output = a.output ? a.output + (int64_t)head.m * a.stride_oy : nullptr;
+  const GemmChoice ca = choose(a), ch = choose(head), ct = choose(tail);
+  auto dma_tile = [](GemmChoice c) {
+    return c == DMA_256x192 || c == DMA_256x128 || c == DMA_128x128 || c == DMA_128x64 ||
+           c == DMA_64x64;
+  };
+  if (!dma_tile(ca) || !dma_tile(ch) || !dma_tile(ct)) return false;
+  // pick()'s cost (tile area on the busiest CU over efficiency) times K is proportional to the
+  // time of a launch; one more launch is priced at 3 us (2.9e6 of those units per us, measured)
+  double whole, first, rest;
+  pick(a, DMA_TILES, 5, &whole);
+  pick(head, DMA_TILES, 5, &first);
+  pick(tail, DMA_TILES, 5, &rest);
+  return (first + rest) * a.k + 8.7e6 < whole * a.k;
+}
+
+bool mfma_gemm_supported(const MatmulArgs& a, const char** name) {
+  MatmulArgs head, tail;
+  if (split_m_tail(a, head, tail)) return choice_name(choose(head), name);
+  return choice_name(choose(a), name);
+}
+
+hipError_t launch_mfma_gemm(hipStream_t stream, const MatmulArgs& a) {
+  MatmulArgs head, tail;
+  if (split_m_tail(a, head, tail)) {
+    const hipError_t e = launch_choice(stream, head, choose(head));
+    if (e != hipSuccess) return e;
+    return launch_choice(stream, tail, choose(tail));
+  }
+  return launch_choice(stream, a, choose(a));
 }
 
 hipError_t launch_gemm_u8_mfma(hipStream_t stream, half_t* out, const half_t* lhs,

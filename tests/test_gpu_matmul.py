@@ -429,6 +429,7 @@ FULL = [
     ("llama_o", 1, 2048, 4096, 4096),
     ("llama_gate", 1, 2048, 4096, 11008),
     ("llama_down", 1, 2048, 11008, 4096),
+    ("llama_qkv_2056_rows", 1, 2056, 4096, 12288),  # issued as 2048 rows + 8 rows
 ]
 
 
@@ -471,6 +472,33 @@ def test_large_tile_kernel_every_k_tail_exact(K):
     assert raw_matmul("adr_matmul_f16", out, a, w, 1, M, K, N, so, sl, sr) == 0
     want = (a.double() @ w.double().t()).half()
     assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+
+
+def test_row_tail_split_keeps_operator_semantics():
+    """A product a few rows past a multiple of 128 goes out as two launches (2048 + 8 rows here);
+    the second one must see its own rows of the previous output and the shared bias."""
+    M, K, N = 2056, 4096, 12288
+    so, sl, sr = nt_strides(M, K, N)
+    gen = torch.Generator(device="cuda").manual_seed(7)
+    a = torch.randn(M, K, generator=gen, device="cuda").half()
+    w = (torch.randn(N, K, generator=gen, device="cuda") * K ** -0.5).half()
+    prev = torch.randn(M, N, generator=gen, device="cuda").half()
+    bias = torch.randn(N, generator=gen, device="cuda").half()
+    out = prev.clone()
+    assert raw_matmul("adr_matmul_f16", out, a, w, 1, M, K, N, so, sl, sr, bias_t=bias, beta=0.5,
+                      store=oracle.STORE_BETA_BIAS) == 0
+    acc16 = (a.float() @ w.float().t()).half().float()
+    want = acc16 + bias.float()[None, :] + 0.5 * prev.float()
+    rms = want.pow(2).mean().sqrt()
+    rel = ((out.float() - want).abs() / torch.maximum(want.abs(), rms)).max().item()
+    assert rel <= TOL, rel
+    # the eight tail rows against the step-for-step kernel on the same rows
+    slow = prev[M - 8:].clone()
+    assert raw_matmul("adr_matmul_f16_slow", slow, a[M - 8:], w, 1, 8, K, N, so, sl, sr,
+                      bias_t=bias, beta=0.5, store=oracle.STORE_BETA_BIAS) == 0
+    rel = ((out[M - 8:].float() - slow.float()).abs() /
+           torch.maximum(slow.float().abs(), rms)).max().item()
+    assert rel <= TOL, rel
 
 
 def test_full_size_attention_products():
