@@ -13,6 +13,7 @@ SYMBOLS = (
     "adr_matmul_nt_fp16u8", "adr_dequantize_absmax_u8", "adr_quantize_absmax_u8",
     "adr_dequantize_absmax_uint8", "adr_quantize_absmax_uint8", "adr_matmul_f16_plan",
     "adr_matmul_nt_fp16u8_plan", "adr_softmax_rows", "adr_error_stats_f16", "adr_error_stats_f32", "adr_attention_f16", "adr_embed_uint8",
+    "adr_microbench_empty", "adr_microbench_mfma_f16", "adr_microbench_stream_read",
     "adr_strerror", "adr_abi_version",
 )
 
@@ -59,6 +60,9 @@ def lib():
     L.adr_matmul_f16_plan.argtypes = [C.c_char_p, i32] + [i32] * 13 + [u32, u32, u32]
     L.adr_matmul_nt_fp16u8_plan.argtypes = [C.c_char_p, i32, i32, i32, i32, i32]
     L.adr_softmax_rows.argtypes = [vp, vp, vp, i32, i32, i32, f32]
+    L.adr_microbench_empty.argtypes = [vp]
+    L.adr_microbench_mfma_f16.argtypes = [vp, i32, i32, i32, vp]
+    L.adr_microbench_stream_read.argtypes = [vp, vp, C.c_int64, i32, vp]
     L.adr_error_stats_f16.argtypes = [vp, TensorDesc, TensorDesc, TensorDesc]
     L.adr_error_stats_f32.argtypes = [vp, TensorDesc, TensorDesc, TensorDesc]
     L.adr_attention_f16.argtypes = [vp, vp, vp, vp, vp] + [i32] * 16 + [f32, f32, u32]

@@ -173,6 +173,10 @@ hipError_t launch_quantize(hipStream_t stream, adr_tensor_desc out, adr_tensor_d
 hipError_t launch_embed_u8(hipStream_t stream, int n_dim, int n_ids, const int16_t* in_ids,
                            half_t* out, const uint8_t* table, const half_t* scales,
                            int block_size);
+hipError_t launch_microbench_empty(hipStream_t stream);
+hipError_t launch_microbench_mfma(hipStream_t stream, int blocks, int times, int pattern, float* sink);
+hipError_t launch_microbench_read(hipStream_t stream, const void* p, int64_t bytes, int blocks,
+                                  uint32_t* sink);
 hipError_t launch_error_stats(hipStream_t stream, float* out, const void* lhs, const void* rhs,
                               int64_t length, int64_t sl, int64_t sr, bool f32);
 hipError_t launch_attention(hipStream_t stream, half_t* out, const half_t* q, const half_t* k,

@@ -276,6 +276,25 @@ static int error_stats_common(adr_stream_t stream, adr_tensor_desc output, adr_t
                                  lhs.shape[0], lhs.strides[0], rhs.strides[0], f32);
 }
 
+int adr_microbench_empty(adr_stream_t stream) {
+  return (int)launch_microbench_empty((hipStream_t)stream);
+}
+
+int adr_microbench_mfma_f16(adr_stream_t stream, int blocks, int times, int pattern, float* sink) {
+  if (blocks <= 0 || times < 0 || (pattern != 0 && pattern != 1)) return ADR_EINVAL_SHAPE;
+  if (!sink) return ADR_ENULL;
+  return (int)launch_microbench_mfma((hipStream_t)stream, blocks, times, pattern, sink);
+}
+
+int adr_microbench_stream_read(adr_stream_t stream, const void* src, int64_t bytes, int blocks,
+                               uint32_t* sink) {
+  if (blocks <= 0 || bytes < 0 || bytes % (16 * (int64_t)blocks) != 0) return ADR_EINVAL_SHAPE;
+  if (bytes == 0) return ADR_OK;
+  if (!src || !sink) return ADR_ENULL;
+  if ((uintptr_t)src % 16 != 0) return ADR_EINVAL_SHAPE;
+  return (int)launch_microbench_read((hipStream_t)stream, src, bytes, blocks, sink);
+}
+
 int adr_error_stats_f16(adr_stream_t stream, adr_tensor_desc output, adr_tensor_desc lhs,
                         adr_tensor_desc rhs) {
   return error_stats_common(stream, output, lhs, rhs, false);

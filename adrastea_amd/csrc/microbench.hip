@@ -1,0 +1,85 @@
+// Device kernels of the microbenchmark (the counterparts of adrastea_kernels/cpp/microbench.cu:28-51,
+// driven like adrastea/src/main.rs:486-553): an empty kernel for the launch overhead, a loop
+// of matrix-core instructions on register operands for the issue peak of this part, and a plain
+// streaming read for the memory peak one launch can reach.  Measurement aids only: nothing in
+// the product calls them.
+#include "adr_common.hpp"
+
+namespace adr {
+
+namespace {
+
+__global__ void empty_kernel(int) {}
+
+// Every wavefront issues `times` x 4 independent v_mfma_f32_32x32x16_f16 (four accumulators keep
+// the pipe full without waiting for a result).  pattern 0: all-zero operands (the instruction
+// rate alone); pattern 1: pseudo-random fp16 operands in [-1, 1) (what the part sustains when
+// the multipliers toggle -- the power limit shows here).
+__global__ __launch_bounds__(256) void mfma_loop_kernel(int times, int pattern, float* sink) {
+  const uint32_t id = blockIdx.x * 256 + threadIdx.x;
+  half8_t a, b;
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    uint32_t h = (id * 8 + e) * 2654435761u;
+    h ^= h >> 15; h *= 2246822519u; h ^= h >> 13;
+    // sign, exponent 14 (values in [0.5, 1)) and ten mantissa bits
+    a[e] = pattern ? bits_to_half((uint16_t)((h & 0x83ffu) | 0x3800u)) : (half_t)0;
+    b[e] = pattern ? bits_to_half((uint16_t)(((h >> 16) & 0x83ffu) | 0x3800u)) : (half_t)0;
+  }
+  float16_t acc[4];
+#pragma unroll
+  for (int q = 0; q < 4; q++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[q][r] = 0.0f;
+  for (int i = 0; i < times; i++) {
+#pragma unroll
+    for (int q = 0; q < 4; q++) acc[q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, acc[q], 0, 0, 0);
+  }
+  float s = 0.0f;
+#pragma unroll
+  for (int q = 0; q < 4; q++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) s += acc[q][r];
+  sink[id] = s;
+}
+
+// Every workgroup reads one contiguous piece with 16-byte streaming loads (the access shape
+// that reads fastest on this part), four loads in flight per lane.
+__global__ __launch_bounds__(256) void stream_read_kernel(const u32x4_t* p, int64_t n16,
+                                                          uint32_t* sink) {
+  const int64_t piece = n16 / gridDim.x;
+  const u32x4_t* q = p + (int64_t)blockIdx.x * piece;
+  u32x4_t acc = {0, 0, 0, 0};
+  int64_t i = threadIdx.x;
+  for (; i + 3 * 256 < piece; i += 4 * 256) {
+    u32x4_t v[4];
+#pragma unroll
+    for (int u = 0; u < 4; u++) v[u] = __builtin_nontemporal_load(q + i + u * 256);
+#pragma unroll
+    for (int u = 0; u < 4; u++) acc ^= v[u];
+  }
+  for (; i < piece; i += 256) acc ^= q[i];
+  const uint32_t r = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
+  if (r == 0x9e3779b9u) sink[0] = r;  // keeps the loads alive; practically never taken
+}
+
+}  // namespace
+
+hipError_t launch_microbench_empty(hipStream_t stream) {
+  hipLaunchKernelGGL(empty_kernel, dim3(1), dim3(1), 0, stream, 0);
+  return hipGetLastError();
+}
+
+hipError_t launch_microbench_mfma(hipStream_t stream, int blocks, int times, int pattern, float* sink) {
+  hipLaunchKernelGGL(mfma_loop_kernel, dim3(blocks), dim3(256), 0, stream, times, pattern, sink);
+  return hipGetLastError();
+}
+
+hipError_t launch_microbench_read(hipStream_t stream, const void* p, int64_t bytes, int blocks,
+                                  uint32_t* sink) {
+  hipLaunchKernelGGL(stream_read_kernel, dim3(blocks), dim3(256), 0, stream, (const u32x4_t*)p,
+                     bytes / 16, sink);
+  return hipGetLastError();
+}
+
+}  // namespace adr

@@ -48,6 +48,9 @@ def main():
                     help="run only the u8 decode GEMV configurations (for profiling that kernel)")
     ap.add_argument("--attention-only", action="store_true",
                     help="run only the attention configuration (QK^T, softmax_rows, P.V, error_stats)")
+    ap.add_argument("--microbenchmark", action="store_true",
+                    help="launch overhead, matrix-core issue peak, streaming-read peak and the "
+                         "2048x4096x4096 products of the reference's microbenchmark()")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain 256 MiB device copy (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters of rocprofv3 --pmc)")
@@ -245,6 +248,75 @@ def main():
 
     if args.attention_only:
         print(json.dumps({"llama7b_attention_fp16": attention_set()}))
+        return
+
+    def microbenchmark():
+        """The list of adrastea/src/main.rs:486-650 (`microbenchmark()`), each entry run for about
+        a second like its bench() (main.rs:409-454): per-call wall time including the
+        synchronisation, reported as fastest / average / slowest rate."""
+        def run(name, ops, call, unit, seconds=1.0):
+            call()
+            torch.cuda.synchronize()
+            times = []
+            t_end = time.perf_counter() + seconds
+            while time.perf_counter() < t_end and len(times) < 100000:
+                t0 = time.perf_counter()
+                call()
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t0)
+            scale = 1e12 if unit == "TFLOP/s" else 1e9 if unit == "GB/s" else 1.0
+            row = {"name": name, "ops": ops, "unit": unit, "runs": len(times)}
+            if unit == "us":
+                row.update(fast=round(min(times) * 1e6, 2), avg=round(sum(times) / len(times) * 1e6, 2),
+                           slow=round(max(times) * 1e6, 2))
+            else:
+                row.update(fast=round(ops / min(times) / scale, 1),
+                           avg=round(ops * len(times) / sum(times) / scale, 1),
+                           slow=round(ops / max(times) / scale, 1))
+            return row
+
+        def ok(rc):
+            if rc != 0:
+                raise RuntimeError(_ffi.strerror(rc))
+        rows = [run("empty_kernel", 1, lambda: ok(lib.adr_microbench_empty(stream())), "us")]
+        blocks, times_ = 512, 20000   # two workgroups of four wavefronts per CU
+        sink = torch.zeros(blocks * 256, dtype=torch.float32, device=dev)
+        flop = blocks * 4 * times_ * 4 * 2 * 32 * 32 * 16
+        for pattern, nm in ((0, "mfma_loop_f32_f16 (zero operands)"), (1, "mfma_loop_f32_f16 (random operands)")):
+            rows.append(run(nm, flop, lambda: ok(lib.adr_microbench_mfma_f16(
+                stream(), blocks, times_, pattern, sink.data_ptr())), "TFLOP/s"))
+        nbytes = 1 << 30
+        src = torch.ones(nbytes, dtype=torch.uint8, device=dev)
+        sink32 = torch.zeros(1, dtype=torch.int32, device=dev)
+        rows.append(run("stream_read 1 GiB", nbytes, lambda: ok(lib.adr_microbench_stream_read(
+            stream(), src.data_ptr(), nbytes, 1024, sink32.data_ptr())), "GB/s"))
+        del src
+        # matmul_f16[_fast]_2048_4096_4096 with a row-major and a permuted right operand
+        M, K, N = 2048, 4096, 4096
+        left, out = randn_h(M, K), torch.zeros(M, N, dtype=torch.float16, device=dev)
+        right = randn_h(K, N, std=K ** -0.5)  # rrr: [K, N] as stored; rrc: the same memory as [N, K]^T
+        for fn_name, label in (("adr_matmul_f16_slow", "matmul_f16"), ("adr_matmul_f16", "matmul_f16_fast")):
+            fn = getattr(lib, fn_name)
+            for layout, (srx, sry) in (("rrr", (1, N)), ("rrc", (K, 1))):
+                rows.append(run(f"{label}_2048_4096_4096_{layout}", 2 * M * K * N, lambda: ok(fn(
+                    stream(), out.data_ptr(), left.data_ptr(), right.data_ptr(), 1, M, K, N, 1, N, 0,
+                    1, K, 0, srx, sry, 0, None, 0.0, 1.0, 0, 0, 0)), "TFLOP/s"))
+        # the library GEMM the reference compares itself with (rocBLAS hgemm there, main.rs:599-648;
+        # torch.matmul dispatches to hipBLASLt / rocBLAS here)
+        rt = right.t().contiguous()
+        rows.append(run("library_hgemm_2048_4096_4096 (torch.matmul)", 2 * M * K * N,
+                        lambda: torch.matmul(left, right), "TFLOP/s"))
+        rows.append(run("library_hgemm_2048_4096_4096_nt (torch.matmul)", 2 * M * K * N,
+                        lambda: torch.matmul(left, rt.t()), "TFLOP/s"))
+        return rows
+
+    if args.microbenchmark:
+        rows = microbenchmark()
+        print("%-48s %14s %12s %12s %12s" % ("name", "ops", "fast", "avg", "slow"), file=sys.stderr)
+        for r in rows:
+            print("%-48s %14d %12s %12s %12s  %s" % (r["name"], r["ops"], r["fast"], r["avg"], r["slow"],
+                                                     r["unit"]), file=sys.stderr)
+        print(json.dumps({"microbenchmark": rows}))
         return
 
     if args.decode_only:

@@ -228,6 +228,24 @@ int adr_matmul_f16_plan(char* name, int32_t cap, int32_t batches, int32_t m, int
 int adr_matmul_nt_fp16u8_plan(char* name, int32_t cap, int32_t m, int32_t p, int32_t n,
                               int32_t block_size);
 
+/*
+ * Microbenchmark aids (the device kernels of adrastea_kernels/cpp/microbench.cu:28-51 -- empty_kernel,
+ * wmma_loop_f32_f16 -- as adrastea/src/main.rs:486-553 drives them, plus a streaming read): the
+ * measured peaks that the fractions of the 2516.6 TFLOP/s and 8 TB/s figures are put beside.
+ *   adr_microbench_empty     one empty launch (launch overhead)
+ *   adr_microbench_mfma_f16  `blocks` workgroups of four wavefronts, each issuing times x 4
+ *                            v_mfma_f32_32x32x16_f16 on register operands: 2*32*32*16 flop each,
+ *                            i.e. blocks * 4 * times * 4 * 32768 flop per launch.  pattern 0:
+ *                            zero operands, 1: pseudo-random fp16 operands.  `sink` receives
+ *                            blocks * 256 floats.
+ *   adr_microbench_stream_read  reads `bytes` (a multiple of 16 * blocks) from `src` with
+ *                            `blocks` workgroups, one contiguous piece each; `sink`: 4 bytes.
+ */
+int adr_microbench_empty(adr_stream_t stream);
+int adr_microbench_mfma_f16(adr_stream_t stream, int blocks, int times, int pattern, float* sink);
+int adr_microbench_stream_read(adr_stream_t stream, const void* src, int64_t bytes, int blocks,
+                               uint32_t* sink);
+
 /* Human-readable text for an ADR_E* code or hipError_t. */
 const char* adr_strerror(int code);
 /* ABI version of this library (bumped on any signature change). */

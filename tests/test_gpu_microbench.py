@@ -1,0 +1,46 @@
+"""The microbenchmark entry points (counterparts of adrastea_kernels/cpp/microbench.cu): they are
+measurement aids, so the checks are about safety of the arguments and that the matrix-core loop
+really multiplies (twice the trips, twice the sums)."""
+import pytest
+import torch
+
+from adrastea_amd import _ffi
+
+pytestmark = pytest.mark.gpu
+
+
+def stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def test_empty_and_argument_checks():
+    L = _ffi.lib()
+    assert L.adr_microbench_empty(stream()) == 0
+    sink = torch.zeros(256, device="cuda")
+    assert L.adr_microbench_mfma_f16(stream(), 0, 1, 0, sink.data_ptr()) == _ffi.ADR_EINVAL_SHAPE
+    assert L.adr_microbench_mfma_f16(stream(), 1, 1, 2, sink.data_ptr()) == _ffi.ADR_EINVAL_SHAPE
+    assert L.adr_microbench_mfma_f16(stream(), 1, 1, 0, None) == _ffi.ADR_ENULL
+    buf = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
+    s32 = torch.zeros(1, dtype=torch.int32, device="cuda")
+    assert L.adr_microbench_stream_read(stream(), buf.data_ptr(), (1 << 20) + 8, 64,
+                                        s32.data_ptr()) == _ffi.ADR_EINVAL_SHAPE
+    assert L.adr_microbench_stream_read(stream(), buf.data_ptr(), 0, 64, s32.data_ptr()) == 0
+    assert L.adr_microbench_stream_read(stream(), buf.data_ptr(), 1 << 20, 64, s32.data_ptr()) == 0
+    torch.cuda.synchronize()
+    assert int(s32.item()) == 0
+
+
+def test_mfma_loop_multiplies():
+    L = _ffi.lib()
+    blocks = 3
+    one = torch.full((blocks * 256,), -1.0, device="cuda")
+    two = torch.full((blocks * 256,), -1.0, device="cuda")
+    zero = torch.full((blocks * 256,), -1.0, device="cuda")
+    assert L.adr_microbench_mfma_f16(stream(), blocks, 1, 1, one.data_ptr()) == 0
+    assert L.adr_microbench_mfma_f16(stream(), blocks, 2, 1, two.data_ptr()) == 0
+    assert L.adr_microbench_mfma_f16(stream(), blocks, 5, 0, zero.data_ptr()) == 0
+    torch.cuda.synchronize()
+    assert torch.all(zero == 0)
+    assert torch.isfinite(one).all() and (one != 0).any()
+    # (the matrix core adds the 16 products of a step to the accumulator in its own order)
+    assert torch.allclose(two, 2 * one, rtol=1e-4, atol=1e-3)
