@@ -1401,7 +1401,22 @@ GemmChoice choose(const MatmulArgs& a) {
                                          {DMA_64x64, 64, 64, 4, 0.50f}};
       return pick(a, shortk, 2);
     }
-    return pick(a, DMA_TILES, 5);
+    const GemmChoice c = pick(a, DMA_TILES, 5);
+    // Short K with one large tile on (nearly) every CU: every workgroup then runs its prologue,
+    // its few slices and its epilogue in step with all the others.  Twice as many tiles of half
+    // the size, two resident per CU, overlap those phases (measured over a sweep of forced
+    // tiles: up to 38 % faster for K <= 1024, e.g. M1024 K320 N8192 17.3 -> 12.6 us).
+    if (a.k <= 1024 && (c == DMA_256x192 || c == DMA_256x128 || c == DMA_128x128)) {
+      auto tiles = [&](int bm, int bn) {
+        return (int64_t)((a.m + bm - 1) / bm) * ((a.n + bn - 1) / bn) * a.batches;
+      };
+      const int64_t now = c == DMA_256x192 ? tiles(256, 192) : c == DMA_256x128 ? tiles(256, 128)
+                                                                                 : tiles(128, 128);
+      const bool to_64 = c == DMA_128x128;
+      const int64_t then = to_64 ? tiles(128, 64) : tiles(128, 128);
+      if (now >= 224 && now <= NUM_CU && then <= 2 * NUM_CU) return to_64 ? DMA_128x64 : DMA_128x128;
+    }
+    return c;
   }
   if (a.rhs_q && a.k % 64 == 0 && a.block_size >= 8 && (a.block_size & (a.block_size - 1)) == 0 &&
       (int64_t)a.m * a.n >= 256 * 1024) {
