@@ -185,7 +185,7 @@ __device__ __forceinline__ void straight_epilogue(const MatmulArgs& a, half_t* o
                       OP == ADR_STORE_BETA_GELU_BIAS || OP == STORE_ACC_BETA;
   constexpr bool nb = OP == ADR_STORE_BETA_BIAS || OP == ADR_STORE_BETA_GELU_BIAS ||
                       OP == ADR_STORE_QUICK_GELU_BIAS;
-  const Epilogue ep{a.bias, a.beta, hscale, OP};
+  const Epilogue ep{a.bias, a.beta, hscale, OP, true};
   const int lrow = lane & 31, g = lane >> 5;
   constexpr int PITCH = TN * 64 + 16;  // bytes per staged row (TN*32 halves + pad)
   constexpr int CPW = TN * 4;          // 16-byte chunks per staged row
@@ -262,7 +262,7 @@ template <int TM, int TN>
 __device__ __forceinline__ void wave_epilogue(const MatmulArgs& a, half_t* out,
                                               float16_t (&acc)[TM][TN], int y0, int x0,
                                               unsigned char* slot, half_t hscale, int lane) {
-  Epilogue ep{a.bias, a.beta, hscale, a.store};
+  Epilogue ep{a.bias, a.beta, hscale, a.store, true};
   const int lrow = lane & 31, g = lane >> 5;
   constexpr int PITCH = TN * 64 + 16;  // bytes per staged row (TN*32 halves + pad)
   constexpr int CPW = TN * 4;          // 16-byte chunks per staged row
@@ -766,7 +766,7 @@ __global__ __launch_bounds__(1024, 1) void gemm_nt_shortk_kernel(MatmulArgs a, S
     const int sw = wave - 4;                       // rows sw*16 .. +15 of a tile
     const int rrow = lane >> 4, rc = lane & 15;    // read round it: row it*4 + rrow, chunk rc
     const half_t hscale = (half_t)a.scale;
-    Epilogue ep{a.bias, a.beta, hscale, a.store};
+    Epilogue ep{a.bias, a.beta, hscale, a.store, true};
     const bool vec = out_vectorizable(a, a.output) && !(a.stride_oz & 7);
     const bool plain = vec && (a.store == ADR_STORE_IDENTITY || a.store == ADR_STORE_SCALE);
     const half_t mul = a.store == ADR_STORE_SCALE ? hscale : (half_t)1.0f;
