@@ -416,6 +416,26 @@ def main():
                         "tflops": round(2.0 * m * K * N / t / 1e12, 1),
                         "frac_mfma_peak": round(2.0 * m * K * N / t / 1e12 / PEAK_F16_TFLOPS, 4),
                         "gbs": round(byts / t / 1e9, 1)}
+        # the same two products with the store operators the CLIP MLP uses
+        # (adrastea_models/src/clip.rs:431-442: QuickGeluBias on the way up, BetaBias 1.0 = residual add
+        # on the way down); the operator runs in the kernel's epilogue
+        for nm, K, N, store, beta in (("vision_mlp_up_quick_gelu_bias", 1024, 4096, 6, 0.0),
+                                     ("vision_mlp_down_beta_bias", 4096, 1024, 3, 1.0)):
+            m = 2056
+            a, w = randn_h(m, K), randn_h(N, K, std=K ** -0.5)
+            bias = randn_h(N)
+            o = torch.zeros(m, N, dtype=torch.float16, device=dev)
+
+            def f_op():
+                rc = lib.adr_matmul_f16(stream(), o.data_ptr(), a.data_ptr(), w.data_ptr(), 1, m, K,
+                                        N, 1, N, 0, 1, K, 0, K, 1, 0, bias.data_ptr(), beta, 1.0,
+                                        store, 0, 0)
+                if rc != 0:
+                    raise RuntimeError(_ffi.strerror(rc))
+            t = timed(f_op, 50, 5)
+            clip[nm] = {"M": m, "K": K, "N": N, "us": round(t * 1e6, 2),
+                        "tflops": round(2.0 * m * K * N / t / 1e12, 1),
+                        "frac_mfma_peak": round(2.0 * m * K * N / t / 1e12 / PEAK_F16_TFLOPS, 4)}
         secondary["clip_fp16"] = clip
 
         attn = attention_set()
