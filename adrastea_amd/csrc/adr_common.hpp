@@ -175,11 +175,32 @@ __device__ __forceinline__ half8_t dequant8(uint32_t w0, uint32_t w1, half2_t s2
   return r;
 }
 
+typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+
+template <int CTRL, int ROWMASK>
+__device__ __forceinline__ float dpp_add(float v) {
+  int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROWMASK, 0xf, true);
+  return v + __builtin_bit_cast(float, t);
+}
+// Sum over the 64 lanes with data-parallel-primitive adds (no LDS); the total is in lane 63.
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+  v = dpp_add<0x111, 0xf>(v);  // row_shr:1
+  v = dpp_add<0x112, 0xf>(v);  // row_shr:2
+  v = dpp_add<0x114, 0xf>(v);  // row_shr:4
+  v = dpp_add<0x118, 0xf>(v);  // row_shr:8   lane 15 of each 16-lane row = row sum
+  v = dpp_add<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+  v = dpp_add<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
+  return v;
+}
+
 // Launchers implemented in the kernel translation units; all return a hipError_t.
 hipError_t launch_matmul_general(hipStream_t stream, const MatmulArgs& a);
 // Returns true and fills `name` when the MFMA kernel family covers these arguments.
 bool mfma_gemm_supported(const MatmulArgs& a, const char** name);
 hipError_t launch_mfma_gemm(hipStream_t stream, const MatmulArgs& a);
+// fp16 skinny matmul (m <= 8, K-contiguous operands): true when the streaming kernel covers it.
+bool gemv_f16_supported(const MatmulArgs& a);
+hipError_t launch_gemv_f16(hipStream_t stream, const MatmulArgs& a);
 
 hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, const uint8_t* rhs,
                           const half_t* scales, int m, int p, int n, int block_size, float beta);

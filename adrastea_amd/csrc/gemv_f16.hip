@@ -1,0 +1,139 @@
+// fp16 skinny matmul for decode, m <= 8 activation rows against a K-contiguous weight matrix:
+// the shape GpuKernels::matmul_f16 is called with once per generated token
+// (adrastea_models/src/llama.rs:485-591: W[N,K].permute([1,0]) on a [tokens, K] activation;
+// kernel arguments adrastea_models/src/kernels.rs:864-887).  The tiled kernels need tens of
+// microseconds for it -- a handful of 64 x 64 tiles walking K slice by slice -- while the job is
+// to read N x K x 2 bytes once.
+//
+// No matrix cores: a wavefront streams whole 1 KiB segments (512 k) of one weight row per load
+// instruction (lane l: 16 bytes at l * 16, streaming loads), keeps the activations of its
+// segments in registers for all rows of the workgroup, and accumulates with v_dot2_f32_f16
+// (exact fp16 products, fp32 sums); lane sums are reduced with DPP adds, the wavefronts of a
+// workgroup through LDS.  Every store operator and the causal mask are applied to the m x RPB
+// results of the workgroup.
+#include "adr_common.hpp"
+
+namespace adr {
+
+namespace {
+
+// MR activation rows, NW wavefronts, RPB weight rows per workgroup, SEGW segments per wavefront
+// (wavefront w owns segments w, w + NW, ...).
+template <int MR, int NW, int RPB, int SEGW>
+__global__ __launch_bounds__(NW * 64) void gemv_f16_dot_kernel(MatmulArgs a) {
+  __shared__ float partial[NW][RPB][MR];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n0 = blockIdx.x * RPB;
+  // All loads of the workgroup are issued up front and unconditionally (a load under a branch
+  // would be waited for at the join): segments past K and rows past m read a valid address and
+  // are zeroed afterwards.  K % 8 == 0, so a lane's eight values are all inside or all outside.
+  bool act[SEGW];
+  u32x4_t xraw[SEGW][MR];
+#pragma unroll
+  for (int j = 0; j < SEGW; j++) {
+    const int k = (wave + j * NW) * 512 + lane * 8;
+    act[j] = k < a.k;
+    const int kc = act[j] ? k : 0;
+#pragma unroll
+    for (int mm = 0; mm < MR; mm++)
+      xraw[j][mm] = *(const u32x4_t*)(a.lhs + (int64_t)min(mm, a.m - 1) * a.stride_ly + kc);
+  }
+  u32x4_t w[RPB][SEGW];
+#pragma unroll
+  for (int r = 0; r < RPB; r++) {
+    const half_t* wp = a.rhs + (int64_t)min(n0 + r, a.n - 1) * a.stride_rx;  // clamped, not stored
+#pragma unroll
+    for (int j = 0; j < SEGW; j++) {
+      const int k = (wave + j * NW) * 512 + lane * 8;
+      // streaming load: a weight is read once per launch
+      w[r][j] = __builtin_nontemporal_load((const u32x4_t*)(wp + (act[j] ? k : 0)));
+    }
+  }
+  u32x4_t x[SEGW][MR];
+#pragma unroll
+  for (int j = 0; j < SEGW; j++)
+#pragma unroll
+    for (int mm = 0; mm < MR; mm++)
+      x[j][mm] = (act[j] && mm < a.m) ? xraw[j][mm] : u32x4_t{0, 0, 0, 0};
+#pragma unroll
+  for (int r = 0; r < RPB; r++) {
+    float tot[MR];
+#pragma unroll
+    for (int mm = 0; mm < MR; mm++) tot[mm] = 0.0f;
+#pragma unroll
+    for (int j = 0; j < SEGW; j++)
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        // (through scalars: a bit_cast applied to a vector element directly reads element 0)
+        const uint32_t wv = w[r][j][e];
+        const h2_t w2 = __builtin_bit_cast(h2_t, wv);
+#pragma unroll
+        for (int mm = 0; mm < MR; mm++) {
+          const uint32_t xv = x[j][mm][e];
+          tot[mm] = __builtin_amdgcn_fdot2(w2, __builtin_bit_cast(h2_t, xv), tot[mm], false);
+        }
+      }
+#pragma unroll
+    for (int mm = 0; mm < MR; mm++) {
+      const float v = wave_sum_dpp(tot[mm]);
+      if (lane == 63) partial[wave][r][mm] = v;
+    }
+  }
+  __syncthreads();
+  const Epilogue ep{a.bias, a.beta, (half_t)a.scale, a.store, true};
+  for (int e = tid; e < RPB * MR; e += NW * 64) {
+    const int y = e / RPB, r = e % RPB, xcol = n0 + r;  // consecutive threads -> consecutive columns
+    if (y >= a.m || xcol >= a.n) continue;
+    half_t* o = a.output + (int64_t)y * a.stride_oy + (int64_t)xcol * a.stride_ox;
+    if (a.mask == ADR_MASK_CAUSAL && xcol > y) {  // matmul.cu:210-213
+      *o = neg_inf_half();
+      continue;
+    }
+    float sum = 0.0f;
+#pragma unroll
+    for (int w2 = 0; w2 < NW; w2++) sum += partial[w2][r][y];
+    const half_t prev = Epilogue::needs_prev(a.store) ? *o : (half_t)0;
+    const half_t bias_x = Epilogue::needs_bias(a.store) ? a.bias[xcol] : (half_t)0;
+    *o = ep.apply(sum, prev, bias_x);
+  }
+}
+
+template <int MR, int NW, int RPB, int SEGW>
+hipError_t launch(hipStream_t stream, const MatmulArgs& a) {
+  hipLaunchKernelGGL((gemv_f16_dot_kernel<MR, NW, RPB, SEGW>), dim3((a.n + RPB - 1) / RPB),
+                     dim3(NW * 64), 0, stream, a);
+  return hipGetLastError();
+}
+
+// rows of activations the instantiation for m rows is built for
+int rows_class(int m) { return m <= 1 ? 1 : m <= 2 ? 2 : m <= 4 ? 4 : 8; }
+
+}  // namespace
+
+bool gemv_f16_supported(const MatmulArgs& a) {
+  if (a.rhs_q || a.load != ADR_LOAD_IDENTITY || a.batches != 1) return false;
+  // from nine rows on the dot products cost more than the tiled kernels' slower loads
+  // (sixteen rows: 46 us against 31 us for K4096 N11008)
+  if (a.m < 1 || a.m > 8 || a.k % 8 != 0 || a.k < 512) return false;
+  if (a.stride_lx != 1 || a.stride_ry != 1) return false;
+  if ((a.stride_ly | a.stride_rx) & 7) return false;
+  if (a.lhs && (((uintptr_t)a.lhs | (uintptr_t)a.rhs) & 15)) return false;
+  // worth it where the weight matrix is the traffic: at least 1 MiB of it
+  if ((int64_t)a.n * a.k < (1 << 19)) return false;
+  const int nseg = (a.k + 511) / 512;
+  // segments the instantiations hold: 4 wavefronts x 2 or 8 x 3
+  return nseg <= 24;
+}
+
+hipError_t launch_gemv_f16(hipStream_t stream, const MatmulArgs& a) {
+  const int nseg = (a.k + 511) / 512;
+  const bool small = nseg <= 8;
+  switch (rows_class(a.m)) {
+    case 1: return small ? launch<1, 4, 4, 2>(stream, a) : launch<1, 8, 4, 3>(stream, a);
+    case 2: return small ? launch<2, 4, 4, 2>(stream, a) : launch<2, 8, 4, 3>(stream, a);
+    case 4: return small ? launch<4, 4, 4, 2>(stream, a) : launch<4, 8, 4, 3>(stream, a);
+    default: return small ? launch<8, 4, 2, 2>(stream, a) : launch<8, 8, 2, 3>(stream, a);
+  }
+}
+
+}  // namespace adr

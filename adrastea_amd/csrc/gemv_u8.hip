@@ -460,24 +460,6 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_ring_loop_kernel(half_t* __re
   }
 }
 
-typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
-
-template <int CTRL, int ROWMASK>
-__device__ __forceinline__ float dpp_add(float v) {
-  int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROWMASK, 0xf, true);
-  return v + __builtin_bit_cast(float, t);
-}
-// Sum over the 64 lanes with data-parallel-primitive adds (no LDS); the total is in lane 63.
-__device__ __forceinline__ float wave_sum_dpp(float v) {
-  v = dpp_add<0x111, 0xf>(v);  // row_shr:1
-  v = dpp_add<0x112, 0xf>(v);  // row_shr:2
-  v = dpp_add<0x114, 0xf>(v);  // row_shr:4
-  v = dpp_add<0x118, 0xf>(v);  // row_shr:8   lane 15 of each 16-lane row = row sum
-  v = dpp_add<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
-  v = dpp_add<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3
-  return v;
-}
-
 // MR activation rows, NW wavefronts, RPB weight rows per workgroup, SEGW 1 KiB K segments per
 // wavefront (wavefront w owns segments w, w+NW, ...).
 template <int MR, int NW, int RPB, int SEGW>

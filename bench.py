@@ -149,6 +149,31 @@ def main():
         t = timed_graph(f, 2 * nbuf, max(2, iters // (2 * nbuf)))
         return t, per + m * K * 2 + m * N * 2
 
+    # ---- the same decode shapes with fp16 weights: the call the reference's LLaMA makes once per
+    # generated token (matmul_f16 on a [tokens, K] activation, llama.rs:485-591)
+    def f16_decode_set():
+        rows = []
+        for K, N in DECODE_SET:
+            per = N * K * 2
+            nbuf = max(2, int(600e6 // per) + 1)
+            ws = [randn_h(N, K, std=K ** -0.5) for _ in range(nbuf)]
+            for m in (1, 4, 8):
+                a = randn_h(m, K)
+                o = torch.zeros(m, N, dtype=torch.float16, device=dev)
+                i = [0]
+
+                def f():
+                    j = i[0] % nbuf
+                    i[0] += 1
+                    mm(o, a, ws[j], m, K, N)
+                t = timed_graph(f, 2 * nbuf, max(2, 200 // (2 * nbuf)))
+                byts = per + m * K * 2 + m * N * 2
+                rows.append({"M": m, "K": K, "N": N, "us": round(t * 1e6, 2),
+                             "gbs": round(byts / t / 1e9, 1),
+                             "frac_hbm_peak": round(byts / t / 1e9 / PEAK_HBM_GBS, 4)})
+            del ws
+        return rows
+
     def decode_set():
         gemv = []
         for K, N in DECODE_SET:
@@ -320,7 +345,7 @@ def main():
         return
 
     if args.decode_only:
-        print(json.dumps({"u8_decode_gemv": decode_set()}))
+        print(json.dumps({"u8_decode_gemv": decode_set(), "f16_decode_gemv": f16_decode_set()}))
         return
 
     # ---------------- primary workload: the fp16 layer GEMM set at M = 2048
@@ -380,6 +405,8 @@ def main():
         best = max(gemv, key=lambda r: r["gbs"])
         secondary["u8_decode_gemv_best"] = {"gbs": best["gbs"], "frac_hbm_peak": best["frac_hbm_peak"],
                                             "shape": [best["M"], best["K"], best["N"]]}
+
+        secondary["f16_decode_gemv"] = f16_decode_set()
 
         # ---- u8 prefill GEMMs (configs[4], u8 half)
         u8p = {}
