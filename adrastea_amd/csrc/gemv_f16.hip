@@ -128,11 +128,16 @@ bool gemv_f16_supported(const MatmulArgs& a) {
 hipError_t launch_gemv_f16(hipStream_t stream, const MatmulArgs& a) {
   const int nseg = (a.k + 511) / 512;
   const bool small = nseg <= 8;
+  // Weight rows per workgroup: every workgroup fetches the activations of all m rows again
+  // (from L2), so with eight rows a workgroup has to cover more weight rows to keep that
+  // traffic below the weights' own (m=8, K4096 N12288: 32.3 us with two rows, 25.0 with eight).
   switch (rows_class(a.m)) {
     case 1: return small ? launch<1, 4, 4, 2>(stream, a) : launch<1, 8, 4, 3>(stream, a);
     case 2: return small ? launch<2, 4, 4, 2>(stream, a) : launch<2, 8, 4, 3>(stream, a);
     case 4: return small ? launch<4, 4, 4, 2>(stream, a) : launch<4, 8, 4, 3>(stream, a);
-    default: return small ? launch<8, 4, 2, 2>(stream, a) : launch<8, 8, 2, 3>(stream, a);
+    default:
+      if (!small) return launch<8, 8, 8, 3>(stream, a);
+      return a.n >= 8192 ? launch<8, 4, 8, 2>(stream, a) : launch<8, 4, 4, 2>(stream, a);
   }
 }
 
