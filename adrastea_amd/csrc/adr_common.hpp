@@ -198,8 +198,8 @@ hipError_t launch_matmul_general(hipStream_t stream, const MatmulArgs& a);
 // Returns true and fills `name` when the MFMA kernel family covers these arguments.
 bool mfma_gemm_supported(const MatmulArgs& a, const char** name);
 hipError_t launch_mfma_gemm(hipStream_t stream, const MatmulArgs& a);
-// fp16 skinny matmul (m <= 8, K-contiguous operands): true when the streaming kernel covers it.
-bool gemv_f16_supported(const MatmulArgs& a);
+// fp16 skinny matmul (m <= 32, K-contiguous operands): true when a streaming kernel covers it.
+bool gemv_f16_supported(const MatmulArgs& a, const char** name);
 hipError_t launch_gemv_f16(hipStream_t stream, const MatmulArgs& a);
 
 hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, const uint8_t* rhs,

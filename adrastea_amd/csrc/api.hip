@@ -49,7 +49,7 @@ bool empty(const MatmulArgs& a) { return a.batches == 0 || a.m == 0 || a.n == 0;
 int run_matmul(hipStream_t stream, const MatmulArgs& a, bool allow_fast) {
   if (empty(a)) return ADR_OK;
   const char* name;
-  if (allow_fast && gemv_f16_supported(a)) return (int)launch_gemv_f16(stream, a);
+  if (allow_fast && gemv_f16_supported(a, &name)) return (int)launch_gemv_f16(stream, a);
   if (allow_fast && mfma_gemm_supported(a, &name)) return (int)launch_mfma_gemm(stream, a);
   return (int)launch_matmul_general(stream, a);  // also the k == 0 case: store(0)
 }
@@ -141,8 +141,8 @@ int adr_matmul_f16_plan(char* name, int32_t cap, int32_t batches, int32_t m, int
                       0.0f, 1.0f, store, load, mask);
   if (int rc = validate_matmul(a, false)) return rc;
   const char* chosen = "none (empty)";
-  if (!empty(a) && gemv_f16_supported(a)) chosen = "gemv_f16_dot2_stream";
-  else if (!empty(a) && !mfma_gemm_supported(a, &chosen)) chosen = "matmul_general";
+  if (!empty(a) && !gemv_f16_supported(a, &chosen) && !mfma_gemm_supported(a, &chosen))
+    chosen = "matmul_general";
   if (name && cap > 0) {
     strncpy(name, chosen, (size_t)cap - 1);
     name[cap - 1] = 0;

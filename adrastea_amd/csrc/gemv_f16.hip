@@ -98,6 +98,109 @@ __global__ __launch_bounds__(NW * 64) void gemv_f16_dot_kernel(MatmulArgs a) {
   }
 }
 
+// Nine to thirty-two activation rows: matrix cores.  A workgroup owns 16 * RG weight rows, its
+// wavefronts split K (wavefront w takes the 128-k macro steps w, w + NW, ...) and their partial
+// sums meet in LDS, so every CU has work however few rows there are -- the tiled kernels put a
+// 64 x 64 tile on N / 64 CUs and walk the whole of K on each.  v_mfma_f32_16x16x32_f16 with the
+// weight rows as the A operand and a block of 16 activation rows as the B operand; lane (r, g)
+// holds 8 consecutive k of row r for k-group g of either operand (which 32 k an instruction sums
+// over is free as long as both operands agree).  MB blocks of 16 activation rows reuse the
+// weight fragments, U macro steps are loaded per trip.  K % 128 == 0.
+template <int NW, int RG, int MB, int U>
+__global__ __launch_bounds__(NW * 64) void skinny_f16_mfma_kernel(MatmulArgs a) {
+  constexpr int MACRO = 128;
+  __shared__ float partial[NW][RG][MB][256];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * (16 * RG);
+  const int steps = a.k / MACRO;
+  const half_t* wrow[RG];
+#pragma unroll
+  for (int q = 0; q < RG; q++)  // rows past n are clamped, their sums never stored
+    wrow[q] = a.rhs + (int64_t)min(n0 + q * 16 + r, a.n - 1) * a.stride_rx + g * 8;
+  const half_t* xrow[MB];
+  bool xvalid[MB];
+#pragma unroll
+  for (int b = 0; b < MB; b++) {
+    xvalid[b] = b * 16 + r < a.m;
+    xrow[b] = a.lhs + (int64_t)min(b * 16 + r, a.m - 1) * a.stride_ly + g * 8;
+  }
+  float4_t acc[RG][MB];
+#pragma unroll
+  for (int q = 0; q < RG; q++)
+#pragma unroll
+    for (int b = 0; b < MB; b++) acc[q][b] = float4_t{0, 0, 0, 0};
+  for (int ms0 = wave; ms0 < steps; ms0 += NW * U) {
+    // every load of the trip (U macro steps) is issued before the first multiply; rows past m
+    // read row m - 1 again, steps past K the last step, and are zeroed (a load under a lane
+    // mask or a branch would be waited for on the spot)
+    u32x4_t w[U][RG][4], x[U][MB][4];
+    bool live[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      live[u] = ms0 + u * NW < steps;
+      const int ms = live[u] ? ms0 + u * NW : steps - 1;
+#pragma unroll
+      for (int q = 0; q < RG; q++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          w[u][q][j] = __builtin_nontemporal_load((const u32x4_t*)(wrow[q] + ms * MACRO + j * 32));
+#pragma unroll
+      for (int b = 0; b < MB; b++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) x[u][b][j] = *(const u32x4_t*)(xrow[b] + ms * MACRO + j * 32);
+    }
+#pragma unroll
+    for (int u = 0; u < U; u++)
+#pragma unroll
+      for (int b = 0; b < MB; b++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          const u32x4_t xz = (xvalid[b] && live[u]) ? x[u][b][j] : u32x4_t{0, 0, 0, 0};
+          const half8_t xb = __builtin_bit_cast(half8_t, xz);
+#pragma unroll
+          for (int q = 0; q < RG; q++) {
+            const u32x4_t wv = w[u][q][j];
+            acc[q][b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, wv), xb,
+                                                               acc[q][b], 0, 0, 0);
+          }
+        }
+  }
+  // lane (r, g) holds sums of weight rows 4g .. 4g+3 against activation row r of the block
+#pragma unroll
+  for (int q = 0; q < RG; q++)
+#pragma unroll
+    for (int b = 0; b < MB; b++)
+#pragma unroll
+      for (int v = 0; v < 4; v++) partial[wave][q][b][(4 * g + v) * 16 + r] = acc[q][b][v];
+  __syncthreads();
+  const Epilogue ep{a.bias, a.beta, (half_t)a.scale, a.store, true};
+  for (int e = tid; e < RG * MB * 256; e += NW * 64) {
+    // consecutive threads -> consecutive output columns (weight rows)
+    const int col = e % (16 * RG), y = e / (16 * RG);
+    const int xcol = n0 + col;
+    if (y >= a.m || xcol >= a.n) continue;
+    half_t* o = a.output + (int64_t)y * a.stride_oy + (int64_t)xcol * a.stride_ox;
+    if (a.mask == ADR_MASK_CAUSAL && xcol > y) {
+      *o = neg_inf_half();
+      continue;
+    }
+    float sum = 0.0f;
+#pragma unroll
+    for (int w2 = 0; w2 < NW; w2++) sum += partial[w2][col / 16][y / 16][(col % 16) * 16 + (y % 16)];
+    const half_t prev = Epilogue::needs_prev(a.store) ? *o : (half_t)0;
+    const half_t bias_x = Epilogue::needs_bias(a.store) ? a.bias[xcol] : (half_t)0;
+    *o = ep.apply(sum, prev, bias_x);
+  }
+}
+
+template <int NW, int RG, int MB, int U>
+hipError_t launch_skinny(hipStream_t stream, const MatmulArgs& a) {
+  hipLaunchKernelGGL((skinny_f16_mfma_kernel<NW, RG, MB, U>), dim3((a.n + 16 * RG - 1) / (16 * RG)),
+                     dim3(NW * 64), 0, stream, a);
+  return hipGetLastError();
+}
+
 template <int MR, int NW, int RPB, int SEGW>
 hipError_t launch(hipStream_t stream, const MatmulArgs& a) {
   hipLaunchKernelGGL((gemv_f16_dot_kernel<MR, NW, RPB, SEGW>), dim3((a.n + RPB - 1) / RPB),
@@ -110,22 +213,44 @@ int rows_class(int m) { return m <= 1 ? 1 : m <= 2 ? 2 : m <= 4 ? 4 : 8; }
 
 }  // namespace
 
-bool gemv_f16_supported(const MatmulArgs& a) {
+static bool layout_ok(const MatmulArgs& a) {
   if (a.rhs_q || a.load != ADR_LOAD_IDENTITY || a.batches != 1) return false;
-  // from nine rows on the dot products cost more than the tiled kernels' slower loads
-  // (sixteen rows: 46 us against 31 us for K4096 N11008)
-  if (a.m < 1 || a.m > 8 || a.k % 8 != 0 || a.k < 512) return false;
   if (a.stride_lx != 1 || a.stride_ry != 1) return false;
   if ((a.stride_ly | a.stride_rx) & 7) return false;
   if (a.lhs && (((uintptr_t)a.lhs | (uintptr_t)a.rhs) & 15)) return false;
+  return true;
+}
+
+static bool dot_ok(const MatmulArgs& a) {
+  // from nine rows on the dot products cost more than the matrix-core kernel's slower loads
+  if (a.m < 1 || a.m > 8 || a.k % 8 != 0 || a.k < 512) return false;
   // worth it where the weight matrix is the traffic: at least 1 MiB of it
   if ((int64_t)a.n * a.k < (1 << 19)) return false;
-  const int nseg = (a.k + 511) / 512;
   // segments the instantiations hold: 4 wavefronts x 2 or 8 x 3
-  return nseg <= 24;
+  return (a.k + 511) / 512 <= 24;
+}
+
+static bool skinny_ok(const MatmulArgs& a) {
+  if (a.m < 9 || a.m > 32 || a.k % 128 != 0 || a.k < 1024 || (int64_t)a.n * a.k < (1 << 22)) return false;
+  // up to 16 rows it is never slower than the tiled kernels (K4096 N4096 16.7 against 18.3 us,
+  // K11008 N4096 39.8 against 65.9); with a second block of 16 rows only where K is long and
+  // the tiled kernels' few tiles walk all of it (K11008 N4096, 32 rows: 49.6 against 65.7 us)
+  return a.m <= 16 || a.k >= 8192;
+}
+
+bool gemv_f16_supported(const MatmulArgs& a, const char** name) {
+  if (!layout_ok(a)) return false;
+  if (dot_ok(a)) { *name = "gemv_f16_dot2_stream"; return true; }
+  if (skinny_ok(a)) { *name = "skinny_f16_mfma16_splitk_lds"; return true; }
+  return false;
 }
 
 hipError_t launch_gemv_f16(hipStream_t stream, const MatmulArgs& a) {
+  if (!dot_ok(a)) {
+    // (one macro step per trip: two or three in flight per wavefront measured slower)
+    if (a.m <= 16) return launch_skinny<8, 2, 1, 1>(stream, a);
+    return launch_skinny<8, 2, 2, 1>(stream, a);
+  }
   const int nseg = (a.k + 511) / 512;
   const bool small = nseg <= 8;
   // Weight rows per workgroup: every workgroup fetches the activations of all m rows again

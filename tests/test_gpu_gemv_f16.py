@@ -1,5 +1,6 @@
-"""fp16 skinny matmul (m <= 8 activation rows, the per-token call of llama.rs:485-591) through
-adr_matmul_f16: the streaming dot-product kernel against the CPU oracle."""
+"""fp16 skinny matmul (few activation rows, the per-token call of llama.rs:485-591) through
+adr_matmul_f16: the streaming dot-product kernel (m <= 8) and the matrix-core kernel whose
+wavefronts split K (m = 9..32) against the CPU oracle."""
 import numpy as np
 import pytest
 import torch
@@ -12,6 +13,7 @@ pytestmark = pytest.mark.gpu
 
 TOL = 1e-2
 PLAN = "gemv_f16_dot2_stream"
+PLAN_MFMA = "skinny_f16_mfma16_splitk_lds"
 
 
 def nt(M, K, N):
@@ -22,7 +24,7 @@ def nt(M, K, N):
 @pytest.mark.parametrize("K,N", [(512, 1030), (4096, 259), (4104, 131), (11008, 50), (12288, 44)])
 def test_matches_oracle_and_is_exact_on_exact_inputs(m, K, N):
     so, sl, sr = nt(m, K, N)
-    assert (plan(1, m, K, N, so, sl, sr) == PLAN) == (m <= 8)   # nine rows and more: tiled kernels
+    assert (plan(1, m, K, N, so, sl, sr) == PLAN) == (m <= 8)   # nine rows and more: other kernels
     g = rng(2000 + m * 31 + K + N)
     l, r = randn_f16(g, m * K), randn_f16(g, K * N, K ** -0.5)
     o_t = to_dev(np.full(m * N, 3.0, np.float16))
@@ -98,3 +100,38 @@ def test_nt_entry_point_with_beta():
     want = (l.reshape(m, K).astype(np.float64) @ r.reshape(N, K).astype(np.float64).T
             + 0.5 * prev.reshape(m, N).astype(np.float64))
     assert max_rel_err(to_np(o_t).reshape(m, N), want) <= 2e-3
+
+
+@pytest.mark.parametrize("m,K,N", [(9, 1024, 4100), (16, 4096, 1030), (13, 11008, 400), (17, 8192, 520),
+                                   (32, 11008, 390), (25, 12288, 350)])
+def test_matrix_core_kernel_for_nine_to_thirty_two_rows(m, K, N):
+    so, sl, sr = nt(m, K, N)
+    assert plan(1, m, K, N, so, sl, sr) == PLAN_MFMA
+    g = rng(2400 + m + K + N)
+    l = (g.integers(-8, 9, size=m * K) / 64.0).astype(np.float16)
+    r = (g.integers(-8, 9, size=K * N) / 64.0).astype(np.float16)
+    o_t = to_dev(np.full(m * N, 2.0, np.float16))
+    assert raw_matmul("adr_matmul_f16", o_t, to_dev(l), to_dev(r), 1, m, K, N, so, sl, sr) == 0
+    want = (l.reshape(m, K).astype(np.float64) @ r.reshape(N, K).astype(np.float64).T)
+    assert np.array_equal(to_np(o_t).view(np.uint16), want.astype(np.float16).reshape(-1).view(np.uint16))
+    # random inputs, an operator that reads the previous output and the bias, the causal mask
+    l, r = randn_f16(g, m * K), randn_f16(g, K * N, K ** -0.5)
+    prev, bias = randn_f16(g, m * N), randn_f16(g, N)
+    o_t = to_dev(prev)
+    assert raw_matmul("adr_matmul_f16", o_t, to_dev(l), to_dev(r), 1, m, K, N, so, sl, sr,
+                      bias_t=to_dev(bias), beta=0.5, store=oracle.STORE_BETA_BIAS,
+                      mask=oracle.MASK_CAUSAL) == 0
+    want = oracle_matmul(prev, l, r, 1, m, K, N, so, sl, sr, bias=bias, beta=0.5,
+                         store=oracle.STORE_BETA_BIAS, mask=oracle.MASK_CAUSAL)
+    got = to_np(o_t)
+    masked = np.isneginf(want.astype(np.float32))
+    assert masked.any() and np.array_equal(np.isneginf(got.astype(np.float32)), masked)
+    err = np.abs(got[~masked].astype(np.float64) - want[~masked].astype(np.float64))
+    ref = np.abs(want[~masked].astype(np.float64))
+    assert np.max(err / np.maximum(ref, np.sqrt(np.mean(ref ** 2)))) <= TOL
+
+
+def test_more_rows_or_short_k_stay_on_the_tiled_kernels():
+    for m, K, N in [(17, 4096, 4096), (33, 11008, 4096), (12, 960, 8192)]:
+        so, sl, sr = nt(m, K, N)
+        assert plan(1, m, K, N, so, sl, sr).startswith("gemm_nt_mfma")
