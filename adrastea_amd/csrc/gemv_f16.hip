@@ -231,11 +231,9 @@ static bool dot_ok(const MatmulArgs& a) {
 }
 
 static bool skinny_ok(const MatmulArgs& a) {
-  if (a.m < 9 || a.m > 32 || a.k % 128 != 0 || a.k < 1024 || (int64_t)a.n * a.k < (1 << 22)) return false;
-  // up to 16 rows it is never slower than the tiled kernels (K4096 N4096 16.7 against 18.3 us,
-  // K11008 N4096 39.8 against 65.9); with a second block of 16 rows only where K is long and
-  // the tiled kernels' few tiles walk all of it (K11008 N4096, 32 rows: 49.6 against 65.7 us)
-  return a.m <= 16 || a.k >= 8192;
+  // measured against the tiled kernels for 9..32 rows on N 4096..12288, K 4096 and 11008: never
+  // slower (K11008 N4096 m=16: 27.5 against 65.9 us; K4096 N12288 m=32: 30.8 against 32.8)
+  return a.m >= 9 && a.m <= 32 && a.k % 128 == 0 && a.k >= 1024 && (int64_t)a.n * a.k >= (1 << 22);
 }
 
 bool gemv_f16_supported(const MatmulArgs& a, const char** name) {
@@ -248,8 +246,18 @@ bool gemv_f16_supported(const MatmulArgs& a, const char** name) {
 hipError_t launch_gemv_f16(hipStream_t stream, const MatmulArgs& a) {
   if (!dot_ok(a)) {
     // (one macro step per trip: two or three in flight per wavefront measured slower)
-    if (a.m <= 16) return launch_skinny<8, 2, 1, 1>(stream, a);
-    return launch_skinny<8, 2, 2, 1>(stream, a);
+    // weight rows per workgroup: as few as still give (nearly) every CU a workgroup (N4096: 16
+    // rows, 256 workgroups, K11008 m=16 27.2 us against 39.5 with 32 rows; N12288: 48 rows,
+    // 25.7 against 28.7 with 16; N11008: 48 rows 25.2 against 31.7 with 32)
+    const int rg = a.n >= 40 * 256 ? 3 : a.n >= 24 * 256 ? 2 : 1;
+    if (a.m <= 16) {
+      if (rg == 3) return launch_skinny<8, 3, 1, 1>(stream, a);
+      if (rg == 2) return launch_skinny<8, 2, 1, 1>(stream, a);
+      return launch_skinny<8, 1, 1, 1>(stream, a);
+    }
+    if (rg == 3) return launch_skinny<8, 3, 2, 1>(stream, a);
+    if (rg == 2) return launch_skinny<8, 2, 2, 1>(stream, a);
+    return launch_skinny<8, 1, 2, 1>(stream, a);
   }
   const int nseg = (a.k + 511) / 512;
   const bool small = nseg <= 8;

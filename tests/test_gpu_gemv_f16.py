@@ -103,7 +103,8 @@ def test_nt_entry_point_with_beta():
 
 
 @pytest.mark.parametrize("m,K,N", [(9, 1024, 4100), (16, 4096, 1030), (13, 11008, 400), (17, 8192, 520),
-                                   (32, 11008, 390), (25, 12288, 350)])
+                                   (32, 11008, 390), (25, 12288, 350), (20, 1024, 6200),
+                                   (30, 1152, 10300)])
 def test_matrix_core_kernel_for_nine_to_thirty_two_rows(m, K, N):
     so, sl, sr = nt(m, K, N)
     assert plan(1, m, K, N, so, sl, sr) == PLAN_MFMA
@@ -132,6 +133,6 @@ def test_matrix_core_kernel_for_nine_to_thirty_two_rows(m, K, N):
 
 
 def test_more_rows_or_short_k_stay_on_the_tiled_kernels():
-    for m, K, N in [(17, 4096, 4096), (33, 11008, 4096), (12, 960, 8192)]:
+    for m, K, N in [(33, 4096, 4096), (33, 11008, 4096), (12, 960, 8192)]:
         so, sl, sr = nt(m, K, N)
         assert plan(1, m, K, N, so, sl, sr).startswith("gemm_nt_mfma")
