@@ -363,10 +363,13 @@ __device__ __forceinline__ void fill_masked_tile(const MatmulArgs& a, half_t* ou
 // =============================================================================================
 // Direct-to-LDS kernel
 // =============================================================================================
-template <int BM, int BN, int WM, int WN, int NSTAGE, int MINB, bool NN>
+template <int BM, int BN, int WM, int WN, int NSTAGE, int MINB, bool NN, int BK = 64>
 __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulArgs a,
                                                                          TileMap map) {
-  constexpr int BK = 64, CPR = 8, KK = 4;
+  // K slices of 64 (128 bytes of a row per slice and DMA request), or of 128 for the small tiles
+  // of few-row products, which are bound by how DRAM serves those requests
+  constexpr int CPR = BK / 8, KK = BK / 16;
+  static_assert(BK == 64 || (BK == 128 && !NN && NSTAGE == 3), "slices of 64, or 128 with three stages");
   constexpr int NW = WM * WN, NT = NW * 64;
   constexpr int IA = BM * CPR / NT, IB = BN * CPR / NT;  // DMA instructions per thread and slice
   constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
@@ -1273,11 +1276,11 @@ TileMap make_map(const MatmulArgs& a, int bm, int bn) {
   return map;
 }
 
-template <int BM, int BN, int WM, int WN, int NSTAGE, int MINB, bool NN = false>
+template <int BM, int BN, int WM, int WN, int NSTAGE, int MINB, bool NN = false, int BK = 64>
 hipError_t launch_dma(hipStream_t stream, const MatmulArgs& a) {
   TileMap map = make_map(a, BM, BN);
   if (map.total < 0) return hipErrorInvalidConfiguration;
-  hipLaunchKernelGGL((gemm_nt_dma_kernel<BM, BN, WM, WN, NSTAGE, MINB, NN>),
+  hipLaunchKernelGGL((gemm_nt_dma_kernel<BM, BN, WM, WN, NSTAGE, MINB, NN, BK>),
                      dim3((unsigned)map.total), dim3(WM * WN * 64), 0, stream, a, map);
   return hipGetLastError();
 }
@@ -1335,7 +1338,7 @@ enum GemmChoice {
   GEMM_NONE = 0,
   SHORTK_64, SHORTK_128,
   U8_256x192, U8_256x128,
-  DMA_256x192, DMA_256x128, DMA_128x128, DMA_128x64, DMA_64x64,
+  DMA_256x192, DMA_256x128, DMA_128x128, DMA_128x64, DMA_64x64, DMA_64x64_K128,
   DMA_NN_256x128, DMA_NN_128x128,
   STAGE_256x128, STAGE_128x128, STAGE_64x64,
 };
@@ -1402,6 +1405,14 @@ GemmChoice choose(const MatmulArgs& a) {
       return pick(a, shortk, 2);
     }
     const GemmChoice c = pick(a, DMA_TILES, 5);
+    // At most one 64 x 64 tile per CU (a few dozen to a few hundred rows against a weight
+    // matrix): the product is bound by how DRAM serves the weight requests -- one piece of every
+    // tile row per slice, a whole weight row apart -- and pieces of 256 bytes (slices of 128)
+    // stream better than pieces of 128 (K11008 N4096 m <= 256: 66 -> 46-54 us; K4096 N4096:
+    // 18.5 -> 14 us).  More tiles than CUs, or larger tiles, are better off with slices of 64.
+    if (c == DMA_64x64 && a.k % 128 == 0 && a.k >= 1024 &&
+        (int64_t)((a.m + 63) / 64) * ((a.n + 63) / 64) * a.batches <= NUM_CU)
+      return DMA_64x64_K128;
     // Short K with one large tile on (nearly) every CU: every workgroup then runs its prologue,
     // its few slices and its epilogue in step with all the others.  Twice as many tiles of half
     // the size, two resident per CU, overlap those phases (measured over a sweep of forced
@@ -1442,6 +1453,7 @@ static bool choice_name(GemmChoice c, const char** name) {
     case DMA_128x128: *name = "gemm_nt_mfma_dma_128x128x64"; return true;
     case DMA_128x64: *name = "gemm_nt_mfma_dma_128x64x64"; return true;
     case DMA_64x64: *name = "gemm_nt_mfma_dma_64x64x64"; return true;
+    case DMA_64x64_K128: *name = "gemm_nt_mfma_dma_64x64x128"; return true;
     case DMA_NN_256x128: *name = "gemm_nn_mfma_dma_256x128x64"; return true;
     case DMA_NN_128x128: *name = "gemm_nn_mfma_dma_128x128x64"; return true;
     case STAGE_256x128: *name = "gemm_nt_mfma_stage_256x128x32"; return true;
@@ -1462,6 +1474,7 @@ static hipError_t launch_choice(hipStream_t stream, const MatmulArgs& a, GemmCho
     case DMA_128x128: return launch_dma<128, 128, 2, 2, 3, 1>(stream, a);
     case DMA_128x64: return launch_dma<128, 64, 2, 2, 3, 2>(stream, a);
     case DMA_64x64: return launch_dma<64, 64, 2, 2, 3, 3>(stream, a);
+    case DMA_64x64_K128: return launch_dma<64, 64, 2, 2, 3, 1, false, 128>(stream, a);
     case DMA_NN_256x128: return launch_dma<256, 128, 4, 2, 3, 1, true>(stream, a);
     case DMA_NN_128x128: return launch_dma<128, 128, 2, 2, 2, 2, true>(stream, a);
     case STAGE_256x128: return launch_stage<256, 128, 32, 2, 2, 2>(stream, a);

@@ -501,6 +501,22 @@ def test_row_tail_split_keeps_operator_semantics():
     assert rel <= TOL, rel
 
 
+@pytest.mark.parametrize("shape", [(33, 1024, 4100), (200, 4096, 4096), (64, 1152, 12288), (256, 11008, 4096)])
+def test_few_row_products_with_slices_of_128(shape):
+    """At most one 64 x 64 tile per CU and K % 128 == 0: the 64 x 64 kernel with K slices of
+    128; exact on inputs whose sums are exact, ragged edges included."""
+    M, K, N = shape
+    so, sl, sr = nt_strides(M, K, N)
+    assert plan(1, M, K, N, so, sl, sr) == "gemm_nt_mfma_dma_64x64x128"
+    gen = torch.Generator(device="cuda").manual_seed(M + K)
+    a = (torch.randint(-8, 9, (M, K), generator=gen, device="cuda").float() / 64).half()
+    w = (torch.randint(-8, 9, (N, K), generator=gen, device="cuda").float() / 64).half()
+    out = torch.full((M, N), 9.0, dtype=torch.float16, device="cuda")
+    assert raw_matmul("adr_matmul_f16", out, a, w, 1, M, K, N, so, sl, sr) == 0
+    want = (a.double() @ w.double().t()).half()
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+
+
 def test_full_size_attention_products():
     """benchmark config 4: 32 heads, head_dim 128, seq 2048.  QK^T scaled by 1/sqrt(128) with the
     causal mask; P.V with softmaxed scores.  Checked per head against an fp32 batched GEMM."""
