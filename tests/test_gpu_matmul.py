@@ -501,13 +501,15 @@ def test_row_tail_split_keeps_operator_semantics():
     assert rel <= TOL, rel
 
 
-@pytest.mark.parametrize("shape", [(33, 1024, 4100), (200, 4096, 4096), (64, 1152, 12288), (256, 11008, 4096)])
+@pytest.mark.parametrize("shape", [(33, 1024, 4100, "64x64"), (200, 4096, 4096, "64x64"),
+                                   (64, 1152, 12288, "64x64"), (256, 11008, 4096, "64x64"),
+                                   (120, 1024, 12200, "128x64"), (500, 11008, 4096, "128x64")])
 def test_few_row_products_with_slices_of_128(shape):
-    """At most one 64 x 64 tile per CU and K % 128 == 0: the 64 x 64 kernel with K slices of
-    128; exact on inputs whose sums are exact, ragged edges included."""
-    M, K, N = shape
+    """At most one 64 x 64 (or 128 x 64) tile per CU and K % 128 == 0: the kernel with K slices
+    of 128; exact on inputs whose sums are exact, ragged edges included."""
+    M, K, N, tile = shape
     so, sl, sr = nt_strides(M, K, N)
-    assert plan(1, M, K, N, so, sl, sr) == "gemm_nt_mfma_dma_64x64x128"
+    assert plan(1, M, K, N, so, sl, sr) == f"gemm_nt_mfma_dma_{tile}x128"
     gen = torch.Generator(device="cuda").manual_seed(M + K)
     a = (torch.randint(-8, 9, (M, K), generator=gen, device="cuda").float() / 64).half()
     w = (torch.randint(-8, 9, (N, K), generator=gen, device="cuda").float() / 64).half()
