@@ -157,7 +157,7 @@ def main():
             per = N * K * 2
             nbuf = max(2, int(600e6 // per) + 1)
             ws = [randn_h(N, K, std=K ** -0.5) for _ in range(nbuf)]
-            for m in (1, 4, 8):
+            for m in (1, 4, 8, 16):
                 a = randn_h(m, K)
                 o = torch.zeros(m, N, dtype=torch.float16, device=dev)
                 i = [0]
