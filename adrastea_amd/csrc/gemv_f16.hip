@@ -194,6 +194,118 @@ __global__ __launch_bounds__(NW * 64) void skinny_f16_mfma_kernel(MatmulArgs a) 
   }
 }
 
+// Up to sixteen activation rows, K = 128 * NW * HS: the weights come in by global -> LDS DMA, four
+// whole 256-byte row pieces per instruction (the register path above touches sixteen rows with 64
+// bytes each per instruction, which DRAM serves a third slower).  A wavefront owns HS macro steps
+// x RG row groups = HS * RG tiles of 4 KiB ([16 rows][16 chunks of 16 bytes], chunk c of row r at
+// position c ^ r so that fragment reads spread over all banks) and streams them through a private
+// ring of RING tiles: nothing but its own vmcnt orders the DMA against its reads.  The
+// activations are loaded into registers before the first DMA, so the count of outstanding loads
+// at any later point is a multiple of the four DMA instructions of a tile.
+#define ADR_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
+#define ADR_GLB_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
+
+template <int NW, int RG, int HS, int RING>
+__global__ __launch_bounds__(NW * 64) void skinny_f16_ring_kernel(MatmulArgs a) {
+  constexpr int TILE = 16 * 256, MACRO = 128;
+  constexpr int UNITS = HS * RG;
+  static_assert(RING <= UNITS && NW * RG * 256 * 4 <= NW * RING * TILE, "partials reuse the ring");
+  __shared__ __attribute__((aligned(1024))) unsigned char ring[NW * RING * TILE];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * (16 * RG);
+  const bool xvalid = r < a.m;
+  const half_t* xrow = a.lhs + (int64_t)min(r, a.m - 1) * a.stride_ly + g * 8;
+  unsigned char* const mine = ring + wave * RING * TILE;
+  // registers first: the activations of all macro steps of the wavefront (rows past m read row
+  // m - 1 again and are zeroed when used)
+  u32x4_t x[HS][4];
+#pragma unroll
+  for (int h = 0; h < HS; h++)
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      x[h][j] = *(const u32x4_t*)(xrow + (int64_t)(wave + h * NW) * MACRO + j * 32);
+  // DMA instruction i of a tile fills its chunks [64 i, 64 i + 64): rows 4i .. 4i+3
+  auto issue = [&](int u) {  // tile u = (macro step u / RG of the wavefront, row group u % RG)
+    const int h = u / RG, q = u % RG;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int row = 4 * i + (lane >> 4), kc = (lane & 15) ^ row;
+      const half_t* src = a.rhs + (int64_t)min(n0 + q * 16 + row, a.n - 1) * a.stride_rx +
+                          (int64_t)(wave + h * NW) * MACRO + kc * 8;
+      __builtin_amdgcn_global_load_lds(ADR_GLB_PTR(src),
+                                       ADR_LDS_PTR(mine + (u % RING) * TILE + i * 1024), 16, 0, 0);
+    }
+  };
+  int roff[4];  // fragment read j of the lane: logical chunk 4j + g of row r
+#pragma unroll
+  for (int j = 0; j < 4; j++) roff[j] = r * 256 + (((4 * j + g) ^ r) << 4);
+  float4_t acc[RG];
+#pragma unroll
+  for (int q = 0; q < RG; q++) acc[q] = float4_t{0, 0, 0, 0};
+#pragma unroll
+  for (int u = 0; u < RING; u++) issue(u);
+#pragma unroll
+  for (int u = 0; u < UNITS; u++) {
+    // tiles u+1 .. min(u+RING-1, UNITS-1) may still be in flight: four DMA instructions each
+    const int later = (u + RING - 1 < UNITS ? RING - 1 : UNITS - 1 - u) * 4;
+    if (later == 12) __builtin_amdgcn_s_waitcnt(0x0F70 | 12);
+    else if (later == 8) __builtin_amdgcn_s_waitcnt(0x0F70 | 8);
+    else if (later == 4) __builtin_amdgcn_s_waitcnt(0x0F70 | 4);
+    else __builtin_amdgcn_s_waitcnt(0x0F70 | 0);
+    const int h = u / RG, q = u % RG;
+    const unsigned char* tile = mine + (u % RING) * TILE;
+    u32x4_t w[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) w[j] = *(const u32x4_t*)(tile + roff[j]);
+    // the tile is in registers before its slot is refilled
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+    __builtin_amdgcn_sched_barrier(0);
+    if (u + RING < UNITS) issue(u + RING);
+    __builtin_amdgcn_sched_barrier(0);
+    const u32x4_t z = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const u32x4_t xv = xvalid ? x[h][j] : z;
+      const u32x4_t wv = w[j];
+      acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, wv),
+                                                      __builtin_bit_cast(half8_t, xv), acc[q], 0, 0, 0);
+    }
+  }
+  // the ring is dead: its memory takes the per-wavefront partial sums [NW][RG][256]
+  __syncthreads();
+  float* partial = (float*)ring;
+#pragma unroll
+  for (int q = 0; q < RG; q++)
+#pragma unroll
+    for (int v = 0; v < 4; v++) partial[(wave * RG + q) * 256 + (4 * g + v) * 16 + r] = acc[q][v];
+  __syncthreads();
+  const Epilogue ep{a.bias, a.beta, (half_t)a.scale, a.store, true};
+  for (int e = tid; e < RG * 256; e += NW * 64) {
+    const int col = e % (16 * RG), y = e / (16 * RG);  // consecutive threads -> consecutive columns
+    const int xcol = n0 + col;
+    if (y >= a.m || xcol >= a.n) continue;
+    half_t* o = a.output + (int64_t)y * a.stride_oy + (int64_t)xcol * a.stride_ox;
+    if (a.mask == ADR_MASK_CAUSAL && xcol > y) {
+      *o = neg_inf_half();
+      continue;
+    }
+    float sum = 0.0f;
+#pragma unroll
+    for (int w2 = 0; w2 < NW; w2++) sum += partial[(w2 * RG + col / 16) * 256 + (col % 16) * 16 + y];
+    const half_t prev = Epilogue::needs_prev(a.store) ? *o : (half_t)0;
+    const half_t bias_x = Epilogue::needs_bias(a.store) ? a.bias[xcol] : (half_t)0;
+    *o = ep.apply(sum, prev, bias_x);
+  }
+}
+
+template <int NW, int RG, int HS, int RING>
+hipError_t launch_ring(hipStream_t stream, const MatmulArgs& a) {
+  hipLaunchKernelGGL((skinny_f16_ring_kernel<NW, RG, HS, RING>), dim3((a.n + 16 * RG - 1) / (16 * RG)),
+                     dim3(NW * 64), 0, stream, a);
+  return hipGetLastError();
+}
+
 template <int NW, int RG, int MB, int U>
 hipError_t launch_skinny(hipStream_t stream, const MatmulArgs& a) {
   hipLaunchKernelGGL((skinny_f16_mfma_kernel<NW, RG, MB, U>), dim3((a.n + 16 * RG - 1) / (16 * RG)),
@@ -250,6 +362,20 @@ hipError_t launch_gemv_f16(hipStream_t stream, const MatmulArgs& a) {
     // rows, 256 workgroups, K11008 m=16 27.2 us against 39.5 with 32 rows; N12288: 48 rows,
     // 25.7 against 28.7 with 16; N11008: 48 rows 25.2 against 31.7 with 32)
     const int rg = a.n >= 40 * 256 ? 3 : a.n >= 24 * 256 ? 2 : 1;
+    // K = 1024 * HS for the values of HS built here: weights through the per-wavefront LDS ring
+    // (m=16: K4096 N4096 12.4 -> 9.7 us, N11008 24.8 -> 20.3, N12288 25.9 -> 22.1)
+    if (a.m <= 16 && a.k % 1024 == 0) {
+      switch (a.k / 1024) {
+#define ADR_RING_CASE(HS)                                                  \
+        case HS:                                                           \
+          if (rg == 3) return launch_ring<8, 3, HS, 3>(stream, a);         \
+          if (rg == 2) return launch_ring<8, 2, HS, 3>(stream, a);         \
+          return launch_ring<8, 1, HS, 2>(stream, a);
+        ADR_RING_CASE(2) ADR_RING_CASE(4) ADR_RING_CASE(5) ADR_RING_CASE(8)
+#undef ADR_RING_CASE
+        default: break;
+      }
+    }
     if (a.m <= 16) {
       if (rg == 3) return launch_skinny<8, 3, 1, 1>(stream, a);
       if (rg == 2) return launch_skinny<8, 2, 1, 1>(stream, a);

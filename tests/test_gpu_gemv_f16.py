@@ -104,7 +104,11 @@ def test_nt_entry_point_with_beta():
 
 @pytest.mark.parametrize("m,K,N", [(9, 1024, 4100), (16, 4096, 1030), (13, 11008, 400), (17, 8192, 520),
                                    (32, 11008, 390), (25, 12288, 350), (20, 1024, 6200),
-                                   (30, 1152, 10300)])
+                                   (30, 1152, 10300),
+                                   # K = 1024 * {2, 4, 5, 8}, up to 16 rows: the LDS-ring variant,
+                                   # one, two and three groups of 16 weight rows per workgroup
+                                   (9, 2048, 4100), (16, 4096, 6200), (12, 5120, 10300),
+                                   (11, 8192, 1000), (16, 4096, 12288)])
 def test_matrix_core_kernel_for_nine_to_thirty_two_rows(m, K, N):
     so, sl, sr = nt(m, K, N)
     assert plan(1, m, K, N, so, sl, sr) == PLAN_MFMA
