@@ -334,7 +334,7 @@ static bool layout_ok(const MatmulArgs& a) {
 }
 
 static bool dot_ok(const MatmulArgs& a) {
-  // from nine rows on the dot products cost more than the matrix-core kernel's slower loads
+  // (the matrix-core kernels below take five rows and more where K allows)
   if (a.m < 1 || a.m > 8 || a.k % 8 != 0 || a.k < 512) return false;
   // worth it where the weight matrix is the traffic: at least 1 MiB of it
   if ((int64_t)a.n * a.k < (1 << 19)) return false;
@@ -344,19 +344,30 @@ static bool dot_ok(const MatmulArgs& a) {
 
 static bool skinny_ok(const MatmulArgs& a) {
   // measured against the tiled kernels for 9..32 rows on N 4096..12288, K 4096 and 11008: never
-  // slower (K11008 N4096 m=16: 27.5 against 65.9 us; K4096 N12288 m=32: 30.8 against 32.8)
-  return a.m >= 9 && a.m <= 32 && a.k % 128 == 0 && a.k >= 1024 && (int64_t)a.n * a.k >= (1 << 22);
+  // slower (K11008 N4096 m=16: 27.5 against 65.9 us; K4096 N12288 m=32: 30.8 against 32.8);
+  // from five rows on also ahead of the dot-product kernel (m=8, K4096 N12288: 21 against 24.9)
+  return a.m >= 5 && a.m <= 32 && a.k % 128 == 0 && a.k >= 1024 && (int64_t)a.n * a.k >= (1 << 22);
+}
+
+enum SkinnyChoice { SKINNY_NONE, SKINNY_DOT, SKINNY_MFMA };
+
+static SkinnyChoice choose_skinny(const MatmulArgs& a) {
+  if (!layout_ok(a)) return SKINNY_NONE;
+  if (a.m <= 4 && dot_ok(a)) return SKINNY_DOT;
+  if (skinny_ok(a)) return SKINNY_MFMA;
+  return dot_ok(a) ? SKINNY_DOT : SKINNY_NONE;
 }
 
 bool gemv_f16_supported(const MatmulArgs& a, const char** name) {
-  if (!layout_ok(a)) return false;
-  if (dot_ok(a)) { *name = "gemv_f16_dot2_stream"; return true; }
-  if (skinny_ok(a)) { *name = "skinny_f16_mfma16_splitk_lds"; return true; }
-  return false;
+  switch (choose_skinny(a)) {
+    case SKINNY_DOT: *name = "gemv_f16_dot2_stream"; return true;
+    case SKINNY_MFMA: *name = "skinny_f16_mfma16_splitk_lds"; return true;
+    default: return false;
+  }
 }
 
 hipError_t launch_gemv_f16(hipStream_t stream, const MatmulArgs& a) {
-  if (!dot_ok(a)) {
+  if (choose_skinny(a) == SKINNY_MFMA) {
     // (one macro step per trip: two or three in flight per wavefront measured slower)
     // weight rows per workgroup: as few as still give (nearly) every CU a workgroup (N4096: 16
     // rows, 256 workgroups, K11008 m=16 27.2 us against 39.5 with 32 rows; N12288: 48 rows,

@@ -21,10 +21,17 @@ def nt(M, K, N):
 
 
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 8, 9, 16])
-@pytest.mark.parametrize("K,N", [(512, 1030), (4096, 259), (4104, 131), (11008, 50), (12288, 44)])
+@pytest.mark.parametrize("K,N", [(512, 1030), (4096, 259), (4104, 131), (11008, 50), (12288, 44),
+                                 (4096, 1100), (11008, 400)])
 def test_matches_oracle_and_is_exact_on_exact_inputs(m, K, N):
     so, sl, sr = nt(m, K, N)
-    assert (plan(1, m, K, N, so, sl, sr) == PLAN) == (m <= 8)   # nine rows and more: other kernels
+    # up to four rows: dot products; five to eight: dot products only where K is no multiple of 128
+    # (or the matrix is small); more: other kernels
+    mfma = m >= 5 and K % 128 == 0 and K >= 1024 and N * K >= (1 << 22)
+    if mfma:
+        assert plan(1, m, K, N, so, sl, sr) == PLAN_MFMA
+    elif m <= 8:
+        assert plan(1, m, K, N, so, sl, sr) == PLAN
     g = rng(2000 + m * 31 + K + N)
     l, r = randn_f16(g, m * K), randn_f16(g, K * N, K ** -0.5)
     o_t = to_dev(np.full(m * N, 3.0, np.float16))
@@ -47,7 +54,7 @@ STORES = [oracle.STORE_IDENTITY, oracle.STORE_SCALE, oracle.STORE_ADD, oracle.ST
 @pytest.mark.parametrize("store", STORES)
 @pytest.mark.parametrize("mask", [oracle.MASK_NONE, oracle.MASK_CAUSAL])
 def test_operators_and_mask(store, mask):
-    m, K, N = 6, 1024, 520
+    m, K, N = 6, 1032, 520
     so, sl, sr = nt(m, K, N)
     assert plan(1, m, K, N, so, sl, sr, store=store, mask=mask) == PLAN
     g = rng(2100 + store * 5 + mask)
@@ -108,8 +115,10 @@ def test_nt_entry_point_with_beta():
                                    # K = 1024 * {2, 4, 5, 8}, up to 16 rows: the LDS-ring variant,
                                    # one, two and three groups of 16 weight rows per workgroup
                                    (9, 2048, 4100), (16, 4096, 6200), (12, 5120, 10300),
-                                   (11, 8192, 1000), (16, 4096, 12288)])
-def test_matrix_core_kernel_for_nine_to_thirty_two_rows(m, K, N):
+                                   (11, 8192, 1000), (16, 4096, 12288),
+                                   # five to eight rows take these kernels too
+                                   (5, 4096, 4100), (8, 11008, 4096), (7, 1152, 4000)])
+def test_matrix_core_kernel_for_five_to_thirty_two_rows(m, K, N):
     so, sl, sr = nt(m, K, N)
     assert plan(1, m, K, N, so, sl, sr) == PLAN_MFMA
     g = rng(2400 + m + K + N)
