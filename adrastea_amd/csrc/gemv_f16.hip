@@ -194,7 +194,9 @@ __global__ __launch_bounds__(NW * 64) void skinny_f16_mfma_kernel(MatmulArgs a) 
   }
 }
 
-// Up to sixteen activation rows, K = 128 * NW * HS: the weights come in by global -> LDS DMA, four
+// Up to sixteen activation rows, K = 128 * pieces with NW * (HS - 1) < pieces <= NW * HS (the
+// wavefronts that have no piece in the last round read the last piece again against zeroed
+// activations): the weights come in by global -> LDS DMA, four
 // whole 256-byte row pieces per instruction (the register path above touches sixteen rows with 64
 // bytes each per instruction, which DRAM serves a third slower).  A wavefront owns HS macro steps
 // x RG row groups = HS * RG tiles of 4 KiB ([16 rows][16 chunks of 16 bytes], chunk c of row r at
@@ -217,22 +219,29 @@ __global__ __launch_bounds__(NW * 64) void skinny_f16_ring_kernel(MatmulArgs a) 
   const bool xvalid = r < a.m;
   const half_t* xrow = a.lhs + (int64_t)min(r, a.m - 1) * a.stride_ly + g * 8;
   unsigned char* const mine = ring + wave * RING * TILE;
+  const int pieces = a.k / MACRO;
+  const bool last_valid = wave + (HS - 1) * NW < pieces;
+  const int last_piece = min(wave + (HS - 1) * NW, pieces - 1);
   // registers first: the activations of all macro steps of the wavefront (rows past m read row
   // m - 1 again and are zeroed when used)
   u32x4_t x[HS][4];
 #pragma unroll
   for (int h = 0; h < HS; h++)
 #pragma unroll
-    for (int j = 0; j < 4; j++)
-      x[h][j] = *(const u32x4_t*)(xrow + (int64_t)(wave + h * NW) * MACRO + j * 32);
+    for (int j = 0; j < 4; j++) {
+      const int piece = h == HS - 1 ? last_piece : wave + h * NW;
+      x[h][j] = *(const u32x4_t*)(xrow + (int64_t)piece * MACRO + j * 32);
+      if (h == HS - 1 && !last_valid) x[h][j] = u32x4_t{0, 0, 0, 0};
+    }
   // DMA instruction i of a tile fills its chunks [64 i, 64 i + 64): rows 4i .. 4i+3
   auto issue = [&](int u) {  // tile u = (macro step u / RG of the wavefront, row group u % RG)
     const int h = u / RG, q = u % RG;
+    const int piece = h == HS - 1 ? last_piece : wave + h * NW;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const int row = 4 * i + (lane >> 4), kc = (lane & 15) ^ row;
       const half_t* src = a.rhs + (int64_t)min(n0 + q * 16 + row, a.n - 1) * a.stride_rx +
-                          (int64_t)(wave + h * NW) * MACRO + kc * 8;
+                          (int64_t)piece * MACRO + kc * 8;
       __builtin_amdgcn_global_load_lds(ADR_GLB_PTR(src),
                                        ADR_LDS_PTR(mine + (u % RING) * TILE + i * 1024), 16, 0, 0);
     }
@@ -373,17 +382,22 @@ hipError_t launch_gemv_f16(hipStream_t stream, const MatmulArgs& a) {
     // rows, 256 workgroups, K11008 m=16 27.2 us against 39.5 with 32 rows; N12288: 48 rows,
     // 25.7 against 28.7 with 16; N11008: 48 rows 25.2 against 31.7 with 32)
     const int rg = a.n >= 40 * 256 ? 3 : a.n >= 24 * 256 ? 2 : 1;
-    // K = 1024 * HS for the values of HS built here: weights through the per-wavefront LDS ring
-    // (m=16: K4096 N4096 12.4 -> 9.7 us, N11008 24.8 -> 20.3, N12288 25.9 -> 22.1)
-    if (a.m <= 16 && a.k % 1024 == 0) {
-      switch (a.k / 1024) {
+    // K in (1024 * (HS - 1), 1024 * HS] for the values of HS built here: weights through the
+    // per-wavefront LDS ring (m=16: K4096 N4096 12.4 -> 9.7 us, N11008 24.8 -> 20.3, N12288
+    // 25.9 -> 22.1)
+    if (a.m <= 16) {
+      switch ((a.k + 1023) / 1024) {
 #define ADR_RING_CASE(HS)                                                  \
         case HS:                                                           \
           if (rg == 3) return launch_ring<8, 3, HS, 3>(stream, a);         \
           if (rg == 2) return launch_ring<8, 2, HS, 3>(stream, a);         \
           return launch_ring<8, 1, HS, 2>(stream, a);
-        ADR_RING_CASE(2) ADR_RING_CASE(4) ADR_RING_CASE(5) ADR_RING_CASE(8)
+        ADR_RING_CASE(2) ADR_RING_CASE(3) ADR_RING_CASE(4) ADR_RING_CASE(5) ADR_RING_CASE(8)
 #undef ADR_RING_CASE
+        // (eleven steps, K 11008, with one row group: 23.8 / 27.2 us for 8 / 16 rows with a ring
+        // of four against 23.3 / 26.4 from registers, so not built: with 16 weight rows per
+        // workgroup the activations every workgroup re-reads through L2 weigh as much as the
+        // weights, whichever way those arrive)
         default: break;
       }
     }

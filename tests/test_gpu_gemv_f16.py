@@ -116,6 +116,9 @@ def test_nt_entry_point_with_beta():
                                    # one, two and three groups of 16 weight rows per workgroup
                                    (9, 2048, 4100), (16, 4096, 6200), (12, 5120, 10300),
                                    (11, 8192, 1000), (16, 4096, 12288),
+                                   # K between multiples of 1024: the wavefronts without a piece in
+                                   # the last round (K 11008: 86 pieces for 8 x 11)
+                                   (16, 11008, 4096), (10, 2176, 6200), (14, 4992, 10300), (9, 10368, 800),
                                    # five to eight rows take these kernels too
                                    (5, 4096, 4100), (8, 11008, 4096), (7, 1152, 4000)])
 def test_matrix_core_kernel_for_five_to_thirty_two_rows(m, K, N):
