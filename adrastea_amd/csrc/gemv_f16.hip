@@ -194,7 +194,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_f16_mfma_kernel(MatmulArgs a) 
   }
 }
 
-// Up to sixteen activation rows, K = 128 * pieces with NW * (HS - 1) < pieces <= NW * HS (the
+// Up to sixteen activation rows per block of MB, K = 128 * pieces with NW * (HS - 1) < pieces <= NW * HS (the
 // wavefronts that have no piece in the last round read the last piece again against zeroed
 // activations): the weights come in by global -> LDS DMA, four
 // whole 256-byte row pieces per instruction (the register path above touches sixteen rows with 64
@@ -207,32 +207,39 @@ __global__ __launch_bounds__(NW * 64) void skinny_f16_mfma_kernel(MatmulArgs a) 
 #define ADR_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 #define ADR_GLB_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
 
-template <int NW, int RG, int HS, int RING>
+template <int NW, int RG, int HS, int RING, int MB>
 __global__ __launch_bounds__(NW * 64) void skinny_f16_ring_kernel(MatmulArgs a) {
   constexpr int TILE = 16 * 256, MACRO = 128;
   constexpr int UNITS = HS * RG;
-  static_assert(RING <= UNITS && NW * RG * 256 * 4 <= NW * RING * TILE, "partials reuse the ring");
+  static_assert(RING <= UNITS && NW * MB * RG * 256 * 4 <= NW * RING * TILE, "partials reuse the ring");
   __shared__ __attribute__((aligned(1024))) unsigned char ring[NW * RING * TILE];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * (16 * RG);
-  const bool xvalid = r < a.m;
-  const half_t* xrow = a.lhs + (int64_t)min(r, a.m - 1) * a.stride_ly + g * 8;
+  bool xvalid[MB];  // MB blocks of sixteen activation rows
+  const half_t* xrow[MB];
+#pragma unroll
+  for (int b = 0; b < MB; b++) {
+    xvalid[b] = b * 16 + r < a.m;
+    xrow[b] = a.lhs + (int64_t)min(b * 16 + r, a.m - 1) * a.stride_ly + g * 8;
+  }
   unsigned char* const mine = ring + wave * RING * TILE;
   const int pieces = a.k / MACRO;
   const bool last_valid = wave + (HS - 1) * NW < pieces;
   const int last_piece = min(wave + (HS - 1) * NW, pieces - 1);
   // registers first: the activations of all macro steps of the wavefront (rows past m read row
   // m - 1 again and are zeroed when used)
-  u32x4_t x[HS][4];
+  u32x4_t x[MB][HS][4];
 #pragma unroll
-  for (int h = 0; h < HS; h++)
+  for (int b = 0; b < MB; b++)
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const int piece = h == HS - 1 ? last_piece : wave + h * NW;
-      x[h][j] = *(const u32x4_t*)(xrow + (int64_t)piece * MACRO + j * 32);
-      if (h == HS - 1 && !last_valid) x[h][j] = u32x4_t{0, 0, 0, 0};
-    }
+    for (int h = 0; h < HS; h++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const int piece = h == HS - 1 ? last_piece : wave + h * NW;
+        x[b][h][j] = *(const u32x4_t*)(xrow[b] + (int64_t)piece * MACRO + j * 32);
+        if (h == HS - 1 && !last_valid) x[b][h][j] = u32x4_t{0, 0, 0, 0};
+      }
   // DMA instruction i of a tile fills its chunks [64 i, 64 i + 64): rows 4i .. 4i+3
   auto issue = [&](int u) {  // tile u = (macro step u / RG of the wavefront, row group u % RG)
     const int h = u / RG, q = u % RG;
@@ -249,9 +256,11 @@ __global__ __launch_bounds__(NW * 64) void skinny_f16_ring_kernel(MatmulArgs a) 
   int roff[4];  // fragment read j of the lane: logical chunk 4j + g of row r
 #pragma unroll
   for (int j = 0; j < 4; j++) roff[j] = r * 256 + (((4 * j + g) ^ r) << 4);
-  float4_t acc[RG];
+  float4_t acc[MB][RG];
 #pragma unroll
-  for (int q = 0; q < RG; q++) acc[q] = float4_t{0, 0, 0, 0};
+  for (int b = 0; b < MB; b++)
+#pragma unroll
+    for (int q = 0; q < RG; q++) acc[b][q] = float4_t{0, 0, 0, 0};
 #pragma unroll
   for (int u = 0; u < RING; u++) issue(u);
 #pragma unroll
@@ -275,22 +284,28 @@ __global__ __launch_bounds__(NW * 64) void skinny_f16_ring_kernel(MatmulArgs a) 
     const u32x4_t z = {0, 0, 0, 0};
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-      const u32x4_t xv = xvalid ? x[h][j] : z;
       const u32x4_t wv = w[j];
-      acc[q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, wv),
-                                                      __builtin_bit_cast(half8_t, xv), acc[q], 0, 0, 0);
+#pragma unroll
+      for (int b = 0; b < MB; b++) {
+        const u32x4_t xv = xvalid[b] ? x[b][h][j] : z;
+        acc[b][q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+            __builtin_bit_cast(half8_t, wv), __builtin_bit_cast(half8_t, xv), acc[b][q], 0, 0, 0);
+      }
     }
   }
-  // the ring is dead: its memory takes the per-wavefront partial sums [NW][RG][256]
+  // the ring is dead: its memory takes the per-wavefront partial sums [NW][MB][RG][256]
   __syncthreads();
   float* partial = (float*)ring;
 #pragma unroll
-  for (int q = 0; q < RG; q++)
+  for (int b = 0; b < MB; b++)
 #pragma unroll
-    for (int v = 0; v < 4; v++) partial[(wave * RG + q) * 256 + (4 * g + v) * 16 + r] = acc[q][v];
+    for (int q = 0; q < RG; q++)
+#pragma unroll
+      for (int v = 0; v < 4; v++)
+        partial[((wave * MB + b) * RG + q) * 256 + (4 * g + v) * 16 + r] = acc[b][q][v];
   __syncthreads();
   const Epilogue ep{a.bias, a.beta, (half_t)a.scale, a.store, true};
-  for (int e = tid; e < RG * 256; e += NW * 64) {
+  for (int e = tid; e < MB * RG * 256; e += NW * 64) {
     const int col = e % (16 * RG), y = e / (16 * RG);  // consecutive threads -> consecutive columns
     const int xcol = n0 + col;
     if (y >= a.m || xcol >= a.n) continue;
@@ -301,16 +316,17 @@ __global__ __launch_bounds__(NW * 64) void skinny_f16_ring_kernel(MatmulArgs a) 
     }
     float sum = 0.0f;
 #pragma unroll
-    for (int w2 = 0; w2 < NW; w2++) sum += partial[(w2 * RG + col / 16) * 256 + (col % 16) * 16 + y];
+    for (int w2 = 0; w2 < NW; w2++)
+      sum += partial[((w2 * MB + y / 16) * RG + col / 16) * 256 + (col % 16) * 16 + y % 16];
     const half_t prev = Epilogue::needs_prev(a.store) ? *o : (half_t)0;
     const half_t bias_x = Epilogue::needs_bias(a.store) ? a.bias[xcol] : (half_t)0;
     *o = ep.apply(sum, prev, bias_x);
   }
 }
 
-template <int NW, int RG, int HS, int RING>
+template <int NW, int RG, int HS, int RING, int MB = 1>
 hipError_t launch_ring(hipStream_t stream, const MatmulArgs& a) {
-  hipLaunchKernelGGL((skinny_f16_ring_kernel<NW, RG, HS, RING>), dim3((a.n + 16 * RG - 1) / (16 * RG)),
+  hipLaunchKernelGGL((skinny_f16_ring_kernel<NW, RG, HS, RING, MB>), dim3((a.n + 16 * RG - 1) / (16 * RG)),
                      dim3(NW * 64), 0, stream, a);
   return hipGetLastError();
 }
@@ -398,6 +414,20 @@ hipError_t launch_gemv_f16(hipStream_t stream, const MatmulArgs& a) {
         // of four against 23.3 / 26.4 from registers, so not built: with 16 weight rows per
         // workgroup the activations every workgroup re-reads through L2 weigh as much as the
         // weights, whichever way those arrive)
+        default: break;
+      }
+    }
+    // 17 to 32 rows: two blocks of activations in registers, so K up to 4096 only (m=32, K4096:
+    // N4096 15.0 -> 13.6 us, N11008 29.1 -> 24.6, N12288 30.8 -> 26.3)
+    if (a.m > 16) {
+      switch ((a.k + 1023) / 1024) {
+#define ADR_RING_CASE(HS)                                                  \
+        case HS:                                                           \
+          if (rg == 3) return launch_ring<8, 3, HS, 3, 2>(stream, a);      \
+          if (rg == 2) return launch_ring<8, 2, HS, 3, 2>(stream, a);      \
+          return launch_ring<8, 1, HS, 2, 2>(stream, a);
+        ADR_RING_CASE(2) ADR_RING_CASE(3) ADR_RING_CASE(4)
+#undef ADR_RING_CASE
         default: break;
       }
     }
