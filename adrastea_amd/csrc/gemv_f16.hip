@@ -207,10 +207,14 @@ __global__ __launch_bounds__(NW * 64) void skinny_f16_mfma_kernel(MatmulArgs a) 
 #define ADR_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 #define ADR_GLB_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
 
-template <int NW, int RG, int HS, int RING, int MB>
+template <int NW, int RG, int HS, int RING, int MB, bool XR>
 __global__ __launch_bounds__(NW * 64) void skinny_f16_ring_kernel(MatmulArgs a) {
   constexpr int TILE = 16 * 256, MACRO = 128;
-  constexpr int UNITS = HS * RG;
+  // XR: the activations of a macro step travel through the ring as MB more tiles ahead of the
+  // step's weight tiles (whole 256-byte row pieces from L2 instead of 64-byte ones, and sixteen
+  // registers of activations per block instead of sixteen per block and macro step)
+  constexpr int PER = XR ? RG + MB : RG;
+  constexpr int UNITS = HS * PER;
   static_assert(RING <= UNITS && NW * MB * RG * 256 * 4 <= NW * RING * TILE, "partials reuse the ring");
   __shared__ __attribute__((aligned(1024))) unsigned char ring[NW * RING * TILE];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -229,11 +233,11 @@ __global__ __launch_bounds__(NW * 64) void skinny_f16_ring_kernel(MatmulArgs a) 
   const int last_piece = min(wave + (HS - 1) * NW, pieces - 1);
   // registers first: the activations of all macro steps of the wavefront (rows past m read row
   // m - 1 again and are zeroed when used)
-  u32x4_t x[MB][HS][4];
+  u32x4_t x[MB][XR ? 1 : HS][4];
 #pragma unroll
   for (int b = 0; b < MB; b++)
 #pragma unroll
-    for (int h = 0; h < HS; h++)
+    for (int h = 0; h < (XR ? 0 : HS); h++)
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         const int piece = h == HS - 1 ? last_piece : wave + h * NW;
@@ -242,12 +246,13 @@ __global__ __launch_bounds__(NW * 64) void skinny_f16_ring_kernel(MatmulArgs a) 
       }
   // DMA instruction i of a tile fills its chunks [64 i, 64 i + 64): rows 4i .. 4i+3
   auto issue = [&](int u) {  // tile u = (macro step u / RG of the wavefront, row group u % RG)
-    const int h = u / RG, q = u % RG;
+    const int h = u / PER, q = u % PER - (XR ? MB : 0);  // q < 0: activation block q + MB
     const int piece = h == HS - 1 ? last_piece : wave + h * NW;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
       const int row = 4 * i + (lane >> 4), kc = (lane & 15) ^ row;
-      const half_t* src = a.rhs + (int64_t)min(n0 + q * 16 + row, a.n - 1) * a.stride_rx +
+      const half_t* src = (q < 0 ? a.lhs + (int64_t)min((q + MB) * 16 + row, a.m - 1) * a.stride_ly
+                                 : a.rhs + (int64_t)min(n0 + q * 16 + row, a.n - 1) * a.stride_rx) +
                           (int64_t)piece * MACRO + kc * 8;
       __builtin_amdgcn_global_load_lds(ADR_GLB_PTR(src),
                                        ADR_LDS_PTR(mine + (u % RING) * TILE + i * 1024), 16, 0, 0);
@@ -271,7 +276,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_f16_ring_kernel(MatmulArgs a) 
     else if (later == 8) __builtin_amdgcn_s_waitcnt(0x0F70 | 8);
     else if (later == 4) __builtin_amdgcn_s_waitcnt(0x0F70 | 4);
     else __builtin_amdgcn_s_waitcnt(0x0F70 | 0);
-    const int h = u / RG, q = u % RG;
+    const int h = u / PER, q = u % PER - (XR ? MB : 0);
     const unsigned char* tile = mine + (u % RING) * TILE;
     u32x4_t w[4];
 #pragma unroll
@@ -282,12 +287,17 @@ __global__ __launch_bounds__(NW * 64) void skinny_f16_ring_kernel(MatmulArgs a) 
     if (u + RING < UNITS) issue(u + RING);
     __builtin_amdgcn_sched_barrier(0);
     const u32x4_t z = {0, 0, 0, 0};
+    if (q < 0) {  // the step's activations
+#pragma unroll
+      for (int j = 0; j < 4; j++) x[q < 0 ? q + MB : 0][0][j] = (h == HS - 1 && !last_valid) ? z : w[j];
+      continue;
+    }
 #pragma unroll
     for (int j = 0; j < 4; j++) {
       const u32x4_t wv = w[j];
 #pragma unroll
       for (int b = 0; b < MB; b++) {
-        const u32x4_t xv = xvalid[b] ? x[b][h][j] : z;
+        const u32x4_t xv = xvalid[b] ? x[b][XR ? 0 : h][j] : z;
         acc[b][q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
             __builtin_bit_cast(half8_t, wv), __builtin_bit_cast(half8_t, xv), acc[b][q], 0, 0, 0);
       }
@@ -324,9 +334,9 @@ __global__ __launch_bounds__(NW * 64) void skinny_f16_ring_kernel(MatmulArgs a) 
   }
 }
 
-template <int NW, int RG, int HS, int RING, int MB = 1>
+template <int NW, int RG, int HS, int RING, int MB = 1, bool XR = false>
 hipError_t launch_ring(hipStream_t stream, const MatmulArgs& a) {
-  hipLaunchKernelGGL((skinny_f16_ring_kernel<NW, RG, HS, RING, MB>), dim3((a.n + 16 * RG - 1) / (16 * RG)),
+  hipLaunchKernelGGL((skinny_f16_ring_kernel<NW, RG, HS, RING, MB, XR>), dim3((a.n + 16 * RG - 1) / (16 * RG)),
                      dim3(NW * 64), 0, stream, a);
   return hipGetLastError();
 }
@@ -398,35 +408,34 @@ hipError_t launch_gemv_f16(hipStream_t stream, const MatmulArgs& a) {
     // rows, 256 workgroups, K11008 m=16 27.2 us against 39.5 with 32 rows; N12288: 48 rows,
     // 25.7 against 28.7 with 16; N11008: 48 rows 25.2 against 31.7 with 32)
     const int rg = a.n >= 40 * 256 ? 3 : a.n >= 24 * 256 ? 2 : 1;
-    // K in (1024 * (HS - 1), 1024 * HS] for the values of HS built here: weights through the
-    // per-wavefront LDS ring (m=16: K4096 N4096 12.4 -> 9.7 us, N11008 24.8 -> 20.3, N12288
-    // 25.9 -> 22.1)
+    // K in (1024 * (HS - 1), 1024 * HS] for the values of HS built here: weights, and the
+    // activations with them, through the per-wavefront LDS ring (m=16, weights alone: K4096
+    // N4096 12.4 -> 9.7 us, N11008 24.8 -> 20.3, N12288 25.9 -> 22.1; activations too: 9.9 ->
+    // 8.7, 21.2 -> 19.7, 23.2 -> 21.9, K11008 N4096 27.7 -> 23.5)
     if (a.m <= 16) {
       switch ((a.k + 1023) / 1024) {
-#define ADR_RING_CASE(HS)                                                  \
-        case HS:                                                           \
-          if (rg == 3) return launch_ring<8, 3, HS, 3>(stream, a);         \
-          if (rg == 2) return launch_ring<8, 2, HS, 3>(stream, a);         \
-          return launch_ring<8, 1, HS, 2>(stream, a);
+#define ADR_RING_CASE(HS)                                                         \
+        case HS:                                                                  \
+          if (rg == 3) return launch_ring<8, 3, HS, 4, 1, true>(stream, a);       \
+          if (rg == 2) return launch_ring<8, 2, HS, 3, 1, true>(stream, a);       \
+          return launch_ring<8, 1, HS, 4, 1, true>(stream, a);
         ADR_RING_CASE(2) ADR_RING_CASE(3) ADR_RING_CASE(4) ADR_RING_CASE(5) ADR_RING_CASE(8)
+        ADR_RING_CASE(11)
 #undef ADR_RING_CASE
-        // (eleven steps, K 11008, with one row group: 23.8 / 27.2 us for 8 / 16 rows with a ring
-        // of four against 23.3 / 26.4 from registers, so not built: with 16 weight rows per
-        // workgroup the activations every workgroup re-reads through L2 weigh as much as the
-        // weights, whichever way those arrive)
         default: break;
       }
     }
-    // 17 to 32 rows: two blocks of activations in registers, so K up to 4096 only (m=32, K4096:
-    // N4096 15.0 -> 13.6 us, N11008 29.1 -> 24.6, N12288 30.8 -> 26.3)
+    // 17 to 32 rows: two blocks of activations (m=32, K4096, in registers: N4096 15.0 -> 13.6 us,
+    // N11008 29.1 -> 24.6, N12288 30.8 -> 26.3)
     if (a.m > 16) {
       switch ((a.k + 1023) / 1024) {
-#define ADR_RING_CASE(HS)                                                  \
-        case HS:                                                           \
-          if (rg == 3) return launch_ring<8, 3, HS, 3, 2>(stream, a);      \
-          if (rg == 2) return launch_ring<8, 2, HS, 3, 2>(stream, a);      \
-          return launch_ring<8, 1, HS, 2, 2>(stream, a);
-        ADR_RING_CASE(2) ADR_RING_CASE(3) ADR_RING_CASE(4)
+#define ADR_RING_CASE(HS)                                                         \
+        case HS:                                                                  \
+          if (rg == 3) return launch_ring<8, 3, HS, 4, 2, true>(stream, a);       \
+          if (rg == 2) return launch_ring<8, 2, HS, 4, 2, true>(stream, a);       \
+          return launch_ring<8, 1, HS, 3, 2, true>(stream, a);
+        ADR_RING_CASE(2) ADR_RING_CASE(3) ADR_RING_CASE(4) ADR_RING_CASE(5) ADR_RING_CASE(8)
+        ADR_RING_CASE(11)
 #undef ADR_RING_CASE
         default: break;
       }

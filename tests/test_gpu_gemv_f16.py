@@ -121,7 +121,7 @@ def test_nt_entry_point_with_beta():
                                    (16, 11008, 4096), (10, 2176, 6200), (14, 4992, 10300), (9, 10368, 800),
                                    # 17 to 32 rows through the ring: K up to 4096
                                    (17, 4096, 6200), (32, 2048, 12288), (25, 3072, 4100), (32, 4096, 12288),
-                                   (20, 3968, 10300),
+                                   (20, 3968, 10300), (32, 11008, 4096), (19, 8192, 6200), (27, 5120, 10300),
                                    # five to eight rows take these kernels too
                                    (5, 4096, 4100), (8, 11008, 4096), (7, 1152, 4000)])
 def test_matrix_core_kernel_for_five_to_thirty_two_rows(m, K, N):
