@@ -194,26 +194,26 @@ __global__ __launch_bounds__(NW * 64) void skinny_f16_mfma_kernel(MatmulArgs a) 
   }
 }
 
-// Up to sixteen activation rows per block of MB, K = 128 * pieces with NW * (HS - 1) < pieces <= NW * HS (the
-// wavefronts that have no piece in the last round read the last piece again against zeroed
-// activations): the weights come in by global -> LDS DMA, four
-// whole 256-byte row pieces per instruction (the register path above touches sixteen rows with 64
-// bytes each per instruction, which DRAM serves a third slower).  A wavefront owns HS macro steps
-// x RG row groups = HS * RG tiles of 4 KiB ([16 rows][16 chunks of 16 bytes], chunk c of row r at
-// position c ^ r so that fragment reads spread over all banks) and streams them through a private
-// ring of RING tiles: nothing but its own vmcnt orders the DMA against its reads.  The
-// activations are loaded into registers before the first DMA, so the count of outstanding loads
-// at any later point is a multiple of the four DMA instructions of a tile.
+// MB blocks of up to sixteen activation rows, K = 128 * pieces with NW * (HS - 1) < pieces <=
+// NW * HS (the wavefronts that have no piece in the last round read the last piece again against
+// zeroed activations).  Weights and activations come in by global -> LDS DMA, four whole 256-byte
+// row pieces per instruction (the register path above touches sixteen rows with 64 bytes each per
+// instruction, which DRAM serves a third slower).  A wavefront owns HS macro steps x (MB blocks
+// of activations + RG groups of sixteen weight rows) tiles of 4 KiB ([16 rows][16 chunks of 16
+// bytes], chunk c of row r at position c ^ r so that fragment reads spread over all banks) and
+// streams them through a private ring of RING tiles: nothing but its own vmcnt orders the DMA
+// against its reads, and every outstanding load is one of the four DMA instructions of a tile.
 #define ADR_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 #define ADR_GLB_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
 
-template <int NW, int RG, int HS, int RING, int MB, bool XR>
+template <int NW, int RG, int HS, int RING, int MB>
 __global__ __launch_bounds__(NW * 64) void skinny_f16_ring_kernel(MatmulArgs a) {
   constexpr int TILE = 16 * 256, MACRO = 128;
-  // XR: the activations of a macro step travel through the ring as MB more tiles ahead of the
-  // step's weight tiles (whole 256-byte row pieces from L2 instead of 64-byte ones, and sixteen
-  // registers of activations per block instead of sixteen per block and macro step)
-  constexpr int PER = XR ? RG + MB : RG;
+  // the activations of a macro step travel through the ring as MB more tiles ahead of the
+  // step's weight tiles (loaded straight into registers in MFMA layout they came as 64-byte
+  // pieces from L2 and took sixteen registers per block and macro step: m=16 K11008 N4096
+  // 27.7 us against 23.5)
+  constexpr int PER = RG + MB;
   constexpr int UNITS = HS * PER;
   static_assert(RING <= UNITS && NW * MB * RG * 256 * 4 <= NW * RING * TILE, "partials reuse the ring");
   __shared__ __attribute__((aligned(1024))) unsigned char ring[NW * RING * TILE];
@@ -221,32 +221,18 @@ __global__ __launch_bounds__(NW * 64) void skinny_f16_ring_kernel(MatmulArgs a) 
   const int r = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * (16 * RG);
   bool xvalid[MB];  // MB blocks of sixteen activation rows
-  const half_t* xrow[MB];
 #pragma unroll
-  for (int b = 0; b < MB; b++) {
-    xvalid[b] = b * 16 + r < a.m;
-    xrow[b] = a.lhs + (int64_t)min(b * 16 + r, a.m - 1) * a.stride_ly + g * 8;
-  }
+  for (int b = 0; b < MB; b++) xvalid[b] = b * 16 + r < a.m;
   unsigned char* const mine = ring + wave * RING * TILE;
   const int pieces = a.k / MACRO;
   const bool last_valid = wave + (HS - 1) * NW < pieces;
   const int last_piece = min(wave + (HS - 1) * NW, pieces - 1);
-  // registers first: the activations of all macro steps of the wavefront (rows past m read row
-  // m - 1 again and are zeroed when used)
-  u32x4_t x[MB][XR ? 1 : HS][4];
-#pragma unroll
-  for (int b = 0; b < MB; b++)
-#pragma unroll
-    for (int h = 0; h < (XR ? 0 : HS); h++)
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const int piece = h == HS - 1 ? last_piece : wave + h * NW;
-        x[b][h][j] = *(const u32x4_t*)(xrow[b] + (int64_t)piece * MACRO + j * 32);
-        if (h == HS - 1 && !last_valid) x[b][h][j] = u32x4_t{0, 0, 0, 0};
-      }
+  u32x4_t x[MB][4];  // the activations of the current macro step (rows past m read row m - 1
+                     // and are zeroed when used)
   // DMA instruction i of a tile fills its chunks [64 i, 64 i + 64): rows 4i .. 4i+3
-  auto issue = [&](int u) {  // tile u = (macro step u / RG of the wavefront, row group u % RG)
-    const int h = u / PER, q = u % PER - (XR ? MB : 0);  // q < 0: activation block q + MB
+  auto issue = [&](int u) {  // tile u: macro step u / PER of the wavefront, then MB activation
+                             // blocks and RG weight row groups in turn
+    const int h = u / PER, q = u % PER - MB;  // q < 0: activation block q + MB
     const int piece = h == HS - 1 ? last_piece : wave + h * NW;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
@@ -276,7 +262,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_f16_ring_kernel(MatmulArgs a) 
     else if (later == 8) __builtin_amdgcn_s_waitcnt(0x0F70 | 8);
     else if (later == 4) __builtin_amdgcn_s_waitcnt(0x0F70 | 4);
     else __builtin_amdgcn_s_waitcnt(0x0F70 | 0);
-    const int h = u / PER, q = u % PER - (XR ? MB : 0);
+    const int h = u / PER, q = u % PER - MB;
     const unsigned char* tile = mine + (u % RING) * TILE;
     u32x4_t w[4];
 #pragma unroll
@@ -289,7 +275,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_f16_ring_kernel(MatmulArgs a) 
     const u32x4_t z = {0, 0, 0, 0};
     if (q < 0) {  // the step's activations
 #pragma unroll
-      for (int j = 0; j < 4; j++) x[q < 0 ? q + MB : 0][0][j] = (h == HS - 1 && !last_valid) ? z : w[j];
+      for (int j = 0; j < 4; j++) x[q < 0 ? q + MB : 0][j] = (h == HS - 1 && !last_valid) ? z : w[j];
       continue;
     }
 #pragma unroll
@@ -297,7 +283,7 @@ __global__ __launch_bounds__(NW * 64) void skinny_f16_ring_kernel(MatmulArgs a) 
       const u32x4_t wv = w[j];
 #pragma unroll
       for (int b = 0; b < MB; b++) {
-        const u32x4_t xv = xvalid[b] ? x[b][XR ? 0 : h][j] : z;
+        const u32x4_t xv = xvalid[b] ? x[b][j] : z;
         acc[b][q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
             __builtin_bit_cast(half8_t, wv), __builtin_bit_cast(half8_t, xv), acc[b][q], 0, 0, 0);
       }
@@ -334,9 +320,9 @@ __global__ __launch_bounds__(NW * 64) void skinny_f16_ring_kernel(MatmulArgs a) 
   }
 }
 
-template <int NW, int RG, int HS, int RING, int MB = 1, bool XR = false>
+template <int NW, int RG, int HS, int RING, int MB>
 hipError_t launch_ring(hipStream_t stream, const MatmulArgs& a) {
-  hipLaunchKernelGGL((skinny_f16_ring_kernel<NW, RG, HS, RING, MB, XR>), dim3((a.n + 16 * RG - 1) / (16 * RG)),
+  hipLaunchKernelGGL((skinny_f16_ring_kernel<NW, RG, HS, RING, MB>), dim3((a.n + 16 * RG - 1) / (16 * RG)),
                      dim3(NW * 64), 0, stream, a);
   return hipGetLastError();
 }
@@ -416,9 +402,9 @@ hipError_t launch_gemv_f16(hipStream_t stream, const MatmulArgs& a) {
       switch ((a.k + 1023) / 1024) {
 #define ADR_RING_CASE(HS)                                                         \
         case HS:                                                                  \
-          if (rg == 3) return launch_ring<8, 3, HS, 4, 1, true>(stream, a);       \
-          if (rg == 2) return launch_ring<8, 2, HS, 3, 1, true>(stream, a);       \
-          return launch_ring<8, 1, HS, 4, 1, true>(stream, a);
+          if (rg == 3) return launch_ring<8, 3, HS, 4, 1>(stream, a);             \
+          if (rg == 2) return launch_ring<8, 2, HS, 3, 1>(stream, a);             \
+          return launch_ring<8, 1, HS, 4, 1>(stream, a);      
         ADR_RING_CASE(2) ADR_RING_CASE(3) ADR_RING_CASE(4) ADR_RING_CASE(5) ADR_RING_CASE(8)
         ADR_RING_CASE(11)
 #undef ADR_RING_CASE
@@ -431,9 +417,9 @@ hipError_t launch_gemv_f16(hipStream_t stream, const MatmulArgs& a) {
       switch ((a.k + 1023) / 1024) {
 #define ADR_RING_CASE(HS)                                                         \
         case HS:                                                                  \
-          if (rg == 3) return launch_ring<8, 3, HS, 4, 2, true>(stream, a);       \
-          if (rg == 2) return launch_ring<8, 2, HS, 4, 2, true>(stream, a);       \
-          return launch_ring<8, 1, HS, 3, 2, true>(stream, a);
+          if (rg == 3) return launch_ring<8, 3, HS, 4, 2>(stream, a);             \
+          if (rg == 2) return launch_ring<8, 2, HS, 4, 2>(stream, a);             \
+          return launch_ring<8, 1, HS, 3, 2>(stream, a);      
         ADR_RING_CASE(2) ADR_RING_CASE(3) ADR_RING_CASE(4) ADR_RING_CASE(5) ADR_RING_CASE(8)
         ADR_RING_CASE(11)
 #undef ADR_RING_CASE
