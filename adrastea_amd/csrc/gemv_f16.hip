@@ -367,7 +367,11 @@ static bool skinny_ok(const MatmulArgs& a) {
   // measured against the tiled kernels for 9..32 rows on N 4096..12288, K 4096 and 11008: never
   // slower (K11008 N4096 m=16: 27.5 against 65.9 us; K4096 N12288 m=32: 30.8 against 32.8);
   // from five rows on also ahead of the dot-product kernel (m=8, K4096 N12288: 21 against 24.9)
-  return a.m >= 5 && a.m <= 32 && a.k % 128 == 0 && a.k >= 1024 && (int64_t)a.n * a.k >= (1 << 22);
+  if (a.k % 128 != 0 || a.k < 1024 || (int64_t)a.n * a.k < (1 << 22)) return false;
+  if (a.m >= 5 && a.m <= 32) return true;
+  // 33 to 64 rows: only the ring kernel, for the K classes built with three and four blocks
+  const int hs = (a.k + 1023) / 1024;
+  return a.m > 32 && a.m <= 64 && (hs == 4 || hs == 11);
 }
 
 enum SkinnyChoice { SKINNY_NONE, SKINNY_DOT, SKINNY_MFMA };
@@ -409,6 +413,26 @@ hipError_t launch_gemv_f16(hipStream_t stream, const MatmulArgs& a) {
         ADR_RING_CASE(11)
 #undef ADR_RING_CASE
         default: break;
+      }
+    }
+    // 33 to 64 rows, three and four blocks of activations, against the tiled kernels: K11008
+    // N4096 m=33 46.3 -> 27.7 us, m=64 53.0 -> 34.1; K4096 N4096 13.8 -> 11.3, 14.4 -> 13.3; N12288
+    // 25.7 -> 25.0, 29.0 -> 29.3
+    if (a.m > 32) {
+      switch ((a.k + 1023) / 1024) {
+#define ADR_RING_CASE(HS)                                                                          \
+        case HS:                                                                                   \
+          if (a.m <= 48) {                                                                         \
+            if (rg == 3) return launch_ring<8, 3, HS, 4, 3>(stream, a);                            \
+            if (rg == 2) return launch_ring<8, 2, HS, 4, 3>(stream, a);                            \
+            return launch_ring<8, 1, HS, 4, 3>(stream, a);                                         \
+          }                                                                                        \
+          if (rg == 3) return launch_ring<8, 3, HS, 4, 4>(stream, a);                              \
+          if (rg == 2) return launch_ring<8, 2, HS, 4, 4>(stream, a);                              \
+          return launch_ring<8, 1, HS, 4, 4>(stream, a);
+        ADR_RING_CASE(4) ADR_RING_CASE(11)
+#undef ADR_RING_CASE
+        default: return hipErrorInvalidValue;
       }
     }
     // 17 to 32 rows: two blocks of activations (m=32, K4096, in registers: N4096 15.0 -> 13.6 us,

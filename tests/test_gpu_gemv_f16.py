@@ -122,9 +122,12 @@ def test_nt_entry_point_with_beta():
                                    # 17 to 32 rows through the ring: K up to 4096
                                    (17, 4096, 6200), (32, 2048, 12288), (25, 3072, 4100), (32, 4096, 12288),
                                    (20, 3968, 10300), (32, 11008, 4096), (19, 8192, 6200), (27, 5120, 10300),
+                                   # 33 to 64 rows: three and four blocks, K classes of 4096 and 11008
+                                   (33, 4096, 4100), (48, 4096, 6200), (49, 3968, 12288), (64, 11008, 4096),
+                                   (40, 10368, 1000), (64, 4096, 12288),
                                    # five to eight rows take these kernels too
                                    (5, 4096, 4100), (8, 11008, 4096), (7, 1152, 4000)])
-def test_matrix_core_kernel_for_five_to_thirty_two_rows(m, K, N):
+def test_matrix_core_kernel_for_five_to_sixty_four_rows(m, K, N):
     so, sl, sr = nt(m, K, N)
     assert plan(1, m, K, N, so, sl, sr) == PLAN_MFMA
     g = rng(2400 + m + K + N)
@@ -152,6 +155,6 @@ def test_matrix_core_kernel_for_five_to_thirty_two_rows(m, K, N):
 
 
 def test_more_rows_or_short_k_stay_on_the_tiled_kernels():
-    for m, K, N in [(33, 4096, 4096), (33, 11008, 4096), (12, 960, 8192)]:
+    for m, K, N in [(65, 4096, 4096), (65, 11008, 4096), (33, 2048, 8192), (12, 960, 8192)]:
         so, sl, sr = nt(m, K, N)
         assert plan(1, m, K, N, so, sl, sr).startswith("gemm_nt_mfma")
