@@ -378,6 +378,13 @@ enum SkinnyChoice { SKINNY_NONE, SKINNY_DOT, SKINNY_MFMA };
 
 static SkinnyChoice choose_skinny(const MatmulArgs& a) {
   if (!layout_ok(a)) return SKINNY_NONE;
+  // three and four rows on a matrix of at most 256 groups of 16 weight rows (one workgroup per
+  // CU) and K up to 4096: the ring kernel is ahead already (m=4: K4096 N4096 9.4 -> 7.8 us, K2048
+  // N4096 6.9 -> 5.6, K3072 N3072 7.0 -> 5.3; with N 6000 12.3 -> 13.0 and with K 11008 19.3 ->
+  // 22.2, so not there; two rows: 7.7 either way)
+  const bool narrow = a.m >= 3 && a.m <= 4 && a.n <= 16 * 256 && a.k <= 4096 && a.k > 1024 &&
+                      a.k % 128 == 0 && (int64_t)a.n * a.k >= (1 << 22);
+  if (narrow) return SKINNY_MFMA;
   if (a.m <= 4 && dot_ok(a)) return SKINNY_DOT;
   if (skinny_ok(a)) return SKINNY_MFMA;
   return dot_ok(a) ? SKINNY_DOT : SKINNY_NONE;
@@ -418,6 +425,7 @@ hipError_t launch_gemv_f16(hipStream_t stream, const MatmulArgs& a) {
     // 33 to 64 rows, three and four blocks of activations, against the tiled kernels: K11008
     // N4096 m=33 46.3 -> 27.7 us, m=64 53.0 -> 34.1; K4096 N4096 13.8 -> 11.3, 14.4 -> 13.3; N12288
     // 25.7 -> 25.0, 29.0 -> 29.3
+    if (a.m > 64) return hipErrorInvalidValue;  // (never chosen)
     if (a.m > 32) {
       switch ((a.k + 1023) / 1024) {
 #define ADR_RING_CASE(HS)                                                                          \

@@ -25,9 +25,11 @@ def nt(M, K, N):
                                  (4096, 1100), (11008, 400)])
 def test_matches_oracle_and_is_exact_on_exact_inputs(m, K, N):
     so, sl, sr = nt(m, K, N)
-    # up to four rows: dot products; five to eight: dot products only where K is no multiple of 128
-    # (or the matrix is small); more: other kernels
-    mfma = m >= 5 and K % 128 == 0 and K >= 1024 and N * K >= (1 << 22)
+    # up to four rows: dot products, but for three and four rows on a narrow matrix with K up to
+    # 4096; five to eight: dot products only where K is no multiple of 128 (or the matrix is
+    # small); more: other kernels
+    mfma = K % 128 == 0 and K >= 1024 and N * K >= (1 << 22) and (
+        m >= 5 or (m >= 3 and N <= 4096 and 1024 < K <= 4096))
     if mfma:
         assert plan(1, m, K, N, so, sl, sr) == PLAN_MFMA
     elif m <= 8:
@@ -125,7 +127,8 @@ def test_nt_entry_point_with_beta():
                                    # 33 to 64 rows: three and four blocks, K classes of 4096 and 11008
                                    (33, 4096, 4100), (48, 4096, 6200), (49, 3968, 12288), (64, 11008, 4096),
                                    (40, 10368, 1000), (64, 4096, 12288),
-                                   # five to eight rows take these kernels too
+                                   # three and four rows on narrow matrices, five to eight rows
+                                   (3, 4096, 4096), (4, 2048, 4000), (4, 3072, 3072),
                                    (5, 4096, 4100), (8, 11008, 4096), (7, 1152, 4000)])
 def test_matrix_core_kernel_for_five_to_sixty_four_rows(m, K, N):
     so, sl, sr = nt(m, K, N)
