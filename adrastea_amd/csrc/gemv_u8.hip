@@ -358,15 +358,20 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_ring_kernel(half_t* __restric
 // whether or not the wavefront has a macro step left (the surplus ones read one 16-byte line and
 // are multiplied with zero scales), so the wait before a slot's use is "all but the 13 (RING - 1)
 // youngest" and no load sits under a branch.
-template <int NW, int RING, int ROUNDS>
+// XR: the slot's activations come through LDS too, as two more tiles of the slot ([16 rows][128
+// halves] each, same chunk swizzle) by eight DMA instructions in place of the eight loads, so
+// the count per slot stays thirteen; a slot is then 12 KiB, which fits with four wavefronts.
+template <int NW, int RING, int ROUNDS, bool XR>
 __global__ __launch_bounds__(NW * 64) void gemv_u8_ring_loop_kernel(half_t* __restrict__ out,
                                                                     const half_t* __restrict__ lhs,
                                                                     const uint8_t* __restrict__ rhs,
                                                                     const half_t* __restrict__ scales,
                                                                     int m, int p, int n, float beta) {
   constexpr int TILE = ROWS * MACRO_K;
+  constexpr int SLOT = XR ? 3 * TILE : TILE;  // weight tile, then the two activation tiles
   constexpr int PER = 8 + 1 + 4;  // activation loads, scale load, DMA instructions per slot
-  __shared__ __attribute__((aligned(1024))) unsigned char ring[NW * RING * TILE];
+  static_assert(NW * RING * SLOT <= 160 * 1024 && NW * 256 * 4 <= NW * RING * SLOT, "LDS");
+  __shared__ __attribute__((aligned(1024))) unsigned char ring[NW * RING * SLOT];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * ROWS;
@@ -375,30 +380,47 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_ring_loop_kernel(half_t* __re
   const int steps = p / MACRO_K;
   const half_t* xrow = lhs + (int64_t)min(r, m - 1) * p + g * 16;
   const half_t* srow = scales + (int64_t)min(n0 + r, n - 1) * nblk;
-  unsigned char* const mine = ring + wave * RING * TILE;
+  unsigned char* const mine = ring + wave * RING * SLOT;
   // DMA instruction i of a tile fills its chunks [64 i, 64 i + 64): rows 4i .. 4i+3
   const uint8_t* wsrc[4];
+  const half_t* xsrc[4];
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     const int row = 4 * i + (lane >> 4), kc = (lane & 15) ^ row;
     wsrc[i] = rhs + (int64_t)min(n0 + row, n - 1) * p + kc * 16;
+    xsrc[i] = lhs + (int64_t)min(row, m - 1) * p + kc * 8;
   }
   int roff[4];  // fragment read j of the lane: logical chunk 4j + g of row r
 #pragma unroll
   for (int j = 0; j < 4; j++) roff[j] = r * 256 + (((4 * j + g) ^ r) << 4);
+  int xoff[4];  // activation fragment 2 jj + e of a tile: logical chunk 8 jj + 2 g + e of row r
+#pragma unroll
+  for (int f = 0; f < 4; f++) xoff[f] = r * 256 + (((8 * (f >> 1) + 2 * g + (f & 1)) ^ r) << 4);
 
-  u32x4_t x[RING][8];
+  u32x4_t x[XR ? 1 : RING][8];
   u32x4_t sc[RING];
   auto issue = [&](int slot, int ms) {
     const bool live = ms < steps;  // wave-uniform
     const int64_t koff = live ? (int64_t)ms * MACRO_K : 0;
     const half_t* xp = xrow + koff;
+    if constexpr (XR) {
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-      // lanes beyond m read row m-1 again (the same addresses as its own lanes) and are zeroed
-      // when used: a load under a lane mask would be waited for where the lanes rejoin
-      x[slot][2 * j] = *(const u32x4_t*)(xp + j * 64);
-      x[slot][2 * j + 1] = *(const u32x4_t*)(xp + j * 64 + 8);
+      for (int t = 0; t < 2; t++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          // (rows beyond m read row m - 1 again and are zeroed when used)
+          const half_t* src = live ? xsrc[i] + koff + t * 128 : lhs;
+          __builtin_amdgcn_global_load_lds(
+              ADR_GLB_PTR(src), ADR_LDS_PTR(mine + slot * SLOT + (1 + t) * TILE + i * 1024), 16, 0, 0);
+        }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        // lanes beyond m read row m-1 again (the same addresses as its own lanes) and are zeroed
+        // when used: a load under a lane mask would be waited for where the lanes rejoin
+        x[slot][2 * j] = *(const u32x4_t*)(xp + j * 64);
+        x[slot][2 * j + 1] = *(const u32x4_t*)(xp + j * 64 + 8);
+      }
     }
     sc[slot] = *(const u32x4_t*)(srow + (live ? ms * (MACRO_K / 32) : 0));
 #pragma unroll
@@ -406,7 +428,7 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_ring_loop_kernel(half_t* __re
       // a surplus slot fetches one 16-byte line (all lanes the same address)
       const uint8_t* src = live ? wsrc[i] + koff : rhs;
       __builtin_amdgcn_global_load_lds(ADR_GLB_PTR(src),
-                                       ADR_LDS_PTR(mine + slot * TILE + i * 1024), 16, 0, 0);
+                                       ADR_LDS_PTR(mine + slot * SLOT + i * 1024), 16, 0, 0);
     }
   };
   float4_t acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
@@ -424,10 +446,16 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_ring_loop_kernel(half_t* __re
       if (later == 2 * PER) __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * PER) & 0xF) | (((2 * PER) >> 4) << 14));
       else if (later == PER) __builtin_amdgcn_s_waitcnt(0x0F70 | (PER & 0xF) | ((PER >> 4) << 14));
       else __builtin_amdgcn_s_waitcnt(0x0F70);
-      const unsigned char* tile = mine + i * TILE;
+      const unsigned char* tile = mine + i * SLOT;
       u32x4_t w[4];
 #pragma unroll
       for (int j = 0; j < 4; j++) w[j] = *(const u32x4_t*)(tile + roff[j]);
+      if constexpr (XR) {
+#pragma unroll
+        for (int f = 0; f < 8; f++) x[0][f] = *(const u32x4_t*)(tile + (1 + f / 4) * TILE + xoff[f % 4]);
+        // tile and activations are in registers before the slot is refilled below
+        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+      }
       // zero scales for a surplus slot: it adds nothing (selected here, not where the scales
       // are loaded: a use right behind the load would wait for it and everything before it)
       const u32x4_t z = {0, 0, 0, 0};
@@ -438,8 +466,8 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_ring_loop_kernel(half_t* __re
         const half_t sv = g < 2 ? s8[2 * j] : s8[2 * j + 1];
         const half2_t s2 = {sv, sv};
         const half8_t a0 = dequant8(w[j][0], w[j][1], s2), a1 = dequant8(w[j][2], w[j][3], s2);
-        const half8_t b0 = __builtin_bit_cast(half8_t, xvalid ? x[i][2 * j] : z);
-        const half8_t b1 = __builtin_bit_cast(half8_t, xvalid ? x[i][2 * j + 1] : z);
+        const half8_t b0 = __builtin_bit_cast(half8_t, xvalid ? x[XR ? 0 : i][2 * j] : z);
+        const half8_t b1 = __builtin_bit_cast(half8_t, xvalid ? x[XR ? 0 : i][2 * j + 1] : z);
         acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, b0, acc0, 0, 0, 0);
         acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, b1, acc1, 0, 0, 0);
       }
@@ -684,16 +712,23 @@ hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, co
                            lhs, rhs, scales, m, p, n, beta);
         return hipGetLastError();
       }
+      // ten rows and more, K 9472 .. 12288: four wavefronts, activations through LDS (K11008
+      // N4096: m=16 19.7 -> 17.1 us, m=12 17.8 -> 16.5; m=8 16.3 -> 16.9, so not below ten)
+      if (steps > 16 && m >= 10 && ((steps + 3) / 4 + 2) / 3 == 4) {
+        hipLaunchKernelGGL((gemv_u8_ring_loop_kernel<4, 3, 4, true>), dim3(blocks), dim3(256), 0, stream,
+                           out, lhs, rhs, scales, m, p, n, beta);
+        return hipGetLastError();
+      }
       if (steps > 16) {
         const int rounds = ((steps + 7) / 8 + 2) / 3;
         if (rounds == 1)
-          hipLaunchKernelGGL((gemv_u8_ring_loop_kernel<8, 3, 1>), dim3(blocks), dim3(512), 0, stream,
+          hipLaunchKernelGGL((gemv_u8_ring_loop_kernel<8, 3, 1, false>), dim3(blocks), dim3(512), 0, stream,
                              out, lhs, rhs, scales, m, p, n, beta);
         else if (rounds == 2)
-          hipLaunchKernelGGL((gemv_u8_ring_loop_kernel<8, 3, 2>), dim3(blocks), dim3(512), 0, stream,
+          hipLaunchKernelGGL((gemv_u8_ring_loop_kernel<8, 3, 2, false>), dim3(blocks), dim3(512), 0, stream,
                              out, lhs, rhs, scales, m, p, n, beta);
         else if (rounds == 3)
-          hipLaunchKernelGGL((gemv_u8_ring_loop_kernel<8, 3, 3>), dim3(blocks), dim3(512), 0, stream,
+          hipLaunchKernelGGL((gemv_u8_ring_loop_kernel<8, 3, 3, false>), dim3(blocks), dim3(512), 0, stream,
                              out, lhs, rhs, scales, m, p, n, beta);
         if (rounds <= 3) return hipGetLastError();
       }

@@ -313,6 +313,29 @@ def test_decode_shapes_full_size(kern, kn, m):
     assert torch.equal(out2, (out * 2).half())
 
 
+@pytest.mark.parametrize("m", [10, 13, 16])
+@pytest.mark.parametrize("kn", [(11008, 1000), (9472, 530), (12288, 700)])
+def test_decode_ten_rows_and_more_long_k(kern, kn, m):
+    """K 9472 .. 12288 with ten to sixteen rows: the kernel whose activations travel through LDS;
+    ragged N, surplus ring slots (K 9472: 37 steps for 4 x 12 slots), previous output added."""
+    p, n = kn
+    gen = torch.Generator(device="cuda").manual_seed(46 + m + p)
+    q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)
+    s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
+    a = torch.randn(m, p, generator=gen, device="cuda").half()
+    prev = torch.randn(m, n, generator=gen, device="cuda").half()
+    assert u8_plan(m, p, n, 32) == "gemv_u8_mfma16_dma"
+    out = prev.clone()
+    assert _ffi.lib().adr_matmul_nt_fp16u8(torch.cuda.current_stream().cuda_stream, out.data_ptr(),
+                                           a.data_ptr(), q.data_ptr(), s.data_ptr(), m, p, n, 32, 0.5) == 0
+    w = torch.zeros(n, p, dtype=torch.float16, device="cuda")
+    kern.dequantize_absmax_uint8(w, s, q)
+    ref32 = a.float() @ w.float().t() + 0.5 * prev.float()
+    rms = ref32.pow(2).mean().sqrt()
+    rel = ((out.float() - ref32).abs() / torch.maximum(ref32.abs(), rms)).max().item()
+    assert rel <= 2e-3, rel
+
+
 def test_prefill_u8_gemm_full_size(kern):
     """benchmark config 5 (u8 variant), the O projection: M=2048, K=4096, N=4096."""
     m, p, n = 2048, 4096, 4096
