@@ -657,6 +657,15 @@ U8Choice choose_u8(const void* lhs, const void* rhs, const void* scales, int m, 
   return U8_NAIVE;
 }
 
+// 17 to 64 activation rows against at least 4 MiB of weights: the sixteen-row kernels once per
+// block of sixteen rows.  The tiled GEMM walks K on N / 64 .. N / 128 CUs for these (K4096 N4096
+// m=17..32 42.9 us, m=64 58.4; N12288 53.4 .. 67.0; K11008 N4096 133 .. 166) where a sixteen-row
+// launch takes 7.2 / 15.3 / 17.1 us.
+bool rows_in_blocks_of_16(int m, int p, int n, int block_size) {
+  return m > 16 && m <= 64 && (int64_t)n * p >= (1 << 22) &&
+         choose_u8(nullptr, nullptr, nullptr, 16, p, n, block_size) == U8_GEMV;
+}
+
 }  // namespace
 
 hipError_t launch_gemm_u8_mfma(hipStream_t stream, half_t* out, const half_t* lhs,
@@ -664,6 +673,7 @@ hipError_t launch_gemm_u8_mfma(hipStream_t stream, half_t* out, const half_t* lh
                                int block_size, float beta);
 
 const char* gemm_u8_plan(int m, int p, int n, int block_size) {
+  if (rows_in_blocks_of_16(m, p, n, block_size)) m = 16;
   switch (choose_u8(nullptr, nullptr, nullptr, m, p, n, block_size)) {
     case U8_DOT: return "gemv_u8_dot2_stream";
     case U8_GEMV:
@@ -677,6 +687,16 @@ const char* gemm_u8_plan(int m, int p, int n, int block_size) {
 
 hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, const uint8_t* rhs,
                           const half_t* scales, int m, int p, int n, int block_size, float beta) {
+  if (rows_in_blocks_of_16(m, p, n, block_size) &&
+      choose_u8(lhs, rhs, scales, 16, p, n, block_size) == U8_GEMV) {
+    // (p is a multiple of 256 here, so every block of rows starts 16-byte aligned)
+    for (int r0 = 0; r0 < m; r0 += 16) {
+      const hipError_t e = launch_gemm_u8(stream, out + (int64_t)r0 * n, lhs + (int64_t)r0 * p, rhs,
+                                          scales, min(16, m - r0), p, n, block_size, beta);
+      if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+  }
   switch (choose_u8(lhs, rhs, scales, m, p, n, block_size)) {
     case U8_DOT: {
       const bool wide = n > 6144;

@@ -336,6 +336,31 @@ def test_decode_ten_rows_and_more_long_k(kern, kn, m):
     assert rel <= 2e-3, rel
 
 
+@pytest.mark.parametrize("m", [17, 32, 33, 50, 64])
+@pytest.mark.parametrize("kn", [(4096, 4100), (4096, 8200), (11008, 1000), (2048, 2100)])
+def test_seventeen_to_sixty_four_rows_in_blocks_of_sixteen(kern, kn, m):
+    """17 to 64 rows on matrices of 4 MiB and more run the sixteen-row kernels per block of rows
+    (a last block of one or two rows takes the dot-product kernel); 65 rows stay on the tiled
+    GEMM.  Previous output added, ragged N."""
+    p, n = kn
+    assert u8_plan(m, p, n, 32) == u8_plan(16, p, n, 32)
+    assert u8_plan(65, p, n, 32) == "gemm_nt_u8_mfma"
+    gen = torch.Generator(device="cuda").manual_seed(47 + m + p)
+    q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)
+    s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
+    a = torch.randn(m, p, generator=gen, device="cuda").half()
+    prev = torch.randn(m, n, generator=gen, device="cuda").half()
+    out = prev.clone()
+    assert _ffi.lib().adr_matmul_nt_fp16u8(torch.cuda.current_stream().cuda_stream, out.data_ptr(),
+                                           a.data_ptr(), q.data_ptr(), s.data_ptr(), m, p, n, 32, 0.5) == 0
+    w = torch.zeros(n, p, dtype=torch.float16, device="cuda")
+    kern.dequantize_absmax_uint8(w, s, q)
+    ref32 = a.float() @ w.float().t() + 0.5 * prev.float()
+    rms = ref32.pow(2).mean().sqrt()
+    rel = ((out.float() - ref32).abs() / torch.maximum(ref32.abs(), rms)).max().item()
+    assert rel <= 2e-3, rel
+
+
 def test_prefill_u8_gemm_full_size(kern):
     """benchmark config 5 (u8 variant), the O projection: M=2048, K=4096, N=4096."""
     m, p, n = 2048, 4096, 4096
