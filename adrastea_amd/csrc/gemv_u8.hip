@@ -657,12 +657,13 @@ U8Choice choose_u8(const void* lhs, const void* rhs, const void* scales, int m, 
   return U8_NAIVE;
 }
 
-// 17 to 64 activation rows against at least 4 MiB of weights: the sixteen-row kernels once per
-// block of sixteen rows.  The tiled GEMM walks K on N / 64 .. N / 128 CUs for these (K4096 N4096
-// m=17..32 42.9 us, m=64 58.4; N12288 53.4 .. 67.0; K11008 N4096 133 .. 166) where a sixteen-row
-// launch takes 7.2 / 15.3 / 17.1 us.
+// 17 to 64 activation rows (to 128 on matrices under 8192 rows) against at least 4 MiB of
+// weights: the sixteen-row kernels once per block of sixteen rows.  The tiled GEMM walks K on
+// N / 64 .. N / 128 CUs for these (K4096 N4096 m=17..32 42.9 us, m=64..128 58.5; N12288 53.4 ..
+// 68.5; K11008 N4096 133 .. 171) where a sixteen-row launch takes 7.2 / 15.3 / 17.1 us (N12288
+// m=96: 78.4 us in blocks against 68.3 tiled, hence the narrower bound there).
 bool rows_in_blocks_of_16(int m, int p, int n, int block_size) {
-  return m > 16 && m <= 64 && (int64_t)n * p >= (1 << 22) &&
+  return m > 16 && m <= (n < 8192 ? 128 : 64) && (int64_t)n * p >= (1 << 22) &&
          choose_u8(nullptr, nullptr, nullptr, 16, p, n, block_size) == U8_GEMV;
 }
 

@@ -336,15 +336,16 @@ def test_decode_ten_rows_and_more_long_k(kern, kn, m):
     assert rel <= 2e-3, rel
 
 
-@pytest.mark.parametrize("m", [17, 32, 33, 50, 64])
+@pytest.mark.parametrize("m", [17, 32, 33, 50, 64, 100, 128])
 @pytest.mark.parametrize("kn", [(4096, 4100), (4096, 8200), (11008, 1000), (2048, 2100)])
-def test_seventeen_to_sixty_four_rows_in_blocks_of_sixteen(kern, kn, m):
-    """17 to 64 rows on matrices of 4 MiB and more run the sixteen-row kernels per block of rows
-    (a last block of one or two rows takes the dot-product kernel); 65 rows stay on the tiled
-    GEMM.  Previous output added, ragged N."""
+def test_seventeen_and_more_rows_in_blocks_of_sixteen(kern, kn, m):
+    """17 to 64 rows (to 128 where N < 8192) on matrices of 4 MiB and more run the sixteen-row
+    kernels per block of rows (a last block of one or two rows takes the dot-product kernel);
+    more rows stay on the tiled GEMM.  Previous output added, ragged N."""
     p, n = kn
-    assert u8_plan(m, p, n, 32) == u8_plan(16, p, n, 32)
-    assert u8_plan(65, p, n, 32) == "gemm_nt_u8_mfma"
+    limit = 128 if n < 8192 else 64
+    assert u8_plan(m, p, n, 32) == (u8_plan(16, p, n, 32) if m <= limit else "gemm_nt_u8_mfma")
+    assert u8_plan(limit + 1, p, n, 32) == "gemm_nt_u8_mfma"
     gen = torch.Generator(device="cuda").manual_seed(47 + m + p)
     q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)
     s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
