@@ -1435,7 +1435,11 @@ GemmChoice choose(const MatmulArgs& a) {
     return c;
   }
   if (a.rhs_q && a.k % 64 == 0 && a.block_size >= 8 && (a.block_size & (a.block_size - 1)) == 0 &&
-      (int64_t)a.m * a.n >= 256 * 1024) {
+      (int64_t)a.m * a.n >= 256 * 1024 &&
+      // (with at most 64 of its 256 x 128 tiles the staged kernels' smaller tiles reach more CUs:
+      // N4096 m=129..512, K4096 59..65 -> 43..50 us, K11008 171..187 -> 129..141; with 96 tiles and
+      // more, N12288, they lose: 69..76 -> 91..126)
+      (int64_t)((a.m + 255) / 256) * ((a.n + 127) / 128) > 64) {
     static const Candidate u8[] = {{U8_256x192, 256, 192, 1, 1.10f}, {U8_256x128, 256, 128, 1, 1.00f}};
     return pick(a, u8, 2);
   }

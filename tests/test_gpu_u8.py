@@ -362,6 +362,29 @@ def test_seventeen_and_more_rows_in_blocks_of_sixteen(kern, kn, m):
     assert rel <= 2e-3, rel
 
 
+@pytest.mark.parametrize("mpn", [(300, 4096, 4096), (512, 2048, 4090), (129, 11008, 1000)])
+def test_mid_row_counts_take_the_smaller_staged_tiles(kern, mpn):
+    """With at most 64 tiles of 256 x 128 the u8 product runs on the staged kernels' smaller tiles;
+    same arithmetic bar as the large-tile kernel."""
+    m, p, n = mpn
+    assert (m + 255) // 256 * ((n + 127) // 128) <= 64
+    assert u8_plan(m, p, n, 32) == "gemm_nt_u8_mfma"   # (one name for all tiled u8 kernels)
+    gen = torch.Generator(device="cuda").manual_seed(48 + m)
+    q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)
+    s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
+    a = torch.randn(m, p, generator=gen, device="cuda").half()
+    prev = torch.randn(m, n, generator=gen, device="cuda").half()
+    out = prev.clone()
+    assert _ffi.lib().adr_matmul_nt_fp16u8(torch.cuda.current_stream().cuda_stream, out.data_ptr(),
+                                           a.data_ptr(), q.data_ptr(), s.data_ptr(), m, p, n, 32, 0.5) == 0
+    w = torch.zeros(n, p, dtype=torch.float16, device="cuda")
+    kern.dequantize_absmax_uint8(w, s, q)
+    ref32 = a.float() @ w.float().t() + 0.5 * prev.float()
+    rms = ref32.pow(2).mean().sqrt()
+    rel = ((out.float() - ref32).abs() / torch.maximum(ref32.abs(), rms)).max().item()
+    assert rel <= 2e-3, rel
+
+
 def test_prefill_u8_gemm_full_size(kern):
     """benchmark config 5 (u8 variant), the O projection: M=2048, K=4096, N=4096."""
     m, p, n = 2048, 4096, 4096
