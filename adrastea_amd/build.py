@@ -21,7 +21,8 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
 
 SOURCES = ["api.hip", "matmul_general.hip", "gemm_mfma.hip", "gemv_u8.hip", "quantize.hip",
-           "softmax.hip", "attention.hip", "error_stats.hip", "microbench.hip", "gemv_f16.hip"]
+           "softmax.hip", "attention.hip", "error_stats.hip", "microbench.hip", "gemv_f16.hip",
+           "device.hip"]
 
 # packed-fp32 instructions are switched off for all device code (some forms have produced
 # wrong results on this hardware generation); the host pass warns that it does not know the

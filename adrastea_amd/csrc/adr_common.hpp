@@ -193,6 +193,18 @@ __device__ __forceinline__ float wave_sum_dpp(float v) {
   return v;
 }
 
+// The current device as the launchers see it (device.hip): status is ADR_OK on a gfx950 device,
+// ADR_EUNSUPPORTED_DEVICE on any other, or the hipError_t of the failed query; cus / xcds are the
+// device's compute-unit and die (XCD) counts -- MI355X: 256 and 8, which are also the values
+// reported beside a non-zero status.  Queried once per device, immutable afterwards.
+struct DeviceInfo {
+  int status;
+  int cus;
+  int xcds;
+};
+DeviceInfo device_info();
+DeviceInfo device_info_for_plan();  // as above, but an MI355X where no usable device is current
+
 // Launchers implemented in the kernel translation units; all return a hipError_t.
 hipError_t launch_matmul_general(hipStream_t stream, const MatmulArgs& a);
 // Returns true and fills `name` when the MFMA kernel family covers these arguments.

@@ -15,6 +15,21 @@ int validate_matmul(const MatmulArgs& a, bool check_ptrs) {
     return ADR_EINVAL_ENUM;
   if (a.store == ADR_STORE_GELU_BIAS) return ADR_ENOTIMPL;
   if (a.batches < 0 || a.m < 0 || a.n < 0 || a.k < 0) return ADR_EINVAL_SHAPE;
+  // Element offsets are 32-bit integers in the reference (every kernel argument is an i32,
+  // kernels.rs:864-887, and its kernels index with int): a view whose farthest element lies at or
+  // beyond 2^31 elements cannot be addressed there, and is rejected here rather than wrapped.
+  if (a.batches && a.m && a.n) {
+    auto span = [](int64_t d0, int64_t s0, int64_t d1, int64_t s1, int64_t d2, int64_t s2) {
+      auto mag = [](int64_t v) { return v < 0 ? -v : v; };
+      return (d0 ? (d0 - 1) * mag(s0) : 0) + (d1 ? (d1 - 1) * mag(s1) : 0) +
+             (d2 ? (d2 - 1) * mag(s2) : 0);
+    };
+    const int64_t lim = (int64_t)1 << 31;
+    if (span(a.n, a.stride_ox, a.m, a.stride_oy, a.batches, a.stride_oz) >= lim ||
+        span(a.k, a.stride_lx, a.m, a.stride_ly, a.batches, a.stride_lz) >= lim ||
+        span(a.n, a.stride_rx, a.k, a.stride_ry, a.batches, a.stride_rz) >= lim)
+      return ADR_EINVAL_SHAPE;
+  }
   if (check_ptrs) {
     if (a.batches && a.m && a.n) {
       if (!a.output || (a.k && (!a.lhs || !a.rhs))) return ADR_ENULL;
@@ -46,8 +61,13 @@ MatmulArgs pack(uint16_t* output, const uint16_t* lhs, const uint16_t* rhs, int3
 
 bool empty(const MatmulArgs& a) { return a.batches == 0 || a.m == 0 || a.n == 0; }
 
+// Every launching entry point starts here: ADR_EUNSUPPORTED_DEVICE unless the current device is
+// a gfx950 (the kernels are built for nothing else), or the error of the failed device query.
+int check_device() { return device_info().status; }
+
 int run_matmul(hipStream_t stream, const MatmulArgs& a, bool allow_fast) {
   if (empty(a)) return ADR_OK;
+  if (int rc = check_device()) return rc;
   const char* name;
   if (allow_fast && gemv_f16_supported(a, &name)) return (int)launch_gemv_f16(stream, a);
   if (allow_fast && mfma_gemm_supported(a, &name)) return (int)launch_mfma_gemm(stream, a);
@@ -155,6 +175,9 @@ int adr_matmul_nt_f16(adr_stream_t stream, uint16_t* output, const uint16_t* lhs
   if (m < 0 || p < 0 || n < 0) return ADR_EINVAL_SHAPE;
   if (m == 0 || n == 0) return ADR_OK;
   if (!output || (p && (!lhs || !rhs))) return ADR_ENULL;
+  if ((int64_t)m * n >= ((int64_t)1 << 31) || (int64_t)m * p >= ((int64_t)1 << 31) ||
+      (int64_t)n * p >= ((int64_t)1 << 31))
+    return ADR_EINVAL_SHAPE;  // (32-bit element offsets, as in adr_matmul_f16)
   MatmulArgs a = pack(output, lhs, rhs, 1, m, p, n, 1, n, 0, 1, p, 0, p, 1, 0, nullptr, beta, 1.0f,
                       STORE_ACC_BETA, ADR_LOAD_IDENTITY, ADR_MASK_NONE);
   return run_matmul((hipStream_t)stream, a, true);
@@ -167,6 +190,10 @@ int adr_matmul_nt_fp16u8(adr_stream_t stream, uint16_t* output, const uint16_t* 
   if (p % block_size != 0) return ADR_EDIVISIBILITY;
   if (m == 0 || n == 0) return ADR_OK;
   if (!output || (p && (!lhs || !rhs || !scales))) return ADR_ENULL;
+  if ((int64_t)m * n >= ((int64_t)1 << 31) || (int64_t)m * p >= ((int64_t)1 << 31) ||
+      (int64_t)n * p >= ((int64_t)1 << 31))
+    return ADR_EINVAL_SHAPE;  // (32-bit element offsets, as in adr_matmul_f16)
+  if (int rc = check_device()) return rc;
   return (int)launch_gemm_u8((hipStream_t)stream, (half_t*)output, (const half_t*)lhs, rhs,
                              (const half_t*)scales, m, p, n, block_size, beta);
 }
@@ -187,6 +214,7 @@ int adr_dequantize_absmax_uint8(adr_stream_t stream, adr_tensor_desc output,
                                 adr_tensor_desc scales, adr_tensor_desc input) {
   if (int rc = validate_quant(output, scales, input)) return rc;
   if (output.shape[0] == 0 || output.shape[1] == 0) return ADR_OK;
+  if (int rc = check_device()) return rc;
   return (int)launch_dequantize((hipStream_t)stream, output, scales, input);
 }
 
@@ -194,6 +222,7 @@ int adr_quantize_absmax_uint8(adr_stream_t stream, adr_tensor_desc output, adr_t
                               adr_tensor_desc input) {
   if (int rc = validate_quant(output, scales, input)) return rc;
   if (output.shape[0] == 0 || output.shape[1] == 0) return ADR_OK;
+  if (int rc = check_device()) return rc;
   return (int)launch_quantize((hipStream_t)stream, output, scales, input);
 }
 
@@ -225,6 +254,7 @@ int adr_embed_uint8(adr_stream_t stream, int32_t n_dim, int32_t n_ids, const int
   if (n_dim % block_size != 0) return ADR_EDIVISIBILITY;
   if (n_dim == 0 || n_ids == 0) return ADR_OK;
   if (!in_ids || !out_embeddings || !embeddings_table || !scales) return ADR_ENULL;
+  if (int rc = check_device()) return rc;
   return (int)launch_embed_u8((hipStream_t)stream, n_dim, n_ids, in_ids, (half_t*)out_embeddings,
                               embeddings_table, (const half_t*)scales, block_size);
 }
@@ -234,6 +264,7 @@ int adr_softmax_rows(adr_stream_t stream, uint16_t* output, const uint16_t* inpu
   if (heads < 0 || h < 0 || w < 0) return ADR_EINVAL_SHAPE;
   if (heads == 0 || h == 0 || w == 0) return ADR_OK;
   if (!output || !input) return ADR_ENULL;
+  if (int rc = check_device()) return rc;
   return (int)launch_softmax_rows((hipStream_t)stream, (half_t*)output, (const half_t*)input,
                                   (int64_t)heads * h, w, temp);
 }
@@ -261,6 +292,7 @@ int adr_attention_f16(adr_stream_t stream, uint16_t* output, const uint16_t* que
     return ADR_EUNSUPPORTED_LAYOUT;
   if (!(scale > 0.0f) || !(temp > 0.0f)) return ADR_EUNSUPPORTED_LAYOUT;
   // largest element offsets stay within int64 trivially; rows are addressed with 64-bit products
+  if (int rc = check_device()) return rc;
   return (int)launch_attention((hipStream_t)stream, (half_t*)output, (const half_t*)query,
                                (const half_t*)key, (const half_t*)value, heads, m, n, d,
                                stride_oy, stride_oz, stride_qy, stride_qz, stride_ky, stride_kz,
@@ -274,17 +306,20 @@ static int error_stats_common(adr_stream_t stream, adr_tensor_desc output, adr_t
     return ADR_EINVAL_SHAPE;
   if (lhs.shape[0] == 0) return ADR_OK;
   if (!output.ptr || !lhs.ptr || !rhs.ptr) return ADR_ENULL;
+  if (int rc = check_device()) return rc;
   return (int)launch_error_stats((hipStream_t)stream, (float*)output.ptr, lhs.ptr, rhs.ptr,
                                  lhs.shape[0], lhs.strides[0], rhs.strides[0], f32);
 }
 
 int adr_microbench_empty(adr_stream_t stream) {
+  if (int rc = check_device()) return rc;
   return (int)launch_microbench_empty((hipStream_t)stream);
 }
 
 int adr_microbench_mfma_f16(adr_stream_t stream, int blocks, int times, int pattern, float* sink) {
   if (blocks <= 0 || times < 0 || (pattern != 0 && pattern != 1)) return ADR_EINVAL_SHAPE;
   if (!sink) return ADR_ENULL;
+  if (int rc = check_device()) return rc;
   return (int)launch_microbench_mfma((hipStream_t)stream, blocks, times, pattern, sink);
 }
 
@@ -294,6 +329,7 @@ int adr_microbench_stream_read(adr_stream_t stream, const void* src, int64_t byt
   if (bytes == 0) return ADR_OK;
   if (!src || !sink) return ADR_ENULL;
   if ((uintptr_t)src % 16 != 0) return ADR_EINVAL_SHAPE;
+  if (int rc = check_device()) return rc;
   return (int)launch_microbench_read((hipStream_t)stream, src, bytes, blocks, sink);
 }
 

@@ -33,7 +33,8 @@ namespace adr {
 
 namespace {
 
-constexpr int XCDS = 8;  // MI355X: 8 accelerator dies, workgroup i is dispatched to die i % 8
+// MI355X has 8 accelerator dies (XCDs), each with its own L2; workgroup i is dispatched to die
+// i % 8.  The count comes from the device query (TileMap::xcds).
 
 #define ADR_LDS_PTR(p) ((__attribute__((address_space(3))) void*)(p))
 #define ADR_GLB_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
@@ -59,6 +60,7 @@ __device__ __forceinline__ void lds_chunk_inv(int phys, int& row, int& kc) {
 struct TileMap {
   int tiles_m, tiles_n, tiles_per_batch, total;
   int group_m;  // tile rows per L2-reuse group
+  int xcds;     // dies of the device: workgroup i runs on die i % xcds
 };
 
 // blockIdx.x -> (batch, tile_m, tile_n).  Consecutive ids land on different dies, so ids are
@@ -67,6 +69,7 @@ struct TileMap {
 __device__ __forceinline__ void map_tile(const TileMap& map, int& batch, int& tile_m,
                                          int& tile_n) {
   int id = blockIdx.x;
+  const int XCDS = map.xcds;
   const int per = (map.total + XCDS - 1) / XCDS;
   const int tall = map.total % XCDS == 0 ? XCDS : map.total % XCDS;
   const int xcd = id % XCDS, local = id / XCDS;
@@ -654,6 +657,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
 struct ShortKMap {
   int tiles_m, tiles_n, rows;   // rows = batches * tiles_m
   int seg, segs_per_row, units; // a unit is `seg` consecutive tiles of one tile row
+  int xcds;                     // dies of the device
 };
 
 template <int CPR>  // 16-byte chunks per row: 8 (K = 64) or 16 (K = 128)
@@ -673,6 +677,7 @@ __global__ __launch_bounds__(1024, 1) void gemm_nt_shortk_kernel(MatmulArgs a, S
   // Workgroup g runs on die g % 8: the workgroups of a die take neighbouring units (they share
   // right panels in the die's L2).  Odd rounds walk the workgroups backwards, which pairs long
   // and short rows of a causal product.
+  const int XCDS = map.xcds;
   const int gl = G % XCDS == 0 ? (blockIdx.x % XCDS) * (G / XCDS) + blockIdx.x / XCDS : blockIdx.x;
 
   // Cursor over this workgroup's units and the tiles in them, in processing order.
@@ -1273,6 +1278,7 @@ TileMap make_map(const MatmulArgs& a, int bm, int bn) {
   const int64_t total = (int64_t)map.tiles_per_batch * a.batches;
   map.total = total > 0x7fffffffLL ? -1 : (int)total;
   map.group_m = map.tiles_m < 8 ? map.tiles_m : 8;
+  map.xcds = device_info_for_plan().xcds;
   return map;
 }
 
@@ -1313,11 +1319,14 @@ hipError_t launch_u8(hipStream_t stream, const MatmulArgs& a) {
   return hipGetLastError();
 }
 
-constexpr int NUM_CU = 256;
+// compute units of the current device (MI355X: 256)
+static int num_cu() { return device_info_for_plan().cus; }
 
 template <int CPR>
 hipError_t launch_shortk(hipStream_t stream, const MatmulArgs& a) {
   ShortKMap map;
+  const int NUM_CU = num_cu();
+  map.xcds = device_info_for_plan().xcds;
   map.tiles_m = (a.m + 127) / 128;
   map.tiles_n = (a.n + 127) / 128;
   const int64_t rows = (int64_t)map.tiles_m * a.batches;
@@ -1356,6 +1365,7 @@ struct Candidate {
 GemmChoice pick(const MatmulArgs& a, const Candidate* c, int n, double* cost_out = nullptr) {
   GemmChoice best = GEMM_NONE;
   double best_cost = 0;
+  const int NUM_CU = num_cu();
   for (int i = 0; i < n; i++) {
     const int64_t tiles = (int64_t)((a.m + c[i].bm - 1) / c[i].bm) * ((a.n + c[i].bn - 1) / c[i].bn) *
                           a.batches;
@@ -1377,6 +1387,7 @@ const Candidate DMA_TILES[] = {
 
 // The MFMA family needs 16-byte aligned, K-contiguous rows on both operands.
 GemmChoice choose(const MatmulArgs& a) {
+  const int NUM_CU = num_cu();
   // "NN": both the left operand (k contiguous) and the right operand (n contiguous) are row
   // major, e.g. P.V on the head views of llama.rs:552-554
   if (a.stride_lx == 1 && a.stride_rx == 1 && a.stride_ry != 1 && a.stride_ox == 1 && !a.rhs_q &&
@@ -1430,7 +1441,7 @@ GemmChoice choose(const MatmulArgs& a) {
                                                                                  : tiles(128, 128);
       const bool to_64 = c == DMA_128x128;
       const int64_t then = to_64 ? tiles(128, 64) : tiles(128, 128);
-      if (now >= 224 && now <= NUM_CU && then <= 2 * NUM_CU) return to_64 ? DMA_128x64 : DMA_128x128;
+      if (now >= NUM_CU - 32 && now <= NUM_CU && then <= 2 * NUM_CU) return to_64 ? DMA_128x64 : DMA_128x128;
     }
     return c;
   }
@@ -1451,7 +1462,15 @@ GemmChoice choose(const MatmulArgs& a) {
 
 }  // namespace
 
-static bool choice_name(GemmChoice c, const char** name) {
+static bool choice_name(GemmChoice c, const char** name, bool u8 = false) {
+  if (u8) {
+    switch (c) {
+      case STAGE_256x128: *name = "gemm_nt_u8_stage_256x128x32"; return true;
+      case STAGE_128x128: *name = "gemm_nt_u8_stage_128x128x32"; return true;
+      case STAGE_64x64: *name = "gemm_nt_u8_stage_64x64x64"; return true;
+      default: break;
+    }
+  }
   switch (c) {
     case SHORTK_64: *name = "gemm_nt_mfma_persistent_128x128_k64"; return true;
     case SHORTK_128: *name = "gemm_nt_mfma_persistent_128x128_k128"; return true;
@@ -1542,9 +1561,8 @@ hipError_t launch_mfma_gemm(hipStream_t stream, const MatmulArgs& a) {
   return launch_choice(stream, a, choose(a));
 }
 
-hipError_t launch_gemm_u8_mfma(hipStream_t stream, half_t* out, const half_t* lhs,
-                               const uint8_t* rhs, const half_t* scales, int m, int p, int n,
-                               int block_size, float beta) {
+static MatmulArgs u8_args(half_t* out, const half_t* lhs, const uint8_t* rhs, const half_t* scales,
+                          int m, int p, int n, int block_size, float beta) {
   MatmulArgs a{};
   a.output = out;
   a.lhs = lhs;
@@ -1560,7 +1578,27 @@ hipError_t launch_gemm_u8_mfma(hipStream_t stream, half_t* out, const half_t* lh
   a.rhs_q = rhs;
   a.scales = scales;
   a.block_size = block_size;
-  return launch_mfma_gemm(stream, a);
+  return a;
+}
+
+// Name of the tiled kernel the u8 product would run on (nullptr: none covers it).  The plan query
+// has no pointers: a non-null marker stands for the weights, alignment is assumed.
+const char* gemm_u8_mfma_plan(int m, int p, int n, int block_size) {
+  const MatmulArgs a = u8_args(nullptr, nullptr, (const uint8_t*)16, nullptr, m, p, n, block_size, 0.0f);
+  const char* name = nullptr;
+  return choice_name(choose(a), &name, true) ? name : nullptr;
+}
+
+bool gemm_u8_mfma_supported(const half_t* lhs, const uint8_t* rhs, const half_t* scales, int m, int p,
+                            int n, int block_size) {
+  const MatmulArgs a = u8_args(nullptr, lhs, rhs, scales, m, p, n, block_size, 0.0f);
+  return choose(a) != GEMM_NONE;
+}
+
+hipError_t launch_gemm_u8_mfma(hipStream_t stream, half_t* out, const half_t* lhs,
+                               const uint8_t* rhs, const half_t* scales, int m, int p, int n,
+                               int block_size, float beta) {
+  return launch_mfma_gemm(stream, u8_args(out, lhs, rhs, scales, m, p, n, block_size, beta));
 }
 
 }  // namespace adr

@@ -382,7 +382,8 @@ static SkinnyChoice choose_skinny(const MatmulArgs& a) {
   // CU) and K up to 4096: the ring kernel is ahead already (m=4: K4096 N4096 9.4 -> 7.8 us, K2048
   // N4096 6.9 -> 5.6, K3072 N3072 7.0 -> 5.3; with N 6000 12.3 -> 13.0 and with K 11008 19.3 ->
   // 22.2, so not there; two rows: 7.7 either way)
-  const bool narrow = a.m >= 3 && a.m <= 4 && a.n <= 16 * 256 && a.k <= 4096 && a.k > 1024 &&
+  const int cus = device_info_for_plan().cus;  // MI355X: 256
+  const bool narrow = a.m >= 3 && a.m <= 4 && a.n <= 16 * cus && a.k <= 4096 && a.k > 1024 &&
                       a.k % 128 == 0 && (int64_t)a.n * a.k >= (1 << 22);
   if (narrow) return SKINNY_MFMA;
   if (a.m <= 4 && dot_ok(a)) return SKINNY_DOT;
@@ -404,7 +405,8 @@ hipError_t launch_gemv_f16(hipStream_t stream, const MatmulArgs& a) {
     // weight rows per workgroup: as few as still give (nearly) every CU a workgroup (N4096: 16
     // rows, 256 workgroups, K11008 m=16 27.2 us against 39.5 with 32 rows; N12288: 48 rows,
     // 25.7 against 28.7 with 16; N11008: 48 rows 25.2 against 31.7 with 32)
-    const int rg = a.n >= 40 * 256 ? 3 : a.n >= 24 * 256 ? 2 : 1;
+    const int cus = device_info_for_plan().cus;  // MI355X: 256
+    const int rg = a.n >= 40 * cus ? 3 : a.n >= 24 * cus ? 2 : 1;
     // K in (1024 * (HS - 1), 1024 * HS] for the values of HS built here: weights, and the
     // activations with them, through the per-wavefront LDS ring (m=16, weights alone: K4096
     // N4096 12.4 -> 9.7 us, N11008 24.8 -> 20.3, N12288 25.9 -> 22.1; activations too: 9.9 ->

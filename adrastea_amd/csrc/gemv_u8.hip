@@ -659,7 +659,8 @@ U8Choice choose_u8(const void* lhs, const void* rhs, const void* scales, int m, 
                    int block_size) {
   const bool aligned = ((uintptr_t)lhs % 16 == 0) && ((uintptr_t)rhs % 16 == 0) &&
                        ((uintptr_t)scales % 16 == 0);
-  if (!aligned) return U8_NAIVE;
+  // (p == 0: the operands may be null pointers; the per-output kernel then never reads them)
+  if (!aligned || p == 0) return U8_NAIVE;
   // dot-product kernel: 16 weights of a lane share one scale; at most 16 segments of 1 KiB.
   // It wins for one or two activation rows; from three on its VALU work (dot products and lane
   // reductions per activation row) costs more than the MFMA kernels' less coalesced loads.
@@ -685,6 +686,9 @@ bool rows_in_blocks_of_16(int m, int p, int n, int block_size) {
 hipError_t launch_gemm_u8_mfma(hipStream_t stream, half_t* out, const half_t* lhs,
                                const uint8_t* rhs, const half_t* scales, int m, int p, int n,
                                int block_size, float beta);
+const char* gemm_u8_mfma_plan(int m, int p, int n, int block_size);
+bool gemm_u8_mfma_supported(const half_t* lhs, const uint8_t* rhs, const half_t* scales, int m, int p,
+                            int n, int block_size);
 
 const char* gemm_u8_plan(int m, int p, int n, int block_size) {
   if (rows_in_blocks_of_16(m, p, n, block_size)) m = 16;
@@ -694,7 +698,11 @@ const char* gemm_u8_plan(int m, int p, int n, int block_size) {
       if (p == 16 * MACRO_K) return n < 8192 ? "gemv_u8_mfma16_dma" : "gemv_u8_mfma16_wide_dma";
       if (n < 8192 && p > 16 * MACRO_K && p <= 72 * MACRO_K) return "gemv_u8_mfma16_dma";
       return n < 8192 ? "gemv_u8_mfma16_stream" : "gemv_u8_mfma16_wide";
-    case U8_GEMM: return "gemm_nt_u8_mfma";
+    case U8_GEMM: {
+      // the tile is part of the name: "gemm_nt_u8_mfma_256x192x64", "gemm_nt_u8_stage_128x128x32", ...
+      const char* tiled = gemm_u8_mfma_plan(m, p, n, block_size);
+      return tiled ? tiled : "gemm_u8_naive";
+    }
     default: return "gemm_u8_naive";
   }
 }
@@ -791,7 +799,9 @@ hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, co
       return hipGetLastError();
     }
     case U8_GEMM:
-      return launch_gemm_u8_mfma(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
+      if (gemm_u8_mfma_supported(lhs, rhs, scales, m, p, n, block_size))
+        return launch_gemm_u8_mfma(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
+      [[fallthrough]];  // no tiled kernel takes these operands: one thread per output
     default: {
       if ((m + 3) / 4 > 65535) return hipErrorInvalidConfiguration;
       hipLaunchKernelGGL(gemm_u8_naive_kernel, dim3((n + 63) / 64, (m + 3) / 4), dim3(256), 0,

@@ -6,7 +6,10 @@
  * (NULL = the null stream, which is what the reference uses: `stream: None`,
  * adrastea_models/src/kernels.rs:862), never synchronises, never allocates, and returns
  * 0 on success, a positive hipError_t, or a negative ADR_E* code.  Invalid requests are
- * rejected on the host; no entry point traps on the device.
+ * rejected on the host; no entry point traps on the device.  The kernels exist for gfx950 only:
+ * with any other device current, every launching entry point returns ADR_EUNSUPPORTED_DEVICE
+ * (the device's architecture, compute-unit and die counts are queried once per device and
+ * cached; that cache is the only state the library keeps).
  *
  * fp16 data is passed as uint16_t bit patterns (Rust `half::f16` is repr(transparent) u16).
  * All strides are in ELEMENTS.  `x` is the last tensor dimension, `y` the second to last,
@@ -218,7 +221,11 @@ int adr_attention_f16(adr_stream_t stream, uint16_t* output, const uint16_t* que
  *
  * adr_matmul_f16_plan: writes the name of the kernel adr_matmul_f16 would launch for these
  * arguments into `name` (at most `cap` bytes, NUL-terminated) without touching the device.
- * Same validation and return codes as adr_matmul_f16 minus the pointer checks.
+ * Same validation and return codes as adr_matmul_f16 minus the pointer checks.  Without pointers
+ * the plan assumes 16-byte aligned operands; a call with unaligned ones runs on the general
+ * (u8: the per-output) kernel whatever the plan says.  On a machine without a device the plan
+ * is the one for an MI355X.  adr_matmul_nt_fp16u8_plan names the tile of a tiled kernel
+ * ("gemm_nt_u8_mfma_256x192x64", "gemm_nt_u8_stage_128x128x32", ...).
  */
 int adr_matmul_f16_plan(char* name, int32_t cap, int32_t batches, int32_t m, int32_t k,
                         int32_t n, int32_t stride_ox, int32_t stride_oy, int32_t stride_oz,

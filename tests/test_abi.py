@@ -81,7 +81,54 @@ def test_u8_plan():
     assert plan(4, 4096, 12288, 32) == (0, "gemv_u8_mfma16_wide_dma")
     assert plan(4, 2048, 12288, 32) == (0, "gemv_u8_mfma16_wide")
     assert plan(16, 4096, 4096, 32) == (0, "gemv_u8_mfma16_dma")
-    assert plan(2048, 4096, 4096, 32) == (0, "gemm_nt_u8_mfma")
-    assert plan(8, 4096, 4096, 64)[1] == "gemm_nt_u8_mfma"
+    # tiled kernels: the name carries the tile
+    assert plan(2048, 4096, 4096, 32) == (0, "gemm_nt_u8_mfma_256x128x64")
+    assert plan(2048, 4096, 12288, 32) == (0, "gemm_nt_u8_mfma_256x192x64")
+    assert plan(2048, 4096, 11008, 32) == (0, "gemm_nt_u8_mfma_256x192x64")
+    assert plan(2048, 11008, 4096, 32) == (0, "gemm_nt_u8_mfma_256x128x64")
+    assert plan(300, 4096, 4096, 32)[1].startswith("gemm_nt_u8_stage_")
+    assert plan(8, 4096, 4096, 64)[1].startswith("gemm_nt_u8_stage_")
+    assert plan(8, 36, 64, 12) == (0, "gemm_u8_naive")
     assert plan(4, 4100, 64, 32)[0] == _ffi.ADR_EDIVISIBILITY
     assert plan(4, 64, 64, 0)[0] == _ffi.ADR_EINVAL_SHAPE
+
+
+def test_offsets_beyond_int32_are_rejected():
+    """Element offsets are i32 in the reference (kernels.rs:864-887): a view whose farthest
+    element lies at 2^31 elements or more returns ADR_EINVAL_SHAPE."""
+    big = 1 << 16
+    ok = ((1, 32767, 0), (1, 64, 0), (64, 1, 0))
+    assert _plan(1, 32768, 64, 32767, *ok)[0] == 0
+    too_far_out = ((1, big, 0), (1, 64, 0), (64, 1, 0))
+    assert _plan(1, 32769, 64, big, *too_far_out)[0] == _ffi.ADR_EINVAL_SHAPE
+    far_batch = ((1, 64, 1 << 30), (1, 64, 0), (64, 1, 0))
+    assert _plan(3, 64, 64, 64, *far_batch)[0] == _ffi.ADR_EINVAL_SHAPE
+    assert _plan(2, 64, 64, 64, *far_batch)[0] == 0
+    neg = ((1, 64, 0), (1, -(1 << 25), 0), (64, 1, 0))
+    assert _plan(1, 65, 64, 64, *neg)[0] == _ffi.ADR_EINVAL_SHAPE
+    lib = _ffi.lib()
+    # the contiguous entry points: n * p elements of weights
+    assert lib.adr_matmul_nt_fp16u8(None, 8, 8, 8, 8, 1, 1 << 16, 1 << 15, 32, 0.0) == _ffi.ADR_EINVAL_SHAPE
+    assert lib.adr_matmul_nt_f16(None, 8, 8, 8, 1, 1 << 16, 1 << 15, 0.0) == _ffi.ADR_EINVAL_SHAPE
+
+
+def test_no_usable_device_is_an_error_not_a_crash():
+    """On a machine without a gfx950 device a launching entry point returns
+    ADR_EUNSUPPORTED_DEVICE or the runtime's error code; it never launches and never aborts."""
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    lib = _ffi.lib()
+    rc = lib.adr_matmul_nt_f16(None, 16, 16, 16, 4, 64, 4, 0.0)
+    assert rc != 0
+    assert _ffi.strerror(rc)
+    assert lib.adr_microbench_empty(None) == rc
+
+
+def test_integration_source_list_matches_the_build():
+    """INTEGRATION.md's build.rs recipe must name every source the library is built from."""
+    from adrastea_amd import build
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    block = text[text.index("let src = ["):]
+    block = block[:block.index("];")]
+    assert sorted(re.findall(r'"([a-z0-9_]+\.hip)"', block)) == sorted(build.SOURCES)

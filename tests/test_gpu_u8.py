@@ -143,10 +143,16 @@ def test_fused_dequant_in_gemv_is_bit_exact_for_every_q_and_finite_scale(kern, m
         assert np.all((got[z] & 0x7FFF) == 0)
 
 
-def test_fused_dequant_in_u8_gemm_is_bit_exact_for_every_q_and_finite_scale(kern):
+@pytest.mark.parametrize("tile", ["256x128", "256x192"])
+def test_fused_dequant_in_u8_gemm_is_bit_exact_for_every_q_and_finite_scale(kern, tile):
+    """One-hot rows extract every weight of the tiled u8 kernel: all 49154 finite scales make 385
+    tiles of 256 x 128; the first 49152 of them exactly 256 tiles of 256 x 192 (the two scales
+    left out are covered by the other tile and by the stand-alone kernel)."""
     scales_bits = _finite_scale_rows()
+    if tile == "256x192":
+        scales_bits = scales_bits[:192 * 256]
     n, p, bs, m = scales_bits.size, 256, 32, 256
-    assert u8_plan(m, p, n, bs) == "gemm_nt_u8_mfma"
+    assert u8_plan(m, p, n, bs) == f"gemm_nt_u8_mfma_{tile}x64"
     q = np.tile(np.arange(256, dtype=np.uint8), (n, 1))
     s = np.repeat(scales_bits.view(np.float16).reshape(n, 1), p // bs, axis=1)
     lhs = np.eye(m, dtype=np.float16)
@@ -250,11 +256,13 @@ def test_u8_matmul_random_matches_oracle_and_reference_kernel(kern, ref, m):
                                   (260, 320, 1100, 64), (1024, 384, 300, 128), (1024, 448, 300, 64), (256, 832, 1024, 32),
                                   (700, 768, 400, 256)],
                          ids=lambda c: "M%d_K%d_N%d_bs%d" % c)
-def test_u8_prefill_kernel_ragged_tiles_and_k_tails_bit_exact(kern, case):
-    """The DMA + dequant-while-staging kernel (m*n >= 256 Ki, K % 64 == 0, power-of-two blocks):
-    partial tiles in M and N, every remainder of the six-slice unrolled K loop, block sizes
-    below, at and above the slice depth, and the beta path -- exact inputs, compared bit for bit."""
+def test_u8_staged_kernels_ragged_tiles_and_k_tails_bit_exact(kern, case):
+    """Products with at most 64 tiles of 256 x 128 run on the register-staged kernels (dequantised
+    while staging): partial tiles in M and N, K slices of 32 and 64 with and without a tail, block
+    sizes below, at and above the slice depth, and the beta path -- exact inputs, compared bit for
+    bit.  (The DMA kernel's tiles: test_u8_dma_kernel_* below.)"""
     m, p, n, bs = case
+    assert u8_plan(m, p, n, bs).startswith("gemm_nt_u8_stage_")
     g = rng(640 + m + p)
     a, q, s = _u8_case(g, m, p, n, bs, exact=True)
     for beta in (0.0, 1.0):
@@ -264,6 +272,75 @@ def test_u8_prefill_kernel_ragged_tiles_and_k_tails_bit_exact(kern, case):
         out = to_dev(prev)
         kern.matmul_nt_fp16u8(out, to_dev(a), to_dev(q), to_dev(s), bs, beta=beta)
         assert np.array_equal(to_np(out).view(np.uint16), want.view(np.uint16)), (case, beta)
+
+
+@pytest.mark.parametrize("p", [320, 384, 448, 512, 576, 640, 1024])
+@pytest.mark.parametrize("tile_mn", [("256x192", 520, 11000), ("256x128", 520, 2900)],
+                         ids=lambda t: t[0])
+def test_u8_dma_kernel_ragged_tiles_and_every_k_remainder_bit_exact(kern, tile_mn, p):
+    """gemm_nt_u8_kernel<256,192> and <256,128> (more than 64 tiles of 256 x 128): a ragged last
+    tile row (520 = 2 x 256 + 8) and tile column, K / 64 = 5 .. 10 and 16 slices, i.e. every
+    remainder of the six-slice unrolled loop, beta 0 and 1, block sizes 32 and 64 -- exact inputs,
+    compared bit for bit.  Expected values: one rounding of the float64 product on the oracle's
+    dequantised weights (every sum is exactly representable), cross-checked with the oracle's
+    own matmul on the rows around the tile borders."""
+    tile, m, n = tile_mn
+    bs = 64 if p % 128 == 0 else 32
+    assert u8_plan(m, p, n, bs) == f"gemm_nt_u8_mfma_{tile}x64"
+    g = rng(1640 + p + n)
+    a, q, s = _u8_case(g, m, p, n, bs, exact=True)
+    w64 = oracle.dequantize_absmax_u8(q, s, bs).astype(np.float64)
+    prod = a.astype(np.float64) @ w64.T
+    rows = np.array([0, 1, 31, 32, 255, 256, 257, 511, 512, 519])
+    a_t, q_t, s_t = to_dev(a), to_dev(q), to_dev(s)
+    for beta in (0.0, 1.0):
+        prev = (g.integers(-8, 9, size=(m, n)) / 4.0).astype(np.float16)
+        want = (prod + beta * prev.astype(np.float64)).astype(np.float16)
+        chk = prev[rows].copy()
+        oracle.matmul_nt_fp16u8(chk, a[rows], q, s, bs, beta=beta, threads=8)
+        assert np.array_equal(chk.view(np.uint16), want[rows].view(np.uint16))
+        out = to_dev(prev)
+        kern.matmul_nt_fp16u8(out, a_t, q_t, s_t, bs, beta=beta)
+        got = to_np(out)
+        bad = np.argwhere(got.view(np.uint16) != want.view(np.uint16))
+        assert bad.size == 0, (tile, p, beta, bad[:5])
+
+
+CFG5_U8 = [("qkv", 4096, 12288, "256x192"), ("o", 4096, 4096, "256x128"),
+           ("gate_up", 4096, 11008, "256x192"), ("down", 11008, 4096, "256x128")]
+
+
+@pytest.mark.parametrize("case", CFG5_U8, ids=[c[0] for c in CFG5_U8])
+def test_prefill_u8_gemm_layer_set_full_size(kern, case):
+    """benchmark config 5 (u8 half) at full size, M = 2048: every product of the layer set on the
+    tile the benchmark measures (asserted through the plan), against an fp32 GEMM on the
+    bit-exactly dequantised weights, both on the device; plus f(2a) = 2 f(a) exactly."""
+    _, p, n, tile = case
+    m = 2048
+    assert u8_plan(m, p, n, 32) == f"gemm_nt_u8_mfma_{tile}x64"
+    gen = torch.Generator(device="cuda").manual_seed(45 + n)
+    q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)
+    s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
+    a = torch.randn(m, p, generator=gen, device="cuda").half()
+    out = torch.zeros(m, n, dtype=torch.float16, device="cuda")
+    kern.matmul_nt_fp16u8(out, a, q, s, 32)
+    w = torch.zeros(n, p, dtype=torch.float16, device="cuda")
+    kern.dequantize_absmax_uint8(w, s, q)
+    ref32 = a.float() @ w.float().t()
+    rms = ref32.pow(2).mean().sqrt()
+    err = (out.float() - ref32).abs()
+    rel = (err / torch.maximum(ref32.abs(), rms)).max().item()
+    assert rel <= 2e-3, rel
+    # the unfloored ratio on every element of at least typical magnitude
+    big = ref32.abs() >= rms
+    assert (err[big] / ref32.abs()[big]).max().item() <= TOL
+    out2 = torch.zeros_like(out)
+    kern.matmul_nt_fp16u8(out2, (a * 2).half(), q, s, 32)
+    # (powers of two commute with the rounding of normal numbers; among 8 to 25 million outputs
+    # a few dozen are subnormal, where they do not)
+    normal = out.abs() >= 2.0 ** -13
+    assert torch.equal(out2[normal], (out * 2).half()[normal])
+    assert (out2[~normal].float() - 2 * out[~normal].float()).abs().max().item() <= 2.0 ** -23
 
 
 def test_u8_other_block_sizes_and_fallbacks(kern):
@@ -282,6 +359,12 @@ def test_u8_other_block_sizes_and_fallbacks(kern):
                                     1, 40, 1, 32, 0.0) == -5   # p % block_size
     assert lib.adr_matmul_nt_fp16u8(None, None, z.data_ptr(), z.data_ptr(), z.data_ptr(),
                                     1, 32, 1, 32, 0.0) == -4
+    # p == 0: an empty sum; the operands may be null, the output becomes beta * out for any m
+    for m in (1, 4, 40):
+        prev = torch.full((m, 24), 2.0, dtype=torch.float16, device="cuda")
+        assert lib.adr_matmul_nt_fp16u8(torch.cuda.current_stream().cuda_stream, prev.data_ptr(),
+                                        None, None, None, m, 0, 24, 32, 0.5) == 0
+        assert torch.all(prev == 1.0)
 
 
 DECODE = [(4096, 4096), (4096, 11008), (4096, 12288), (11008, 4096)]
@@ -344,8 +427,9 @@ def test_seventeen_and_more_rows_in_blocks_of_sixteen(kern, kn, m):
     more rows stay on the tiled GEMM.  Previous output added, ragged N."""
     p, n = kn
     limit = 128 if n < 8192 else 64
-    assert u8_plan(m, p, n, 32) == (u8_plan(16, p, n, 32) if m <= limit else "gemm_nt_u8_mfma")
-    assert u8_plan(limit + 1, p, n, 32) == "gemm_nt_u8_mfma"
+    assert (u8_plan(m, p, n, 32) == u8_plan(16, p, n, 32)) if m <= limit else \
+        u8_plan(m, p, n, 32).startswith("gemm_nt_u8_")
+    assert u8_plan(limit + 1, p, n, 32).startswith("gemm_nt_u8_")
     gen = torch.Generator(device="cuda").manual_seed(47 + m + p)
     q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)
     s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
@@ -368,7 +452,7 @@ def test_mid_row_counts_take_the_smaller_staged_tiles(kern, mpn):
     same arithmetic bar as the large-tile kernel."""
     m, p, n = mpn
     assert (m + 255) // 256 * ((n + 127) // 128) <= 64
-    assert u8_plan(m, p, n, 32) == "gemm_nt_u8_mfma"   # (one name for all tiled u8 kernels)
+    assert u8_plan(m, p, n, 32).startswith("gemm_nt_u8_stage_")
     gen = torch.Generator(device="cuda").manual_seed(48 + m)
     q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)
     s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
@@ -380,23 +464,6 @@ def test_mid_row_counts_take_the_smaller_staged_tiles(kern, mpn):
     w = torch.zeros(n, p, dtype=torch.float16, device="cuda")
     kern.dequantize_absmax_uint8(w, s, q)
     ref32 = a.float() @ w.float().t() + 0.5 * prev.float()
-    rms = ref32.pow(2).mean().sqrt()
-    rel = ((out.float() - ref32).abs() / torch.maximum(ref32.abs(), rms)).max().item()
-    assert rel <= 2e-3, rel
-
-
-def test_prefill_u8_gemm_full_size(kern):
-    """benchmark config 5 (u8 variant), the O projection: M=2048, K=4096, N=4096."""
-    m, p, n = 2048, 4096, 4096
-    gen = torch.Generator(device="cuda").manual_seed(45)
-    q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)
-    s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
-    a = torch.randn(m, p, generator=gen, device="cuda").half()
-    out = torch.zeros(m, n, dtype=torch.float16, device="cuda")
-    kern.matmul_nt_fp16u8(out, a, q, s, 32)
-    w = torch.zeros(n, p, dtype=torch.float16, device="cuda")
-    kern.dequantize_absmax_uint8(w, s, q)
-    ref32 = a.float() @ w.float().t()
     rms = ref32.pow(2).mean().sqrt()
     rel = ((out.float() - ref32).abs() / torch.maximum(ref32.abs(), rms)).max().item()
     assert rel <= 2e-3, rel
