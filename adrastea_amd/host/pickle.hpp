@@ -19,6 +19,7 @@
 
 #include <cstdint>
 #include <cstring>
+#include <algorithm>
 #include <map>
 #include <memory>
 #include <stdexcept>
@@ -101,37 +102,46 @@ inline std::map<std::string, ZipMember> read_zip_directory(const uint8_t* d, siz
     // zip64: locator (0x07064b50) sits right before the record and points at the zip64 record
     if (eocd < 20 || rd32(d + eocd - 20) != 0x07064b50u) throw std::runtime_error("zip64 locator missing");
     const uint64_t rec = rd64(d + eocd - 20 + 8);
-    if (rec + 56 > n || rd32(d + rec) != 0x06064b50u) throw std::runtime_error("zip64 record missing");
+    if (n < 56 || rec > n - 56 || rd32(d + rec) != 0x06064b50u) throw std::runtime_error("zip64 record missing");
     entries = rd64(d + rec + 32);
     cd_size = rd64(d + rec + 40);
     cd_off = rd64(d + rec + 48);
   }
-  if (cd_off + cd_size > n) throw std::runtime_error("zip: central directory out of range");
+  // (every bound below is written as a subtraction: the fields come from the file, and a sum of
+  // two 64-bit values chosen by the file can wrap)
+  if (cd_off > n || cd_size > n - cd_off) throw std::runtime_error("zip: central directory out of range");
   std::map<std::string, ZipMember> out;
   size_t p = cd_off;
   for (uint64_t i = 0; i < entries; i++) {
-    if (p + 46 > n || rd32(d + p) != 0x02014b50u) throw std::runtime_error("zip: bad central entry");
+    if (p > n || n - p < 46 || rd32(d + p) != 0x02014b50u) throw std::runtime_error("zip: bad central entry");
     const uint16_t method = rd16(d + p + 10);
     uint64_t csize = rd32(d + p + 20), usize = rd32(d + p + 24), lho = rd32(d + p + 42);
     const uint16_t nlen = rd16(d + p + 28), xlen = rd16(d + p + 30), clen = rd16(d + p + 32);
-    if (p + 46 + nlen + xlen + clen > n) throw std::runtime_error("zip: truncated central entry");
+    if (n - p - 46 < (size_t)nlen + xlen + clen) throw std::runtime_error("zip: truncated central entry");
     const std::string name((const char*)d + p + 46, nlen);
     // zip64 extended information (header id 1): the fields that were 0xFFFFFFFF, in this order
     const uint8_t* x = d + p + 46 + nlen;
     for (size_t q = 0; q + 4 <= xlen;) {
       const uint16_t id = rd16(x + q), len = rd16(x + q + 2);
       if (id == 1) {
+        // each 8-byte field must lie inside this extra field and inside the extra area
+        const size_t lim = std::min((size_t)xlen, q + 4 + (size_t)len);
         size_t o = q + 4;
-        if (usize == 0xFFFFFFFFu) { usize = rd64(x + o); o += 8; }
-        if (csize == 0xFFFFFFFFu) { csize = rd64(x + o); o += 8; }
-        if (lho == 0xFFFFFFFFu) { lho = rd64(x + o); o += 8; }
+        auto field = [&](uint64_t& v) {
+          if (o + 8 > lim) throw std::runtime_error("zip64: truncated extended information");
+          v = rd64(x + o);
+          o += 8;
+        };
+        if (usize == 0xFFFFFFFFu) field(usize);
+        if (csize == 0xFFFFFFFFu) field(csize);
+        if (lho == 0xFFFFFFFFu) field(lho);
       }
       q += 4 + (size_t)len;
     }
     if (method != 0) throw std::runtime_error("pytorch archives should not contain compressed files");
-    if (lho + 30 > n || rd32(d + lho) != 0x04034b50u) throw std::runtime_error("zip: bad local header");
+    if (n < 30 || lho > n - 30 || rd32(d + lho) != 0x04034b50u) throw std::runtime_error("zip: bad local header");
     const size_t start = lho + 30 + rd16(d + lho + 26) + rd16(d + lho + 28);
-    if (start + usize > n) throw std::runtime_error("zip: member out of range");
+    if (start > n || usize > n - start) throw std::runtime_error("zip: member out of range");
     const size_t slash = name.find_last_of('/');
     const std::string base = slash == std::string::npos ? name : name.substr(slash + 1);
     if (!base.empty()) out[base] = ZipMember{start, (size_t)usize};
@@ -358,7 +368,7 @@ class PickledModel {
           a[2]->items.size() != a[3]->items.size())
         throw std::runtime_error("entry " + kv.first->s + ": unexpected tensor record");
       const int64_t off = a[1]->i;
-      if (off < 0 || (uint64_t)off * el > t.end - t.begin) throw std::runtime_error("invalid storage offset");
+      if (off < 0 || (uint64_t)off > (t.end - t.begin) / el) throw std::runtime_error("invalid storage offset");
       t.begin += (size_t)off * el;
       size_t largest = 0;
       for (size_t k = 0; k < a[2]->items.size(); k++) {
@@ -368,12 +378,17 @@ class PickledModel {
         t.shape.push_back((size_t)a[2]->items[k]->i);
         t.stride.push_back((size_t)a[3]->items[k]->i);
         if (t.shape.back() == 0) throw std::runtime_error("entry " + kv.first->s + ": empty dimension");
-        largest += (t.shape.back() - 1) * t.stride.back();
+        size_t reach;
+        if (__builtin_mul_overflow(t.shape.back() - 1, t.stride.back(), &reach) ||
+            __builtin_add_overflow(largest, reach, &largest))
+          throw std::runtime_error("invalid tensor size");
       }
       if (!t.shape.empty()) {
         // trimmed to the addressed span (pickle.rs:160-168)
-        const size_t span = (largest + 1) * el;
-        if (span > t.end - t.begin) throw std::runtime_error("invalid tensor size");
+        size_t span;
+        if (__builtin_add_overflow(largest, (size_t)1, &span) || __builtin_mul_overflow(span, el, &span) ||
+            span > t.end - t.begin)
+          throw std::runtime_error("invalid tensor size");
         t.end = t.begin + span;
       }
       tensors.emplace(kv.first->s, std::move(t));

@@ -157,18 +157,12 @@ def test_checkpoint_to_u8_on_the_device(tmp_path):
     assert float(fields[-1]) <= 0.5 + 2 * 127.5 * 2.0 ** -11 + 1e-3
 
 
-def test_zip64_records(tmp_path):
-    """Archives beyond 4 GiB carry their sizes and offsets in zip64 records.  A small archive is
-    rewritten here with EVERY size and offset moved into those records (legal for any size), so
-    the reader's zip64 branch is exercised without a 4 GiB file."""
+def _zip64_archive(members, cd_off_delta=0, rec_off=None, lho=None, usize=None, extra_len=24,
+                   extra_fields=3):
+    """A zip archive with EVERY size and offset moved into zip64 records (legal for any size).
+    The keyword arguments falsify single fields, for the hostile-archive tests."""
     import struct
     import zipfile
-    state = {"w": torch.arange(24, dtype=torch.float32).reshape(4, 6).half(),
-             "b": torch.arange(5, dtype=torch.int64)}
-    src = str(tmp_path / "small.pt")
-    torch.save(state, src)
-    with zipfile.ZipFile(src) as z:
-        members = [(i.filename, z.read(i.filename)) for i in z.infolist()]
     blob, central = b"", b""
     for name, data in members:
         nb = name.encode()
@@ -177,18 +171,38 @@ def test_zip64_records(tmp_path):
         extra = struct.pack("<HHQQ", 1, 16, len(data), len(data))
         blob += struct.pack("<IHHHHHIIIHH", 0x04034b50, 45, 0, 0, 0, 0, zipfile.crc32(data),
                             0xFFFFFFFF, 0xFFFFFFFF, len(nb), len(extra)) + nb + extra + data
-        cextra = struct.pack("<HHQQQ", 1, 24, len(data), len(data), off)
+        fields = [len(data) if usize is None else usize, len(data), off if lho is None else lho]
+        cextra = struct.pack("<HH", 1, extra_len) + b"".join(struct.pack("<Q", f)
+                                                              for f in fields[:extra_fields])
         central += struct.pack("<IHHHHHHIIIHHHHHII", 0x02014b50, 45, 45, 0, 0, 0, 0,
                                zipfile.crc32(data), 0xFFFFFFFF, 0xFFFFFFFF, len(nb), len(cextra),
                                0, 0, 0, 0, 0xFFFFFFFF) + nb + cextra
     cd_off = len(blob)
-    rec_off = cd_off + len(central)
+    real_rec = cd_off + len(central)
     rec = struct.pack("<IQHHIIQQQQ", 0x06064b50, 44, 45, 45, 0, 0, len(members), len(members),
-                      len(central), cd_off)
-    loc = struct.pack("<IIQI", 0x07064b50, 0, rec_off, 1)
+                      len(central), (cd_off + cd_off_delta) & 0xFFFFFFFFFFFFFFFF)
+    loc = struct.pack("<IIQI", 0x07064b50, 0, real_rec if rec_off is None else rec_off, 1)
     eocd = struct.pack("<IHHHHIIH", 0x06054b50, 0, 0, 0xFFFF, 0xFFFF, 0xFFFFFFFF, 0xFFFFFFFF, 0)
+    return blob + central + rec + loc + eocd
+
+
+def _members_of(path):
+    import zipfile
+    with zipfile.ZipFile(path) as z:
+        return [(i.filename, z.read(i.filename)) for i in z.infolist()]
+
+
+def test_zip64_records(tmp_path):
+    """Archives beyond 4 GiB carry their sizes and offsets in zip64 records.  A small archive is
+    rewritten here with every size and offset moved into those records, so the reader's zip64
+    branch is exercised without a 4 GiB file."""
+    import zipfile
+    state = {"w": torch.arange(24, dtype=torch.float32).reshape(4, 6).half(),
+             "b": torch.arange(5, dtype=torch.int64)}
+    src = str(tmp_path / "small.pt")
+    torch.save(state, src)
     dst = str(tmp_path / "zip64.pt")
-    open(dst, "wb").write(blob + central + rec + loc + eocd)
+    open(dst, "wb").write(_zip64_archive(_members_of(src)))
     with zipfile.ZipFile(dst) as z:                        # Python's reader accepts it too
         assert z.testzip() is None
     rc, out = run("pickle", dst)
@@ -199,3 +213,49 @@ def test_zip64_records(tmp_path):
     strip = lambda ls: [" ".join(l.split()[:-3]) + " " + l.split()[-1] for l in ls]
     assert ref_rc == 0 and strip(lines) == strip(ref_out.strip().splitlines())
     check(out, state)
+
+
+@pytest.mark.parametrize("knob", [
+    dict(cd_off_delta=-(1 << 20)),                 # directory offset wraps to just below 2^64
+    dict(cd_off_delta=1 << 40),                    # ... or lies far beyond the file
+    dict(rec_off=(1 << 64) - 40),                  # zip64 record offset + 56 wraps
+    dict(lho=(1 << 64) - 16),                      # local header offset + 30 wraps
+    dict(usize=(1 << 64) - 8),                     # member size: start + size wraps
+    dict(usize=1 << 50),                           # ... or simply runs past the end
+    dict(extra_len=24, extra_fields=1),            # zip64 extra field shorter than it claims
+    dict(extra_len=8, extra_fields=3),             # ... and fields beyond the declared length
+], ids=lambda k: "_".join(k))
+def test_hostile_zip_fields_are_rejected_not_followed(tmp_path, knob):
+    """Offsets and sizes come from the file: a crafted value must fail the range check (also
+    where a sum of two such values would wrap around 2^64), never be used as an address."""
+    src = str(tmp_path / "small.pt")
+    torch.save({"w": torch.arange(24, dtype=torch.float32).reshape(4, 6).half()}, src)
+    dst = str(tmp_path / "hostile.pt")
+    open(dst, "wb").write(_zip64_archive(_members_of(src), **knob))
+    rc, out = run("pickle", dst)
+    assert rc == 2 and "ERROR" in out, (rc, out)
+
+
+@pytest.mark.parametrize("dim0", [1 << 62, (1 << 64) // 6 + 2, 1 << 40])
+def test_tensor_span_overflow_is_rejected(tmp_path, dim0):
+    """A shape whose byte span wraps around 2^64 (or merely exceeds its storage) must not pass
+    the span check with a small wrapped value."""
+    import zipfile
+    src = str(tmp_path / "small.pt")
+    torch.save({"w": torch.arange(24, dtype=torch.float32).reshape(4, 6).half()}, src)
+    members = _members_of(src)
+    patched = []
+    for name, data in members:
+        if name.endswith("data.pkl"):
+            old = b"K\x04K\x06\x86"                     # the shape tuple (4, 6)
+            assert data.count(old) == 1
+            data = data.replace(old, b"\x8a\x09" + dim0.to_bytes(9, "little")[:9] + b"K\x06\x86"
+                                if dim0 >= 1 << 63 else
+                                b"\x8a\x08" + dim0.to_bytes(8, "little") + b"K\x06\x86")
+        patched.append((name, data))
+    dst = str(tmp_path / "span.pt")
+    with zipfile.ZipFile(dst, "w", zipfile.ZIP_STORED) as z:
+        for name, data in patched:
+            z.writestr(name, data)
+    rc, out = run("pickle", dst)
+    assert rc == 2 and "ERROR" in out, (rc, out)
