@@ -4,7 +4,7 @@
 // (adrastea_kernels/cpp/matmul_nt_fp16u8.cu:4-24 and
 // matmul_nt_wmma_16x128x256_fp16u8.cu:5-7, 43-83; format quantize.cu:3-56).
 //
-// The problem is bound by streaming the u8 weights from HBM once.  Two kernels:
+// The problem is bound by streaming the u8 weights from HBM once.  Kernels:
 //
 //  gemv_u8_dot_kernel (m <= 2)   no matrix cores.  A wavefront streams whole 1 KiB segments of
 //      one weight row per load instruction (lane l: 16 bytes at l*16, perfectly coalesced),
@@ -16,15 +16,21 @@
 //      once.  This is the arithmetic of the reference's naive kernel (unrounded weights,
 //      matmul_nt_fp16u8.cu:17-21) in fp32.  Lane sums are reduced with DPP adds.
 //
-//  gemv_u8_kernel (m <= 16)      v_mfma_f32_16x16x32_f16 with the 16 weight rows of the
-//      workgroup as the A operand and the activations as the B operand (rows beyond m are
-//      zero).  Per 256-element macro step a lane (row r = lane % 16, group g = lane / 16)
-//      loads 4 x 16 weight bytes such that the four lanes of a row cover 64 contiguous bytes
-//      per instruction, dequantises them in registers to fp16 exactly as the stand-alone
-//      dequantise kernel does (the WMMA kernel's arithmetic) and issues two MFMAs per load.
-//      The k slots of an MFMA may hold any 32 distinct k as long as both operands agree,
-//      which is what lets a lane use 16 contiguous bytes.  Wavefronts split K; partial sums
-//      are reduced through LDS.
+//  gemv_u8_regstream_kernel (3 <= m <= 16, block size 32, K % 256 == 0)   the same arithmetic on
+//      the matrix cores: one v_mfma_f32_16x16x32_f16 per scale block of 32 weights on the
+//      integers 1024 + q, its accumulator input preset to -1151.5 * (sum of the block's
+//      activations), the four results scaled in fp32.  Weights and activations are fetched in
+//      pieces of 4 rows x 256 bytes per instruction (what DRAM serves at the streaming rate; the
+//      matrix-core operand layout itself would ask for 16 rows x 64 bytes) into registers, and a
+//      private 4 KiB LDS tile per wavefront turns them into operand layout.  Requests run a
+//      fixed distance ahead of their use: a compute unit holds only some 64 KiB of requests in
+//      flight whatever is asked, oldest wavefront first, so asking for everything up front
+//      starves the younger wavefronts and leaves all arithmetic to the end.
+//
+//  gemv_u8_ring_kernel (17 .. 32 rows per pass, K = 4096)   v_mfma_f32_16x16x32_f16 on weights
+//      dequantised to fp16 in registers exactly as the stand-alone dequantise kernel does (the
+//      WMMA kernel's arithmetic), two blocks of sixteen activation rows per pass over the
+//      weights, operands through a per-wavefront LDS ring filled by global -> LDS DMA.
 #include "adr_common.hpp"
 
 namespace adr {
@@ -34,194 +40,9 @@ namespace {
 constexpr int MACRO_K = 256;  // k elements per macro step
 constexpr int ROWS = 16;      // weight rows per workgroup
 
-struct Stage {
-  u32x4_t w[4];   // 4 x 16 weight bytes of this lane's row
-  u32x4_t sc;     // the eight fp16 scales (block_size 32) of the macro step
-  u32x4_t x[8];   // 4 x 16 activation halves of this lane's activation row
-};
-
-template <int NW>
-__global__ __launch_bounds__(NW * 64) void gemv_u8_kernel(half_t* __restrict__ out,
-                                                          const half_t* __restrict__ lhs,
-                                                          const uint8_t* __restrict__ rhs,
-                                                          const half_t* __restrict__ scales,
-                                                          int m, int p, int n, float beta) {
-  __shared__ float partial[NW][ROWS * 16];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int r = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * ROWS;
-  const int row = min(n0 + r, n - 1);  // tail rows are clamped; their sums are not stored
-  const int nblk = p / 32;
-  // load j of a macro step takes bytes j*64 + g*16 .. +16 of the row: the four lanes of a row
-  // cover 64 contiguous bytes per instruction
-  const uint8_t* wrow = rhs + (int64_t)row * p + g * 16;
-  const half_t* srow = scales + (int64_t)row * nblk;
-  const bool xvalid = r < m;
-  const half_t* xrow = lhs + (int64_t)min(r, m - 1) * p + g * 16;
-  const int steps = p / MACRO_K;
-
-  auto load = [&](Stage& s, int ms) {
-    const uint8_t* wp = wrow + (int64_t)ms * MACRO_K;
-#pragma unroll
-    for (int j = 0; j < 4; j++) s.w[j] = *(const u32x4_t*)(wp + j * 64);
-    s.sc = *(const u32x4_t*)(srow + ms * (MACRO_K / 32));
-    const half_t* xp = xrow + (int64_t)ms * MACRO_K;
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-      // (lanes beyond m load row m-1 again -- same addresses as its own lanes, no extra
-      // traffic -- and are zeroed: a load under a branch would be waited for at the join)
-      const u32x4_t x0 = *(const u32x4_t*)(xp + j * 64), x1 = *(const u32x4_t*)(xp + j * 64 + 8);
-      s.x[2 * j] = xvalid ? x0 : u32x4_t{0, 0, 0, 0};
-      s.x[2 * j + 1] = xvalid ? x1 : u32x4_t{0, 0, 0, 0};
-    }
-  };
-
-  float4_t acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
-  auto compute = [&](const Stage& s) {
-    const half8_t sc = __builtin_bit_cast(half8_t, s.sc);
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-      // the lane's 16 weights of load j sit in scale block 2j (g < 2) or 2j + 1
-      const half_t sv = g < 2 ? sc[2 * j] : sc[2 * j + 1];
-      const half2_t s2 = {sv, sv};
-      half8_t a0 = dequant8(s.w[j][0], s.w[j][1], s2);
-      half8_t a1 = dequant8(s.w[j][2], s.w[j][3], s2);
-      half8_t b0 = __builtin_bit_cast(half8_t, s.x[2 * j]);
-      half8_t b1 = __builtin_bit_cast(half8_t, s.x[2 * j + 1]);
-      acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, b0, acc0, 0, 0, 0);
-      acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, b1, acc1, 0, 0, 0);
-    }
-  };
-
-  // two-stage software pipeline over this wavefront's macro steps (wave, wave+NW, ...)
-  Stage s0, s1;
-  int ms = wave;
-  if (ms < steps) load(s0, ms);
-  while (ms < steps) {
-    const int nxt = ms + NW;
-    if (nxt < steps) load(s1, nxt);
-    compute(s0);
-    ms = nxt;
-    if (ms >= steps) break;
-    const int nxt2 = ms + NW;
-    if (nxt2 < steps) load(s0, nxt2);
-    compute(s1);
-    ms = nxt2;
-  }
-
-  // accumulator element i of lane (col = lane % 16, grp = lane / 16) is D[4*grp + i][col]:
-  // weight row 4*grp + i, activation row col
-#pragma unroll
-  for (int i = 0; i < 4; i++) partial[wave][(4 * g + i) * 16 + r] = acc0[i] + acc1[i];
-  __syncthreads();
-  for (int e = tid; e < ROWS * 16; e += NW * 64) {
-    const int mm = e / ROWS, nn = e % ROWS;  // consecutive threads -> consecutive output columns
-    if (mm < m && n0 + nn < n) {
-      float sum = 0.0f;
-#pragma unroll
-      for (int w = 0; w < NW; w++) sum += partial[w][nn * 16 + mm];
-      half_t* o = out + (int64_t)mm * n + n0 + nn;
-      // the previous output is read even for beta == 0, as the reference does
-      *o = (half_t)(sum + beta * (float)*o);
-    }
-  }
-}
-
-
-// Variant for wide matrices: a workgroup covers RG groups of 16 weight rows, and a wavefront keeps
-// the activation fragments of its macro step in registers while it walks the RG groups, so the
-// activations are fetched once per 16*RG weight rows instead of once per 16.
-struct WStage {
-  u32x4_t w[4];  // 4 x 16 weight bytes of this lane's row
-  u32x4_t sc;    // the eight fp16 scales (block_size 32) of the macro step
-};
-
-template <int NW, int RG>
-__global__ __launch_bounds__(NW * 64) void gemv_u8_wide_kernel(half_t* __restrict__ out,
-                                                               const half_t* __restrict__ lhs,
-                                                               const uint8_t* __restrict__ rhs,
-                                                               const half_t* __restrict__ scales,
-                                                               int m, int p, int n, float beta) {
-  __shared__ float partial[NW][RG][ROWS * 16];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int r = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * (ROWS * RG);
-  const int nblk = p / 32;
-  const bool xvalid = r < m;
-  const half_t* xrow = lhs + (int64_t)min(r, m - 1) * p + g * 16;
-  const int steps = p / MACRO_K;
-  const uint8_t* wrow[RG];
-  const half_t* srow[RG];
-#pragma unroll
-  for (int q = 0; q < RG; q++) {
-    const int row = min(n0 + q * ROWS + r, n - 1);  // tail rows are clamped, never stored
-    wrow[q] = rhs + (int64_t)row * p + g * 16;
-    srow[q] = scales + (int64_t)row * nblk;
-  }
-  auto load_w = [&](WStage& s, int q, int ms) {
-    const uint8_t* wp = wrow[q] + (int64_t)ms * MACRO_K;
-#pragma unroll
-    for (int j = 0; j < 4; j++) s.w[j] = *(const u32x4_t*)(wp + j * 64);
-    s.sc = *(const u32x4_t*)(srow[q] + ms * (MACRO_K / 32));
-  };
-  auto load_x = [&](u32x4_t (&x)[8], int ms) {
-    const half_t* xp = xrow + (int64_t)ms * MACRO_K;
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-      // (under the lane mask on purpose: measured faster here than unconditional loads of a
-      // clamped row, which is what the 16-row kernel does)
-      x[2 * j] = xvalid ? *(const u32x4_t*)(xp + j * 64) : u32x4_t{0, 0, 0, 0};
-      x[2 * j + 1] = xvalid ? *(const u32x4_t*)(xp + j * 64 + 8) : u32x4_t{0, 0, 0, 0};
-    }
-  };
-  float4_t acc[RG][2];
-#pragma unroll
-  for (int q = 0; q < RG; q++) acc[q][0] = acc[q][1] = float4_t{0, 0, 0, 0};
-  auto compute = [&](const WStage& s, const u32x4_t (&x)[8], float4_t (&a)[2]) {
-    const half8_t sc = __builtin_bit_cast(half8_t, s.sc);
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-      const half_t sv = g < 2 ? sc[2 * j] : sc[2 * j + 1];
-      const half2_t s2 = {sv, sv};
-      half8_t a0 = dequant8(s.w[j][0], s.w[j][1], s2);
-      half8_t a1 = dequant8(s.w[j][2], s.w[j][3], s2);
-      a[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, __builtin_bit_cast(half8_t, x[2 * j]), a[0], 0, 0, 0);
-      a[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, __builtin_bit_cast(half8_t, x[2 * j + 1]), a[1], 0, 0, 0);
-    }
-  };
-
-  // all weight loads of a macro step are issued before its first use
-  for (int ms = wave; ms < steps; ms += NW) {
-    u32x4_t x[8];
-    WStage s[RG];
-    load_x(x, ms);
-#pragma unroll
-    for (int q = 0; q < RG; q++) load_w(s[q], q, ms);
-#pragma unroll
-    for (int q = 0; q < RG; q++) compute(s[q], x, acc[q]);
-  }
-
-#pragma unroll
-  for (int q = 0; q < RG; q++)
-#pragma unroll
-    for (int i = 0; i < 4; i++) partial[wave][q][(4 * g + i) * 16 + r] = acc[q][0][i] + acc[q][1][i];
-  __syncthreads();
-  for (int e = tid; e < RG * ROWS * 16; e += NW * 64) {
-    const int mm = e / (RG * ROWS), nn = e % (RG * ROWS);  // consecutive threads -> consecutive columns
-    if (mm < m && n0 + nn < n) {
-      float sum = 0.0f;
-#pragma unroll
-      for (int w = 0; w < NW; w++) sum += partial[w][nn / ROWS][(nn % ROWS) * 16 + mm];
-      half_t* o = out + (int64_t)mm * n + n0 + nn;
-      // the previous output is read even for beta == 0, as the reference does
-      *o = (half_t)(sum + beta * (float)*o);
-    }
-  }
-}
-
-// K = 4096: weights and activations come in by global -> LDS DMA, four whole 256-byte row
-// pieces per instruction (the register path touches sixteen rows with 64 bytes each per
-// instruction, which moves the same bytes about a quarter slower).  A wavefront owns two macro
+// K = 4096, 17 to 32 activation rows per pass (MB = 2 blocks of sixteen): weights and activations
+// come in by global -> LDS DMA, four whole 256-byte row pieces per instruction, the weights are
+// dequantised to fp16 in registers (the WMMA kernel's arithmetic).  A wavefront owns two macro
 // steps x (2 activation tiles + RG weight row groups) tiles of 4 KiB ([16 rows][16 chunks of 16
 // bytes], chunk c of row r at position c ^ r so that fragment reads spread over all banks) and
 // streams them through a private ring of RING tiles: nothing but its own vmcnt orders the DMA
@@ -364,149 +185,197 @@ __global__ __launch_bounds__(NW * 64) void gemv_u8_ring_kernel(half_t* __restric
   }
 }
 
-// Other K (multiples of 256), sixteen weight rows per workgroup: the same private ring, walked
-// ROUNDS times.  Wavefront w owns macro steps w, w + NW, ...; every ring slot holds one macro step:
-// its 4 KiB weight tile in LDS and its activations and scales in registers.  A slot is refilled
-// right after it has been multiplied, and every refill issues the same 13 memory instructions
-// whether or not the wavefront has a macro step left (the surplus ones read one 16-byte line and
-// are multiplied with zero scales), so the wait before a slot's use is "all but the 13 (RING - 1)
-// youngest" and no load sits under a branch.
-// XR: the slot's activations come through LDS too, as two more tiles of the slot ([16 rows][128
-// halves] each, same chunk swizzle) by eight DMA instructions in place of the eight loads, so
-// the count per slot stays thirteen; a slot is then 12 KiB, which fits with four wavefronts.
-template <int NW, int RING, int ROUNDS, bool XR>
-__global__ __launch_bounds__(NW * 64) void gemv_u8_ring_loop_kernel(half_t* __restrict__ out,
-                                                                    const half_t* __restrict__ lhs,
-                                                                    const uint8_t* __restrict__ rhs,
-                                                                    const half_t* __restrict__ scales,
-                                                                    int m, int p, int n, float beta) {
-  constexpr int TILE = ROWS * MACRO_K;
-  constexpr int SLOT = XR ? 3 * TILE : TILE;  // weight tile, then the two activation tiles
-  constexpr int PER = 8 + 1 + 4;  // activation loads, scale load, DMA instructions per slot
-  static_assert(NW * RING * SLOT <= 160 * 1024 && NW * 256 * 4 <= NW * RING * SLOT, "LDS");
-  __shared__ __attribute__((aligned(1024))) unsigned char ring[NW * RING * SLOT];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int r = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * ROWS;
-  const int nblk = p / 32;
-  const bool xvalid = r < m;
-  const int steps = p / MACRO_K;
-  const half_t* xrow = lhs + (int64_t)min(r, m - 1) * p + g * 16;
-  const half_t* srow = scales + (int64_t)min(n0 + r, n - 1) * nblk;
-  unsigned char* const mine = ring + wave * RING * SLOT;
-  // DMA instruction i of a tile fills its chunks [64 i, 64 i + 64): rows 4i .. 4i+3
-  const uint8_t* wsrc[4];
-  const half_t* xsrc[4];
+// 3 to 16 activation rows, any K % 256 == 0, block size 32.  A workgroup of eight wavefronts owns
+// RG groups of sixteen weight rows; wavefront w owns the macro steps (256 k) w, w + 8, ...  Per
+// macro step a wavefront handles PER = 2 + RG tiles of 4 KiB ([16 rows][256 bytes]): two of
+// activations (k 0..127 and 128..255 of the step as fp16) and RG of weights.  Tile u of every
+// step has its own four registers per lane; the request for a tile is issued three tiles before
+// its use (two with one row group), as four instructions of 4 rows x 256 contiguous bytes (quarter a of the wavefront takes
+// row 4i + a, lane x of the quarter the 16-byte chunk x).  On arrival the tile goes through the
+// wavefront's private LDS tile (chunk c of row r at position c ^ r: both directions free of bank
+// conflicts) and comes back in matrix-core operand layout: lane (r, g) gets, of row r, the 8
+// weights g of a scale block, or the 8 activations g of its 32.
+// Arithmetic per scale block b of a weight row (the naive kernel's formula, matmul_nt_fp16u8.cu:
+// 17-21, in fp32):  sum_k x_k (q_k - 127.5) s_b = s_b (sum_k x_k (1024 + q_k) - 1151.5 sum_k x_k).
+// The activations are the FIRST matrix-core operand, so a lane's four results are four
+// activation rows of ONE weight row (lane % 16) and take one scale; sum_k x_k comes from a
+// product with an all-ones operand once per step and enters the block's product as accumulator
+// input, times -1151.5.  Every product x_k (1024 + q_k) is exact in fp32.
+// MQ: groups of four activation rows that exist (requests for the others are left out at compile
+// time; the LDS tile then holds stale rows there, which only reach results that are not stored).
+template <int RG, int MQ>
+__global__ __launch_bounds__(512) void gemv_u8_regstream_kernel(half_t* __restrict__ out,
+                                                                const half_t* __restrict__ lhs,
+                                                                const uint8_t* __restrict__ rhs,
+                                                                const half_t* __restrict__ scales,
+                                                                int m, int p, int n, float beta) {
+  constexpr int NW = 8, TILE = ROWS * MACRO_K, RB = ROWS * RG, PER = 2 + RG;
+  constexpr int DIST = PER - 1 < 3 ? PER - 1 : 3;  // tiles between a request and its use
+  __shared__ __attribute__((aligned(1024))) unsigned char shuf[NW][TILE];
+  __shared__ float partial[NW][RG][256];
+  const int tid = threadIdx.x, lane = tid & 63;
+  // (wave-uniform by construction; said so, the step's addresses live in scalar registers)
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int a = lane >> 4, x = lane & 15;  // request role: quarter a takes row 4i + a, chunk x
+  const int r = lane & 15, g = lane >> 4;  // operand role: row r, group g of 8 within a block of 32
+  const int n0 = blockIdx.x * RB;
+  const int nblk = p / 32, steps = p / MACRO_K, last = steps - 1;
+  unsigned char* const mine = shuf[wave];
+  // the previous output of the elements this thread will store, requested before anything else
+  // (unconditionally, from a clamped address: a load under a lane mask is waited for where the
+  // lanes rejoin); read even for beta == 0, as the reference does
+  constexpr int EPT = (RB * 16 + NW * 64 - 1) / (NW * 64);
+  half_t prev[EPT];
 #pragma unroll
-  for (int i = 0; i < 4; i++) {
-    const int row = 4 * i + (lane >> 4), kc = (lane & 15) ^ row;
-    wsrc[i] = rhs + (int64_t)min(n0 + row, n - 1) * p + kc * 16;
-    xsrc[i] = lhs + (int64_t)min(row, m - 1) * p + kc * 8;
+  for (int k = 0; k < EPT; k++) {
+    const int e = tid + k * NW * 64, mm = e / RB, nn = e % RB;
+    prev[k] = out[(int64_t)min(mm, m - 1) * n + min(n0 + nn, n - 1)];
   }
-  int roff[4];  // fragment read j of the lane: logical chunk 4j + g of row r
+  // scales of a step: the eight blocks of row q * 16 + r (16 bytes), requested a whole step ahead
+  uint32_t so[RG];
 #pragma unroll
-  for (int j = 0; j < 4; j++) roff[j] = r * 256 + (((4 * j + g) ^ r) << 4);
-  int xoff[4];  // activation fragment 2 jj + e of a tile: logical chunk 8 jj + 2 g + e of row r
+  for (int q = 0; q < RG; q++) so[q] = (uint32_t)min(q * ROWS + r, n - 1 - n0) * (uint32_t)nblk * 2u;
+  const unsigned char* const sbase = (const unsigned char*)(scales + (int64_t)n0 * nblk);
+  u32x4_t sc[RG], sc_next[RG];
 #pragma unroll
-  for (int f = 0; f < 4; f++) xoff[f] = r * 256 + (((8 * (f >> 1) + 2 * g + (f & 1)) ^ r) << 4);
-
-  u32x4_t x[XR ? 1 : RING][8];
-  u32x4_t sc[RING];
-  auto issue = [&](int slot, int ms) {
-    const bool live = ms < steps;  // wave-uniform
-    const int64_t koff = live ? (int64_t)ms * MACRO_K : 0;
-    const half_t* xp = xrow + koff;
-    if constexpr (XR) {
+  for (int q = 0; q < RG; q++) sc[q] = *(const u32x4_t*)(sbase + min(wave, last) * 16 + so[q]);
+  // Request addresses: a uniform base per step (scalar registers) plus one 32-bit byte offset per
+  // lane and instruction.  Rows beyond m read row m - 1 again and rows beyond n row n - 1 (their
+  // products are never stored).
+  uint32_t xo[MQ], wo[RG][4];
 #pragma unroll
-      for (int t = 0; t < 2; t++)
+  for (int i = 0; i < MQ; i++) xo[i] = (uint32_t)min(4 * i + a, m - 1) * (uint32_t)p * 2u + x * 16;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-          // (rows beyond m read row m - 1 again and are zeroed when used)
-          const half_t* src = live ? xsrc[i] + koff + t * 128 : lhs;
-          __builtin_amdgcn_global_load_lds(
-              ADR_GLB_PTR(src), ADR_LDS_PTR(mine + slot * SLOT + (1 + t) * TILE + i * 1024), 16, 0, 0);
-        }
-    } else {
+  for (int q = 0; q < RG; q++)
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        // lanes beyond m read row m-1 again (the same addresses as its own lanes) and are zeroed
-        // when used: a load under a lane mask would be waited for where the lanes rejoin
-        x[slot][2 * j] = *(const u32x4_t*)(xp + j * 64);
-        x[slot][2 * j + 1] = *(const u32x4_t*)(xp + j * 64 + 8);
-      }
-    }
-    sc[slot] = *(const u32x4_t*)(srow + (live ? ms * (MACRO_K / 32) : 0));
+    for (int i = 0; i < 4; i++)
+      wo[q][i] = (uint32_t)min(q * ROWS + 4 * i + a, n - 1 - n0) * (uint32_t)p + x * 16;
+  const unsigned char* const xbase = (const unsigned char*)lhs;
+  const unsigned char* const wbase = rhs + (int64_t)n0 * p;
+  u32x4_t ld[PER][4];
+  auto request = [&](int ms, int u) {  // tile u of macro step ms into its registers
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-      // a surplus slot fetches one 16-byte line (all lanes the same address)
-      const uint8_t* src = live ? wsrc[i] + koff : rhs;
-      __builtin_amdgcn_global_load_lds(ADR_GLB_PTR(src),
-                                       ADR_LDS_PTR(mine + slot * SLOT + i * 1024), 16, 0, 0);
+      if (u < 2) {
+        if (i < MQ) ld[u][i] = *(const u32x4_t*)(xbase + (int64_t)ms * (MACRO_K * 2) + u * 256 + xo[i]);
+      } else {
+        // streaming load: a weight byte is read once per launch
+        ld[u][i] = __builtin_nontemporal_load(
+            (const u32x4_t*)(wbase + (int64_t)ms * MACRO_K + wo[u - 2][i]));
+      }
     }
   };
-  float4_t acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
 #pragma unroll
-  for (int i = 0; i < RING; i++) issue(i, wave + i * NW);
-  // ROUNDS = ceil(ceil(steps / NW) / RING), the same for every wavefront; unrolled, because the
-  // compiler drains all loads at the head of a run-time loop that carries loads in registers
+  for (int u = 0; u < DIST; u++) request(min(wave, last), u);
+
+  int woff[4], roff[8], xoff[4];
 #pragma unroll
-  for (int rd = 0; rd < ROUNDS; rd++) {
+  for (int i = 0; i < 4; i++) woff[i] = (4 * i + a) * 256 + ((x ^ (4 * i + a)) << 4);
+  // weights of block b = bytes 32 b .. 32 b + 31 of the row: lane (r, g) takes bytes 8 g .. 8 g + 7
 #pragma unroll
-    for (int i = 0; i < RING; i++) {
-      // slots issued after this one: RING - 1, fewer at the very end
-      const int later = PER * (rd + 1 < ROUNDS ? RING - 1 : RING - 1 - i);
-      static_assert(RING == 3, "the three wait immediates below");
-      if (later == 2 * PER) __builtin_amdgcn_s_waitcnt(0x0F70 | ((2 * PER) & 0xF) | (((2 * PER) >> 4) << 14));
-      else if (later == PER) __builtin_amdgcn_s_waitcnt(0x0F70 | (PER & 0xF) | ((PER >> 4) << 14));
-      else __builtin_amdgcn_s_waitcnt(0x0F70);
-      const unsigned char* tile = mine + i * SLOT;
-      u32x4_t w[4];
+  for (int b = 0; b < 8; b++) roff[b] = r * 256 + (((2 * b + (g >> 1)) ^ r) << 4) + (g & 1) * 8;
+  // activations of block b = chunks 4 b .. 4 b + 3 of the step: tile b / 4, chunk 4 (b % 4) + g
 #pragma unroll
-      for (int j = 0; j < 4; j++) w[j] = *(const u32x4_t*)(tile + roff[j]);
-      if constexpr (XR) {
+  for (int b = 0; b < 4; b++) xoff[b] = r * 256 + (((4 * b + g) ^ r) << 4);
+
+  float4_t acc[RG];
 #pragma unroll
-        for (int f = 0; f < 8; f++) x[0][f] = *(const u32x4_t*)(tile + (1 + f / 4) * TILE + xoff[f % 4]);
-        // tile and activations are in registers before the slot is refilled below
-        __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
-      }
-      // zero scales for a surplus slot: it adds nothing (selected here, not where the scales
-      // are loaded: a use right behind the load would wait for it and everything before it)
-      const u32x4_t z = {0, 0, 0, 0};
-      const bool live = wave + (rd * RING + i) * NW < steps;
-      const half8_t s8 = __builtin_bit_cast(half8_t, live ? sc[i] : z);
+  for (int q = 0; q < RG; q++) acc[q] = float4_t{0, 0, 0, 0};
+  const half_t one = (half_t)1.0f;
+  const half8_t ones = {one, one, one, one, one, one, one, one};
+  half8_t xf[8];    // activation operands of the step's eight blocks
+  float4_t c0[8];   // -1151.5 * their sums, in result layout
+
+#pragma unroll 1
+  for (int ms = wave; ms < steps; ms += NW) {
+    const int ms_next = min(ms + NW, last);  // (past the end: the last step again, never used)
 #pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const half_t sv = g < 2 ? s8[2 * j] : s8[2 * j + 1];
-        const half2_t s2 = {sv, sv};
-        const half8_t a0 = dequant8(w[j][0], w[j][1], s2), a1 = dequant8(w[j][2], w[j][3], s2);
-        const half8_t b0 = __builtin_bit_cast(half8_t, xvalid ? x[XR ? 0 : i][2 * j] : z);
-        const half8_t b1 = __builtin_bit_cast(half8_t, xvalid ? x[XR ? 0 : i][2 * j + 1] : z);
-        acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, b0, acc0, 0, 0, 0);
-        acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, b1, acc1, 0, 0, 0);
-      }
-      // the slot's tile and registers have been consumed: refill it
+    for (int u = 0; u < PER; u++) {
       __builtin_amdgcn_sched_barrier(0);
-      if (rd + 1 < ROUNDS) issue(i, wave + ((rd + 1) * RING + i) * NW);
+      if (u + DIST < PER) request(ms, u + DIST); else request(ms_next, u + DIST - PER);
+      if (u == 0) {
+#pragma unroll
+        for (int q = 0; q < RG; q++) sc_next[q] = *(const u32x4_t*)(sbase + ms_next * 16 + so[q]);
+      }
       __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+        if (u >= 2 || i < MQ) *(u32x4_t*)(mine + woff[i]) = ld[u][i];
+      if (u < 2) {
+#pragma unroll
+        for (int b = 0; b < 4; b++) xf[4 * u + b] = *(const half8_t*)(mine + xoff[b]);
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+          const float4_t z = {0, 0, 0, 0};
+          c0[4 * u + b] =
+              __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[4 * u + b], ones, z, 0, 0, 0) * -1151.5f;
+        }
+      } else {
+        const int q = u - 2;
+        const half8_t s8 = __builtin_bit_cast(half8_t, sc[q]);
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          u32x2_t w[4];
+#pragma unroll
+          for (int b = 0; b < 4; b++) w[b] = *(const u32x2_t*)(mine + roff[4 * h + b]);
+#pragma unroll
+          for (int b = 0; b < 4; b++) {
+            // bytes b0..b3 of a dword -> halves (1024 + b0, 1024 + b1) and (1024 + b2, 1024 + b3)
+            u32x4_t v;
+            v[0] = __builtin_amdgcn_perm(0x64646464u, w[b][0], 0x07010700u);
+            v[1] = __builtin_amdgcn_perm(0x64646464u, w[b][0], 0x07030702u);
+            v[2] = __builtin_amdgcn_perm(0x64646464u, w[b][1], 0x07010700u);
+            v[3] = __builtin_amdgcn_perm(0x64646464u, w[b][1], 0x07030702u);
+            const float4_t d = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                xf[4 * h + b], __builtin_bit_cast(half8_t, v), c0[4 * h + b], 0, 0, 0);
+            acc[q] += d * (float)s8[4 * h + b];
+          }
+        }
+      }
     }
+#pragma unroll
+    for (int q = 0; q < RG; q++) sc[q] = sc_next[q];
   }
 
-  __syncthreads();
-  float* partial = (float*)ring;  // [NW][256]
+  // lane (weight row r, group g): acc[q][i] belongs to activation row 4 g + i
 #pragma unroll
-  for (int i = 0; i < 4; i++) partial[wave * 256 + (4 * g + i) * 16 + r] = acc0[i] + acc1[i];
-  __syncthreads();
-  for (int e = tid; e < ROWS * 16; e += NW * 64) {
-    const int mm = e / ROWS, nn = e % ROWS;  // consecutive threads -> consecutive output columns
-    if (mm < m && n0 + nn < n) {
+  for (int q = 0; q < RG; q++)
+#pragma unroll
+    for (int i = 0; i < 4; i++) partial[wave][q][r * 16 + 4 * g + i] = acc[q][i];
+  // (not __syncthreads(): its fence would wait for the surplus requests of the last step)
+  __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): the partial sums are in LDS
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int k = 0; k < EPT; k++) {
+    const int e = tid + k * NW * 64, mm = e / RB, nn = e % RB;  // consecutive threads -> consecutive columns
+    if (e < RB * 16 && mm < m && n0 + nn < n) {
       float sum = 0.0f;
 #pragma unroll
-      for (int w2 = 0; w2 < NW; w2++) sum += partial[w2 * 256 + nn * 16 + mm];
-      half_t* o = out + (int64_t)mm * n + n0 + nn;
-      // the previous output is read even for beta == 0, as the reference does
-      *o = (half_t)(sum + beta * (float)*o);
+      for (int w2 = 0; w2 < NW; w2++) sum += partial[w2][nn / ROWS][(nn % ROWS) * 16 + mm];
+      out[(int64_t)mm * n + n0 + nn] = (half_t)(sum + beta * (float)prev[k]);
     }
   }
+}
+
+template <int RG>
+hipError_t launch_regstream(hipStream_t stream, half_t* out, const half_t* lhs, const uint8_t* rhs,
+                            const half_t* scales, int m, int p, int n, float beta) {
+  const dim3 grid((n + ROWS * RG - 1) / (ROWS * RG)), block(512);
+  switch ((m + 3) / 4) {
+    case 1: hipLaunchKernelGGL((gemv_u8_regstream_kernel<RG, 1>), grid, block, 0, stream, out, lhs, rhs, scales, m, p, n, beta); break;
+    case 2: hipLaunchKernelGGL((gemv_u8_regstream_kernel<RG, 2>), grid, block, 0, stream, out, lhs, rhs, scales, m, p, n, beta); break;
+    case 3: hipLaunchKernelGGL((gemv_u8_regstream_kernel<RG, 3>), grid, block, 0, stream, out, lhs, rhs, scales, m, p, n, beta); break;
+    default: hipLaunchKernelGGL((gemv_u8_regstream_kernel<RG, 4>), grid, block, 0, stream, out, lhs, rhs, scales, m, p, n, beta); break;
+  }
+  return hipGetLastError();
+}
+
+// groups of sixteen weight rows per workgroup: as many as still give every compute unit a
+// workgroup (at most three: 48 rows share one fetch of the activations)
+int regstream_row_groups(int n) {
+  const int cus = device_info_for_plan().cus;
+  const int groups = (n + ROWS - 1) / ROWS;
+  return groups >= 3 * cus - cus / 2 ? 3 : groups >= 2 * cus - cus / 2 ? 2 : 1;
 }
 
 // MR activation rows, NW wavefronts, RPB weight rows per workgroup, SEGW 1 KiB K segments per
@@ -672,9 +541,9 @@ U8Choice choose_u8(const void* lhs, const void* rhs, const void* scales, int m, 
 }
 
 // 17 to 64 activation rows (to 128 on matrices under 8192 rows) against at least 4 MiB of
-// weights: the sixteen-row kernels once per block of sixteen rows.  The tiled GEMM walks K on
+// weights: the sixteen-row kernels once per block of rows.  The tiled GEMM walks K on
 // N / 64 .. N / 128 CUs for these (K4096 N4096 m=17..32 42.9 us, m=64..128 58.5; N12288 53.4 ..
-// 68.5; K11008 N4096 133 .. 171) where a sixteen-row launch takes 7.2 / 15.3 / 17.1 us (N12288
+// 68.5; K11008 N4096 133 .. 171) where a sixteen-row launch takes 7 / 14 / 15 us (N12288
 // m=96: 78.4 us in blocks against 68.3 tiled, hence the narrower bound there).
 bool rows_in_blocks_of_16(int m, int p, int n, int block_size) {
   return m > 16 && m <= (n < 8192 ? 128 : 64) && (int64_t)n * p >= (1 << 22) &&
@@ -691,13 +560,11 @@ bool gemm_u8_mfma_supported(const half_t* lhs, const uint8_t* rhs, const half_t*
                             int n, int block_size);
 
 const char* gemm_u8_plan(int m, int p, int n, int block_size) {
-  if (rows_in_blocks_of_16(m, p, n, block_size)) m = 16;
+  if (rows_in_blocks_of_16(m, p, n, block_size))
+    return p == 16 * MACRO_K ? "gemv_u8_mfma16_dma_32rows" : "gemv_u8_mfma16_regstream";
   switch (choose_u8(nullptr, nullptr, nullptr, m, p, n, block_size)) {
     case U8_DOT: return "gemv_u8_dot2_stream";
-    case U8_GEMV:
-      if (p == 16 * MACRO_K) return n < 8192 ? "gemv_u8_mfma16_dma" : "gemv_u8_mfma16_wide_dma";
-      if (n < 8192 && p > 16 * MACRO_K && p <= 72 * MACRO_K) return "gemv_u8_mfma16_dma";
-      return n < 8192 ? "gemv_u8_mfma16_stream" : "gemv_u8_mfma16_wide";
+    case U8_GEMV: return "gemv_u8_mfma16_regstream";
     case U8_GEMM: {
       // the tile is part of the name: "gemm_nt_u8_mfma_256x192x64", "gemm_nt_u8_stage_128x128x32", ...
       const char* tiled = gemm_u8_mfma_plan(m, p, n, block_size);
@@ -751,53 +618,12 @@ hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, co
       if (m == 1) return launch_dot<1, 8, 4, 2>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
       return launch_dot<2, 8, 4, 2>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
     }
-    case U8_GEMV: {
-      const int blocks = (n + ROWS - 1) / ROWS;
-      const int steps = p / MACRO_K;
-      // enough wavefronts per workgroup to keep every macro step of a small problem in flight
-      // wide matrices: 48 weight rows per workgroup share one fetch of the activations
-      if (n >= 8192) {
-        if (steps == 16)
-          hipLaunchKernelGGL((gemv_u8_ring_kernel<8, 3, 4, 1>), dim3((n + 3 * ROWS - 1) / (3 * ROWS)),
-                             dim3(512), 0, stream, out, lhs, rhs, scales, m, p, n, beta);
-        else
-          hipLaunchKernelGGL((gemv_u8_wide_kernel<8, 3>), dim3((n + 3 * ROWS - 1) / (3 * ROWS)),
-                             dim3(512), 0, stream, out, lhs, rhs, scales, m, p, n, beta);
-        return hipGetLastError();
+    case U8_GEMV:
+      switch (regstream_row_groups(n)) {
+        case 3: return launch_regstream<3>(stream, out, lhs, rhs, scales, m, p, n, beta);
+        case 2: return launch_regstream<2>(stream, out, lhs, rhs, scales, m, p, n, beta);
+        default: return launch_regstream<1>(stream, out, lhs, rhs, scales, m, p, n, beta);
       }
-      if (steps == 16) {
-        hipLaunchKernelGGL((gemv_u8_ring_kernel<8, 1, 4, 1>), dim3(blocks), dim3(512), 0, stream, out,
-                           lhs, rhs, scales, m, p, n, beta);
-        return hipGetLastError();
-      }
-      // ten rows and more, K 9472 .. 12288: four wavefronts, activations through LDS (K11008
-      // N4096: m=16 19.7 -> 17.1 us, m=12 17.8 -> 16.5; m=8 16.3 -> 16.9, so not below ten)
-      if (steps > 16 && m >= 10 && ((steps + 3) / 4 + 2) / 3 == 4) {
-        hipLaunchKernelGGL((gemv_u8_ring_loop_kernel<4, 3, 4, true>), dim3(blocks), dim3(256), 0, stream,
-                           out, lhs, rhs, scales, m, p, n, beta);
-        return hipGetLastError();
-      }
-      if (steps > 16) {
-        const int rounds = ((steps + 7) / 8 + 2) / 3;
-        if (rounds == 1)
-          hipLaunchKernelGGL((gemv_u8_ring_loop_kernel<8, 3, 1, false>), dim3(blocks), dim3(512), 0, stream,
-                             out, lhs, rhs, scales, m, p, n, beta);
-        else if (rounds == 2)
-          hipLaunchKernelGGL((gemv_u8_ring_loop_kernel<8, 3, 2, false>), dim3(blocks), dim3(512), 0, stream,
-                             out, lhs, rhs, scales, m, p, n, beta);
-        else if (rounds == 3)
-          hipLaunchKernelGGL((gemv_u8_ring_loop_kernel<8, 3, 3, false>), dim3(blocks), dim3(512), 0, stream,
-                             out, lhs, rhs, scales, m, p, n, beta);
-        if (rounds <= 3) return hipGetLastError();
-      }
-      if (steps >= 16 && blocks <= 1024)
-        hipLaunchKernelGGL(gemv_u8_kernel<8>, dim3(blocks), dim3(512), 0, stream, out, lhs, rhs,
-                           scales, m, p, n, beta);
-      else
-        hipLaunchKernelGGL(gemv_u8_kernel<4>, dim3(blocks), dim3(256), 0, stream, out, lhs, rhs,
-                           scales, m, p, n, beta);
-      return hipGetLastError();
-    }
     case U8_GEMM:
       if (gemm_u8_mfma_supported(lhs, rhs, scales, m, p, n, block_size))
         return launch_gemm_u8_mfma(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);

@@ -74,13 +74,15 @@ def test_u8_plan():
     for m in (1, 2):
         assert plan(m, 4096, 4096, 32) == (0, "gemv_u8_dot2_stream")
         assert plan(m, 11008, 4096, 32) == (0, "gemv_u8_dot2_stream")
-    for m in (4, 16):
-        assert plan(m, 4096, 4096, 32) == (0, "gemv_u8_mfma16_dma")
-        assert plan(m, 11008, 4096, 32) == (0, "gemv_u8_mfma16_dma")
+    for m in (3, 4, 16):
+        assert plan(m, 4096, 4096, 32) == (0, "gemv_u8_mfma16_regstream")
+        assert plan(m, 11008, 4096, 32) == (0, "gemv_u8_mfma16_regstream")
+        assert plan(m, 4096, 12288, 32) == (0, "gemv_u8_mfma16_regstream")
+        assert plan(m, 256, 16, 32) == (0, "gemv_u8_mfma16_regstream")
     assert plan(2, 4096, 12288, 32) == (0, "gemv_u8_dot2_stream")
-    assert plan(4, 4096, 12288, 32) == (0, "gemv_u8_mfma16_wide_dma")
-    assert plan(4, 2048, 12288, 32) == (0, "gemv_u8_mfma16_wide")
-    assert plan(16, 4096, 4096, 32) == (0, "gemv_u8_mfma16_dma")
+    # 17 to 64 rows in blocks of rows: 32 per pass for K = 4096, 16 otherwise
+    assert plan(32, 4096, 12288, 32) == (0, "gemv_u8_mfma16_dma_32rows")
+    assert plan(32, 11008, 4096, 32) == (0, "gemv_u8_mfma16_regstream")
     # tiled kernels: the name carries the tile
     assert plan(2048, 4096, 4096, 32) == (0, "gemm_nt_u8_mfma_256x128x64")
     assert plan(2048, 4096, 12288, 32) == (0, "gemm_nt_u8_mfma_256x192x64")

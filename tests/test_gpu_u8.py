@@ -120,11 +120,10 @@ def _finite_scale_rows():
 @pytest.mark.parametrize("every", [1, 8], ids=["all_scales", "every_8th_scale"])
 def test_fused_dequant_in_gemv_is_bit_exact_for_every_q_and_finite_scale(kern, m, every):
     """One-hot activations pick single weights out of the matmul: out[r, c] = w[c, k_r].
-    All finite scales make a wide matrix (48-row workgroups), every 8th a narrow one."""
+    All finite scales make a wide matrix (48-row workgroups), every 8th a narrower one (32)."""
     scales_bits = _finite_scale_rows()[::every]
     n, p, bs = scales_bits.size, 256, 32
-    assert u8_plan(m, p, n, bs) == ("gemv_u8_dot2_stream" if m <= 2 else
-                                    "gemv_u8_mfma16_wide" if n >= 8192 else "gemv_u8_mfma16_stream")
+    assert u8_plan(m, p, n, bs) == ("gemv_u8_dot2_stream" if m <= 2 else "gemv_u8_mfma16_regstream")
     q = np.tile(np.arange(256, dtype=np.uint8), (n, 1))
     s = np.repeat(scales_bits.view(np.float16).reshape(n, 1), p // bs, axis=1)
     table = oracle.dequant_table()  # [q][scale bits]
@@ -177,7 +176,7 @@ def _u8_case(g, m, p, n, bs, exact):
     return a, q, s
 
 
-@pytest.mark.parametrize("m", [1, 2, 4, 7, 16])
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 7, 8, 9, 12, 13, 16])
 @pytest.mark.parametrize("pn", [(256, 16), (512, 100), (1024, 33), (2816, 48), (4096, 52),
                                 (5120, 40), (11008, 24)])
 def test_gemv_bit_exact_on_exact_inputs(kern, m, pn):
@@ -195,11 +194,11 @@ def test_gemv_bit_exact_on_exact_inputs(kern, m, pn):
 
 @pytest.mark.parametrize("m", [3, 16])
 def test_wide_dma_gemv_bit_exact_on_exact_inputs(kern, m):
-    """K = 4096 on a wide matrix: the weights stream through the per-wavefront LDS ring; ragged
-    last workgroup (8251 = 171 * 48 + 43 rows), beta path."""
-    p, n = 4096, 8251
+    """K = 4096 on a wide matrix (48 rows per workgroup, two macro steps per wavefront); ragged
+    last workgroup (12251 = 255 * 48 + 11 rows), beta path."""
+    p, n = 4096, 12251
     g = rng(990 + m)
-    assert u8_plan(m, p, n, 32) == "gemv_u8_mfma16_wide_dma"
+    assert u8_plan(m, p, n, 32) == "gemv_u8_mfma16_regstream"
     a, q, s = _u8_case(g, m, p, n, 32, exact=True)
     for beta in (0.0, 1.0):
         prev = (g.integers(-8, 9, size=(m, n)) / 4.0).astype(np.float16)
@@ -213,10 +212,11 @@ def test_wide_dma_gemv_bit_exact_on_exact_inputs(kern, m):
 @pytest.mark.parametrize("m", [3, 7, 16])
 @pytest.mark.parametrize("pn", [(256, 8192), (768, 8200), (1024, 8251)])
 def test_wide_gemv_bit_exact_on_exact_inputs(kern, m, pn):
-    """The 48-rows-per-workgroup variant (n >= 8192): ragged last workgroup, beta path."""
+    """32 rows per workgroup (n around 8192) with one to four macro steps, i.e. wavefronts
+    without any step of their own: ragged last workgroup, beta path."""
     p, n = pn
     g = rng(660 + m + p)
-    assert u8_plan(m, p, n, 32) == "gemv_u8_mfma16_wide"
+    assert u8_plan(m, p, n, 32) == "gemv_u8_mfma16_regstream"
     a, q, s = _u8_case(g, m, p, n, 32, exact=True)
     for beta in (0.0, 1.0):
         prev = (g.integers(-8, 9, size=(m, n)) / 4.0).astype(np.float16)
@@ -380,8 +380,7 @@ def test_decode_shapes_full_size(kern, kn, m):
     q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)
     s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
     a = torch.randn(m, p, generator=gen, device="cuda").half()
-    assert u8_plan(m, p, n, 32) in ("gemv_u8_mfma16_stream", "gemv_u8_mfma16_wide",
-                                    "gemv_u8_mfma16_wide_dma", "gemv_u8_mfma16_dma", "gemv_u8_dot2_stream")
+    assert u8_plan(m, p, n, 32) == ("gemv_u8_dot2_stream" if m <= 2 else "gemv_u8_mfma16_regstream")
     out = torch.zeros(m, n, dtype=torch.float16, device="cuda")
     kern.matmul_nt_fp16u8(out, a, q, s, 32)
     w = torch.zeros(n, p, dtype=torch.float16, device="cuda")
@@ -399,15 +398,16 @@ def test_decode_shapes_full_size(kern, kn, m):
 @pytest.mark.parametrize("m", [10, 13, 16])
 @pytest.mark.parametrize("kn", [(11008, 1000), (9472, 530), (12288, 700)])
 def test_decode_ten_rows_and_more_long_k(kern, kn, m):
-    """K 9472 .. 12288 with ten to sixteen rows: the kernel whose activations travel through LDS;
-    ragged N, surplus ring slots (K 9472: 37 steps for 4 x 12 slots), previous output added."""
+    """K 9472 .. 12288 with ten to sixteen rows: five and six macro steps per wavefront with
+    uneven counts over the wavefronts (37, 43 and 48 steps over eight), ragged N, previous output
+    added."""
     p, n = kn
     gen = torch.Generator(device="cuda").manual_seed(46 + m + p)
     q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)
     s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
     a = torch.randn(m, p, generator=gen, device="cuda").half()
     prev = torch.randn(m, n, generator=gen, device="cuda").half()
-    assert u8_plan(m, p, n, 32) == "gemv_u8_mfma16_dma"
+    assert u8_plan(m, p, n, 32) == "gemv_u8_mfma16_regstream"
     out = prev.clone()
     assert _ffi.lib().adr_matmul_nt_fp16u8(torch.cuda.current_stream().cuda_stream, out.data_ptr(),
                                            a.data_ptr(), q.data_ptr(), s.data_ptr(), m, p, n, 32, 0.5) == 0
@@ -427,7 +427,8 @@ def test_seventeen_and_more_rows_in_blocks_of_sixteen(kern, kn, m):
     more rows stay on the tiled GEMM.  Previous output added, ragged N."""
     p, n = kn
     limit = 128 if n < 8192 else 64
-    assert (u8_plan(m, p, n, 32) == u8_plan(16, p, n, 32)) if m <= limit else \
+    blocks = "gemv_u8_mfma16_dma_32rows" if p == 4096 else "gemv_u8_mfma16_regstream"
+    assert (u8_plan(m, p, n, 32) == blocks) if m <= limit else \
         u8_plan(m, p, n, 32).startswith("gemm_nt_u8_")
     assert u8_plan(limit + 1, p, n, 32).startswith("gemm_nt_u8_")
     gen = torch.Generator(device="cuda").manual_seed(47 + m + p)
