@@ -8,10 +8,13 @@ A "step" is one pass over the LLaMA-7B per-layer GEMM set at prefill M=2048 in f
 every launch going through the C ABI (adr_matmul_f16) with operands resident in HBM.
 Prints ONE JSON line.  `value` is the fp16 TFLOP/s of that step; `roofline` is the dominant
 kernel (the MFMA GEMM on the QKV shape) timed with HIP events on the launch stream;
-`cpu_baseline` is the CPU oracle (a scalar restatement of the reference kernel, OpenMP over
-rows) on a bounded sample of the same workload, timed on this machine's host cores;
-`secondary` carries the other benchmark configurations: the u8 decode GEMV in GB/s against
-the HBM peak, the u8 prefill GEMMs, the CLIP GEMMs and the attention products.
+`roofline_u8_gemv` is the same for the u8 decode GEMV (the other half of the metric), with a
+plain streaming read of the same bytes timed beside it; `cpu_baseline` is the CPU side of every
+benchmark configuration on bounded samples, timed on this machine's host cores: torch-CPU fp32
+matmul on the same seeded fp16 inputs (the style of the reference's py/gen_tests generator), a
+blocked OpenMP fp32 GEMM (the counterpart of its host sgemm) and the scalar restatement of its
+kernel; `secondary` carries the other benchmark configurations: the u8 decode GEMV in GB/s
+against the HBM peak, the u8 prefill GEMMs, the CLIP GEMMs and the attention products.
 
 Input data is synthetic (seeded): activations ~ N(0,1), weights ~ N(0,1/sqrt(K)) in fp16;
 u8 weights uniform with fp16 scales ~ U(0.001, 0.02) per 32 weights.
@@ -36,6 +39,25 @@ LAYER_SET = [  # (name, K, N) at M = 2048
     ("down", 11008, 4096),
 ]
 DECODE_SET = [(4096, 4096), (4096, 11008), (4096, 12288), (11008, 4096)]
+
+
+def profile_figures(name):
+    """The machine-readable lines of a rocprofv3 summary under profiles/: `@bench key=value ...`
+    (figures measured with counters, which this script cannot collect itself)."""
+    out = {}
+    try:
+        with open(os.path.join(ROOT, "profiles", name)) as f:
+            for line in f:
+                if line.startswith("@bench "):
+                    for item in line.split()[1:]:
+                        k, _, v = item.partition("=")
+                        try:
+                            out[k] = float(v)
+                        except ValueError:
+                            out[k] = v
+    except OSError:
+        pass
+    return out
 
 
 def main():
@@ -128,7 +150,7 @@ def main():
 
     # ---- u8 decode GEMV (benchmark configs[2]): weight buffers rotate through > 256 MB so
     # that repeats stream from HBM, not from the Infinity Cache
-    def u8_case(m, K, N, iters):
+    def u8_case(m, K, N, iters, probe=False):
         per = N * K + N * (K // 32) * 2
         nbuf = max(2, int(600e6 // per) + 1)
         qs = [torch.randint(0, 256, (N, K), generator=gen, device=dev, dtype=torch.uint8)
@@ -147,7 +169,28 @@ def main():
             if rc != 0:
                 raise RuntimeError(_ffi.strerror(rc))
         t = timed_graph(f, 2 * nbuf, max(2, iters // (2 * nbuf)))
-        return t, per + m * K * 2 + m * N * 2
+        t_probe = None
+        if probe:
+            # a plain streaming read of the same weight bytes (one contiguous piece per workgroup,
+            # nothing computed, nothing written) through the same rotation and the same graph
+            # replays: what this part delivers for this many bytes in one launch
+            sink = torch.zeros(1, dtype=torch.int32, device=dev)
+            best = None
+            for blocks in (1024, 2048, 4096):
+                if (N * K) % (16 * blocks):
+                    continue
+
+                def g():
+                    j = i[0] % nbuf
+                    i[0] += 1
+                    rc = lib.adr_microbench_stream_read(stream(), qs[j].data_ptr(), N * K, blocks,
+                                                        sink.data_ptr())
+                    if rc != 0:
+                        raise RuntimeError(_ffi.strerror(rc))
+                tp = timed_graph(g, 2 * nbuf, max(2, iters // (2 * nbuf)))
+                best = tp if best is None else min(best, tp)
+            t_probe = best
+        return t, per + m * K * 2 + m * N * 2, t_probe
 
     # ---- the same decode shapes with fp16 weights: the call the reference's LLaMA makes once per
     # generated token (matmul_f16 on a [tokens, K] activation, llama.rs:485-591)
@@ -178,10 +221,13 @@ def main():
         gemv = []
         for K, N in DECODE_SET:
             for m in (1, 4, 16):
-                t, byts = u8_case(m, K, N, 200)
-                gemv.append({"M": m, "K": K, "N": N, "us": round(t * 1e6, 2),
-                             "gbs": round(byts / t / 1e9, 1),
-                             "frac_hbm_peak": round(byts / t / 1e9 / PEAK_HBM_GBS, 4)})
+                t, byts, tp = u8_case(m, K, N, 200, probe=(m == 1))
+                row = {"M": m, "K": K, "N": N, "us": round(t * 1e6, 2),
+                       "gbs": round(byts / t / 1e9, 1),
+                       "frac_hbm_peak": round(byts / t / 1e9 / PEAK_HBM_GBS, 4)}
+                if tp is not None:
+                    row["plain_read_of_the_weights_us"] = round(tp * 1e6, 2)
+                gemv.append(row)
         return gemv
 
     def attention_set():
@@ -360,12 +406,24 @@ def main():
         for name, K, N in LAYER_SET:
             mm(outs[name], acts[K], weights[name], M, K, N)
 
-    for _ in range(args.warmup):
+    # The five launches of a step are recorded once into a HIP graph (the entry points neither
+    # allocate nor synchronise, so they can be captured) and the step is replayed: the timed
+    # region then holds the device work of K steps, not the rate at which Python can call.
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()  # first call outside capture (lazy module loading)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    step_graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(step_graph):
         step()
+    for _ in range(args.warmup):
+        step_graph.replay()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        step()
+        step_graph.replay()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     step_flops = sum(2.0 * M * K * N for _, K, N in LAYER_SET)
@@ -376,19 +434,22 @@ def main():
     name, K, N = LAYER_SET[0]
     t_qkv = timed(lambda: mm(outs[name], acts[K], weights[name], M, K, N), 200, 20)
     qkv_flops = 2.0 * M * K * N
+    prof = profile_figures("gemm_nt_dma_llama7b_layer_set.txt")
     roofline = {
-        "kernel": "gemm_nt_dma_kernel<256,192,4,2,5,1> (qkv: M2048 K4096 N12288)",
+        "kernel": prof.get("kernel", "gemm_nt_dma_kernel") + " (qkv: M2048 K4096 N12288)",
         "bound": "mfma", "achieved": round(qkv_flops / t_qkv / 1e12, 2),
         "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
         "frac": round(qkv_flops / t_qkv / 1e12 / PEAK_F16_TFLOPS, 4),
         "launch_us": round(t_qkv * 1e6, 2),
-        # bytes moved between L2 and the memory fabric per qkv launch, from the rocprofv3 --pmc
-        # FETCH_SIZE and WRITE_SIZE passes recorded in profiles/gemm_nt_dma_llama7b_layer_set.txt
-        # (scaled by a plain device copy); the algorithmic figure is 167.8e6
-        "traffic": 426.1e6, "traffic_algorithmic": 167.8e6,
+        # bytes moved between L2 and the memory fabric per qkv launch: rocprofv3 --pmc FETCH_SIZE and
+        # WRITE_SIZE passes (scaled by a plain device copy), read from the summary under profiles/
+        "traffic": prof.get("traffic_bytes"),
+        "traffic_algorithmic": float((M * K + N * K + M * N) * 2),
+        "traffic_source": "profiles/gemm_nt_dma_llama7b_layer_set.txt",
     }
 
     secondary = {}
+    roofline_u8 = None
     if not args.quick:
         per_gemm = {}
         for name, K, N in LAYER_SET:
@@ -405,6 +466,21 @@ def main():
         best = max(gemv, key=lambda r: r["gbs"])
         secondary["u8_decode_gemv_best"] = {"gbs": best["gbs"], "frac_hbm_peak": best["frac_hbm_peak"],
                                             "shape": [best["M"], best["K"], best["N"]]}
+        # the other half of the metric: the dominant u8 decode kernel (one token, the widest
+        # matrix of the layer) against the HBM peak
+        dk = next(r for r in gemv if (r["M"], r["K"], r["N"]) == (1, 4096, 12288))
+        dprof = profile_figures("gemv_u8_decode_llama7b.txt")
+        roofline_u8 = {
+            "kernel": "gemv_u8_dot_kernel<1,4,4,1> (M1 K4096 N12288)", "bound": "hbm",
+            "achieved": dk["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "frac": dk["frac_hbm_peak"], "launch_us": dk["us"],
+            "traffic": dprof.get("traffic_bytes_m1_n12288"),
+            "traffic_algorithmic": float(12288 * 4096 + 12288 * 128 * 2 + 4096 * 2 + 12288 * 2),
+            "traffic_source": "profiles/gemv_u8_decode_llama7b.txt",
+            "plain_read_of_the_weights_us": dk.get("plain_read_of_the_weights_us"),
+            "rows_4": next(r for r in gemv if (r["M"], r["K"], r["N"]) == (4, 4096, 12288)),
+            "rows_16": next(r for r in gemv if (r["M"], r["K"], r["N"]) == (16, 4096, 12288)),
+        }
 
         secondary["f16_decode_gemv"] = f16_decode_set()
 
@@ -468,36 +544,117 @@ def main():
         attn = attention_set()
         secondary["llama7b_attention_fp16"] = attn
 
-    # ---------------- CPU baseline: the oracle on a bounded sample of the same workload
+    # ---------------- CPU baseline: every configuration on bounded samples, this machine's cores
     cpu_baseline = None
     if not args.quick:
         import numpy as np
         import oracle  # checker / baseline only; never on the product path
-        cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
-        rows = 128
-        name, K, N = LAYER_SET[0]
-        a_np = acts[K][:rows].cpu().numpy()
-        w_np = weights[name].cpu().numpy()
-        o_np = np.zeros(rows * N, np.float16)
+        nproc = os.cpu_count() or 1
+        threads = max(1, min(nproc, int(os.environ.get("OMP_NUM_THREADS", "16"))))
+        torch.set_num_threads(threads)
+        g_cpu = torch.Generator().manual_seed(42)   # seeded CPU generator, as py/gen_tests does
+
+        def cpu_mm(m, K, N, reps, batch=None):
+            """torch-CPU fp32 matmul on fp16-rounded inputs of the configuration's distribution."""
+            shape_a, shape_w = ((m, K), (N, K)) if batch is None else ((batch, m, K), (batch, N, K))
+            a32 = torch.randn(*shape_a, generator=g_cpu).half().float()
+            w32 = (torch.randn(*shape_w, generator=g_cpu) * K ** -0.5).half().float()
+            torch.matmul(a32, w32.transpose(-1, -2))  # warm-up
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                torch.matmul(a32, w32.transpose(-1, -2))
+            return (time.perf_counter() - t0) / reps
+
+        per_config = {}
+        t = cpu_mm(77, 768, 2304, 50)
+        per_config["configs[0] clip_text_qkv_M77_K768_N2304"] = {
+            "sample": "whole problem, 50 runs", "ms": round(t * 1e3, 3),
+            "tflops": round(2.0 * 77 * 768 * 2304 / t / 1e12, 4)}
+        for nm, K, N in (("up_K1024_N4096", 1024, 4096), ("down_K4096_N1024", 4096, 1024)):
+            t = cpu_mm(2056, K, N, 3)
+            per_config[f"configs[1] clip_vision_mlp_M2056_{nm}"] = {
+                "sample": "whole problem, 3 runs", "ms": round(t * 1e3, 2),
+                "tflops": round(2.0 * 2056 * K * N / t / 1e12, 4)}
+        # u8 decode: dequantise (the format's formula in fp32) + fp32 matmul, from the u8 weights
+        Kd, Nd = 4096, 4096
+        q_c = torch.randint(0, 256, (Nd, Kd), generator=g_cpu, dtype=torch.uint8)
+        s_c = (torch.rand(Nd, Kd // 32, generator=g_cpu) * 0.019 + 0.001).half()
+        for m in (1, 16):
+            a_c = torch.randn(m, Kd, generator=g_cpu).half().float()
+            t0 = time.perf_counter()
+            w_c = (q_c.float() - 127.5) * s_c.float().repeat_interleave(32, dim=1)
+            torch.matmul(a_c, w_c.t())
+            t = time.perf_counter() - t0
+            byts = Nd * Kd + Nd * (Kd // 32) * 2 + m * Kd * 2 + m * Nd * 2
+            per_config[f"configs[2] u8_decode_M{m}_K4096_N4096"] = {
+                "sample": "whole problem, dequantise + matmul, 1 run", "ms": round(t * 1e3, 2),
+                "gbs": round(byts / t / 1e9, 2)}
+        del q_c, s_c, w_c
+        # attention products: 4 of the 32 heads (the heads are independent: time x 8 for the layer)
+        S_, D_ = 2048, 128
+        qh = torch.randn(4, S_, D_, generator=g_cpu).half().float()
+        kh = torch.randn(4, S_, D_, generator=g_cpu).half().float()
         t0 = time.perf_counter()
-        oracle.matmul_f16(o_np, a_np, w_np, 1, rows, K, N, (1, N, 0), (1, K, 0), (K, 1, 0),
-                          mode=oracle.FAITHFUL, threads=cores)
+        sc_ = torch.matmul(qh, kh.transpose(1, 2)) * D_ ** -0.5
+        t_qk = time.perf_counter() - t0
+        p_ = torch.softmax(sc_, dim=-1)
+        t0 = time.perf_counter()
+        torch.matmul(p_, qh)
+        t_pv = time.perf_counter() - t0
+        per_config["configs[3] attention_S2048_H32_D128"] = {
+            "sample": "4 of 32 heads, 1 run (heads are independent: whole layer = 8 x)",
+            "qk_t_ms_4_heads": round(t_qk * 1e3, 2), "pv_ms_4_heads": round(t_pv * 1e3, 2),
+            "qk_t_tflops": round(2.0 * 4 * S_ * S_ * D_ / t_qk / 1e12, 4),
+            "pv_tflops": round(2.0 * 4 * S_ * S_ * D_ / t_pv / 1e12, 4)}
+        del qh, kh, sc_, p_
+        # the layer set (headline workload): the first 512 of the 2048 rows of each product
+        rows = 512
+        t_set, fl_set = 0.0, 0.0
+        for nm, K, N in LAYER_SET:
+            t = cpu_mm(rows, K, N, 1)
+            t_set += t
+            fl_set += 2.0 * rows * K * N
+        per_config["configs[4] llama7b_layer_set_fp16_M2048"] = {
+            "sample": f"first {rows} of 2048 rows of each of the five products, 1 run each "
+                      "(rows are independent: whole step = 4 x)",
+            "ms_sample": round(t_set * 1e3, 1), "tflops": round(fl_set / t_set / 1e12, 4)}
+        torch_value = fl_set / t_set / 1e12
+
+        # the same qkv sample on the blocked OpenMP fp32 GEMM (counterpart of the reference's host
+        # sgemm) and on the scalar restatement of its kernel (fp16 products, fp32 sum)
+        name, K, N = LAYER_SET[0]
+        a_np = acts[K][:128].cpu().numpy()
+        w_np = weights[name].cpu().numpy()
+        t0 = time.perf_counter()
+        oracle.sgemm_nt(a_np.astype(np.float32), w_np.astype(np.float32), threads=threads)
         dt = time.perf_counter() - t0
-        cpu_baseline = {
-            "value": round(2.0 * rows * K * N / dt / 1e12, 6), "unit": "TFLOP/s", "cores": cores,
-            "kind": "port",
-            "sample": f"first {rows} of 2048 activation rows of the qkv GEMM (K4096 N12288), "
-                      f"{2.0 * rows * K * N / 1e9:.1f} GFLOP in {dt:.1f} s, reference-faithful "
-                      "scalar arithmetic (fp16 products, fp32 sum)",
-        }
-        # parity spot check of the sample against a fresh device result
+        sgemm = {"tflops": round(2.0 * 128 * K * N / dt / 1e12, 5), "seconds": round(dt, 2),
+                 "sample": "first 128 rows of the qkv GEMM (K4096 N12288), plain-C blocked OpenMP fp32 GEMM"}
+        rows_f = 64
+        o_np = np.zeros(rows_f * N, np.float16)
+        t0 = time.perf_counter()
+        oracle.matmul_f16(o_np, a_np[:rows_f], w_np, 1, rows_f, K, N, (1, N, 0), (1, K, 0), (K, 1, 0),
+                          mode=oracle.FAITHFUL, threads=threads)
+        dt = time.perf_counter() - t0
+        faithful = {"tflops": round(2.0 * rows_f * K * N / dt / 1e12, 6), "seconds": round(dt, 2),
+                    "sample": f"first {rows_f} rows of the qkv GEMM, reference-faithful scalar arithmetic "
+                              "(soft fp16 products, fp32 sum), OpenMP over rows"}
+        # parity spot check of that sample against a fresh device result
         mm(outs[name], acts[K], weights[name], M, K, N)
         torch.cuda.synchronize()
-        got = outs[name][:rows].cpu().numpy().astype(np.float64)
-        ref = o_np.reshape(rows, N).astype(np.float64)
+        got = outs[name][:rows_f].cpu().numpy().astype(np.float64)
+        ref = o_np.reshape(rows_f, N).astype(np.float64)
         rms = np.sqrt(np.mean(ref ** 2))
-        cpu_baseline["max_rel_err_gpu_vs_cpu"] = float(
+        faithful["max_rel_err_gpu_vs_cpu"] = float(
             np.max(np.abs(got - ref) / np.maximum(np.abs(ref), rms)))
+        cpu_baseline = {
+            "value": round(torch_value, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "threads": threads, "nproc": nproc,
+            "sample": per_config["configs[4] llama7b_layer_set_fp16_M2048"]["sample"] +
+                      "; torch-CPU fp32 matmul on fp16-rounded inputs",
+            "per_config_torch_cpu_fp32": per_config,
+            "blocked_openmp_sgemm": sgemm, "faithful_scalar_port": faithful,
+        }
 
     line = {
         "metric": METRIC, "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1,
@@ -508,7 +665,8 @@ def main():
                                "fp16 weights: qkv, o, gate, up, down)",
                    "gflop_per_step": round(step_flops / 1e9, 1),
                    "frac_mfma_peak": round(value / PEAK_F16_TFLOPS, 4)},
-        "roofline": roofline, "cpu_baseline": cpu_baseline, "secondary": secondary,
+        "roofline": roofline, "roofline_u8_gemv": roofline_u8, "cpu_baseline": cpu_baseline,
+        "secondary": secondary,
     }
     print(json.dumps(line))
 

@@ -75,6 +75,8 @@ def lib():
         L.adr_o_embed_uint8.restype = None
         L.adr_o_error_stats.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
         L.adr_o_softmax_rows.argtypes = [u16p, u16p, C.c_int64, C.c_int, C.c_float, C.c_int]
+        L.adr_o_sgemm_nt.argtypes = [f32p, f32p, f32p, C.c_int, C.c_int, C.c_int, C.c_int]
+        L.adr_o_sgemm_nt.restype = None
         _lib = L
     return _lib
 
@@ -137,6 +139,21 @@ def matmul_nt_fp16u8(out, lhs, rhs_q, scales, block_size, beta=0.0, threads=1, n
     fn = lib().adr_o_matmul_nt_fp16u8_naive if naive else lib().adr_o_matmul_nt_fp16u8
     fn(_p16(out.view(np.uint16)), _p16(lhs.view(np.uint16)), _p8(rhs_q),
        _p16(scales.view(np.uint16)), m, p, n, block_size, float(beta), threads)
+    return out
+
+
+def sgemm_nt(a, b, threads=1):
+    """out[m,n] = a[m,k] . b[n,k]^T in fp32 (blocked, OpenMP): the host-GEMM leg of the CPU
+    baseline (the reference's matrixmultiply::sgemm, adrastea_core/src/mel.rs:142-157)."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    b = np.ascontiguousarray(b, dtype=np.float32)
+    m, k = a.shape
+    n = b.shape[0]
+    assert b.shape[1] == k
+    out = np.empty((m, n), np.float32)
+    f32p = C.POINTER(C.c_float)
+    lib().adr_o_sgemm_nt(out.ctypes.data_as(f32p), a.ctypes.data_as(f32p), b.ctypes.data_as(f32p),
+                         m, k, n, int(threads))
     return out
 
 

@@ -408,3 +408,52 @@ void adr_o_error_stats(float* out, const void* lhs, const void* rhs, int64_t len
   out[1] = mx;
   out[2] = (float)(sum / (double)length);
 }
+
+/* ---- blocked fp32 GEMM, the CPU-baseline counterpart of the reference's only host GEMM ------
+ * (matrixmultiply::sgemm with its `threading` feature, adrastea_core/src/mel.rs:142-157 and
+ * adrastea_core/Cargo.toml:12): out[m,n] = sum_k a[m,k] * b[n,k], all row-major fp32, B given as
+ * [n,k] like the weights of the path.  Cache blocking (64 x 256 panels of B, 4 x 4 register
+ * tiles over k) and OpenMP over row blocks; plain C, no intrinsics.  Baseline material for
+ * bench.py only -- no parity claim rests on it beyond its test against numpy. */
+void adr_o_sgemm_nt(float* out, const float* a, const float* b, int m, int k, int n, int threads) {
+  enum { MB = 64, NB = 64, KB = 256 };
+  if (threads < 1) threads = 1;
+#pragma omp parallel for num_threads(threads) schedule(dynamic, 1) collapse(2)
+  for (int i0 = 0; i0 < m; i0 += MB)
+    for (int j0 = 0; j0 < n; j0 += NB) {
+      const int i1 = i0 + MB < m ? i0 + MB : m, j1 = j0 + NB < n ? j0 + NB : n;
+      for (int i = i0; i < i1; i++)
+        for (int j = j0; j < j1; j++) out[(int64_t)i * n + j] = 0.0f;
+      for (int k0 = 0; k0 < k; k0 += KB) {
+        const int k1 = k0 + KB < k ? k0 + KB : k;
+        int i = i0;
+        for (; i + 4 <= i1; i += 4) {
+          int j = j0;
+          for (; j + 4 <= j1; j += 4) {
+            float c[4][4] = {{0}};
+            for (int kk = k0; kk < k1; kk++) {
+              float av[4], bv[4];
+              for (int u = 0; u < 4; u++) av[u] = a[(int64_t)(i + u) * k + kk];
+              for (int v = 0; v < 4; v++) bv[v] = b[(int64_t)(j + v) * k + kk];
+              for (int u = 0; u < 4; u++)
+                for (int v = 0; v < 4; v++) c[u][v] += av[u] * bv[v];
+            }
+            for (int u = 0; u < 4; u++)
+              for (int v = 0; v < 4; v++) out[(int64_t)(i + u) * n + j + v] += c[u][v];
+          }
+          for (; j < j1; j++)
+            for (int u = 0; u < 4; u++) {
+              float c = 0.0f;
+              for (int kk = k0; kk < k1; kk++) c += a[(int64_t)(i + u) * k + kk] * b[(int64_t)j * k + kk];
+              out[(int64_t)(i + u) * n + j] += c;
+            }
+        }
+        for (; i < i1; i++)
+          for (int j = j0; j < j1; j++) {
+            float c = 0.0f;
+            for (int kk = k0; kk < k1; kk++) c += a[(int64_t)i * k + kk] * b[(int64_t)j * k + kk];
+            out[(int64_t)i * n + j] += c;
+          }
+      }
+    }
+}

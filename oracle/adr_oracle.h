@@ -106,6 +106,10 @@ void adr_o_softmax_rows(uint16_t* output, const uint16_t* input, int64_t rows, i
  * is_f32 selects fp32 inputs (else fp16 bit patterns). */
 void adr_o_error_stats(float* out, const void* lhs, const void* rhs, int64_t length, int is_f32);
 
+/* Blocked OpenMP fp32 GEMM out[m,n] = a[m,k] . b[n,k]^T: the CPU-baseline counterpart of the
+ * reference's host GEMM (matrixmultiply::sgemm, adrastea_core/src/mel.rs:142-157). */
+void adr_o_sgemm_nt(float* out, const float* a, const float* b, int m, int k, int n, int threads);
+
 /* exhaustive dequant table: out[q * 65536 + s] = dequant(q, scale bits s) */
 void adr_o_dequant_table(uint16_t* out);
 

@@ -330,3 +330,19 @@ def test_overflow_saturates_to_infinity():
     out = np.zeros(1, np.float16)
     run(out, a, b, 1, 1, 4, 1, (1, 1, 0), (1, 4, 0), (1, 1, 0), mode=oracle.EXACT)
     assert out.view(np.uint16)[0] == 0x7C00
+
+
+@pytest.mark.parametrize("mkn", [(1, 1, 1), (5, 300, 7), (64, 256, 64), (70, 513, 131), (130, 64, 3)])
+def test_blocked_sgemm_baseline_matches_numpy(mkn):
+    """The OpenMP fp32 GEMM that bench.py times as a CPU baseline: ragged panels in all three
+    dimensions against numpy's float64 product, and small integers exactly."""
+    m, k, n = mkn
+    g = rng(7000 + m + k + n)
+    a = g.standard_normal((m, k)).astype(np.float32)
+    b = g.standard_normal((n, k)).astype(np.float32)
+    got = oracle.sgemm_nt(a, b, threads=4)
+    ref = a.astype(np.float64) @ b.astype(np.float64).T
+    assert np.max(np.abs(got - ref)) <= 1e-4 * max(1.0, np.max(np.abs(ref)))
+    ai = g.integers(-8, 9, size=(m, k)).astype(np.float32)
+    bi = g.integers(-8, 9, size=(n, k)).astype(np.float32)
+    assert np.array_equal(oracle.sgemm_nt(ai, bi, threads=3), ai @ bi.T)
