@@ -10,6 +10,7 @@ LIB_PATH = os.path.join(HERE, "lib", "libadrastea_kernels_hip.so")
 # every symbol include/adrastea_kernels.h declares
 SYMBOLS = (
     "adr_matmul_f16", "adr_matmul_f16_slow", "adr_matmul_f16_raw", "adr_matmul_nt_f16",
+    "adr_matmul_f16_ws", "adr_matmul_f16_workspace_bytes", "adr_matmul_f16_ws_plan",
     "adr_matmul_nt_fp16u8", "adr_dequantize_absmax_u8", "adr_quantize_absmax_u8",
     "adr_dequantize_absmax_uint8", "adr_quantize_absmax_uint8", "adr_matmul_f16_plan",
     "adr_matmul_nt_fp16u8_plan", "adr_softmax_rows", "adr_error_stats_f16", "adr_error_stats_f32", "adr_attention_f16", "adr_embed_uint8",
@@ -50,6 +51,9 @@ def lib():
     mm = [vp, vp, vp, vp] + [i32] * 13 + [vp, f32, f32, u32, u32, u32]
     L.adr_matmul_f16.argtypes = mm
     L.adr_matmul_f16_slow.argtypes = mm
+    L.adr_matmul_f16_ws.argtypes = mm + [vp, C.c_int64]
+    L.adr_matmul_f16_workspace_bytes.argtypes = [i32] * 13 + [u32, u32, u32]
+    L.adr_matmul_f16_ws_plan.argtypes = [C.c_char_p, i32] + [i32] * 13 + [u32, u32, u32, C.c_int64]
     L.adr_matmul_f16_raw.argtypes = [vp, vp, vp, vp] + [i32] * 13
     L.adr_matmul_nt_f16.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32]
     L.adr_matmul_nt_fp16u8.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, f32]
@@ -73,6 +77,7 @@ def lib():
     for name in SYMBOLS:
         if name not in ("adr_strerror",):
             getattr(L, name).restype = C.c_int
+    L.adr_matmul_f16_workspace_bytes.restype = C.c_int64
     _lib = L
     return L
 

@@ -34,6 +34,10 @@ struct MatmulArgs {
   const uint8_t* rhs_q;
   const half_t* scales;
   int block_size;
+  // caller-provided scratch for kernels that split K over workgroups (adr_matmul_f16_ws): fp32
+  // partial tiles, fully rewritten by every launch that uses them; null / 0: no such kernel
+  float* workspace;
+  int64_t workspace_bytes;
 };
 
 // Internal store operator of the contiguous NT entry points (matmul_nt_wmma_16x128x256.cu:63-66):
@@ -210,6 +214,9 @@ hipError_t launch_matmul_general(hipStream_t stream, const MatmulArgs& a);
 // Returns true and fills `name` when the MFMA kernel family covers these arguments.
 bool mfma_gemm_supported(const MatmulArgs& a, const char** name);
 hipError_t launch_mfma_gemm(hipStream_t stream, const MatmulArgs& a);
+// Scratch bytes the split-K form of these arguments would use (0: no split pays here); the
+// kernel family splits only when a.workspace holds at least this much.
+int64_t mfma_gemm_workspace_bytes(const MatmulArgs& a);
 // fp16 skinny matmul (m <= 32, K-contiguous operands): true when a streaming kernel covers it.
 bool gemv_f16_supported(const MatmulArgs& a, const char** name);
 hipError_t launch_gemv_f16(hipStream_t stream, const MatmulArgs& a);

@@ -129,6 +129,37 @@ int adr_matmul_f16(adr_stream_t stream, uint16_t* output, const uint16_t* lhs, c
   return run_matmul((hipStream_t)stream, a, true);
 }
 
+int adr_matmul_f16_ws(adr_stream_t stream, uint16_t* output, const uint16_t* lhs, const uint16_t* rhs,
+                      int32_t batches, int32_t m, int32_t k, int32_t n, int32_t stride_ox,
+                      int32_t stride_oy, int32_t stride_oz, int32_t stride_lx, int32_t stride_ly,
+                      int32_t stride_lz, int32_t stride_rx, int32_t stride_ry, int32_t stride_rz,
+                      const uint16_t* bias, float beta, float scale, uint32_t store, uint32_t load,
+                      uint32_t mask, void* workspace, int64_t workspace_bytes) {
+  MatmulArgs a = pack(output, lhs, rhs, batches, m, k, n, stride_ox, stride_oy, stride_oz,
+                      stride_lx, stride_ly, stride_lz, stride_rx, stride_ry, stride_rz, bias, beta,
+                      scale, store, load, mask);
+  if (int rc = validate_matmul(a, true)) return rc;
+  if (workspace_bytes < 0 || (workspace_bytes > 0 && !workspace)) return ADR_ENULL;
+  if ((uintptr_t)workspace % 16 != 0) return ADR_EINVAL_SHAPE;
+  a.workspace = (float*)workspace;
+  a.workspace_bytes = workspace_bytes;
+  return run_matmul((hipStream_t)stream, a, true);
+}
+
+int64_t adr_matmul_f16_workspace_bytes(int32_t batches, int32_t m, int32_t k, int32_t n,
+                                       int32_t stride_ox, int32_t stride_oy, int32_t stride_oz,
+                                       int32_t stride_lx, int32_t stride_ly, int32_t stride_lz,
+                                       int32_t stride_rx, int32_t stride_ry, int32_t stride_rz,
+                                       uint32_t store, uint32_t load, uint32_t mask) {
+  MatmulArgs a = pack(nullptr, nullptr, nullptr, batches, m, k, n, stride_ox, stride_oy, stride_oz,
+                      stride_lx, stride_ly, stride_lz, stride_rx, stride_ry, stride_rz, nullptr,
+                      0.0f, 1.0f, store, load, mask);
+  if (int rc = validate_matmul(a, false)) return rc;
+  const char* name;
+  if (empty(a) || gemv_f16_supported(a, &name)) return 0;
+  return mfma_gemm_workspace_bytes(a);
+}
+
 int adr_matmul_f16_slow(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
                         const uint16_t* rhs, int32_t batches, int32_t m, int32_t k, int32_t n,
                         int32_t stride_ox, int32_t stride_oy, int32_t stride_oz, int32_t stride_lx,
@@ -160,6 +191,27 @@ int adr_matmul_f16_plan(char* name, int32_t cap, int32_t batches, int32_t m, int
                       stride_lx, stride_ly, stride_lz, stride_rx, stride_ry, stride_rz, nullptr,
                       0.0f, 1.0f, store, load, mask);
   if (int rc = validate_matmul(a, false)) return rc;
+  const char* chosen = "none (empty)";
+  if (!empty(a) && !gemv_f16_supported(a, &chosen) && !mfma_gemm_supported(a, &chosen))
+    chosen = "matmul_general";
+  if (name && cap > 0) {
+    strncpy(name, chosen, (size_t)cap - 1);
+    name[cap - 1] = 0;
+  }
+  return ADR_OK;
+}
+
+int adr_matmul_f16_ws_plan(char* name, int32_t cap, int32_t batches, int32_t m, int32_t k, int32_t n,
+                           int32_t stride_ox, int32_t stride_oy, int32_t stride_oz,
+                           int32_t stride_lx, int32_t stride_ly, int32_t stride_lz,
+                           int32_t stride_rx, int32_t stride_ry, int32_t stride_rz, uint32_t store,
+                           uint32_t load, uint32_t mask, int64_t workspace_bytes) {
+  MatmulArgs a = pack(nullptr, nullptr, nullptr, batches, m, k, n, stride_ox, stride_oy, stride_oz,
+                      stride_lx, stride_ly, stride_lz, stride_rx, stride_ry, stride_rz, nullptr,
+                      0.0f, 1.0f, store, load, mask);
+  if (int rc = validate_matmul(a, false)) return rc;
+  if (workspace_bytes < 0) return ADR_EINVAL_SHAPE;
+  a.workspace_bytes = workspace_bytes;
   const char* chosen = "none (empty)";
   if (!empty(a) && !gemv_f16_supported(a, &chosen) && !mfma_gemm_supported(a, &chosen))
     chosen = "matmul_general";

@@ -25,6 +25,7 @@
 // output columns; the epilogue narrows them to fp16, transposes through a per-wavefront LDS
 // slot and writes whole 16-byte chunks of output rows, applying the store operator, the bias
 // and the causal mask on the way.
+#include <stdint.h>
 #include <type_traits>
 
 #include "adr_common.hpp"
@@ -61,14 +62,14 @@ struct TileMap {
   int tiles_m, tiles_n, tiles_per_batch, total;
   int group_m;  // tile rows per L2-reuse group
   int xcds;     // dies of the device: workgroup i runs on die i % xcds
+  int splits;   // K is cut into this many pieces, one workgroup each (1: no split)
 };
 
 // blockIdx.x -> (batch, tile_m, tile_n).  Consecutive ids land on different dies, so ids are
 // first regrouped per die; inside a batch, tiles are walked column by column within groups of
 // `group_m` tile rows so that the tiles resident on one die share A and B panels in its L2.
 __device__ __forceinline__ void map_tile(const TileMap& map, int& batch, int& tile_m,
-                                         int& tile_n) {
-  int id = blockIdx.x;
+                                         int& tile_n, int id = blockIdx.x) {
   const int XCDS = map.xcds;
   const int per = (map.total + XCDS - 1) / XCDS;
   const int tall = map.total % XCDS == 0 ? XCDS : map.total % XCDS;
@@ -366,7 +367,11 @@ __device__ __forceinline__ void fill_masked_tile(const MatmulArgs& a, half_t* ou
 // =============================================================================================
 // Direct-to-LDS kernel
 // =============================================================================================
-template <int BM, int BN, int WM, int WN, int NSTAGE, int MINB, bool NN, int BK = 64>
+// SPLIT: the grid holds map.splits workgroups per tile, each multiplying its own piece of K and
+// leaving the fp32 accumulators in a.workspace ([piece][tile][register chunk][thread] float4, so
+// that consecutive threads store consecutive 16 bytes); splitk_reduce_kernel sums the pieces in
+// a fixed order and runs the epilogue.
+template <int BM, int BN, int WM, int WN, int NSTAGE, int MINB, bool NN, int BK = 64, bool SPLIT = false>
 __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulArgs a,
                                                                          TileMap map) {
   // K slices of 64 (128 bytes of a row per slice and DMA request), or of 128 for the small tiles
@@ -393,19 +398,27 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   __shared__ __attribute__((aligned(1024))) unsigned char sB2[NSTAGE >= 3 ? BN * BK * 2 : 1024];
 
   int batch, tile_m, tile_n;
-  map_tile(map, batch, tile_m, tile_n);
+  const int tile_id = SPLIT ? (int)(blockIdx.x % (unsigned)map.total) : (int)blockIdx.x;
+  const int piece = SPLIT ? (int)(blockIdx.x / (unsigned)map.total) : 0;
+  map_tile(map, batch, tile_m, tile_n, tile_id);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
   half_t* const out = a.output + (int64_t)batch * a.stride_oz;
 
   if (a.mask == ADR_MASK_CAUSAL && n0 > m0 + BM - 1) {
-    fill_masked_tile<BM, BN, NT>(a, out, m0, n0, tid);
+    // (split: the reduction kernel fills the tile; nothing is left in the workspace for it)
+    if (!SPLIT) fill_masked_tile<BM, BN, NT>(a, out, m0, n0, tid);
     return;
   }
 
-  const half_t* const A = a.lhs + (int64_t)batch * a.stride_lz;
-  const half_t* const B = a.rhs + (int64_t)batch * a.stride_rz;
+  // K slices of this workgroup: all of them, or piece `piece` of map.splits nearly equal ones
+  const int KT_all = a.k / BK;
+  const int kt_begin = SPLIT ? (int)((int64_t)KT_all * piece / map.splits) : 0;
+  const int kt_end = SPLIT ? (int)((int64_t)KT_all * (piece + 1) / map.splits) : KT_all;
+  const half_t* const A = a.lhs + (int64_t)batch * a.stride_lz + (int64_t)kt_begin * BK;
+  const half_t* const B = a.rhs + (int64_t)batch * a.stride_rz +
+                          (int64_t)kt_begin * (NN ? (int64_t)BK * a.stride_ry : BK);
 
   // DMA instruction i of this wavefront fills LDS chunks [(i*NW + wave)*64, +64) of a stage,
   // lane l the l-th of them; the lane fetches whatever (row, k-chunk) the swizzle puts there.
@@ -434,7 +447,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
     }
   }
   const int64_t b_slice = NN ? (int64_t)BK * a.stride_ry : BK;  // elements per K slice
-  const int KT = a.k / BK;
+  const int KT = kt_end - kt_begin;
   int kload = 0;  // next slice to fetch; past the end the last slice is fetched again (unused)
   auto dmaA = [&](int ks, unsigned char* dA) {
 #pragma unroll
@@ -633,8 +646,68 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   // drain the trailing (redundant) DMA before the stages are reused by the epilogue
   wait_dma_barrier(std::integral_constant<int, 0>{});
 
+  if (SPLIT) {
+    float4_t* const ws = (float4_t*)a.workspace +
+                         ((int64_t)piece * map.total + tile_id) * (TM * TN * 4) * NT + tid;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          const float4_t v = {acc[i][j][4 * c], acc[i][j][4 * c + 1], acc[i][j][4 * c + 2],
+                              acc[i][j][4 * c + 3]};
+          ws[(int64_t)((i * TN + j) * 4 + c) * NT] = v;
+        }
+    return;
+  }
   unsigned char* slot = (wave < NW / 2 ? sA0 : sA1) + (wave % (NW / 2)) * SLOT;
   wave_epilogue<TM, TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, slot, (half_t)a.scale, lane);
+}
+
+// Second launch of a split product: one workgroup per tile, with the geometry of the kernel that
+// wrote the pieces.  Every thread sums its accumulator registers over the pieces (always in the
+// order 0, 1, 2, ...: the result does not depend on which workgroup finished first) and the
+// epilogue of the unsplit kernel stores the tile.
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64) void splitk_reduce_kernel(MatmulArgs a, TileMap map) {
+  constexpr int NW = WM * WN, NT = NW * 64;
+  constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
+  constexpr int SLOT = 32 * (TN * 64 + 16);
+  __shared__ __attribute__((aligned(1024))) unsigned char slots[NW * SLOT];
+  int batch, tile_m, tile_n;
+  map_tile(map, batch, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  half_t* const out = a.output + (int64_t)batch * a.stride_oz;
+  if (a.mask == ADR_MASK_CAUSAL && n0 > m0 + BM - 1) {
+    fill_masked_tile<BM, BN, NT>(a, out, m0, n0, tid);
+    return;
+  }
+  float16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+  for (int piece = 0; piece < map.splits; piece++) {
+    const float4_t* const ws = (const float4_t*)a.workspace +
+                               ((int64_t)piece * map.total + blockIdx.x) * (TM * TN * 4) * NT + tid;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          const float4_t v = ws[(int64_t)((i * TN + j) * 4 + c) * NT];
+#pragma unroll
+          for (int e = 0; e < 4; e++) acc[i][j][4 * c + e] += v[e];
+        }
+  }
+  wave_epilogue<TM, TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, slots + wave * SLOT,
+                        (half_t)a.scale, lane);
 }
 
 // =============================================================================================
@@ -1279,6 +1352,7 @@ TileMap make_map(const MatmulArgs& a, int bm, int bn) {
   map.total = total > 0x7fffffffLL ? -1 : (int)total;
   map.group_m = map.tiles_m < 8 ? map.tiles_m : 8;
   map.xcds = device_info_for_plan().xcds;
+  map.splits = 1;
   return map;
 }
 
@@ -1288,6 +1362,27 @@ hipError_t launch_dma(hipStream_t stream, const MatmulArgs& a) {
   if (map.total < 0) return hipErrorInvalidConfiguration;
   hipLaunchKernelGGL((gemm_nt_dma_kernel<BM, BN, WM, WN, NSTAGE, MINB, NN, BK>),
                      dim3((unsigned)map.total), dim3(WM * WN * 64), 0, stream, a, map);
+  return hipGetLastError();
+}
+
+// Bytes of workspace a split product on BM x BN tiles with `splits` pieces needs.
+int64_t split_workspace_bytes(const MatmulArgs& a, int bm, int bn, int splits) {
+  const int64_t tiles = (int64_t)((a.m + bm - 1) / bm) * ((a.n + bn - 1) / bn) * a.batches;
+  return tiles * splits * bm * bn * 4;
+}
+
+template <int BM, int BN, int WM, int WN, int NSTAGE, int MINB>
+hipError_t launch_dma_split(hipStream_t stream, const MatmulArgs& a, int splits) {
+  TileMap map = make_map(a, BM, BN);
+  if (map.total < 0 || (int64_t)map.total * splits > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+  if (!a.workspace || a.workspace_bytes < split_workspace_bytes(a, BM, BN, splits)) return hipErrorInvalidValue;
+  map.splits = splits;
+  hipLaunchKernelGGL((gemm_nt_dma_kernel<BM, BN, WM, WN, NSTAGE, MINB, false, 64, true>),
+                     dim3((unsigned)(map.total * splits)), dim3(WM * WN * 64), 0, stream, a, map);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL((splitk_reduce_kernel<BM, BN, WM, WN>), dim3((unsigned)map.total),
+                     dim3(WM * WN * 64), 0, stream, a, map);
   return hipGetLastError();
 }
 
@@ -1460,6 +1555,65 @@ GemmChoice choose(const MatmulArgs& a) {
   return pick(a, stage, 3);
 }
 
+// Splitting K over workgroups (needs a workspace): a product with few tiles and a long K keeps
+// most compute units idle while a few walk all of K.  With `splits` workgroups per tile every
+// one of them walks K / splits; a second launch sums the pieces.  The estimate is pick()'s cost
+// (tile area on the busiest compute unit over the tile's efficiency) times K, 2.9e6 units per
+// microsecond, plus the second launch and the fp32 pieces written and read again.
+struct SplitChoice {
+  GemmChoice tile;
+  int splits;
+  int bm, bn;
+};
+
+SplitChoice choose_split(const MatmulArgs& a, int64_t avail_bytes) {
+  const SplitChoice none = {GEMM_NONE, 1, 0, 0};
+  if (avail_bytes <= 0 || a.rhs_q || a.load != ADR_LOAD_IDENTITY || a.k % 64 != 0 || a.k < 1024)
+    return none;
+  const GemmChoice whole = choose(a);
+  if (whole != DMA_128x128 && whole != DMA_128x64 && whole != DMA_64x64 && whole != DMA_64x64_K128 &&
+      whole != DMA_128x64_K128 && whole != DMA_256x128)
+    return none;
+  const int NUM_CU = num_cu();
+  double whole_cost;
+  pick(a, DMA_TILES, 5, &whole_cost);
+  whole_cost *= a.k;
+  // With about one small tile per compute unit the time is set by the latency of the K slices,
+  // not by the tile's arithmetic: 0.38 us per slice of 64 (measured: K4160 N4096 m=130 25.7 us),
+  // 0.25 us where the tile walks K in slices of 128.
+  const double US = 2.9e6;
+  auto latency_floor = [&](int k, double us_per_slice) { return ((k / 64) * us_per_slice + 2.0) * US; };
+  if (whole != DMA_256x128 && whole != DMA_128x128) {
+    const bool k128 = whole == DMA_64x64_K128 || whole == DMA_128x64_K128;
+    const double f = latency_floor(a.k, k128 ? 0.25 : 0.38);
+    if (f > whole_cost) whole_cost = f;
+  }
+  static const Candidate tiles[] = {{DMA_128x128, 128, 128, 2, 0.80f}, {DMA_128x64, 128, 64, 2, 0.60f},
+                                    {DMA_64x64, 64, 64, 4, 0.40f}};
+  SplitChoice best = none;
+  double best_cost = whole_cost * 0.85;  // (a split has to win clearly)
+  for (const Candidate& t : tiles) {
+    const int64_t nt = (int64_t)((a.m + t.bm - 1) / t.bm) * ((a.n + t.bn - 1) / t.bn) * a.batches;
+    for (int sp = 2; sp <= 16; sp++) {
+      if (a.k / sp < 256) break;  // at least four slices per piece
+      if (nt * sp > 4 * (int64_t)NUM_CU) break;
+      const int64_t bytes = nt * sp * t.bm * t.bn * 4;
+      if (bytes > avail_bytes) break;
+      const int64_t per_cu = (nt * sp + NUM_CU - 1) / NUM_CU;
+      double mm = (double)per_cu * t.bm * t.bn / t.eff * ((double)a.k / sp);
+      const double f = latency_floor(a.k / sp, t.id == DMA_128x128 ? 0.48 : t.id == DMA_128x64 ? 0.42 : 0.38);
+      if (f > mm) mm = f;
+      // second launch (4 us) + pieces written and read at some 4 TB/s
+      const double extra = (4.0 + 2.0 * (double)bytes / 4.0e6) * US;
+      if (mm + extra < best_cost) {
+        best_cost = mm + extra;
+        best = {t.id, sp, t.bm, t.bn};
+      }
+    }
+  }
+  return best;
+}
+
 }  // namespace
 
 static bool choice_name(GemmChoice c, const char** name, bool u8 = false) {
@@ -1545,13 +1699,49 @@ static bool split_m_tail(const MatmulArgs& a, MatmulArgs& head, MatmulArgs& tail
   return (first + rest) * a.k + 8.7e6 < whole * a.k;
 }
 
+static const char* split_name(const SplitChoice& sc) {
+  // "gemm_nt_mfma_dma_128x128x64_splitk4": the tile, then the number of pieces
+  static const char* const names[3][15] = {
+      {"gemm_nt_mfma_dma_128x128x64_splitk2", "gemm_nt_mfma_dma_128x128x64_splitk3", "gemm_nt_mfma_dma_128x128x64_splitk4",
+       "gemm_nt_mfma_dma_128x128x64_splitk5", "gemm_nt_mfma_dma_128x128x64_splitk6", "gemm_nt_mfma_dma_128x128x64_splitk7",
+       "gemm_nt_mfma_dma_128x128x64_splitk8", "gemm_nt_mfma_dma_128x128x64_splitk9", "gemm_nt_mfma_dma_128x128x64_splitk10",
+       "gemm_nt_mfma_dma_128x128x64_splitk11", "gemm_nt_mfma_dma_128x128x64_splitk12", "gemm_nt_mfma_dma_128x128x64_splitk13",
+       "gemm_nt_mfma_dma_128x128x64_splitk14", "gemm_nt_mfma_dma_128x128x64_splitk15", "gemm_nt_mfma_dma_128x128x64_splitk16"},
+      {"gemm_nt_mfma_dma_128x64x64_splitk2", "gemm_nt_mfma_dma_128x64x64_splitk3", "gemm_nt_mfma_dma_128x64x64_splitk4",
+       "gemm_nt_mfma_dma_128x64x64_splitk5", "gemm_nt_mfma_dma_128x64x64_splitk6", "gemm_nt_mfma_dma_128x64x64_splitk7",
+       "gemm_nt_mfma_dma_128x64x64_splitk8", "gemm_nt_mfma_dma_128x64x64_splitk9", "gemm_nt_mfma_dma_128x64x64_splitk10",
+       "gemm_nt_mfma_dma_128x64x64_splitk11", "gemm_nt_mfma_dma_128x64x64_splitk12", "gemm_nt_mfma_dma_128x64x64_splitk13",
+       "gemm_nt_mfma_dma_128x64x64_splitk14", "gemm_nt_mfma_dma_128x64x64_splitk15", "gemm_nt_mfma_dma_128x64x64_splitk16"},
+      {"gemm_nt_mfma_dma_64x64x64_splitk2", "gemm_nt_mfma_dma_64x64x64_splitk3", "gemm_nt_mfma_dma_64x64x64_splitk4",
+       "gemm_nt_mfma_dma_64x64x64_splitk5", "gemm_nt_mfma_dma_64x64x64_splitk6", "gemm_nt_mfma_dma_64x64x64_splitk7",
+       "gemm_nt_mfma_dma_64x64x64_splitk8", "gemm_nt_mfma_dma_64x64x64_splitk9", "gemm_nt_mfma_dma_64x64x64_splitk10",
+       "gemm_nt_mfma_dma_64x64x64_splitk11", "gemm_nt_mfma_dma_64x64x64_splitk12", "gemm_nt_mfma_dma_64x64x64_splitk13",
+       "gemm_nt_mfma_dma_64x64x64_splitk14", "gemm_nt_mfma_dma_64x64x64_splitk15", "gemm_nt_mfma_dma_64x64x64_splitk16"}};
+  const int t = sc.tile == DMA_128x128 ? 0 : sc.tile == DMA_128x64 ? 1 : 2;
+  return names[t][sc.splits - 2];
+}
+
+int64_t mfma_gemm_workspace_bytes(const MatmulArgs& a) {
+  const SplitChoice sc = choose_split(a, INT64_MAX);
+  return sc.tile == GEMM_NONE ? 0 : split_workspace_bytes(a, sc.bm, sc.bn, sc.splits);
+}
+
 bool mfma_gemm_supported(const MatmulArgs& a, const char** name) {
+  const SplitChoice sc = choose_split(a, a.workspace_bytes);
+  if (sc.tile != GEMM_NONE) {
+    *name = split_name(sc);
+    return true;
+  }
   MatmulArgs head, tail;
   if (split_m_tail(a, head, tail)) return choice_name(choose(head), name);
   return choice_name(choose(a), name);
 }
 
 hipError_t launch_mfma_gemm(hipStream_t stream, const MatmulArgs& a) {
+  const SplitChoice sc = choose_split(a, a.workspace ? a.workspace_bytes : 0);
+  if (sc.tile == DMA_128x128) return launch_dma_split<128, 128, 2, 2, 3, 1>(stream, a, sc.splits);
+  if (sc.tile == DMA_128x64) return launch_dma_split<128, 64, 2, 2, 3, 2>(stream, a, sc.splits);
+  if (sc.tile == DMA_64x64) return launch_dma_split<64, 64, 2, 2, 3, 3>(stream, a, sc.splits);
   MatmulArgs head, tail;
   if (split_m_tail(a, head, tail)) {
     const hipError_t e = launch_choice(stream, head, choose(head));

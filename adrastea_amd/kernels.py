@@ -175,13 +175,21 @@ def _current_stream() -> int:
 
 
 class GpuKernels(CommonKernels):
-    """Launches through the C ABI on torch's current HIP stream.  Holds no mutable state."""
+    """Launches through the C ABI on torch's current HIP stream.
 
-    def __init__(self):
+    `workspace_bytes` > 0 gives the instance a scratch buffer of that size, owned like any other
+    tensor of the host (in the reference: one more GpuBuffer held by GpuKernels); matmul_f16 then
+    goes through adr_matmul_f16_ws, which may split K over workgroups for products with few
+    output tiles and a long K.  The buffer carries nothing between calls; one instance must not
+    be used from streams that run concurrently."""
+
+    def __init__(self, workspace_bytes: int = 0):
         self._lib = _ffi.lib()
         import torch
         if not torch.cuda.is_available():
             raise RuntimeError("adrastea_amd.GpuKernels needs a GPU; there is no CPU fallback")
+        self._workspace = (torch.empty(workspace_bytes, dtype=torch.uint8, device="cuda")
+                           if workspace_bytes > 0 else None)
 
     def _matmul(self, fn, what, output, left, right, options):
         low = lower_matmul(output.layout, left.layout, right.layout, options)
@@ -193,7 +201,13 @@ class GpuKernels(CommonKernels):
             raise AdrasteaError(rc, what)
 
     def matmul_f16(self, output, left, right, options=MatmulOptions()):
-        self._matmul(self._lib.adr_matmul_f16, "matmul_f16", output, left, right, options)
+        if self._workspace is None:
+            return self._matmul(self._lib.adr_matmul_f16, "matmul_f16", output, left, right, options)
+        ws = self._workspace
+
+        def with_workspace(*args):
+            return self._lib.adr_matmul_f16_ws(*args, ws.data_ptr(), ws.numel())
+        self._matmul(with_workspace, "matmul_f16", output, left, right, options)
 
     def matmul_f16_slow(self, output, left, right, options=MatmulOptions()):
         self._matmul(self._lib.adr_matmul_f16_slow, "matmul_f16_slow", output, left, right,
@@ -319,14 +333,26 @@ def descriptor(view: TensorView) -> _ffi.TensorDesc:
 
 
 def plan_matmul(output: TensorLayout, left: TensorLayout, right: TensorLayout,
-                options: MatmulOptions = MatmulOptions()) -> str:
-    """Name of the kernel adr_matmul_f16 selects for these layouts (no device needed)."""
+                options: MatmulOptions = MatmulOptions(), workspace_bytes: int = 0) -> str:
+    """Name of the kernel adr_matmul_f16 (or, with a workspace, adr_matmul_f16_ws) selects for
+    these layouts (no device needed)."""
     low = lower_matmul(output, left, right, options)
-    buf = C.create_string_buffer(64)
-    rc = _ffi.lib().adr_matmul_f16_plan(buf, 64, *low.scalars(), low.store, low.load, low.mask)
+    buf = C.create_string_buffer(96)
+    rc = _ffi.lib().adr_matmul_f16_ws_plan(buf, 96, *low.scalars(), low.store, low.load, low.mask,
+                                           int(workspace_bytes))
     if rc != 0:
         raise AdrasteaError(rc, "matmul_f16_plan")
     return buf.value.decode()
+
+
+def matmul_workspace_bytes(output: TensorLayout, left: TensorLayout, right: TensorLayout,
+                           options: MatmulOptions = MatmulOptions()) -> int:
+    """Scratch bytes adr_matmul_f16_ws would use for these layouts (0: it would not split K)."""
+    low = lower_matmul(output, left, right, options)
+    n = _ffi.lib().adr_matmul_f16_workspace_bytes(*low.scalars(), low.store, low.load, low.mask)
+    if n < 0:
+        raise AdrasteaError(int(n), "matmul_f16_workspace_bytes")
+    return int(n)
 
 
 class MatmulTracer(CommonKernels):

@@ -87,6 +87,36 @@ int adr_matmul_f16_slow(adr_stream_t stream, uint16_t* output, const uint16_t* l
                         const uint16_t* bias, float beta, float scale, uint32_t store,
                         uint32_t load, uint32_t mask);
 
+/*
+ * adr_matmul_f16 with a caller-provided scratch buffer (no counterpart in the reference, whose
+ * kernel walks all of K in every workgroup: kernels.rs:849-863, matmul.cu:288-381).  Same
+ * arguments, same result, same validation; in addition `workspace` (device memory, 16-byte
+ * aligned) of `workspace_bytes` bytes.  A product with few output tiles and a long K -- a few
+ * dozen to a few hundred rows against a weight matrix, what the reference's LLaMA issues for
+ * every generated token since it keeps no KV cache (llama.rs:456-483) -- then runs as two
+ * launches: K is split over several workgroups per tile that leave fp32 partial tiles in the
+ * workspace, and a second kernel sums them in a fixed order and applies the store operator.
+ * adr_matmul_f16_workspace_bytes tells how much such a product would use at best (0: it would
+ * not be split); with less, K is cut into fewer pieces or not at all, and with
+ * workspace_bytes == 0 the call is adr_matmul_f16.
+ * The workspace is written and read by the two launches only; it carries nothing from one call
+ * to the next, so one buffer serves all calls on a stream.  Calls that may overlap (different
+ * streams) need different buffers.
+ */
+int adr_matmul_f16_ws(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
+                      const uint16_t* rhs, int32_t batches, int32_t m, int32_t k, int32_t n,
+                      int32_t stride_ox, int32_t stride_oy, int32_t stride_oz, int32_t stride_lx,
+                      int32_t stride_ly, int32_t stride_lz, int32_t stride_rx, int32_t stride_ry,
+                      int32_t stride_rz, const uint16_t* bias, float beta, float scale,
+                      uint32_t store, uint32_t load, uint32_t mask, void* workspace,
+                      int64_t workspace_bytes);
+/* Returns the bytes (>= 0) or a negative ADR_E* code; touches no device memory. */
+int64_t adr_matmul_f16_workspace_bytes(int32_t batches, int32_t m, int32_t k, int32_t n,
+                                       int32_t stride_ox, int32_t stride_oy, int32_t stride_oz,
+                                       int32_t stride_lx, int32_t stride_ly, int32_t stride_lz,
+                                       int32_t stride_rx, int32_t stride_ry, int32_t stride_rz,
+                                       uint32_t store, uint32_t load, uint32_t mask);
+
 /* `matmul_f16_raw` (matmul.cu:515-517): identity operators, the 16 common arguments. */
 int adr_matmul_f16_raw(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
                        const uint16_t* rhs, int32_t batches, int32_t m, int32_t k, int32_t n,
@@ -234,6 +264,12 @@ int adr_matmul_f16_plan(char* name, int32_t cap, int32_t batches, int32_t m, int
                         uint32_t load, uint32_t mask);
 int adr_matmul_nt_fp16u8_plan(char* name, int32_t cap, int32_t m, int32_t p, int32_t n,
                               int32_t block_size);
+/* The plan of adr_matmul_f16_ws for a workspace of the given size ("..._splitk4": K in four pieces). */
+int adr_matmul_f16_ws_plan(char* name, int32_t cap, int32_t batches, int32_t m, int32_t k,
+                           int32_t n, int32_t stride_ox, int32_t stride_oy, int32_t stride_oz,
+                           int32_t stride_lx, int32_t stride_ly, int32_t stride_lz,
+                           int32_t stride_rx, int32_t stride_ry, int32_t stride_rz, uint32_t store,
+                           uint32_t load, uint32_t mask, int64_t workspace_bytes);
 
 /*
  * Microbenchmark aids (the device kernels of adrastea_kernels/cpp/microbench.cu:28-51 -- empty_kernel,

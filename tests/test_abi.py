@@ -134,3 +134,29 @@ def test_integration_source_list_matches_the_build():
     block = text[text.index("let src = ["):]
     block = block[:block.index("];")]
     assert sorted(re.findall(r'"([a-z0-9_]+\.hip)"', block)) == sorted(build.SOURCES)
+
+
+def test_workspace_plan_and_size():
+    """adr_matmul_f16_ws splits K only for few output tiles and a long K, and only with enough
+    workspace; the size query and the plan agree."""
+    lib = _ffi.lib()
+
+    def need(m, k, n):
+        return lib.adr_matmul_f16_workspace_bytes(1, m, k, n, 1, n, 0, 1, k, 0, k, 1, 0, 0, 0, 0)
+
+    def plan_ws(m, k, n, ws):
+        buf = C.create_string_buffer(96)
+        assert lib.adr_matmul_f16_ws_plan(buf, 96, 1, m, k, n, 1, n, 0, 1, k, 0, k, 1, 0, 0, 0, 0, ws) == 0
+        return buf.value.decode()
+    b = need(128, 11008, 4096)
+    assert b > 0
+    assert plan_ws(128, 11008, 4096, b).endswith("_splitk4")
+    # less workspace: fewer pieces, then none
+    assert plan_ws(128, 11008, 4096, b - 16).endswith("_splitk3")
+    assert plan_ws(128, 11008, 4096, b // 8) == plan_ws(128, 11008, 4096, 0) == _plan(
+        1, 128, 11008, 4096, (1, 4096, 0), (1, 11008, 0), (11008, 1, 0))[1]
+    # the prefill shapes and the decode shapes are never split
+    assert need(2048, 4096, 12288) == 0 and need(2048, 11008, 4096) == 0
+    assert need(1, 4096, 4096) == 0 and need(16, 11008, 4096) == 0
+    assert need(128, 512, 4096) == 0            # short K
+    assert lib.adr_matmul_f16_workspace_bytes(1, -1, 64, 64, 1, 64, 0, 1, 64, 0, 64, 1, 0, 0, 0, 0) == _ffi.ADR_EINVAL_SHAPE
