@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(HERE, "lib", "libadrastea_kernels_hip.so")
 SYMBOLS = (
     "adr_matmul_f16", "adr_matmul_f16_slow", "adr_matmul_f16_raw", "adr_matmul_nt_f16",
     "adr_matmul_f16_ws", "adr_matmul_f16_workspace_bytes", "adr_matmul_f16_ws_plan",
+    "adr_matmul_f16_noalloc",
     "adr_matmul_nt_fp16u8", "adr_dequantize_absmax_u8", "adr_quantize_absmax_u8",
     "adr_dequantize_absmax_uint8", "adr_quantize_absmax_uint8", "adr_matmul_f16_plan",
     "adr_matmul_nt_fp16u8_plan", "adr_softmax_rows", "adr_error_stats_f16", "adr_error_stats_f32", "adr_attention_f16", "adr_embed_uint8",
@@ -20,7 +21,8 @@ SYMBOLS = (
 
 ADR_OK, ADR_EINVAL_SHAPE, ADR_EINVAL_ENUM, ADR_ENOTIMPL, ADR_ENULL, ADR_EDIVISIBILITY = (
     0, -1, -2, -3, -4, -5)
-ADR_EUNSUPPORTED_DEVICE, ADR_EUNSUPPORTED_LAYOUT = -6, -7
+ADR_EUNSUPPORTED_DEVICE, ADR_EUNSUPPORTED_LAYOUT, ADR_ESCRATCH = -6, -7, -8
+NOALLOC_SCRATCH_BYTES = 16 * 1024 * 1024
 
 
 class TensorDesc(C.Structure):
@@ -52,6 +54,7 @@ def lib():
     L.adr_matmul_f16.argtypes = mm
     L.adr_matmul_f16_slow.argtypes = mm
     L.adr_matmul_f16_ws.argtypes = mm + [vp, C.c_int64]
+    L.adr_matmul_f16_noalloc.argtypes = mm
     L.adr_matmul_f16_workspace_bytes.argtypes = [i32] * 13 + [u32, u32, u32]
     L.adr_matmul_f16_ws_plan.argtypes = [C.c_char_p, i32] + [i32] * 13 + [u32, u32, u32, C.c_int64]
     L.adr_matmul_f16_raw.argtypes = [vp, vp, vp, vp] + [i32] * 13

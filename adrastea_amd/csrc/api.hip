@@ -2,6 +2,8 @@
 // Declarations and the reference interface each one replaces: include/adrastea_kernels.h.
 #include <string.h>
 
+#include <atomic>
+
 #include "adr_common.hpp"
 
 using namespace adr;
@@ -96,6 +98,40 @@ int validate_quant(const adr_tensor_desc& wide, const adr_tensor_desc& scales,
 
 }  // namespace
 
+// ---- scratch of the entry point that allocates nothing ------------------------------------------
+// A file-scope device array: every GPU the library runs on holds its own copy, at its own
+// address, until the process ends.  In host code the array's NAME is only a handle for
+// hipGetSymbolAddress: the kernels get the device address that call returns, kept per device.
+static __device__ __align__(256) unsigned char scratch[ADR_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+
+constexpr int MAX_SCRATCH_DEVICES = 64;
+std::atomic<void*> scratch_address[MAX_SCRATCH_DEVICES];
+
+// Device address of `scratch` on the current device (looked up once per device, with that device
+// current), or null with the error in *err.
+void* scratch_on_current_device(hipError_t* err) {
+  *err = hipSuccess;
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= MAX_SCRATCH_DEVICES) {
+    *err = e != hipSuccess ? e : hipErrorInvalidDevice;
+    return nullptr;
+  }
+  void* p = scratch_address[dev].load(std::memory_order_acquire);
+  if (p) return p;
+  e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || !p) {
+    *err = e != hipSuccess ? e : hipErrorInvalidSymbol;
+    return nullptr;
+  }
+  scratch_address[dev].store(p, std::memory_order_release);  // (racing threads store the same value)
+  return p;
+}
+
+}  // namespace
+
 extern "C" {
 
 int adr_abi_version(void) { return ABI_VERSION; }
@@ -109,6 +145,9 @@ const char* adr_strerror(int code) {
     case ADR_ENULL: return "null tensor pointer or missing bias";
     case ADR_EDIVISIBILITY: return "size not divisible by block_size / unsupported block_size";
     case ADR_EUNSUPPORTED_DEVICE: return "current device is not gfx950";
+    case ADR_ESCRATCH:
+      return "adr_matmul_f16_noalloc: the product would split K with more scratch than the built-in "
+             "ADR_NOALLOC_SCRATCH_BYTES; use adr_matmul_f16 or adr_matmul_f16_ws";
     case ADR_EUNSUPPORTED_LAYOUT:
       return "fused attention covers head dimension 64 or 128, unit x strides, y/z strides that "
              "are multiples of 8 and 16-byte aligned pointers";
@@ -143,6 +182,32 @@ int adr_matmul_f16_ws(adr_stream_t stream, uint16_t* output, const uint16_t* lhs
   if ((uintptr_t)workspace % 16 != 0) return ADR_EINVAL_SHAPE;
   a.workspace = (float*)workspace;
   a.workspace_bytes = workspace_bytes;
+  return run_matmul((hipStream_t)stream, a, true);
+}
+
+int adr_matmul_f16_noalloc(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
+                           const uint16_t* rhs, int32_t batches, int32_t m, int32_t k, int32_t n,
+                           int32_t stride_ox, int32_t stride_oy, int32_t stride_oz, int32_t stride_lx,
+                           int32_t stride_ly, int32_t stride_lz, int32_t stride_rx, int32_t stride_ry,
+                           int32_t stride_rz, const uint16_t* bias, float beta, float scale,
+                           uint32_t store, uint32_t load, uint32_t mask) {
+  MatmulArgs a = pack(output, lhs, rhs, batches, m, k, n, stride_ox, stride_oy, stride_oz,
+                      stride_lx, stride_ly, stride_lz, stride_rx, stride_ry, stride_rz, bias, beta,
+                      scale, store, load, mask);
+  if (int rc = validate_matmul(a, true)) return rc;
+  if (empty(a)) return ADR_OK;
+  if (int rc = check_device()) return rc;
+  // what the product would use with a workspace of any size: it has to fit the built-in one
+  const char* name;
+  const int64_t need = gemv_f16_supported(a, &name) ? 0 : mfma_gemm_workspace_bytes(a);
+  if (need > ADR_NOALLOC_SCRATCH_BYTES) return ADR_ESCRATCH;
+  if (need > 0) {
+    hipError_t e;
+    void* p = scratch_on_current_device(&e);
+    if (!p) return (int)e;
+    a.workspace = (float*)p;
+    a.workspace_bytes = ADR_NOALLOC_SCRATCH_BYTES;
+  }
   return run_matmul((hipStream_t)stream, a, true);
 }
 

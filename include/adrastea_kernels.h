@@ -38,8 +38,10 @@ enum {
   ADR_ENULL = -4,          /* null tensor pointer, or a bias operator without a bias */
   ADR_EDIVISIBILITY = -5,  /* u8 kernels: p % block_size != 0 or block_size not supported */
   ADR_EUNSUPPORTED_DEVICE = -6, /* the current device is not gfx950 */
-  ADR_EUNSUPPORTED_LAYOUT = -7  /* adr_attention_f16: head dimension, stride or alignment that the
+  ADR_EUNSUPPORTED_LAYOUT = -7, /* adr_attention_f16: head dimension, stride or alignment that the
                                    fused kernel does not cover; use the three-call sequence */
+  ADR_ESCRATCH = -8             /* adr_matmul_f16_noalloc: the product needs more scratch than
+                                   ADR_NOALLOC_SCRATCH_BYTES */
 };
 
 /* adrastea_models/src/kernels.rs:81-135, adrastea_kernels/cpp/matmul.cu:26-36 */
@@ -116,6 +118,30 @@ int64_t adr_matmul_f16_workspace_bytes(int32_t batches, int32_t m, int32_t k, in
                                        int32_t stride_lx, int32_t stride_ly, int32_t stride_lz,
                                        int32_t stride_rx, int32_t stride_ry, int32_t stride_rz,
                                        uint32_t store, uint32_t load, uint32_t mask);
+
+/*
+ * adr_matmul_f16_ws without the workspace argument (no counterpart in the reference).  For
+ * callers that cannot allocate device memory around a call: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  The scratch is a fixed array of
+ * ADR_NOALLOC_SCRATCH_BYTES inside the library's device code, one copy per GPU the library runs
+ * on, held until the process ends; the entry point allocates and frees nothing (its first call
+ * on a device looks the array's address up once).  Same arguments, validation and result as
+ * adr_matmul_f16_ws given a workspace of at least adr_matmul_f16_workspace_bytes bytes.
+ * A product that would use more than ADR_NOALLOC_SCRATCH_BYTES (16 MiB: the LLaMA-7B down
+ * projection up to 256 rows fits) returns ADR_ESCRATCH and launches nothing.
+ * All calls on one GPU share that GPU's array: calls that may overlap in time (different streams)
+ * race on it and must be serialised by the caller or use adr_matmul_f16_ws with buffers of their
+ * own.  Nothing in the array has to start at zero and nothing is kept from one call to the next
+ * (every partial tile is written before the reduction reads it).
+ */
+#define ADR_NOALLOC_SCRATCH_BYTES (16 * 1024 * 1024)
+int adr_matmul_f16_noalloc(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
+                           const uint16_t* rhs, int32_t batches, int32_t m, int32_t k, int32_t n,
+                           int32_t stride_ox, int32_t stride_oy, int32_t stride_oz,
+                           int32_t stride_lx, int32_t stride_ly, int32_t stride_lz,
+                           int32_t stride_rx, int32_t stride_ry, int32_t stride_rz,
+                           const uint16_t* bias, float beta, float scale, uint32_t store,
+                           uint32_t load, uint32_t mask);
 
 /* `matmul_f16_raw` (matmul.cu:515-517): identity operators, the 16 common arguments. */
 int adr_matmul_f16_raw(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,

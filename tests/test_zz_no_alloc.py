@@ -1,0 +1,90 @@
+"""adr_matmul_f16_noalloc (the entry point that allocates nothing: its scratch is a fixed array
+inside the library's device code) against adr_matmul_f16_ws (the same kernels with a
+caller-provided workspace), through the C ABI: bit-identical results on two calls in a row, the
+second with a smaller input; the size limit; products that need no scratch."""
+import pytest
+import torch
+
+from adrastea_amd import _ffi
+
+pytestmark = pytest.mark.gpu
+
+
+def nt(M, K, N):
+    return (1, N, 0), (1, K, 0), (K, 1, 0)
+
+
+def call(fn_name, out, a, w, M, K, N, bias=None, beta=0.0, store=0, ws=None):
+    lib = _ffi.lib()
+    so, sl, sr = nt(M, K, N)
+    args = [torch.cuda.current_stream().cuda_stream, out.data_ptr(), a.data_ptr(), w.data_ptr(), 1, M, K, N,
+            *so, *sl, *sr, bias.data_ptr() if bias is not None else None, beta, 1.0, store, 0, 0]
+    if ws is not None:
+        args += [ws.data_ptr(), ws.numel()]
+    return getattr(lib, fn_name)(*args)
+
+
+def test_noalloc_matches_workspace_entry_point_on_two_calls_in_a_row():
+    lib = _ffi.lib()
+    K, N = 11008, 4096
+    gen = torch.Generator(device="cuda").manual_seed(91)
+    w = (torch.randn(N, K, generator=gen, device="cuda") * K ** -0.5).half()
+    bias = torch.randn(N, generator=gen, device="cuda").half()
+    ws = torch.empty(_ffi.NOALLOC_SCRATCH_BYTES, dtype=torch.uint8, device="cuda")
+    results = []
+    for M in (256, 100):   # the second call is smaller and must not see the first one's partials
+        so, sl, sr = nt(M, K, N)
+        need = lib.adr_matmul_f16_workspace_bytes(1, M, K, N, *so, *sl, *sr, 3, 0, 0)
+        assert 0 < need <= _ffi.NOALLOC_SCRATCH_BYTES   # the scratch is really used
+        a = torch.randn(M, K, generator=gen, device="cuda").half()
+        prev = torch.randn(M, N, generator=gen, device="cuda").half()
+        want = prev.clone()
+        assert call("adr_matmul_f16_ws", want, a, w, M, K, N, bias=bias, beta=0.5, store=3, ws=ws) == 0
+        got = prev.clone()
+        assert call("adr_matmul_f16_noalloc", got, a, w, M, K, N, bias=bias, beta=0.5, store=3) == 0
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), M
+        ref = a.float() @ w.float().t() + bias.float() + 0.5 * prev.float()
+        rms = ref.pow(2).mean().sqrt()
+        assert ((got.float() - ref).abs() / torch.maximum(ref.abs(), rms)).max().item() <= 2e-3
+        results.append(got)
+    # the first problem again: same bits as before the smaller call used the scratch
+    M = 256
+    gen = torch.Generator(device="cuda").manual_seed(91)
+    w2 = (torch.randn(N, K, generator=gen, device="cuda") * K ** -0.5).half()
+    bias2 = torch.randn(N, generator=gen, device="cuda").half()
+    a = torch.randn(M, K, generator=gen, device="cuda").half()
+    prev = torch.randn(M, N, generator=gen, device="cuda").half()
+    again = prev.clone()
+    assert call("adr_matmul_f16_noalloc", again, a, w2, M, K, N, bias=bias2, beta=0.5, store=3) == 0
+    assert torch.equal(again, results[0])
+
+
+def test_noalloc_size_limit_and_products_without_scratch():
+    lib = _ffi.lib()
+    # a product whose split would need more than the built-in scratch: rejected, nothing written
+    M, K, N = 300, 22016, 4096
+    so, sl, sr = nt(M, K, N)
+    assert lib.adr_matmul_f16_workspace_bytes(1, M, K, N, *so, *sl, *sr, 0, 0, 0) > _ffi.NOALLOC_SCRATCH_BYTES
+    a = torch.zeros(M, K, dtype=torch.float16, device="cuda")
+    w = torch.zeros(N, K, dtype=torch.float16, device="cuda")
+    out = torch.full((M, N), 3.0, dtype=torch.float16, device="cuda")
+    rc = call("adr_matmul_f16_noalloc", out, a, w, M, K, N)
+    assert rc == _ffi.ADR_ESCRATCH and "ADR_NOALLOC_SCRATCH_BYTES" in _ffi.strerror(rc)
+    torch.cuda.synchronize()
+    assert torch.all(out == 3.0)
+    # products that are not split run as adr_matmul_f16 does: prefill, decode, empty
+    gen = torch.Generator(device="cuda").manual_seed(92)
+    for M, K, N in ((512, 1024, 768), (4, 4096, 4096), (0, 64, 64)):
+        a = torch.randn(max(M, 1), K, generator=gen, device="cuda").half()
+        w = (torch.randn(N, K, generator=gen, device="cuda") * K ** -0.5).half()
+        got = torch.zeros(max(M, 1), N, dtype=torch.float16, device="cuda")
+        want = torch.zeros_like(got)
+        assert call("adr_matmul_f16_noalloc", got, a, w, M, K, N) == 0
+        assert call("adr_matmul_f16", want, a, w, M, K, N) == 0
+        assert torch.equal(got, want)
+    # same validation as the other entry points
+    assert lib.adr_matmul_f16_noalloc(None, None, a.data_ptr(), w.data_ptr(), 1, 4, 64, 64, 1, 64, 0, 1, 64, 0,
+                                      64, 1, 0, None, 0.0, 1.0, 0, 0, 0) == _ffi.ADR_ENULL
+    assert lib.adr_matmul_f16_noalloc(None, got.data_ptr(), a.data_ptr(), w.data_ptr(), 1, 4, 64, 64, 1, 64, 0,
+                                      1, 64, 0, 64, 1, 0, None, 0.0, 1.0, 1, 0, 0) == _ffi.ADR_ENOTIMPL
