@@ -15,6 +15,7 @@
 
 #include "../../adrastea_amd/host/kernels.hpp"
 #include "../../adrastea_amd/host/pickle.hpp"
+#include "../../adrastea_amd/host/llama_loader.hpp"
 
 using namespace adrastea;
 
@@ -225,6 +226,56 @@ static int pickle_dump(int argc, char** argv) {
   return 0;
 }
 
+// Every weight of a LLaMA checkpoint through the model loaders (llama.rs:171-243), one line per
+// address: name dtype rank shape.. stride.. bytes fnv1a64(bytes).
+static void dump_loaded(const std::string& name, const LoadedTensor& t) {
+  static const char* names[] = {"i8", "i64", "f16", "f32", "f64"};
+  uint64_t h = 1469598103934665603ull;
+  for (size_t i = 0; i < t.bytes; i++) h = (h ^ t.data[i]) * 1099511628211ull;
+  printf("%s %s %zu", name.c_str(), names[(int)t.dtype], t.shape.size());
+  for (size_t d : t.shape) printf(" %zu", d);
+  for (size_t d : t.stride) printf(" %zu", d);
+  printf(" %zu %016llx\n", t.bytes, (unsigned long long)h);
+}
+
+template <typename Names, typename Loader>
+static void dump_llama(const Loader& loader, size_t layers) {
+  auto one = [&](const LlamaModelAddress& a) { dump_loaded(Names::resolve(a), loader.load_tensor(a)); };
+  one(LlamaModelAddress::token_embedding());
+  for (size_t l = 0; l < layers; l++) {
+    using B = LlamaTransformerBlockAddress;
+    one(LlamaModelAddress::in_layer(l, B::attention_norm()));
+    for (auto a : {LlamaAttentionAddress::Query, LlamaAttentionAddress::Key, LlamaAttentionAddress::Value,
+                   LlamaAttentionAddress::Out})
+      one(LlamaModelAddress::in_layer(l, B::of(a)));
+    one(LlamaModelAddress::in_layer(l, B::mlp_norm()));
+    for (auto a : {LlamaMLPAddress::Gate, LlamaMLPAddress::Expand, LlamaMLPAddress::Contract})
+      one(LlamaModelAddress::in_layer(l, B::of(a)));
+  }
+  one(LlamaModelAddress::output_norm());
+  one(LlamaModelAddress::token_projection());
+}
+
+// llama-meta <file> <layers> | llama-hf <dir> <layers> <dim> <n_heads>
+static int llama_dump(int argc, char** argv) {
+  try {
+    const size_t layers = (size_t)atoll(argv[3]);
+    if (!strcmp(argv[1], "llama-meta")) {
+      auto m = PickledModel::load_file(argv[2]);
+      dump_llama<MetaTensorNames>(MetaLlamaModelLoader(*m), layers);
+    } else {
+      if (argc < 6) throw std::runtime_error("usage: llama-hf dir layers dim n_heads");
+      auto m = ShardedModel::load_huggingface(argv[2]);
+      dump_llama<HuggingFaceTensorNames>(
+          HuggingFaceLlamaModelLoader(*m, {(size_t)atoll(argv[4]), (size_t)atoll(argv[5])}), layers);
+    }
+  } catch (const std::exception& e) {
+    printf("ERROR %s\n", e.what());
+    return 2;
+  }
+  return 0;
+}
+
 // Checkpoint -> device -> u8: uploads one fp16 [N, K] tensor of the file, quantises it with
 // adr_quantize_absmax_u8 and dequantises it again; prints the largest |x - dq(q(x))| / scale.
 static int pickle_quantize(const char* path, const char* name, int block_size) {
@@ -268,6 +319,7 @@ static int pickle_quantize(const char* path, const char* name, int block_size) {
 
 int main(int argc, char** argv) {
   if (argc > 2 && (!strcmp(argv[1], "pickle") || !strcmp(argv[1], "sharded"))) return pickle_dump(argc, argv);
+  if (argc > 3 && (!strcmp(argv[1], "llama-meta") || !strcmp(argv[1], "llama-hf"))) return llama_dump(argc, argv);
   if (argc > 4 && !strcmp(argv[1], "quantize")) return pickle_quantize(argv[2], argv[3], atoi(argv[4]));
   if (argc > 1 && !strcmp(argv[1], "gpu")) gpu_test(); else cpu_tests();
   printf(failures ? "FAILED (%d)\n" : "OK\n", failures);

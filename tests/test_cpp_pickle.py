@@ -259,3 +259,106 @@ def test_tensor_span_overflow_is_rejected(tmp_path, dim0):
             z.writestr(name, data)
     rc, out = run("pickle", dst)
     assert rc == 2 and "ERROR" in out, (rc, out)
+
+
+# ---- LLaMA tensor names and the Hugging Face query/key row order (llama.rs:70-243) ---------------
+
+LLAMA = dict(dim=16, n_heads=2, hidden=24, vocab=11, layers=2)
+
+
+def _meta_llama_state():
+    g = torch.Generator().manual_seed(17)
+    r = lambda *s: torch.randn(*s, generator=g).half()
+    d, hid, v = LLAMA["dim"], LLAMA["hidden"], LLAMA["vocab"]
+    st = {"tok_embeddings.weight": r(v, d), "norm.weight": r(d), "output.weight": r(v, d)}
+    for l in range(LLAMA["layers"]):
+        st.update({f"layers.{l}.attention_norm.weight": r(d), f"layers.{l}.ffn_norm.weight": r(d),
+                   f"layers.{l}.attention.wq.weight": r(d, d), f"layers.{l}.attention.wk.weight": r(d, d),
+                   f"layers.{l}.attention.wv.weight": r(d, d), f"layers.{l}.attention.wo.weight": r(d, d),
+                   f"layers.{l}.feed_forward.w1.weight": r(hid, d), f"layers.{l}.feed_forward.w2.weight": r(d, hid),
+                   f"layers.{l}.feed_forward.w3.weight": r(hid, d)})
+    return st
+
+
+def _address_order(layers):
+    """(Meta name, Hugging Face name) in the order the C++ driver walks the addresses."""
+    out = [("tok_embeddings.weight", "model.embed_tokens.weight")]
+    for l in range(layers):
+        m, h = f"layers.{l}.", f"model.layers.{l}."
+        out += [(m + "attention_norm.weight", h + "input_layernorm.weight"),
+                (m + "attention.wq.weight", h + "self_attn.q_proj.weight"),
+                (m + "attention.wk.weight", h + "self_attn.k_proj.weight"),
+                (m + "attention.wv.weight", h + "self_attn.v_proj.weight"),
+                (m + "attention.wo.weight", h + "self_attn.o_proj.weight"),
+                (m + "ffn_norm.weight", h + "post_attention_layernorm.weight"),
+                (m + "feed_forward.w1.weight", h + "mlp.gate_proj.weight"),
+                (m + "feed_forward.w3.weight", h + "mlp.up_proj.weight"),
+                (m + "feed_forward.w2.weight", h + "mlp.down_proj.weight")]
+    return out + [("norm.weight", "model.norm.weight"), ("output.weight", "lm_head.weight")]
+
+
+def _check_loaded(stdout, names, state):
+    lines = stdout.strip().splitlines()
+    assert len(lines) == len(names)
+    for line, (name, key) in zip(lines, names):
+        t = state[key].contiguous()
+        parts = line.split()
+        dims = [str(x) for x in t.shape]
+        assert parts[0] == name and parts[1] == "f16" and parts[2] == str(t.dim()), line
+        assert parts[3:3 + t.dim()] == dims, line
+        raw = t.numpy().tobytes()
+        assert int(parts[-2]) == len(raw) and parts[-1] == f"{fnv1a64(raw):016x}", line
+
+
+def test_meta_llama_loader_names(tmp_path):
+    st = _meta_llama_state()
+    path = str(tmp_path / "consolidated.00.pth")
+    torch.save(st, path)
+    rc, out = run("llama-meta", path, str(LLAMA["layers"]))
+    assert rc == 0, out
+    order = _address_order(LLAMA["layers"])
+    _check_loaded(out, [(m, m) for m, _ in order], st)
+    rc, out = run("llama-meta", path, str(LLAMA["layers"] + 1))       # a layer the file lacks
+    assert rc == 2 and "layers.2.attention_norm.weight not found" in out
+
+
+def test_huggingface_llama_loader_restores_meta_row_order(tmp_path):
+    """A Hugging Face style checkpoint made from Meta-layout weights the way the transformers
+    conversion script makes it (query/key rows of each head de-interleaved: view(n_heads,
+    head/2, 2, dim).transpose(1, 2)), split over two shards, one key projection stored
+    transposed (non-unit column stride): the loader must hand back Meta's weights bit for bit
+    under the Hugging Face names, as contiguous [dim, dim] matrices for q and k."""
+    st = _meta_llama_state()
+    d, h = LLAMA["dim"], LLAMA["n_heads"]
+    permute = lambda w: w.view(h, d // h // 2, 2, d).transpose(1, 2).reshape(d, d)
+    order = _address_order(LLAMA["layers"])
+    hf = {}
+    for m, name in order:
+        w = st[m]
+        if name.endswith(("q_proj.weight", "k_proj.weight")):
+            w = permute(w).contiguous()
+            assert not torch.equal(w, st[m])
+        hf[name] = w
+    odd = "model.layers.1.self_attn.k_proj.weight"
+    hf[odd] = hf[odd].t().contiguous().t()                            # strides (1, dim)
+    assert hf[odd].stride() == (1, d)
+    names = sorted(hf)
+    shards = {"pytorch_model-00001-of-00002.bin": names[:len(names) // 2],
+              "pytorch_model-00002-of-00002.bin": names[len(names) // 2:]}
+    for f, ks in shards.items():
+        torch.save({k: hf[k] for k in ks}, str(tmp_path / f))
+    index = {"metadata": {}, "weight_map": {k: f for f, ks in shards.items() for k in ks}}
+    (tmp_path / "pytorch_model.bin.index.json").write_text(json.dumps(index))
+    rc, out = run("llama-hf", str(tmp_path), str(LLAMA["layers"]), str(d), str(h))
+    assert rc == 0, out
+    meta_under_hf_names = {name: st[m] for m, name in order}
+    _check_loaded(out, [(name, name) for _, name in order], meta_under_hf_names)
+    # every q/k line reports the contiguous layout, whatever the file had
+    for line in out.strip().splitlines():
+        if "q_proj" in line or "k_proj" in line:
+            assert line.split()[3:7] == [str(d), str(d), str(d), "1"], line
+    # the head split must divide
+    rc, out = run("llama-hf", str(tmp_path), "1", str(d), "3")
+    assert rc == 2 and "multiple of 2 * n_heads" in out
+    rc, out = run("llama-hf", str(tmp_path), "1", "32", "2")          # wrong dim for the file
+    assert rc == 2 and "not [dim, dim]" in out
