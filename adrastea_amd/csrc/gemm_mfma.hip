@@ -379,14 +379,24 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   constexpr int CPR = BK / 8, KK = BK / 16;
   static_assert(BK == 64 || (BK == 128 && !NN && NSTAGE == 3), "slices of 64, or 128 with three stages");
   constexpr int NW = WM * WN, NT = NW * 64;
-  constexpr int IA = BM * CPR / NT, IB = BN * CPR / NT;  // DMA instructions per thread and slice
+  // DMA instructions per thread and slice.  NSTAGE == 6: the first half of the wavefronts issues
+  // all transfers of the left operand, the second half all of the right one (NWD each)
+  constexpr int NWD = NSTAGE == 6 ? NW / 2 : NW;
+  constexpr int IA = BM * CPR / (NWD * 64), IB = BN * CPR / (NWD * 64);
   constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
   constexpr int SLOT = 32 * (TN * 64 + 16);
-  static_assert(BM * CPR % NT == 0 && BN * CPR % NT == 0, "slices must split evenly over lanes");
+  static_assert(BM * CPR % (NWD * 64) == 0 && BN * CPR % (NWD * 64) == 0,
+                "slices must split evenly over lanes");
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "MFMA 32x32x16 tiling");
-  static_assert((NW / 2) * SLOT <= BM * BK * 2, "epilogue slots must fit in two A stages");
-  static_assert(NSTAGE == 2 || NSTAGE == 3 || NSTAGE == 5,
-                "2 or 3 LDS stages, or 5: two stages of the left and three of the right operand");
+  // epilogue slots: half of the wavefronts in each A stage, or (256 x 256) as many as fit per
+  // stage buffer over the A and then the B stages
+  constexpr bool SLOTS_IN_A = (NW / 2) * SLOT <= BM * BK * 2;
+  constexpr int SLOTS_PER_BUF = (BM * BK * 2) / SLOT;
+  static_assert(SLOTS_IN_A || (BN >= BM && NSTAGE == 5 && 5 * SLOTS_PER_BUF >= NW),
+                "epilogue slots must fit in the stage buffers");
+  static_assert(NSTAGE == 2 || NSTAGE == 3 || NSTAGE == 5 || NSTAGE == 6,
+                "2 or 3 LDS stages, or 5 / 6: two stages of the left and three / four of the right operand");
+  static_assert(NSTAGE != 6 || (!NN && !SPLIT && NW % 2 == 0), "role split: plain NT products");
   static_assert(!NN || BN == 128, "the N-contiguous right operand is staged as [64][128] tiles");
   // Separate objects per stage: the compiler's alias analysis then knows that the asynchronous
   // LDS writes of one stage cannot touch the stage being read, and does not serialise them.
@@ -396,6 +406,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   __shared__ __attribute__((aligned(1024))) unsigned char sB0[BN * BK * 2];
   __shared__ __attribute__((aligned(1024))) unsigned char sB1[BN * BK * 2];
   __shared__ __attribute__((aligned(1024))) unsigned char sB2[NSTAGE >= 3 ? BN * BK * 2 : 1024];
+  __shared__ __attribute__((aligned(1024))) unsigned char sB3[NSTAGE == 6 ? BN * BK * 2 : 1024];
 
   int batch, tile_m, tile_n;
   const int tile_id = SPLIT ? (int)(blockIdx.x % (unsigned)map.total) : (int)blockIdx.x;
@@ -423,12 +434,13 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   // DMA instruction i of this wavefront fills LDS chunks [(i*NW + wave)*64, +64) of a stage,
   // lane l the l-th of them; the lane fetches whatever (row, k-chunk) the swizzle puts there.
   // Rows beyond the matrix are clamped to the last row (their results are never stored).
+  const int dwave = NSTAGE == 6 ? wave % NWD : wave;  // index among the wavefronts issuing an operand
   const half_t* gA[IA];
   const half_t* gB[IB];
 #pragma unroll
   for (int i = 0; i < IA; i++) {
     int row, kc;
-    lds_chunk_inv<CPR>((i * NW + wave) * 64 + lane, row, kc);
+    lds_chunk_inv<CPR>((i * NWD + dwave) * 64 + lane, row, kc);
     gA[i] = A + (int64_t)min(m0 + row, a.m - 1) * a.stride_ly + kc * 8;
   }
 #pragma unroll
@@ -442,7 +454,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
       gB[i] = B + (int64_t)krow * a.stride_ry + min(n0 + c * 8, a.n - 8);
     } else {
       int row, kc;
-      lds_chunk_inv<CPR>((i * NW + wave) * 64 + lane, row, kc);
+      lds_chunk_inv<CPR>((i * NWD + dwave) * 64 + lane, row, kc);
       gB[i] = B + (int64_t)min(n0 + row, a.n - 1) * a.stride_rx + kc * 8;
     }
   }
@@ -453,13 +465,13 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
 #pragma unroll
     for (int i = 0; i < IA; i++)
       __builtin_amdgcn_global_load_lds(ADR_GLB_PTR(gA[i] + ks * BK),
-                                       ADR_LDS_PTR(dA + (i * NW + wave) * 1024), 16, 0, 0);
+                                       ADR_LDS_PTR(dA + (i * NWD + dwave) * 1024), 16, 0, 0);
   };
   auto dmaB = [&](int ks, unsigned char* dB) {
 #pragma unroll
     for (int i = 0; i < IB; i++)
       __builtin_amdgcn_global_load_lds(ADR_GLB_PTR(gB[i] + ks * b_slice),
-                                       ADR_LDS_PTR(dB + (i * NW + wave) * 1024), 16, 0, 0);
+                                       ADR_LDS_PTR(dB + (i * NWD + dwave) * 1024), 16, 0, 0);
   };
   auto dma = [&](unsigned char* dA, unsigned char* dB) {
     const int ks = min(kload, KT - 1);
@@ -570,7 +582,62 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  if (NSTAGE == 5) {
+  if constexpr (NSTAGE == 6) {
+    // Two stages of the left and four of the right operand, and two roles.  A wavefront's
+    // transfers complete in the order it issued them, so a wavefront that issues both operands
+    // cannot leave a right-operand slice in flight across the wait for the next left-operand
+    // slice.  Here wavefronts 0 .. NW/2-1 issue every transfer of the left operand (slice kt+1 at
+    // the head of slice kt, landed at its end) and the others every transfer of the right operand
+    // (slice kt+3 at the head of slice kt; at its end slices kt+2 and kt+3 may still be in
+    // flight): weights that no cache holds get three slices to arrive.  Each role has its own
+    // instruction stream; both pass the same barriers.
+    auto run = [&](auto role_tag) {
+      constexpr bool LEFT = decltype(role_tag)::value;
+      int kA = 0, kB = 0;
+      auto slice6 = [&](const unsigned char* cA, const unsigned char* cB, const unsigned char* nA,
+                        const unsigned char* nB, unsigned char* dA, unsigned char* dB) {
+        if (LEFT) dmaA(min(kA++, KT - 1), dA); else dmaB(min(kB++, KT - 1), dB);
+#pragma unroll
+        for (int kk = 0; kk < KK; kk++) {
+          if (kk + 1 < KK) {
+            load_frags((kk + 1) & 1, cA, cB, kk + 1);
+            mfmas(kk & 1);
+#pragma unroll
+            for (int q = 0; q < TM * TN; q++) {
+              __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+              __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+              if (kk * TM * TN + q < (LEFT ? IA : IB)) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+            }
+          } else {
+            mfmas(kk & 1);
+          }
+        }
+        wait_dma_barrier(std::integral_constant<int, LEFT ? 0 : 2 * IB>{});
+        load_frags(0, nA, nB, 0);
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      if (LEFT) {
+        dmaA(min(kA++, KT - 1), sA0);
+      } else {
+        dmaB(min(kB++, KT - 1), sB0);
+        dmaB(min(kB++, KT - 1), sB1);
+        dmaB(min(kB++, KT - 1), sB2);
+      }
+      wait_dma_barrier(std::integral_constant<int, LEFT ? 0 : 2 * IB>{});
+      load_frags(0, sA0, sB0, 0);
+      int kt = 0;
+      for (; kt + 4 <= KT; kt += 4) {
+        slice6(sA0, sB0, sA1, sB1, sA1, sB3);
+        slice6(sA1, sB1, sA0, sB2, sA0, sB0);
+        slice6(sA0, sB2, sA1, sB3, sA1, sB1);
+        slice6(sA1, sB3, sA0, sB0, sA0, sB2);
+      }
+      if (kt < KT) { slice6(sA0, sB0, sA1, sB1, sA1, sB3); kt++; }
+      if (kt < KT) { slice6(sA1, sB1, sA0, sB2, sA0, sB0); kt++; }
+      if (kt < KT) { slice6(sA0, sB2, sA1, sB3, sA1, sB1); kt++; }
+    };
+    if (__builtin_amdgcn_readfirstlane(wave) < NW / 2) run(std::true_type{}); else run(std::false_type{});
+  } else if (NSTAGE == 5) {
     // Two stages of the left and three of the right operand: slice kt reads A stage kt % 2 and
     // B stage kt % 3; at its head the DMA of A(kt+1) and then of B(kt+2) is issued, and at its
     // end everything but B(kt+2) has to have landed.  The right operand (weights that no cache
@@ -661,7 +728,14 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
         }
     return;
   }
-  unsigned char* slot = (wave < NW / 2 ? sA0 : sA1) + (wave % (NW / 2)) * SLOT;
+  unsigned char* slot;
+  if (SLOTS_IN_A) {
+    slot = (wave < NW / 2 ? sA0 : sA1) + (wave % (NW / 2)) * SLOT;
+  } else {
+    const int buf = wave / SLOTS_PER_BUF;
+    slot = (buf == 0 ? sA0 : buf == 1 ? sA1 : buf == 2 ? sB0 : buf == 3 ? sB1 : sB2) +
+           (wave % SLOTS_PER_BUF) * SLOT;
+  }
   wave_epilogue<TM, TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, slot, (half_t)a.scale, lane);
 }
 
@@ -1442,7 +1516,7 @@ enum GemmChoice {
   GEMM_NONE = 0,
   SHORTK_64, SHORTK_128,
   U8_256x192, U8_256x128,
-  DMA_256x192, DMA_256x128, DMA_128x128, DMA_128x64, DMA_64x64, DMA_64x64_K128, DMA_128x64_K128,
+  DMA_256x256, DMA_256x192, DMA_256x128, DMA_128x128, DMA_128x64, DMA_64x64, DMA_64x64_K128, DMA_128x64_K128,
   DMA_NN_256x128, DMA_NN_128x128,
   STAGE_256x128, STAGE_128x128, STAGE_64x64,
 };
@@ -1510,7 +1584,19 @@ GemmChoice choose(const MatmulArgs& a) {
                                          {DMA_64x64, 64, 64, 4, 0.50f}};
       return pick(a, shortk, 2);
     }
-    const GemmChoice c = pick(a, DMA_TILES, 5);
+    double cost;
+    GemmChoice c = pick(a, DMA_TILES, 5, &cost);
+    // 256 x 256 tiles move 14 % fewer bytes into LDS per flop than 256 x 192 (2 % faster per
+    // tile area) but are too coarse for most shapes; they win where they fill whole rounds and
+    // the smaller tiles do not (M2048 K4096 N8192: 137 -> 124 us, M4096 N4096: 134 -> 122 us).
+    // Long K only: with few slices one large tile per CU has nothing to overlap its prologue
+    // and epilogue with.
+    if (a.k >= 2048) {
+      static const Candidate big = {DMA_256x256, 256, 256, 1, 1.12f};
+      double cost_big;
+      pick(a, &big, 1, &cost_big);
+      if (cost_big < cost) c = DMA_256x256;
+    }
     // At most one 64 x 64 tile per CU (a few dozen to a few hundred rows against a weight
     // matrix): the product is bound by how DRAM serves the weight requests -- one piece of every
     // tile row per slice, a whole weight row apart -- and pieces of 256 bytes (slices of 128)
@@ -1630,6 +1716,7 @@ static bool choice_name(GemmChoice c, const char** name, bool u8 = false) {
     case SHORTK_128: *name = "gemm_nt_mfma_persistent_128x128_k128"; return true;
     case U8_256x192: *name = "gemm_nt_u8_mfma_256x192x64"; return true;
     case U8_256x128: *name = "gemm_nt_u8_mfma_256x128x64"; return true;
+    case DMA_256x256: *name = "gemm_nt_mfma_dma_256x256x64"; return true;
     case DMA_256x192: *name = "gemm_nt_mfma_dma_256x192x64"; return true;
     case DMA_256x128: *name = "gemm_nt_mfma_dma_256x128x64"; return true;
     case DMA_128x128: *name = "gemm_nt_mfma_dma_128x128x64"; return true;
@@ -1652,7 +1739,8 @@ static hipError_t launch_choice(hipStream_t stream, const MatmulArgs& a, GemmCho
     case SHORTK_128: return launch_shortk<16>(stream, a);
     case U8_256x192: return launch_u8<256, 192, 4, 2>(stream, a);
     case U8_256x128: return launch_u8<256, 128, 4, 2>(stream, a);
-    case DMA_256x192: return launch_dma<256, 192, 4, 2, 5, 1>(stream, a);
+    case DMA_256x256: return launch_dma<256, 256, 4, 2, 5, 1>(stream, a);
+    case DMA_256x192: return launch_dma<256, 192, 4, 2, 6, 1>(stream, a);
     case DMA_256x128: return launch_dma<256, 128, 4, 2, 3, 1>(stream, a);
     case DMA_128x128: return launch_dma<128, 128, 2, 2, 3, 1>(stream, a);
     case DMA_128x64: return launch_dma<128, 64, 2, 2, 3, 2>(stream, a);

@@ -462,9 +462,10 @@ def test_full_size_gemm_against_fp32_gemm_and_slow_kernel(case):
 
 @pytest.mark.parametrize("K", [320, 384, 448, 512, 576, 640])
 def test_large_tile_kernel_every_k_tail_exact(K):
-    """The 256 x 192 kernel rotates two left and three right LDS stages with a period of six
-    slices: every remainder of that loop, on inputs whose fp32 sums are exact, must give the
-    correctly rounded product bit for bit (ragged last tile row and column included)."""
+    """The 256 x 192 kernel rotates two left and four right LDS stages with a period of four
+    slices, half of its wavefronts issuing the left and half the right operand's transfers:
+    every remainder of that loop, on inputs whose fp32 sums are exact, must give the correctly
+    rounded product bit for bit (ragged last tile row and column included)."""
     M, N = 2000, 12200
     so, sl, sr = nt_strides(M, K, N)
     assert plan(1, M, K, N, so, sl, sr) == "gemm_nt_mfma_dma_256x192x64"
@@ -475,6 +476,64 @@ def test_large_tile_kernel_every_k_tail_exact(K):
     assert raw_matmul("adr_matmul_f16", out, a, w, 1, M, K, N, so, sl, sr) == 0
     want = (a.double() @ w.double().t()).half()
     assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.parametrize("K", [2048, 2112, 2176, 2240, 2304, 2368])
+def test_256x256_tile_every_k_tail_exact(K):
+    """The 256 x 256 kernel (long K, whole rounds of 256 tiles) rotates two left and three right
+    LDS stages with a period of six slices; its epilogue slots spill over into the right
+    operand's stages.  Every remainder of the loop on inputs whose fp32 sums are exact, ragged
+    last tile row and column."""
+    M, N = 2000, 8184
+    so, sl, sr = nt_strides(M, K, N)
+    assert plan(1, M, K, N, so, sl, sr) == "gemm_nt_mfma_dma_256x256x64"
+    gen = torch.Generator(device="cuda").manual_seed(K)
+    a = (torch.randint(-4, 5, (M, K), generator=gen, device="cuda").float() / 64).half()
+    w = (torch.randint(-4, 5, (N, K), generator=gen, device="cuda").float() / 64).half()
+    out = torch.full((M, N), 9.0, dtype=torch.float16, device="cuda")
+    assert raw_matmul("adr_matmul_f16", out, a, w, 1, M, K, N, so, sl, sr) == 0
+    want = (a.double() @ w.double().t()).half()
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.parametrize("store", STORES_EXACT + STORES_F32)
+@pytest.mark.parametrize("mask", [oracle.MASK_NONE, oracle.MASK_CAUSAL])
+def test_256x256_tile_epilogues_against_the_slow_kernel(store, mask):
+    """Every store operator and the causal mask through the 256 x 256 tile's epilogue, compared
+    with the step-for-step kernel on bands of rows (first tile row, a diagonal tile, the ragged
+    last rows)."""
+    M, K, N = 4000, 2048, 4090 - 2
+    so, sl, sr = nt_strides(M, K, N)
+    assert plan(1, M, K, N, so, sl, sr, store=store, mask=mask) == "gemm_nt_mfma_dma_256x256x64"
+    gen = torch.Generator(device="cuda").manual_seed(900 + store * 2 + mask)
+    a = torch.randn(M, K, generator=gen, device="cuda").half()
+    w = (torch.randn(N, K, generator=gen, device="cuda") * K ** -0.5).half()
+    prev = torch.randn(M, N, generator=gen, device="cuda").half()
+    bias = torch.randn(N, generator=gen, device="cuda").half()
+    kw = dict(bias_t=bias, beta=0.7, scale=0.2, store=store, mask=mask)
+    out = prev.clone()
+    assert raw_matmul("adr_matmul_f16", out, a, w, 1, M, K, N, so, sl, sr, **kw) == 0
+    for r0, rows in ((0, 40), (1500, 72), (M - 30, 30)):
+        # the causal mask compares absolute row numbers: run the band as a product of its own
+        # with the columns it may see shifted accordingly (a band of the full problem on the
+        # slow kernel = rows r0.. of a, previous output rows r0..)
+        slow = prev[r0:r0 + rows].clone()
+        if mask == oracle.MASK_CAUSAL:
+            # rows 0..r0+rows of the product, keep the band
+            full = prev[:r0 + rows].clone()
+            assert raw_matmul("adr_matmul_f16_slow", full, a[:r0 + rows], w, 1, r0 + rows, K, N, so, sl, sr,
+                              **kw) == 0
+            slow = full[r0:]
+        else:
+            assert raw_matmul("adr_matmul_f16_slow", slow, a[r0:r0 + rows], w, 1, rows, K, N, so, sl, sr,
+                              **kw) == 0
+        got = out[r0:r0 + rows]
+        inf = torch.isinf(slow)
+        assert torch.equal(torch.isinf(got), inf)
+        fin = ~inf
+        scale = slow[fin].float().pow(2).mean().sqrt()
+        err = (got[fin].float() - slow[fin].float()).abs() / torch.maximum(slow[fin].float().abs(), scale)
+        assert err.max().item() <= TOL, (store, mask, r0)
 
 
 def test_row_tail_split_keeps_operator_semantics():
