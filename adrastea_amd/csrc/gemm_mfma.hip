@@ -1130,8 +1130,11 @@ __global__ __launch_bounds__(WM* WN * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a
       __builtin_amdgcn_global_load_lds(ADR_GLB_PTR(gA[i] + k0),
                                        ADR_LDS_PTR(dA + (i * NW + wave) * 1024), 16, 0, 0);
   };
-  u32x2_t rq[2][LB];
-  half_t rs[2][LB];
+  // three register sets: the weights consumed in slice kt+1 were requested at the head of slice
+  // kt-1, so the wait at the end of slice kt-1 (everything but that slice's own requests)
+  // already covers them and nothing in slice kt waits for a load issued a moment ago
+  u32x2_t rq[3][LB];
+  half_t rs[3][LB];
   auto fetchQ = [&](int set) {
     const int ks = min(kloadQ, KT - 1);
     kloadQ++;
@@ -1186,7 +1189,7 @@ __global__ __launch_bounds__(WM* WN * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a
   };
   // Slice kt.  (cA, cB): its stages; (nA, nB): those of slice kt+1 -- nB is filled here from
   // register set `nset`; dA: the A stage refilled with slice kt+2; `fset`: the register set
-  // that receives the weights of slice kt+2 (the one slice kt was dequantised from).
+  // that receives the weights of slice kt+3 (the one slice kt was dequantised from).
   auto slice = [&](const unsigned char* cA, const unsigned char* cB, const unsigned char* nA,
                    unsigned char* nB, unsigned char* dA, int fset, int nset) {
     fetchQ(fset);
@@ -1222,6 +1225,7 @@ __global__ __launch_bounds__(WM* WN * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a
   fetchQ(0);
   fetchQ(1);
   dmaA(sA0);
+  fetchQ(2);
   dmaA(sA1);
   dequant_store(0, sB0);
   {
@@ -1233,17 +1237,17 @@ __global__ __launch_bounds__(WM* WN * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a
   int kt = 0;
   for (; kt + 6 <= KT; kt += 6) {
     slice(sA0, sB0, sA1, sB1, sA2, 0, 1);
-    slice(sA1, sB1, sA2, sB0, sA0, 1, 0);
-    slice(sA2, sB0, sA0, sB1, sA1, 0, 1);
-    slice(sA0, sB1, sA1, sB0, sA2, 1, 0);
-    slice(sA1, sB0, sA2, sB1, sA0, 0, 1);
-    slice(sA2, sB1, sA0, sB0, sA1, 1, 0);
+    slice(sA1, sB1, sA2, sB0, sA0, 1, 2);
+    slice(sA2, sB0, sA0, sB1, sA1, 2, 0);
+    slice(sA0, sB1, sA1, sB0, sA2, 0, 1);
+    slice(sA1, sB0, sA2, sB1, sA0, 1, 2);
+    slice(sA2, sB1, sA0, sB0, sA1, 2, 0);
   }
   if (kt < KT) { slice(sA0, sB0, sA1, sB1, sA2, 0, 1); kt++; }
-  if (kt < KT) { slice(sA1, sB1, sA2, sB0, sA0, 1, 0); kt++; }
-  if (kt < KT) { slice(sA2, sB0, sA0, sB1, sA1, 0, 1); kt++; }
-  if (kt < KT) { slice(sA0, sB1, sA1, sB0, sA2, 1, 0); kt++; }
-  if (kt < KT) { slice(sA1, sB0, sA2, sB1, sA0, 0, 1); kt++; }
+  if (kt < KT) { slice(sA1, sB1, sA2, sB0, sA0, 1, 2); kt++; }
+  if (kt < KT) { slice(sA2, sB0, sA0, sB1, sA1, 2, 0); kt++; }
+  if (kt < KT) { slice(sA0, sB1, sA1, sB0, sA2, 0, 1); kt++; }
+  if (kt < KT) { slice(sA1, sB0, sA2, sB1, sA0, 1, 2); kt++; }
   __builtin_amdgcn_s_waitcnt(0x0070);
   __builtin_amdgcn_s_barrier();
 

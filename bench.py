@@ -70,6 +70,10 @@ def main():
                     help="run only the u8 decode GEMV configurations (for profiling that kernel)")
     ap.add_argument("--attention-only", action="store_true",
                     help="run only the attention configuration (QK^T, softmax_rows, P.V, error_stats)")
+    ap.add_argument("--u8-prefill-only", action="store_true",
+                    help="run only the u8-weight prefill GEMMs of the layer set (for profiling that kernel)")
+    ap.add_argument("--clip-only", action="store_true",
+                    help="run only the CLIP GEMM configurations (for profiling those tiles)")
     ap.add_argument("--microbenchmark", action="store_true",
                     help="launch overhead, matrix-core issue peak, streaming-read peak and the "
                          "2048x4096x4096 products of the reference's microbenchmark()")
@@ -394,6 +398,77 @@ def main():
         print(json.dumps({"u8_decode_gemv": decode_set(), "f16_decode_gemv": f16_decode_set()}))
         return
 
+    def u8_prefill_set():
+        """u8 prefill GEMMs (configs[4], u8 half): the layer set at M = 2048 with u8 weights."""
+        M = 2048
+        act = {4096: randn_h(M, 4096), 11008: randn_h(M, 11008)}
+        u8p = {}
+        for name, K, N in LAYER_SET:
+            if name == "up":
+                continue
+            q = torch.randint(0, 256, (N, K), generator=gen, device=dev, dtype=torch.uint8)
+            s = (torch.rand(N, K // 32, generator=gen, device=dev) * 0.019 + 0.001).half()
+            out = torch.zeros(M, N, dtype=torch.float16, device=dev)
+
+            def f():
+                rc = lib.adr_matmul_nt_fp16u8(stream(), out.data_ptr(), act[K].data_ptr(),
+                                              q.data_ptr(), s.data_ptr(), M, K, N, 32, 0.0)
+                if rc != 0:
+                    raise RuntimeError(_ffi.strerror(rc))
+            t = timed(f, 50, 5)
+            u8p[name] = {"M": M, "K": K, "N": N, "us": round(t * 1e6, 1),
+                         "tflops": round(2.0 * M * K * N / t / 1e12, 1),
+                         "frac_mfma_peak": round(2.0 * M * K * N / t / 1e12 / PEAK_F16_TFLOPS, 4)}
+            del q, s
+        return u8p
+
+    def clip_set():
+        """CLIP GEMMs (configs[0], configs[1])."""
+
+        clip = {}
+        for nm, m, K, N in (("text_qkv_M77", 77, 768, 2304), ("vision_mlp_up", 2056, 1024, 4096),
+                            ("vision_mlp_down", 2056, 4096, 1024)):
+            a, w = randn_h(m, K), randn_h(N, K, std=K ** -0.5)
+            o = torch.zeros(m, N, dtype=torch.float16, device=dev)
+            # (launches of a few microseconds are timed as graph replays: Python cannot issue
+            # them that fast)
+            t = timed_graph(lambda: mm(o, a, w, m, K, N), 50, 20) if m < 256 else \
+                timed(lambda: mm(o, a, w, m, K, N), 50, 5)
+            byts = (m * K + N * K + m * N) * 2
+            clip[nm] = {"M": m, "K": K, "N": N, "us": round(t * 1e6, 2),
+                        "tflops": round(2.0 * m * K * N / t / 1e12, 1),
+                        "frac_mfma_peak": round(2.0 * m * K * N / t / 1e12 / PEAK_F16_TFLOPS, 4),
+                        "gbs": round(byts / t / 1e9, 1)}
+        # the same two products with the store operators the CLIP MLP uses
+        # (adrastea_models/src/clip.rs:431-442: QuickGeluBias on the way up, BetaBias 1.0 = residual add
+        # on the way down); the operator runs in the kernel's epilogue
+        for nm, K, N, store, beta in (("vision_mlp_up_quick_gelu_bias", 1024, 4096, 6, 0.0),
+                                     ("vision_mlp_down_beta_bias", 4096, 1024, 3, 1.0)):
+            m = 2056
+            a, w = randn_h(m, K), randn_h(N, K, std=K ** -0.5)
+            bias = randn_h(N)
+            o = torch.zeros(m, N, dtype=torch.float16, device=dev)
+
+            def f_op():
+                rc = lib.adr_matmul_f16(stream(), o.data_ptr(), a.data_ptr(), w.data_ptr(), 1, m, K,
+                                        N, 1, N, 0, 1, K, 0, K, 1, 0, bias.data_ptr(), beta, 1.0,
+                                        store, 0, 0)
+                if rc != 0:
+                    raise RuntimeError(_ffi.strerror(rc))
+            t = timed(f_op, 50, 5)
+            clip[nm] = {"M": m, "K": K, "N": N, "us": round(t * 1e6, 2),
+                        "tflops": round(2.0 * m * K * N / t / 1e12, 1),
+                        "frac_mfma_peak": round(2.0 * m * K * N / t / 1e12 / PEAK_F16_TFLOPS, 4)}
+        return clip
+
+    if args.u8_prefill_only:
+        print(json.dumps({"llama7b_prefill_u8": u8_prefill_set()}))
+        return
+
+    if args.clip_only:
+        print(json.dumps({"clip_fp16": clip_set()}))
+        return
+
     # ---------------- primary workload: the fp16 layer GEMM set at M = 2048
     M = 2048
     acts = {4096: randn_h(M, 4096), 11008: randn_h(M, 11008)}
@@ -484,62 +559,8 @@ def main():
 
         secondary["f16_decode_gemv"] = f16_decode_set()
 
-        # ---- u8 prefill GEMMs (configs[4], u8 half)
-        u8p = {}
-        for name, K, N in LAYER_SET:
-            if name == "up":
-                continue
-            q = torch.randint(0, 256, (N, K), generator=gen, device=dev, dtype=torch.uint8)
-            s = (torch.rand(N, K // 32, generator=gen, device=dev) * 0.019 + 0.001).half()
-
-            def f():
-                rc = lib.adr_matmul_nt_fp16u8(stream(), outs[name].data_ptr(), acts[K].data_ptr(),
-                                              q.data_ptr(), s.data_ptr(), M, K, N, 32, 0.0)
-                if rc != 0:
-                    raise RuntimeError(_ffi.strerror(rc))
-            t = timed(f, 50, 5)
-            u8p[name] = {"M": M, "K": K, "N": N, "us": round(t * 1e6, 1),
-                         "tflops": round(2.0 * M * K * N / t / 1e12, 1),
-                         "frac_mfma_peak": round(2.0 * M * K * N / t / 1e12 / PEAK_F16_TFLOPS, 4)}
-            del q, s
-        secondary["llama7b_prefill_u8"] = u8p
-
-        # ---- CLIP GEMMs (configs[0], configs[1])
-        clip = {}
-        for nm, m, K, N in (("text_qkv_M77", 77, 768, 2304), ("vision_mlp_up", 2056, 1024, 4096),
-                            ("vision_mlp_down", 2056, 4096, 1024)):
-            a, w = randn_h(m, K), randn_h(N, K, std=K ** -0.5)
-            o = torch.zeros(m, N, dtype=torch.float16, device=dev)
-            # (launches of a few microseconds are timed as graph replays: Python cannot issue
-            # them that fast)
-            t = timed_graph(lambda: mm(o, a, w, m, K, N), 50, 20) if m < 256 else \
-                timed(lambda: mm(o, a, w, m, K, N), 50, 5)
-            byts = (m * K + N * K + m * N) * 2
-            clip[nm] = {"M": m, "K": K, "N": N, "us": round(t * 1e6, 2),
-                        "tflops": round(2.0 * m * K * N / t / 1e12, 1),
-                        "frac_mfma_peak": round(2.0 * m * K * N / t / 1e12 / PEAK_F16_TFLOPS, 4),
-                        "gbs": round(byts / t / 1e9, 1)}
-        # the same two products with the store operators the CLIP MLP uses
-        # (adrastea_models/src/clip.rs:431-442: QuickGeluBias on the way up, BetaBias 1.0 = residual add
-        # on the way down); the operator runs in the kernel's epilogue
-        for nm, K, N, store, beta in (("vision_mlp_up_quick_gelu_bias", 1024, 4096, 6, 0.0),
-                                     ("vision_mlp_down_beta_bias", 4096, 1024, 3, 1.0)):
-            m = 2056
-            a, w = randn_h(m, K), randn_h(N, K, std=K ** -0.5)
-            bias = randn_h(N)
-            o = torch.zeros(m, N, dtype=torch.float16, device=dev)
-
-            def f_op():
-                rc = lib.adr_matmul_f16(stream(), o.data_ptr(), a.data_ptr(), w.data_ptr(), 1, m, K,
-                                        N, 1, N, 0, 1, K, 0, K, 1, 0, bias.data_ptr(), beta, 1.0,
-                                        store, 0, 0)
-                if rc != 0:
-                    raise RuntimeError(_ffi.strerror(rc))
-            t = timed(f_op, 50, 5)
-            clip[nm] = {"M": m, "K": K, "N": N, "us": round(t * 1e6, 2),
-                        "tflops": round(2.0 * m * K * N / t / 1e12, 1),
-                        "frac_mfma_peak": round(2.0 * m * K * N / t / 1e12 / PEAK_F16_TFLOPS, 4)}
-        secondary["clip_fp16"] = clip
+        secondary["llama7b_prefill_u8"] = u8_prefill_set()
+        secondary["clip_fp16"] = clip_set()
 
         attn = attention_set()
         secondary["llama7b_attention_fp16"] = attn

@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 
 TOL = 1e-2
 PLAN = "gemv_f16_dot2_stream"
-PLAN_MFMA = "skinny_f16_mfma16_splitk_lds"
+PLAN_MFMA = "skinny_f16_mfma16_regstream"
 
 
 def nt(M, K, N):
@@ -114,19 +114,22 @@ def test_nt_entry_point_with_beta():
 @pytest.mark.parametrize("m,K,N", [(9, 1024, 4100), (16, 4096, 1030), (13, 11008, 400), (17, 8192, 520),
                                    (32, 11008, 390), (25, 12288, 350), (20, 1024, 6200),
                                    (30, 1152, 10300),
-                                   # K = 1024 * {2, 4, 5, 8}, up to 16 rows: the LDS-ring variant,
                                    # one, two and three groups of 16 weight rows per workgroup
                                    (9, 2048, 4100), (16, 4096, 6200), (12, 5120, 10300),
                                    (11, 8192, 1000), (16, 4096, 12288),
-                                   # K between multiples of 1024: the wavefronts without a piece in
-                                   # the last round (K 11008: 86 pieces for 8 x 11)
+                                   # macro-step counts that do not divide by the eight wavefronts
+                                   # (K 11008: 86 steps), fewer steps than wavefronts + 1
                                    (16, 11008, 4096), (10, 2176, 6200), (14, 4992, 10300), (9, 10368, 800),
-                                   # 17 to 32 rows through the ring: K up to 4096
+                                   (16, 13824, 5120), (12, 6656, 700),
+                                   # 17 to 32 rows: two blocks of activations
                                    (17, 4096, 6200), (32, 2048, 12288), (25, 3072, 4100), (32, 4096, 12288),
                                    (20, 3968, 10300), (32, 11008, 4096), (19, 8192, 6200), (27, 5120, 10300),
-                                   # 33 to 64 rows: three and four blocks, K classes of 4096 and 11008
-                                   (33, 4096, 4100), (48, 4096, 6200), (49, 3968, 12288), (64, 11008, 4096),
-                                   (40, 10368, 1000), (64, 4096, 12288),
+                                   # 33 to 64 rows: three and four blocks (four: at most two row groups)
+                                   (33, 4096, 4100), (48, 4096, 6200), (49, 3968, 8192), (64, 11008, 4096),
+                                   (40, 10368, 1000), (64, 4096, 8192), (48, 5120, 5000), (64, 13824, 1000),
+                                   (48, 8192, 12288), (33, 2048, 8192),
+                                   # one to four rows where K is beyond the dot-product kernel's reach
+                                   (2, 13824, 1000), (4, 16384, 600), (1, 12416, 520),
                                    # three and four rows on narrow matrices, five to eight rows
                                    (3, 4096, 4096), (4, 2048, 4000), (4, 3072, 3072),
                                    (5, 4096, 4100), (8, 11008, 4096), (7, 1152, 4000)])
@@ -158,6 +161,7 @@ def test_matrix_core_kernel_for_five_to_sixty_four_rows(m, K, N):
 
 
 def test_more_rows_or_short_k_stay_on_the_tiled_kernels():
-    for m, K, N in [(65, 4096, 4096), (65, 11008, 4096), (33, 2048, 8192), (12, 960, 8192)]:
+    for m, K, N in [(65, 4096, 4096), (65, 11008, 4096), (33, 2000, 8192), (12, 960, 8192),
+                    (64, 4096, 12288)]:
         so, sl, sr = nt(m, K, N)
         assert plan(1, m, K, N, so, sl, sr).startswith("gemm_nt_mfma")
