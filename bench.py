@@ -523,6 +523,22 @@ def main():
         "traffic_source": "profiles/gemm_nt_dma_llama7b_layer_set.txt",
     }
 
+    if not args.quick:
+        # Two reference points for that figure, same launch, same shape.  (1) Operands of zeros: the
+        # instruction stream and the memory traffic are identical, only the switching activity in
+        # the matrix pipe is gone -- the part is power limited under this kernel, and the
+        # difference is what the power limit costs on real data.  (2) The vendor library
+        # (torch.matmul -> hipBLASLt) on the same random operands.
+        za, zw = torch.zeros_like(acts[K]), torch.zeros_like(weights[name])
+        t_zero = timed(lambda: mm(outs[name], za, zw, M, K, N), 100, 20)
+        wt = weights[name].t()
+        t_lib = timed(lambda: torch.matmul(acts[K], wt, out=outs[name]), 100, 20)
+        roofline["probe"] = {
+            "same_launch_on_zero_operands_tflops": round(qkv_flops / t_zero / 1e12, 1),
+            "library_hgemm_same_operands_tflops": round(qkv_flops / t_lib / 1e12, 1),
+        }
+        del za, zw
+
     secondary = {}
     roofline_u8 = None
     if not args.quick:
