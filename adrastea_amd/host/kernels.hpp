@@ -119,9 +119,20 @@ inline adr_tensor_desc descriptor(const TensorView<T>& v) {
 
 class GpuKernels : public CommonKernels {
  public:
-  explicit GpuKernels(adr_stream_t stream = nullptr) : stream_(stream) {}
+  // `workspace`: optional device buffer (16-byte aligned) the caller owns for as long as this
+  // object lives; with it, products with few output tiles and a long K are split over K
+  // (adr_matmul_f16_ws).  Calls on one object must not overlap in time when it is set.
+  explicit GpuKernels(adr_stream_t stream = nullptr, void* workspace = nullptr, int64_t workspace_bytes = 0)
+      : stream_(stream), workspace_(workspace), workspace_bytes_(workspace ? workspace_bytes : 0) {}
   void matmul_f16(TensorView<f16>& o, const TensorView<const f16>& l, const TensorView<const f16>& r,
-                  const MatmulOptions& opt) override { run(adr_matmul_f16, "matmul_f16", o, l, r, opt); }
+                  const MatmulOptions& opt) override {
+    if (workspace_bytes_ <= 0) return run(adr_matmul_f16, "matmul_f16", o, l, r, opt);
+    LoweredMatmul w = lower_matmul(o.layout, l.layout, r.layout, opt);
+    int rc = adr_matmul_f16_ws(stream_, o.ptr, l.ptr, r.ptr, w.batches, w.m, w.k, w.n, w.so[0], w.so[1], w.so[2],
+                               w.sl[0], w.sl[1], w.sl[2], w.sr[0], w.sr[1], w.sr[2], opt.store_.bias, w.beta,
+                               w.scale, w.store, w.load, w.mask, workspace_, workspace_bytes_);
+    if (rc) throw AdrasteaError(rc, "matmul_f16");
+  }
   void matmul_f16_slow(TensorView<f16>& o, const TensorView<const f16>& l, const TensorView<const f16>& r,
                        const MatmulOptions& opt) override { run(adr_matmul_f16_slow, "matmul_f16_slow", o, l, r, opt); }
   // kernels.rs:892-915: rows = size(-2), heads = size(-3) (1 for rank 2), width = size(-1); like
@@ -185,6 +196,8 @@ class GpuKernels : public CommonKernels {
     if (rc) throw AdrasteaError(rc, what);
   }
   adr_stream_t stream_;
+  void* workspace_;
+  int64_t workspace_bytes_;
 };
 
 // Records the set of (left, right, output) layouts seen, then forwards (kernels.rs:231-359).

@@ -190,6 +190,35 @@ static void gpu_test() {
     CHECK(bad == 0);
     CHECK(throws([&] { tr.attention_f16(av, qv, kv.permute({1, 0}), vv_, 0.125f, 1.0f, MatmulMask::None); }));
   }
+  {
+    // GpuKernels with a workspace: a product with few tiles and a long K is split over K and
+    // must give the bits of the unsplit call (inputs in {-1, 0, 1}: every sum is exact)
+    const int M2 = 100, K2 = 1472, N2 = 1000;
+    const int64_t need = adr_matmul_f16_workspace_bytes(1, M2, K2, N2, 1, N2, 0, 1, K2, 0, K2, 1, 0, 0, 0, 0);
+    CHECK(need > 0);
+    std::vector<uint16_t> a2((size_t)M2 * K2), w2((size_t)N2 * K2), o1((size_t)M2 * N2), o2((size_t)M2 * N2);
+    for (auto& v : a2) v = f2h_small_int(rnd() % 2);
+    for (auto& v : w2) v = f2h_small_int(rnd() % 2);
+    uint16_t *da2, *dw2, *do1, *do2;
+    void* ws;
+    CHECK(hipMalloc((void**)&da2, a2.size() * 2) == 0 && hipMalloc((void**)&dw2, w2.size() * 2) == 0 &&
+          hipMalloc((void**)&do1, o1.size() * 2) == 0 && hipMalloc((void**)&do2, o2.size() * 2) == 0 &&
+          hipMalloc(&ws, (size_t)need) == 0);
+    hipMemcpy(da2, a2.data(), a2.size() * 2, 1); hipMemcpy(dw2, w2.data(), w2.size() * 2, 1);
+    GpuKernels with_ws(nullptr, ws, need);
+    TensorView<f16> ov1(do1, TensorLayout::row_major({(size_t)M2, (size_t)N2}));
+    TensorView<f16> ov2(do2, TensorLayout::row_major({(size_t)M2, (size_t)N2}));
+    TensorView<const f16> lv2(da2, TensorLayout::row_major({(size_t)M2, (size_t)K2}));
+    TensorView<const f16> wv2(dw2, TensorLayout::row_major({(size_t)N2, (size_t)K2}));
+    gk.matmul_f16(ov1, lv2, wv2.permute({1, 0}), MatmulOptions::make());
+    with_ws.matmul_f16(ov2, lv2, wv2.permute({1, 0}), MatmulOptions::make());
+    CHECK(hipDeviceSynchronize() == 0);
+    hipMemcpy(o1.data(), do1, o1.size() * 2, 2); hipMemcpy(o2.data(), do2, o2.size() * 2, 2);
+    CHECK(o1 == o2);
+    int ref = 0;
+    for (int k = 0; k < K2; k++) ref += h2i(a2[(size_t)7 * K2 + k]) * h2i(w2[(size_t)9 * K2 + k]);
+    CHECK(h2i(o2[(size_t)7 * N2 + 9]) == ref);
+  }
   uint16_t bias = 0;
   CHECK(throws([&] { tr.matmul_f16(ov, lv, wv.permute({1, 0}), MatmulOptions::make().store(MatmulStore::GeluBias(&bias))); }));
 }
