@@ -43,6 +43,49 @@ __global__ __launch_bounds__(256) void mfma_loop_kernel(int times, int pattern, 
   sink[id] = s;
 }
 
+// The same count of instructions as a GEMM's inner loop issues them: 2 x 2 sub-tiles, every
+// instruction with another pair of operands, and the operands themselves replaced after every
+// four instructions (rotated through four random fragments each, in registers: still no memory
+// traffic at all).  What the matrix pipe sustains when its inputs switch like a product's do.
+__global__ __launch_bounds__(256) void mfma_rotating_kernel(int times, float* sink) {
+  const uint32_t id = blockIdx.x * 256 + threadIdx.x;
+  half8_t a[4], b[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++)
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      uint32_t h = (id * 64 + i * 8 + e) * 2654435761u;
+      h ^= h >> 15; h *= 2246822519u; h ^= h >> 13;
+      a[i][e] = bits_to_half((uint16_t)((h & 0x83ffu) | 0x3800u));
+      b[i][e] = bits_to_half((uint16_t)(((h >> 16) & 0x83ffu) | 0x3800u));
+    }
+  float16_t acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+  for (int t = 0; t < times; t++) {
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+      for (int j = 0; j < 2; j++)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b[j], a[i], acc[i][j], 0, 0, 0);
+    const half8_t ta = a[0], tb = b[0];
+    a[0] = a[1]; a[1] = a[2]; a[2] = a[3]; a[3] = ta;
+    b[0] = b[1]; b[1] = b[2]; b[2] = b[3]; b[3] = tb;
+  }
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) s += acc[i][j][r];
+  sink[id] = s;
+}
+
 // Every workgroup reads one contiguous piece with 16-byte streaming loads (the access shape
 // that reads fastest on this part), four loads in flight per lane.
 __global__ __launch_bounds__(256) void stream_read_kernel(const u32x4_t* p, int64_t n16,
@@ -71,7 +114,10 @@ hipError_t launch_microbench_empty(hipStream_t stream) {
 }
 
 hipError_t launch_microbench_mfma(hipStream_t stream, int blocks, int times, int pattern, float* sink) {
-  hipLaunchKernelGGL(mfma_loop_kernel, dim3(blocks), dim3(256), 0, stream, times, pattern, sink);
+  if (pattern == 2)
+    hipLaunchKernelGGL(mfma_rotating_kernel, dim3(blocks), dim3(256), 0, stream, times, sink);
+  else
+    hipLaunchKernelGGL(mfma_loop_kernel, dim3(blocks), dim3(256), 0, stream, times, pattern, sink);
   return hipGetLastError();
 }
 

@@ -357,7 +357,8 @@ def main():
         blocks, times_ = 512, 20000   # two workgroups of four wavefronts per CU
         sink = torch.zeros(blocks * 256, dtype=torch.float32, device=dev)
         flop = blocks * 4 * times_ * 4 * 2 * 32 * 32 * 16
-        for pattern, nm in ((0, "mfma_loop_f32_f16 (zero operands)"), (1, "mfma_loop_f32_f16 (random operands)")):
+        for pattern, nm in ((0, "mfma_loop_f32_f16 (zero operands)"), (1, "mfma_loop_f32_f16 (random operands)"),
+                            (2, "mfma_loop_f32_f16 (random operands, changing with every instruction)")):
             rows.append(run(nm, flop, lambda: ok(lib.adr_microbench_mfma_f16(
                 stream(), blocks, times_, pattern, sink.data_ptr())), "TFLOP/s"))
         nbytes = 1 << 30

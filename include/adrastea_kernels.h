@@ -305,8 +305,10 @@ int adr_matmul_f16_ws_plan(char* name, int32_t cap, int32_t batches, int32_t m, 
  *   adr_microbench_mfma_f16  `blocks` workgroups of four wavefronts, each issuing times x 4
  *                            v_mfma_f32_32x32x16_f16 on register operands: 2*32*32*16 flop each,
  *                            i.e. blocks * 4 * times * 4 * 32768 flop per launch.  pattern 0:
- *                            zero operands, 1: pseudo-random fp16 operands.  `sink` receives
- *                            blocks * 256 floats.
+ *                            zero operands, 1: pseudo-random fp16 operands, 2: pseudo-random
+ *                            operands that change with every instruction as in a product's
+ *                            inner loop (2 x 2 sub-tiles, fragments rotated in registers).
+ *                            `sink` receives blocks * 256 floats.
  *   adr_microbench_stream_read  reads `bytes` (a multiple of 16 * blocks) from `src` with
  *                            `blocks` workgroups, one contiguous piece each; `sink`: 4 bytes.
  */

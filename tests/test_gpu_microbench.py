@@ -18,7 +18,7 @@ def test_empty_and_argument_checks():
     assert L.adr_microbench_empty(stream()) == 0
     sink = torch.zeros(256, device="cuda")
     assert L.adr_microbench_mfma_f16(stream(), 0, 1, 0, sink.data_ptr()) == _ffi.ADR_EINVAL_SHAPE
-    assert L.adr_microbench_mfma_f16(stream(), 1, 1, 2, sink.data_ptr()) == _ffi.ADR_EINVAL_SHAPE
+    assert L.adr_microbench_mfma_f16(stream(), 1, 1, 3, sink.data_ptr()) == _ffi.ADR_EINVAL_SHAPE
     assert L.adr_microbench_mfma_f16(stream(), 1, 1, 0, None) == _ffi.ADR_ENULL
     buf = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
     s32 = torch.zeros(1, dtype=torch.int32, device="cuda")
@@ -44,3 +44,12 @@ def test_mfma_loop_multiplies():
     assert torch.isfinite(one).all() and (one != 0).any()
     # (the matrix core adds the 16 products of a step to the accumulator in its own order)
     assert torch.allclose(two, 2 * one, rtol=1e-4, atol=1e-3)
+    # the loop whose operands change with every instruction: four trips rotate the four fragments
+    # of either operand once around, so eight trips sum every product twice
+    r4 = torch.full((blocks * 256,), -1.0, device="cuda")
+    r8 = torch.full((blocks * 256,), -1.0, device="cuda")
+    assert L.adr_microbench_mfma_f16(stream(), blocks, 4, 2, r4.data_ptr()) == 0
+    assert L.adr_microbench_mfma_f16(stream(), blocks, 8, 2, r8.data_ptr()) == 0
+    torch.cuda.synchronize()
+    assert torch.isfinite(r4).all() and (r4 != 0).any()
+    assert torch.allclose(r8, 2 * r4, rtol=1e-4, atol=1e-3)
