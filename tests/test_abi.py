@@ -128,7 +128,7 @@ def test_no_usable_device_is_an_error_not_a_crash():
 
 
 def test_integration_source_list_matches_the_build():
-    """INTEGRATION.md's build.rs recipe must name every source the library is built from."""
+    """The build.rs recipe of the integration guide must name every source the library is built from."""
     from adrastea_amd import build
     text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
     block = text[text.index("let src = ["):]
