@@ -12,7 +12,8 @@ SYMBOLS = (
     "adr_matmul_f16", "adr_matmul_f16_slow", "adr_matmul_f16_raw", "adr_matmul_nt_f16",
     "adr_matmul_f16_ws", "adr_matmul_f16_workspace_bytes", "adr_matmul_f16_ws_plan",
     "adr_matmul_f16_noalloc",
-    "adr_matmul_nt_fp16u8", "adr_dequantize_absmax_u8", "adr_quantize_absmax_u8",
+    "adr_matmul_nt_fp16u8", "adr_matmul_nt_fp16u8_ws", "adr_matmul_nt_fp16u8_workspace_bytes",
+    "adr_dequantize_absmax_u8", "adr_quantize_absmax_u8",
     "adr_dequantize_absmax_uint8", "adr_quantize_absmax_uint8", "adr_matmul_f16_plan",
     "adr_matmul_nt_fp16u8_plan", "adr_softmax_rows", "adr_error_stats_f16", "adr_error_stats_f32", "adr_attention_f16", "adr_embed_uint8",
     "adr_microbench_empty", "adr_microbench_mfma_f16", "adr_microbench_stream_read",
@@ -60,6 +61,9 @@ def lib():
     L.adr_matmul_f16_raw.argtypes = [vp, vp, vp, vp] + [i32] * 13
     L.adr_matmul_nt_f16.argtypes = [vp, vp, vp, vp, i32, i32, i32, f32]
     L.adr_matmul_nt_fp16u8.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, f32]
+    L.adr_matmul_nt_fp16u8_ws.argtypes = [vp, vp, vp, vp, vp, i32, i32, i32, i32, f32, vp, C.c_int64]
+    L.adr_matmul_nt_fp16u8_workspace_bytes.argtypes = [i32, i32, i32, i32]
+    L.adr_matmul_nt_fp16u8_workspace_bytes.restype = C.c_int64
     L.adr_dequantize_absmax_u8.argtypes = [vp, vp, vp, vp, i32, i32, i32]
     L.adr_quantize_absmax_u8.argtypes = [vp, vp, vp, vp, i32, i32, i32]
     L.adr_dequantize_absmax_uint8.argtypes = [vp, TensorDesc, TensorDesc, TensorDesc]

@@ -315,6 +315,37 @@ int adr_matmul_nt_fp16u8(adr_stream_t stream, uint16_t* output, const uint16_t* 
                              (const half_t*)scales, m, p, n, block_size, beta);
 }
 
+// Where dequantising the matrix once and running the fp16 kernels beats the fused kernels
+// (measured over M 129 .. 4096 on N 4096 / 8192 / 12288, K 4096 and 11008): always on narrow
+// matrices, and on wide ones except where one round of the fused 256-row tiles covers the product
+// (N12288: M512 72 against 81 us, M1024 112 against 120; N8192: M768 72 against 75).
+static bool u8_dequantise_first(int m, int p, int n) {
+  if (m < 129 || p == 0) return false;
+  if (m <= 256 || m >= 1536) return true;
+  return m <= 512 ? n <= 10240 : n < 8192;
+}
+
+int64_t adr_matmul_nt_fp16u8_workspace_bytes(int32_t m, int32_t p, int32_t n, int32_t block_size) {
+  if (m < 0 || p < 0 || n < 0 || block_size <= 0) return ADR_EINVAL_SHAPE;
+  if (p % block_size != 0) return ADR_EDIVISIBILITY;
+  return u8_dequantise_first(m, p, n) ? (int64_t)n * p * 2 : 0;
+}
+
+int adr_matmul_nt_fp16u8_ws(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
+                            const uint8_t* rhs, const uint16_t* scales, int32_t m, int32_t p,
+                            int32_t n, int32_t block_size, float beta, void* workspace,
+                            int64_t workspace_bytes) {
+  if (workspace_bytes < 0 || (workspace_bytes > 0 && !workspace)) return ADR_ENULL;
+  if ((uintptr_t)workspace % 16 != 0) return ADR_EINVAL_SHAPE;
+  if (m < 0 || p < 0 || n < 0 || block_size <= 0) return ADR_EINVAL_SHAPE;
+  if (p % block_size != 0) return ADR_EDIVISIBILITY;
+  if (!u8_dequantise_first(m, p, n) || workspace_bytes < (int64_t)n * p * 2)
+    return adr_matmul_nt_fp16u8(stream, output, lhs, rhs, scales, m, p, n, block_size, beta);
+  if (!output || !lhs || !rhs || !scales) return ADR_ENULL;
+  if (int rc = adr_dequantize_absmax_u8(stream, (uint16_t*)workspace, rhs, scales, n, p, block_size)) return rc;
+  return adr_matmul_nt_f16(stream, output, lhs, (const uint16_t*)workspace, m, p, n, beta);
+}
+
 int adr_matmul_nt_fp16u8_plan(char* name, int32_t cap, int32_t m, int32_t p, int32_t n,
                               int32_t block_size) {
   if (m < 0 || p < 0 || n < 0 || block_size <= 0) return ADR_EINVAL_SHAPE;

@@ -281,9 +281,17 @@ class GpuKernels(CommonKernels):
         assert rhs_q.shape[1] == p and tuple(output.shape) == (m, n)
         assert tuple(scales.shape) == (n, p // block_size)
         assert all(t.is_contiguous() for t in (output, lhs, rhs_q, scales))
-        rc = self._lib.adr_matmul_nt_fp16u8(_current_stream(), output.data_ptr(), lhs.data_ptr(),
-                                            rhs_q.data_ptr(), scales.data_ptr(), m, p, n,
-                                            block_size, beta)
+        if self._workspace is None:
+            rc = self._lib.adr_matmul_nt_fp16u8(_current_stream(), output.data_ptr(), lhs.data_ptr(),
+                                                rhs_q.data_ptr(), scales.data_ptr(), m, p, n,
+                                                block_size, beta)
+        else:
+            # with a workspace of n * p * 2 bytes or more, products of 129 rows and more may
+            # dequantise the matrix once and run the fp16 kernels (same bits, less time)
+            rc = self._lib.adr_matmul_nt_fp16u8_ws(_current_stream(), output.data_ptr(), lhs.data_ptr(),
+                                                   rhs_q.data_ptr(), scales.data_ptr(), m, p, n,
+                                                   block_size, beta, self._workspace.data_ptr(),
+                                                   self._workspace.numel())
         if rc != 0:
             raise AdrasteaError(rc, "matmul_nt_fp16u8")
 

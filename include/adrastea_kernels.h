@@ -175,6 +175,24 @@ int adr_matmul_nt_fp16u8(adr_stream_t stream, uint16_t* output, const uint16_t* 
                          int32_t n, int32_t block_size, float beta);
 
 /*
+ * adr_matmul_nt_fp16u8 with a caller-provided workspace (no counterpart in the reference).  From
+ * 129 activation rows on, dequantising the weight matrix once into `workspace` (n * p fp16
+ * values, bit-identical to dequantize_absmax_uint8) and running the fp16 kernels on it is
+ * faster than dequantising every weight once per 256-row tile inside the GEMM: M2048 K4096 N12288
+ * 232 -> 211 us, M512 K11008 N4096 140 -> 88 us, and the result has the same bits.  Fewer rows, or
+ * a few hundred to 1535 rows against a wide matrix (where one round of the fused kernel's tiles
+ * covers the product and it is ahead), or a workspace smaller than
+ * adr_matmul_nt_fp16u8_workspace_bytes reports: exactly adr_matmul_nt_fp16u8.  The workspace (16-byte aligned, device memory) is written by the call
+ * and holds nothing afterwards; calls sharing one must not overlap in time.
+ */
+int adr_matmul_nt_fp16u8_ws(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
+                            const uint8_t* rhs, const uint16_t* scales, int32_t m, int32_t p,
+                            int32_t n, int32_t block_size, float beta, void* workspace,
+                            int64_t workspace_bytes);
+/* Bytes (>= 0; 0: the workspace would not be used) or a negative ADR_E* code. */
+int64_t adr_matmul_nt_fp16u8_workspace_bytes(int32_t m, int32_t p, int32_t n, int32_t block_size);
+
+/*
  * Flat-pointer forms of `dequantize_absmax_uint8` / `quantize_absmax_uint8`
  * (adrastea_kernels/cpp/quantize.cu:46-56 and :3-44) for contiguous [rows, cols] tensors with
  * scales [rows, cols / block_size]:

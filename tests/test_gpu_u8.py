@@ -503,3 +503,43 @@ def test_descriptor_forms_on_strided_views(kern):
     # shape errors
     bad = TensorView(sb, TensorLayout((rows + 1, cols // bs), (cols // bs + 3, 1)))
     assert lib.adr_dequantize_absmax_uint8(None, descriptor(ov), descriptor(bad), descriptor(qv)) == -1
+
+
+@pytest.mark.parametrize("shape", [(129, 4096, 4096), (300, 1024, 8200), (512, 11008, 4096), (1024, 4096, 4096),
+                                   (1100, 448, 12288), (2048, 4096, 12288), (1700, 640, 9000), (128, 4096, 4096)])
+@pytest.mark.parametrize("beta", [0.0, 1.0])
+def test_workspace_variant_gives_the_bits_of_the_fused_call(shape, beta):
+    """adr_matmul_nt_fp16u8_ws (weights dequantised once into the workspace, then the fp16
+    kernels) against adr_matmul_nt_fp16u8 on the same operands: both round every weight to fp16
+    with the reference's dequantisation and sum slices of K in the same order -- the outputs are
+    compared bit for bit, with the previous output added and without, in the regimes where the
+    workspace is used and where it is not (128 rows; 1100 rows against 12288 weight rows)."""
+    m, p, n = shape
+    lib = _ffi.lib()
+    gen = torch.Generator(device="cuda").manual_seed(m + p + n)
+    q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)
+    s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
+    a = torch.randn(m, p, generator=gen, device="cuda").half()
+    prev = torch.randn(m, n, generator=gen, device="cuda").half()
+    need = lib.adr_matmul_nt_fp16u8_workspace_bytes(m, p, n, 32)
+    assert need in (0, n * p * 2)
+    ws = torch.full((max(need, 16),), 0x7f, dtype=torch.uint8, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    want, got = prev.clone(), prev.clone()
+    assert lib.adr_matmul_nt_fp16u8(st, want.data_ptr(), a.data_ptr(), q.data_ptr(), s.data_ptr(), m, p, n, 32, beta) == 0
+    assert lib.adr_matmul_nt_fp16u8_ws(st, got.data_ptr(), a.data_ptr(), q.data_ptr(), s.data_ptr(), m, p, n, 32,
+                                       beta, ws.data_ptr(), ws.numel()) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    if need:
+        # the workspace held the dequantised matrix, bit-identical to the stand-alone kernel
+        w = torch.empty(n, p, dtype=torch.float16, device="cuda")
+        assert lib.adr_dequantize_absmax_u8(st, w.data_ptr(), q.data_ptr(), s.data_ptr(), n, p, 32) == 0
+        assert torch.equal(ws[:need].view(torch.float16).view(n, p), w)
+        # too small a workspace: the fused call, same bits again
+        again = prev.clone()
+        assert lib.adr_matmul_nt_fp16u8_ws(st, again.data_ptr(), a.data_ptr(), q.data_ptr(), s.data_ptr(), m, p, n,
+                                           32, beta, ws.data_ptr(), need - 16) == 0
+        assert torch.equal(again.view(torch.int16), want.view(torch.int16))
+    else:
+        assert torch.all(ws == 0x7f)   # untouched
