@@ -316,11 +316,15 @@ int adr_matmul_nt_fp16u8(adr_stream_t stream, uint16_t* output, const uint16_t* 
 }
 
 // Where dequantising the matrix once and running the fp16 kernels beats the fused kernels
-// (measured over M 129 .. 4096 on N 4096 / 8192 / 12288, K 4096 and 11008): always on narrow
+// (measured over M 33 .. 4096 on N 4096 / 8192 / 12288, K 4096 and 11008): always on narrow
 // matrices, and on wide ones except where one round of the fused 256-row tiles covers the product
 // (N12288: M512 72 against 81 us, M1024 112 against 120; N8192: M768 72 against 75).
 static bool u8_dequantise_first(int m, int p, int n) {
-  if (m < 129 || p == 0) return false;
+  if (m < 65 || p == 0) return false;  // (to 64 rows the streaming kernels read the bytes once)
+  // 65 .. 128 rows: the fused path runs sixteen rows per pass or a few large tiles (K11008 N4096
+  // M128 112 against 62 us, K4096 N12288 M65 61 against 48); on a matrix of 16 M weights or fewer
+  // its passes are short enough to stay ahead up to about 110 rows (K4096 N4096 M96 25 against 28)
+  if (m < 129) return (int64_t)n * p > ((int64_t)1 << 24) || m >= 112;
   if (m <= 256 || m >= 1536) return true;
   return m <= 512 ? n <= 10240 : n < 8192;
 }

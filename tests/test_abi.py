@@ -166,7 +166,7 @@ def test_workspace_plan_and_size():
 
 
 def test_u8_workspace_size_and_validation():
-    """adr_matmul_nt_fp16u8_ws dequantises the matrix first from 129 rows on (not where one round
+    """adr_matmul_nt_fp16u8_ws dequantises the matrix first from 65 rows on (not where one round
     of the fused kernel's tiles covers a wide product); the size query says when, and how much."""
     lib = _ffi.lib()
     need = lib.adr_matmul_nt_fp16u8_workspace_bytes
@@ -176,7 +176,9 @@ def test_u8_workspace_size_and_validation():
     assert need(1024, 4096, 12288, 32) == 0        # the fused 256-row tiles are ahead here
     assert need(512, 4096, 12288, 32) == 0 and need(512, 4096, 8192, 32) == 8192 * 4096 * 2
     assert need(1024, 4096, 8192, 32) == 0 and need(256, 4096, 12288, 32) == 12288 * 4096 * 2
-    assert need(128, 4096, 4096, 32) == 0 and need(1, 4096, 12288, 32) == 0
+    assert need(64, 11008, 4096, 32) == 0 and need(1, 4096, 12288, 32) == 0
+    assert need(65, 11008, 4096, 32) == 4096 * 11008 * 2 and need(65, 4096, 12288, 32) == 12288 * 4096 * 2
+    assert need(96, 4096, 4096, 32) == 0 and need(128, 4096, 4096, 32) == 4096 * 4096 * 2
     assert need(2048, 0, 64, 32) == 0
     assert need(-1, 64, 64, 32) == _ffi.ADR_EINVAL_SHAPE
     assert need(256, 100, 64, 32) == _ffi.ADR_EDIVISIBILITY
