@@ -125,7 +125,7 @@ int64_t adr_matmul_f16_workspace_bytes(int32_t batches, int32_t m, int32_t k, in
  * serving loops, harnesses that forbid hipMalloc.  The scratch is a fixed array of
  * ADR_NOALLOC_SCRATCH_BYTES inside the library's device code, one copy per GPU the library runs
  * on, held until the process ends; the entry point allocates and frees nothing (its first call
- * on a device looks the array's address up once).  Same arguments, validation and result as
+ * on a device looks the array's address up once: make that call before a graph capture begins).  Same arguments, validation and result as
  * adr_matmul_f16_ws given a workspace of at least adr_matmul_f16_workspace_bytes bytes.
  * A product that would use more than ADR_NOALLOC_SCRATCH_BYTES (16 MiB: the LLaMA-7B down
  * projection up to 256 rows fits) returns ADR_ESCRATCH and launches nothing.

@@ -88,3 +88,37 @@ def test_noalloc_size_limit_and_products_without_scratch():
                                       64, 1, 0, None, 0.0, 1.0, 0, 0, 0) == _ffi.ADR_ENULL
     assert lib.adr_matmul_f16_noalloc(None, got.data_ptr(), a.data_ptr(), w.data_ptr(), 1, 4, 64, 64, 1, 64, 0,
                                       1, 64, 0, 64, 1, 0, None, 0.0, 1.0, 1, 0, 0) == _ffi.ADR_ENOTIMPL
+
+
+def test_noalloc_in_a_captured_graph():
+    """What the entry point is for: a split product (partial tiles in the built-in scratch, then
+    the reduction launch) recorded into a HIP graph and replayed, with eager calls that use the
+    same scratch for another product and synchronisations between the replays; every replay
+    reproduces the eager result bit for bit.  (The first call on a device, which looks the
+    scratch address up, is made before the capture.)"""
+    K, N, M = 11008, 4096, 200
+    gen = torch.Generator(device="cuda").manual_seed(93)
+    w = (torch.randn(N, K, generator=gen, device="cuda") * K ** -0.5).half()
+    a = torch.randn(M, K, generator=gen, device="cuda").half()
+    a2 = torch.randn(96, K, generator=gen, device="cuda").half()
+    out = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+    other = torch.zeros(96, N, dtype=torch.float16, device="cuda")
+    so, sl, sr = nt(M, K, N)
+    assert _ffi.lib().adr_matmul_f16_workspace_bytes(1, M, K, N, *so, *sl, *sr, 0, 0, 0) > 0
+    assert call("adr_matmul_f16_noalloc", out, a, w, M, K, N) == 0
+    torch.cuda.synchronize()
+    want = out.clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            assert call("adr_matmul_f16_noalloc", out, a, w, M, K, N) == 0
+    torch.cuda.current_stream().wait_stream(side)
+    for _ in range(3):
+        out.zero_()
+        assert call("adr_matmul_f16_noalloc", other, a2, w, 96, K, N) == 0   # dirties the scratch
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want)
