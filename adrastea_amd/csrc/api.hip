@@ -320,11 +320,11 @@ int adr_matmul_nt_fp16u8(adr_stream_t stream, uint16_t* output, const uint16_t* 
 // matrices, and on wide ones except where one round of the fused 256-row tiles covers the product
 // (N12288: M512 72 against 81 us, M1024 112 against 120; N8192: M768 72 against 75).
 static bool u8_dequantise_first(int m, int p, int n) {
-  if (m < 65 || p == 0) return false;  // (to 64 rows the streaming kernels read the bytes once)
-  // 65 .. 128 rows: the fused path runs sixteen rows per pass or a few large tiles (K11008 N4096
-  // M128 112 against 62 us, K4096 N12288 M65 61 against 48); on a matrix of 16 M weights or fewer
-  // its passes are short enough to stay ahead up to about 110 rows (K4096 N4096 M96 25 against 28)
-  if (m < 129) return (int64_t)n * p > ((int64_t)1 << 24) || m >= 112;
+  // To 95 rows the streaming kernels, which read the bytes once per 64 rows, stay ahead; to 159
+  // rows they still do on narrow matrices (K11008 N4096 M128 53 against 62 us, K4096 N4096 26
+  // against 28) but not on wide ones (K4096 N12288 M96 54 against 49, N8192 M128 46 against 37).
+  if (m < 96 || p == 0) return false;
+  if (m < 160) return n >= 8192;
   if (m <= 256 || m >= 1536) return true;
   return m <= 512 ? n <= 10240 : n < 8192;
 }

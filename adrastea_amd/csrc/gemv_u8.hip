@@ -357,6 +357,182 @@ __global__ __launch_bounds__(512) void gemv_u8_regstream_kernel(half_t* __restri
   }
 }
 
+// 17 to 64 activation rows, block size 32, any K % 256 == 0: the request pipeline of the kernel
+// above with MB blocks of sixteen activation rows per workgroup, so that the weights are read
+// once for all of them.  With two blocks and more the per-block correction term of the kernel
+// above would not fit the register file; the VALU work that trick saves is small beside the
+// time the bytes take anyway, so here every weight is dequantised to fp16 exactly as
+// dequantize_absmax_uint8 does (dequant8, the formula of the reference's WMMA kernel, as in the
+// tiled u8 GEMM) and v_mfma_f32_16x16x32_f16 accumulates straight into the result.  A macro
+// step is 256 k: two tiles of activations per block (k 0..127 and 128..255) and RG tiles of
+// weights.  It is walked in two halves so that only one half's activation operands (16
+// registers per block) are live: the weight tiles stay in the wavefront's LDS slots, one per
+// row group, between the halves.  Request order per step = consumption order: the blocks' first
+// tiles, the weight tiles, the blocks' second tiles.
+template <int RG, int MB>
+__global__ __launch_bounds__(512) void gemv_u8_blocks_kernel(half_t* __restrict__ out,
+                                                             const half_t* __restrict__ lhs,
+                                                             const uint8_t* __restrict__ rhs,
+                                                             const half_t* __restrict__ scales,
+                                                             int m, int p, int n, float beta) {
+  constexpr int NW = 8, TILE = ROWS * MACRO_K, RB = ROWS * RG, PER = 2 * MB + RG;
+  constexpr int DIST = 3;  // tiles between a request and its use
+  static_assert(PER > DIST, "a step holds more tiles than are in flight");
+  // per wavefront: slot 0 for activation tiles, slots 1 .. RG for the step's weight tiles
+  __shared__ __attribute__((aligned(1024))) unsigned char shuf[NW][RG + 1][TILE];
+  static_assert(NW * MB * RG * 256 * 4 <= NW * (RG + 1) * TILE, "the partial sums reuse the tiles");
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int a = lane >> 4, x = lane & 15;  // request role: quarter a takes row 4i + a, chunk x
+  const int r = lane & 15, g = lane >> 4;  // operand role: row r, k-group g of a block of 32
+  const int n0 = blockIdx.x * RB;
+  const int nblk = p / 32, steps = p / MACRO_K, last = steps - 1;
+  unsigned char* const mine = shuf[wave][0];
+
+  // scales of a step: the eight blocks of row q * 16 + r (16 bytes), requested a whole step ahead
+  uint32_t so[RG];
+#pragma unroll
+  for (int q = 0; q < RG; q++) so[q] = (uint32_t)min(q * ROWS + r, n - 1 - n0) * (uint32_t)nblk * 2u;
+  const unsigned char* const sbase = (const unsigned char*)(scales + (int64_t)n0 * nblk);
+  u32x4_t sc[RG], sc_next[RG];
+#pragma unroll
+  for (int q = 0; q < RG; q++) sc[q] = *(const u32x4_t*)(sbase + min(wave, last) * 16 + so[q]);
+  // request addresses: a uniform base per step plus a 32-bit byte offset per lane and instruction
+  // (rows beyond m read row m - 1 again, rows beyond n row n - 1: their products are never stored)
+  uint32_t xo[MB][4], wo[RG][4];
+#pragma unroll
+  for (int b = 0; b < MB; b++)
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      xo[b][i] = (uint32_t)min(b * ROWS + 4 * i + a, m - 1) * (uint32_t)p * 2u + x * 16;
+#pragma unroll
+  for (int q = 0; q < RG; q++)
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      wo[q][i] = (uint32_t)min(q * ROWS + 4 * i + a, n - 1 - n0) * (uint32_t)p + x * 16;
+  const unsigned char* const xbase = (const unsigned char*)lhs;
+  const unsigned char* const wbase = rhs + (int64_t)n0 * p;
+  u32x4_t ld[PER][4];
+  // tile u of a step: u < MB: first half of block u; u < MB + RG: weight group u - MB; else the
+  // second half of block u - MB - RG
+  auto request = [&](int ms, int u) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      if (u < MB)
+        ld[u][i] = *(const u32x4_t*)(xbase + (int64_t)ms * (MACRO_K * 2) + xo[u][i]);
+      else if (u < MB + RG)  // streaming load: a weight byte is read once per launch
+        ld[u][i] = __builtin_nontemporal_load(
+            (const u32x4_t*)(wbase + (int64_t)ms * MACRO_K + wo[u - MB][i]));
+      else
+        ld[u][i] = *(const u32x4_t*)(xbase + (int64_t)ms * (MACRO_K * 2) + 256 + xo[u - MB - RG][i]);
+    }
+  };
+#pragma unroll
+  for (int u = 0; u < DIST; u++) request(min(wave, last), u);
+
+  int woff[4], roff[8], xoff[4];
+#pragma unroll
+  for (int i = 0; i < 4; i++) woff[i] = (4 * i + a) * 256 + ((x ^ (4 * i + a)) << 4);
+  // weights of block b = bytes 32 b .. 32 b + 31 of the row: lane (r, g) takes bytes 8 g .. 8 g + 7
+#pragma unroll
+  for (int b = 0; b < 8; b++) roff[b] = r * 256 + (((2 * b + (g >> 1)) ^ r) << 4) + (g & 1) * 8;
+  // activations of block b of a half = chunks 4 b .. 4 b + 3 of the tile: chunk 4 b + g
+#pragma unroll
+  for (int b = 0; b < 4; b++) xoff[b] = r * 256 + (((4 * b + g) ^ r) << 4);
+
+  float4_t acc[MB][RG];
+#pragma unroll
+  for (int b = 0; b < MB; b++)
+#pragma unroll
+    for (int q = 0; q < RG; q++) acc[b][q] = float4_t{0, 0, 0, 0};
+  half8_t xf[MB][4];  // activation operands of the current half: four blocks of 32 k
+
+  // the weight operands of half h of row group q, from its LDS slot, against every block
+  auto multiply = [&](int q, int h) {
+    const unsigned char* slot = shuf[wave][1 + q];
+    const half8_t s8 = __builtin_bit_cast(half8_t, sc[q]);
+    u32x2_t w[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) w[j] = *(const u32x2_t*)(slot + roff[4 * h + j]);
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const half2_t s2 = {s8[4 * h + j], s8[4 * h + j]};
+      const half8_t wf = dequant8(w[j][0], w[j][1], s2);
+#pragma unroll
+      for (int b = 0; b < MB; b++)
+        acc[b][q] = __builtin_amdgcn_mfma_f32_16x16x32_f16(wf, xf[b][j], acc[b][q], 0, 0, 0);
+    }
+  };
+
+#pragma unroll 1
+  for (int ms = wave; ms < steps; ms += NW) {
+    const int ms_next = min(ms + NW, last);  // (past the end: the last step again, never used)
+#pragma unroll
+    for (int u = 0; u < PER; u++) {
+      __builtin_amdgcn_sched_barrier(0);
+      if (u + DIST < PER) request(ms, u + DIST); else request(ms_next, u + DIST - PER);
+      if (u == 0) {
+#pragma unroll
+        for (int q = 0; q < RG; q++) sc_next[q] = *(const u32x4_t*)(sbase + ms_next * 16 + so[q]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      const bool weights = u >= MB && u < MB + RG;
+      unsigned char* dst = weights ? shuf[wave][1 + (u - MB)] : mine;
+#pragma unroll
+      for (int i = 0; i < 4; i++) *(u32x4_t*)(dst + woff[i]) = ld[u][i];
+      if (!weights) {
+        const int b = u < MB ? u : u - MB - RG;
+#pragma unroll
+        for (int j = 0; j < 4; j++) xf[b][j] = *(const half8_t*)(mine + xoff[j]);
+      }
+      if (u == MB + RG - 1) {  // all of the step's weights and the first halves are in: half 0
+#pragma unroll
+        for (int q = 0; q < RG; q++) multiply(q, 0);
+      }
+      if (u == PER - 1) {      // the second halves are in: half 1
+#pragma unroll
+        for (int q = 0; q < RG; q++) multiply(q, 1);
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < RG; q++) sc[q] = sc_next[q];
+  }
+
+  // lane (r, g): acc[b][q][v] is weight row 4g + v of group q against activation row r of block b
+  // (not __syncthreads(): its fence would wait for the surplus requests of the last step)
+  __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wavefront's tiles are dead
+  __builtin_amdgcn_s_barrier();        // ... and everybody else's
+  float* const partial = (float*)&shuf[0][0][0];  // [NW][MB][RG][256]
+#pragma unroll
+  for (int b = 0; b < MB; b++)
+#pragma unroll
+    for (int q = 0; q < RG; q++)
+#pragma unroll
+      for (int v = 0; v < 4; v++)
+        partial[((wave * MB + b) * RG + q) * 256 + (4 * g + v) * 16 + r] = acc[b][q][v];
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  __builtin_amdgcn_s_barrier();
+  for (int e = tid; e < MB * RG * 256; e += NW * 64) {
+    const int col = e % RB, y = e / RB;  // consecutive threads -> consecutive columns
+    if (y >= m || n0 + col >= n) continue;
+    float sum = 0.0f;
+#pragma unroll
+    for (int w2 = 0; w2 < NW; w2++)
+      sum += partial[((w2 * MB + y / 16) * RG + col / 16) * 256 + (col % 16) * 16 + y % 16];
+    half_t* o = out + (int64_t)y * n + n0 + col;
+    // the previous output is read even for beta == 0, as the reference does
+    *o = (half_t)(sum + beta * (float)*o);
+  }
+}
+
+template <int RG, int MB>
+hipError_t launch_blocks(hipStream_t stream, half_t* out, const half_t* lhs, const uint8_t* rhs,
+                         const half_t* scales, int m, int p, int n, float beta) {
+  hipLaunchKernelGGL((gemv_u8_blocks_kernel<RG, MB>), dim3((n + ROWS * RG - 1) / (ROWS * RG)), dim3(512), 0,
+                     stream, out, lhs, rhs, scales, m, p, n, beta);
+  return hipGetLastError();
+}
+
 template <int RG>
 hipError_t launch_regstream(hipStream_t stream, half_t* out, const half_t* lhs, const uint8_t* rhs,
                             const half_t* scales, int m, int p, int n, float beta) {
@@ -540,14 +716,28 @@ U8Choice choose_u8(const void* lhs, const void* rhs, const void* scales, int m, 
   return U8_NAIVE;
 }
 
-// 17 to 64 activation rows (to 128 on matrices under 8192 rows) against at least 4 MiB of
-// weights: the sixteen-row kernels once per block of rows.  The tiled GEMM walks K on
-// N / 64 .. N / 128 CUs for these (K4096 N4096 m=17..32 42.9 us, m=64..128 58.5; N12288 53.4 ..
-// 68.5; K11008 N4096 133 .. 171) where a sixteen-row launch takes 7 / 14 / 15 us (N12288
-// m=96: 78.4 us in blocks against 68.3 tiled, hence the narrower bound there).
-bool rows_in_blocks_of_16(int m, int p, int n, int block_size) {
-  return m > 16 && m <= (n < 8192 ? 128 : 64) && (int64_t)n * p >= (1 << 22) &&
-         choose_u8(nullptr, nullptr, nullptr, 16, p, n, block_size) == U8_GEMV;
+// 17 activation rows and more against at least 4 MiB of weights: passes of up to 64 rows on the
+// matrix-core streaming kernels, each pass reading the weights once.  The tiled GEMM walks K on
+// N / 64 .. N / 128 CUs for these row counts, which takes about 10 + 0.0105 K us whatever the
+// rows (K4096 N4096 m=65..256: 49.6 .. 52.3 us, K11008 N4096 127 .. 132, K512 N9000 15.4; ten more
+// on N 12288).  A pass of 64 rows is one workgroup per sixteen weight rows, 2 + 0.0023 K us per
+// round of them over the CUs (K4096 N4096 13.1 us, N8192 23.5, N12288 33.9, K11008 N4096 26.4,
+// K5120 N5120 25.7); a last pass of r rows costs 0.55 + 0.45 r / 64 of that.  Up to 64 rows the
+// passes always win; above, where this estimate says so (measured: K4096 N4096 to 256 rows,
+// 25.7 us at m=128 against 49.6; K11008 N4096 m=256 105 against 132; K4096 N12288 to 96 rows, 54
+// against 63; K4096 N8192 and K5120 N5120 to 128, 46 against 53 and 51 against 64).
+bool rows_in_passes(int m, int p, int n, int block_size) {
+  if (m <= 16 || m > 256 || (int64_t)n * p < (1 << 22) ||
+      choose_u8(nullptr, nullptr, nullptr, 16, p, n, block_size) != U8_GEMV)
+    return false;
+  if (m <= 64) return true;
+  const int cus = device_info_for_plan().cus;
+  const int rounds = ((n + ROWS - 1) / ROWS + cus - 1) / cus;
+  const double t64 = fmax(12.0, rounds * (2.0 + 0.0023 * p));
+  const int rem = m % 64;
+  const double passes = (m / 64) * t64 + (rem ? t64 * (0.55 + 0.45 * rem / 64.0) : 0.0);
+  const double tiled = 10.0 + 0.0105 * p + (n > 10240 ? 10.0 : 0.0);
+  return passes < tiled;
 }
 
 }  // namespace
@@ -560,8 +750,8 @@ bool gemm_u8_mfma_supported(const half_t* lhs, const uint8_t* rhs, const half_t*
                             int n, int block_size);
 
 const char* gemm_u8_plan(int m, int p, int n, int block_size) {
-  if (rows_in_blocks_of_16(m, p, n, block_size))
-    return p == 16 * MACRO_K ? "gemv_u8_mfma16_dma_32rows" : "gemv_u8_mfma16_regstream";
+  if (rows_in_passes(m, p, n, block_size))
+    return m <= 32 && p == 16 * MACRO_K ? "gemv_u8_mfma16_dma_32rows" : "gemv_u8_mfma16_blocks";
   switch (choose_u8(nullptr, nullptr, nullptr, m, p, n, block_size)) {
     case U8_DOT: return "gemv_u8_dot2_stream";
     case U8_GEMV: return "gemv_u8_mfma16_regstream";
@@ -576,18 +766,24 @@ const char* gemm_u8_plan(int m, int p, int n, int block_size) {
 
 hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, const uint8_t* rhs,
                           const half_t* scales, int m, int p, int n, int block_size, float beta) {
-  if (rows_in_blocks_of_16(m, p, n, block_size) &&
+  if (rows_in_passes(m, p, n, block_size) &&
       choose_u8(lhs, rhs, scales, 16, p, n, block_size) == U8_GEMV) {
-    // (p is a multiple of 256 here, so every block of rows starts 16-byte aligned)
-    // K 4096: blocks of 32 rows on the ring kernel with two blocks of activations (m=32: N4096
-    // 13.3 -> 8.8 us, N12288 27.5 -> 18.4; m=64: 25.1 -> 16.8, 52.9 -> 34.9)
-    const int step = p == 16 * MACRO_K ? 32 : 16;
-    for (int r0 = 0; r0 < m; r0 += step) {
-      const int mb = min(step, m - r0);
+    // 17 rows and more against 4 MiB of weights and more: passes of up to 64 rows, each reading
+    // the weights once for two to four blocks of sixteen rows (p is a multiple of 256 here, so
+    // every pass starts 16-byte aligned).  Row groups per workgroup as the register file allows:
+    // three with two blocks, two with three, one with four.  K11008 N4096 m=32 / 64 / 128:
+    // 28.5 / 55.1 / 112 us in passes of sixteen rows -> 19.0 / 26.4 / 53.
+    const int rg = regstream_row_groups(n);
+    for (int r0 = 0; r0 < m; r0 += 64) {
+      const int mb = min(64, m - r0);
       half_t* o = out + (int64_t)r0 * n;
       const half_t* l = lhs + (int64_t)r0 * p;
       hipError_t e;
-      if (mb > 16) {
+      if (mb <= 16) {
+        e = launch_gemm_u8(stream, o, l, rhs, scales, mb, p, n, block_size, beta);
+      } else if (mb <= 32 && p == 16 * MACRO_K) {
+        // K 4096, up to 32 rows: the DMA-ring kernel with two blocks is 4-10 % ahead (m=32: N4096
+        // 9.6 against 10.0 us, N12288 18.9 against 21.0)
         if (n >= 8192)
           hipLaunchKernelGGL((gemv_u8_ring_kernel<8, 3, 4, 2>), dim3((n + 3 * ROWS - 1) / (3 * ROWS)),
                              dim3(512), 0, stream, o, l, rhs, scales, mb, p, n, beta);
@@ -595,8 +791,15 @@ hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, co
           hipLaunchKernelGGL((gemv_u8_ring_kernel<8, 1, 4, 2>), dim3((n + ROWS - 1) / ROWS), dim3(512),
                              0, stream, o, l, rhs, scales, mb, p, n, beta);
         e = hipGetLastError();
+      } else if (mb <= 32) {
+        e = rg == 3 ? launch_blocks<3, 2>(stream, o, l, rhs, scales, mb, p, n, beta)
+          : rg == 2 ? launch_blocks<2, 2>(stream, o, l, rhs, scales, mb, p, n, beta)
+                    : launch_blocks<1, 2>(stream, o, l, rhs, scales, mb, p, n, beta);
+      } else if (mb <= 48) {
+        e = rg >= 2 ? launch_blocks<2, 3>(stream, o, l, rhs, scales, mb, p, n, beta)
+                    : launch_blocks<1, 3>(stream, o, l, rhs, scales, mb, p, n, beta);
       } else {
-        e = launch_gemm_u8(stream, o, l, rhs, scales, mb, p, n, block_size, beta);
+        e = launch_blocks<1, 4>(stream, o, l, rhs, scales, mb, p, n, beta);
       }
       if (e != hipSuccess) return e;
     }

@@ -176,15 +176,16 @@ int adr_matmul_nt_fp16u8(adr_stream_t stream, uint16_t* output, const uint16_t* 
 
 /*
  * adr_matmul_nt_fp16u8 with a caller-provided workspace (no counterpart in the reference).  From
- * 65 activation rows on (about 112 against a matrix of 16 M weights or fewer), dequantising the weight matrix once into `workspace` (n * p fp16
- * values, bit-identical to dequantize_absmax_uint8) and running the fp16 kernels on it is
- * faster than dequantising every weight once per 256-row tile inside the GEMM: M2048 K4096 N12288
- * 232 -> 211 us, M512 K11008 N4096 140 -> 88 us, and from 129 rows on the result has the same
- * bits (65 .. 128 rows: the fused call evaluates the reference's naive formula on unrounded
- * weights there, this one its WMMA formula; they differ by < 5e-4 relative).  Fewer rows, or
- * a few hundred to 1535 rows against a wide matrix (where one round of the fused kernel's tiles
- * covers the product and it is ahead), or a workspace smaller than
- * adr_matmul_nt_fp16u8_workspace_bytes reports: exactly adr_matmul_nt_fp16u8.  The workspace (16-byte aligned, device memory) is written by the call
+ * 96 activation rows on (160 against fewer than 8192 weight rows), dequantising the weight
+ * matrix once into `workspace` (n * p fp16 values, bit-identical to dequantize_absmax_uint8) and
+ * running the fp16 kernels on it is faster than dequantising every weight once per 256-row tile
+ * inside the GEMM: M2048 K4096 N12288 232 -> 211 us, M512 K11008 N4096 140 -> 88 us.  Both paths
+ * round every weight to fp16 as dequantize_absmax_uint8 does; from 257 rows on (and below
+ * wherever adr_matmul_nt_fp16u8_plan names a gemm_nt_u8_ kernel) they also sum in the same order
+ * and the result has the same bits.  Fewer rows, or a few hundred to 1535 rows against a wide
+ * matrix (where one round of the fused kernel's tiles covers the product and it is ahead), or a
+ * workspace smaller than adr_matmul_nt_fp16u8_workspace_bytes reports: exactly
+ * adr_matmul_nt_fp16u8.  The workspace (16-byte aligned, device memory) is written by the call
  * and holds nothing afterwards; calls sharing one must not overlap in time.
  */
 int adr_matmul_nt_fp16u8_ws(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,

@@ -82,7 +82,14 @@ def test_u8_plan():
     assert plan(2, 4096, 12288, 32) == (0, "gemv_u8_dot2_stream")
     # 17 to 64 rows in blocks of rows: 32 per pass for K = 4096, 16 otherwise
     assert plan(32, 4096, 12288, 32) == (0, "gemv_u8_mfma16_dma_32rows")
-    assert plan(32, 11008, 4096, 32) == (0, "gemv_u8_mfma16_regstream")
+    assert plan(32, 11008, 4096, 32) == (0, "gemv_u8_mfma16_blocks")
+    assert plan(64, 4096, 12288, 32) == (0, "gemv_u8_mfma16_blocks")
+    # above 64 rows: passes of 64 rows where the estimate puts them ahead of the tiled kernels
+    assert plan(256, 11008, 4096, 32) == (0, "gemv_u8_mfma16_blocks")
+    assert plan(96, 4096, 12288, 32) == (0, "gemv_u8_mfma16_blocks")
+    assert plan(128, 4096, 12288, 32)[1].startswith("gemm_nt_u8_")
+    assert plan(100, 512, 9000, 32)[1].startswith("gemm_nt_u8_")
+    assert plan(257, 11008, 4096, 32)[1].startswith("gemm_nt_u8_")
     # tiled kernels: the name carries the tile
     assert plan(2048, 4096, 4096, 32) == (0, "gemm_nt_u8_mfma_256x128x64")
     assert plan(2048, 4096, 12288, 32) == (0, "gemm_nt_u8_mfma_256x192x64")
@@ -166,7 +173,7 @@ def test_workspace_plan_and_size():
 
 
 def test_u8_workspace_size_and_validation():
-    """adr_matmul_nt_fp16u8_ws dequantises the matrix first from 65 rows on (not where one round
+    """adr_matmul_nt_fp16u8_ws dequantises the matrix first from 96 rows on (160 on narrow matrices; not where one round
     of the fused kernel's tiles covers a wide product); the size query says when, and how much."""
     lib = _ffi.lib()
     need = lib.adr_matmul_nt_fp16u8_workspace_bytes
@@ -176,9 +183,9 @@ def test_u8_workspace_size_and_validation():
     assert need(1024, 4096, 12288, 32) == 0        # the fused 256-row tiles are ahead here
     assert need(512, 4096, 12288, 32) == 0 and need(512, 4096, 8192, 32) == 8192 * 4096 * 2
     assert need(1024, 4096, 8192, 32) == 0 and need(256, 4096, 12288, 32) == 12288 * 4096 * 2
-    assert need(64, 11008, 4096, 32) == 0 and need(1, 4096, 12288, 32) == 0
-    assert need(65, 11008, 4096, 32) == 4096 * 11008 * 2 and need(65, 4096, 12288, 32) == 12288 * 4096 * 2
-    assert need(96, 4096, 4096, 32) == 0 and need(128, 4096, 4096, 32) == 4096 * 4096 * 2
+    assert need(95, 4096, 12288, 32) == 0 and need(1, 4096, 12288, 32) == 0
+    assert need(96, 4096, 12288, 32) == 12288 * 4096 * 2 and need(128, 4096, 8192, 32) == 8192 * 4096 * 2
+    assert need(159, 11008, 4096, 32) == 0 and need(160, 11008, 4096, 32) == 4096 * 11008 * 2
     assert need(2048, 0, 64, 32) == 0
     assert need(-1, 64, 64, 32) == _ffi.ADR_EINVAL_SHAPE
     assert need(256, 100, 64, 32) == _ffi.ADR_EDIVISIBILITY

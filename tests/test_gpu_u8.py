@@ -227,6 +227,26 @@ def test_wide_gemv_bit_exact_on_exact_inputs(kern, m, pn):
         assert np.array_equal(to_np(out).view(np.uint16), want.view(np.uint16)), (m, p, n, beta)
 
 
+@pytest.mark.parametrize("m", [17, 31, 32, 33, 48, 50, 64, 70])
+@pytest.mark.parametrize("pn", [(256, 16400), (768, 8200), (2304, 1900), (11008, 400), (4096, 1030)])
+def test_blocks_kernel_bit_exact_on_exact_inputs(kern, m, pn):
+    """Two to four blocks of sixteen activation rows per workgroup: one, two and three groups of
+    weight rows, macro-step counts from one (wavefronts without a step) to 43, ragged rows of
+    both operands, a second pass for rows 65 .. 70, beta path."""
+    p, n = pn
+    g = rng(1700 + m + p)
+    if m <= 64 or p != 768:    # (70 rows on K 768 x N 8200 are estimated faster on the tiled kernel)
+        assert u8_plan(m, p, n, 32) in ("gemv_u8_mfma16_blocks", "gemv_u8_mfma16_dma_32rows")
+    a, q, s = _u8_case(g, m, p, n, 32, exact=True)
+    for beta in (0.0, 1.0):
+        prev = (g.integers(-8, 9, size=(m, n)) / 4.0).astype(np.float16)
+        want = prev.copy()
+        oracle.matmul_nt_fp16u8(want, a, q, s, 32, beta=beta, threads=8)
+        out = to_dev(prev)
+        kern.matmul_nt_fp16u8(out, to_dev(a), to_dev(q), to_dev(s), 32, beta=beta)
+        assert np.array_equal(to_np(out).view(np.uint16), want.view(np.uint16)), (m, p, n, beta)
+
+
 @pytest.mark.parametrize("m", [1, 4, 16, 17, 100, 300])
 def test_u8_matmul_random_matches_oracle_and_reference_kernel(kern, ref, m):
     g = rng(620 + m)
@@ -422,18 +442,24 @@ def test_decode_ten_rows_and_more_long_k(kern, kn, m):
     assert rel <= 2e-3, rel
 
 
-@pytest.mark.parametrize("m", [17, 32, 33, 50, 64, 100, 128])
+@pytest.mark.parametrize("m", [17, 32, 33, 50, 64, 65, 100, 128, 200, 256])
 @pytest.mark.parametrize("kn", [(4096, 4100), (4096, 8200), (11008, 1000), (2048, 2100)])
-def test_seventeen_and_more_rows_in_blocks_of_sixteen(kern, kn, m):
-    """17 to 64 rows (to 128 where N < 8192) on matrices of 4 MiB and more run the sixteen-row
-    kernels per block of rows (a last block of one or two rows takes the dot-product kernel);
-    more rows stay on the tiled GEMM.  Previous output added, ragged N."""
+def test_seventeen_and_more_rows_in_passes(kern, kn, m):
+    """17 rows and more on matrices of 4 MiB and more run in passes of up to 64 rows, each
+    reading the weights once for two to four blocks of sixteen rows (K = 4096 up to 32 rows: the
+    DMA-ring kernel; a last pass of up to sixteen rows: the sixteen-row kernels); above 64 rows
+    only where that is estimated to beat the tiled GEMM.  Previous output added, ragged N."""
     p, n = kn
-    limit = 128 if n < 8192 else 64
-    blocks = "gemv_u8_mfma16_dma_32rows" if p == 4096 else "gemv_u8_mfma16_regstream"
-    assert (u8_plan(m, p, n, 32) == blocks) if m <= limit else \
-        u8_plan(m, p, n, 32).startswith("gemm_nt_u8_")
-    assert u8_plan(limit + 1, p, n, 32).startswith("gemm_nt_u8_")
+    name = u8_plan(m, p, n, 32)
+    if m <= 64:
+        assert name == ("gemv_u8_mfma16_dma_32rows" if p == 4096 and m <= 32 else "gemv_u8_mfma16_blocks")
+    else:
+        assert name == "gemv_u8_mfma16_blocks" or name.startswith("gemm_nt_u8_")
+    # decisions the estimate must make: a long K keeps the passes to 256 rows, a matrix of three
+    # rounds of workgroups leaves them at 64
+    assert u8_plan(256, 11008, 1000, 32) == "gemv_u8_mfma16_blocks"
+    assert u8_plan(100, 4096, 8200, 32).startswith("gemm_nt_u8_")
+    assert u8_plan(257, 11008, 1000, 32).startswith("gemm_nt_u8_")
     gen = torch.Generator(device="cuda").manual_seed(47 + m + p)
     q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)
     s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
@@ -450,7 +476,7 @@ def test_seventeen_and_more_rows_in_blocks_of_sixteen(kern, kn, m):
     assert rel <= 2e-3, rel
 
 
-@pytest.mark.parametrize("mpn", [(300, 4096, 4096), (512, 2048, 4090), (129, 11008, 1000)])
+@pytest.mark.parametrize("mpn", [(300, 4096, 4096), (512, 2048, 4090), (260, 11008, 1000)])
 def test_mid_row_counts_take_the_smaller_staged_tiles(kern, mpn):
     """With at most 64 tiles of 256 x 128 the u8 product runs on the staged kernels' smaller tiles;
     same arithmetic bar as the large-tile kernel."""
@@ -507,16 +533,18 @@ def test_descriptor_forms_on_strided_views(kern):
 
 @pytest.mark.parametrize("shape", [(129, 4096, 4096), (300, 1024, 8200), (512, 11008, 4096), (1024, 4096, 4096),
                                    (1100, 448, 12288), (2048, 4096, 12288), (1700, 640, 9000), (96, 4096, 4096),
-                                   (65, 11008, 4096), (128, 4096, 4096), (80, 4096, 8200)])
+                                   (65, 11008, 4096), (128, 4096, 4096), (80, 4096, 8200),
+                                   # the fused call in passes of 64 rows, the workspace used
+                                   (200, 11008, 1000), (100, 2048, 8200), (256, 4096, 4100)])
 @pytest.mark.parametrize("beta", [0.0, 1.0])
 def test_workspace_variant_gives_the_bits_of_the_fused_call(shape, beta):
     """adr_matmul_nt_fp16u8_ws (weights dequantised once into the workspace, then the fp16
-    kernels) against adr_matmul_nt_fp16u8 on the same operands: both round every weight to fp16
-    with the reference's dequantisation and sum slices of K in the same order -- from 129 rows on
-    the outputs are compared bit for bit (below: against the fp32 product, see there), with the
-    previous output added and without, in the regimes where the
-    workspace is used and where it is not (96 rows against 16 M weights; 1100 rows against 12288
-    weight rows)."""
+    kernels) against adr_matmul_nt_fp16u8 on the same operands.  Both round every weight to fp16
+    with the reference's dequantisation; where the fused call runs its tiled kernels (always from
+    257 rows on) both also sum slices of K in the same order and the outputs are compared bit for
+    bit, as they are where the workspace is not used.  Where the fused call runs its passes of 64
+    rows (wavefronts split K) both are held to the fp32 product.  With the previous output added
+    and without."""
     m, p, n = shape
     lib = _ffi.lib()
     gen = torch.Generator(device="cuda").manual_seed(m + p + n)
@@ -533,12 +561,12 @@ def test_workspace_variant_gives_the_bits_of_the_fused_call(shape, beta):
     assert lib.adr_matmul_nt_fp16u8_ws(st, got.data_ptr(), a.data_ptr(), q.data_ptr(), s.data_ptr(), m, p, n, 32,
                                        beta, ws.data_ptr(), ws.numel()) == 0
     torch.cuda.synchronize()
-    if m >= 129 or not need:
+    if not need or u8_plan(m, p, n, 32).startswith("gemm_nt_u8_"):
         assert torch.equal(got.view(torch.int16), want.view(torch.int16))
     else:
-        # 65 .. 128 rows: the fused call runs sixteen rows per pass on the kernel that evaluates
-        # the reference's naive formula (unrounded weights), the workspace path its WMMA formula
-        # (weights rounded to fp16): the two differ by less than 5e-4 of the output's magnitude
+        # the fused call's wavefronts split K, the workspace path's do not: same weights, another
+        # order of the fp32 sums
+        assert m <= 256
         w = torch.empty(n, p, dtype=torch.float16, device="cuda")
         assert lib.adr_dequantize_absmax_u8(st, w.data_ptr(), q.data_ptr(), s.data_ptr(), n, p, 32) == 0
         ref = a.float() @ w.float().t() + beta * prev.float()
