@@ -176,21 +176,83 @@ __device__ __forceinline__ bool epilogue_is_straight(const MatmulArgs& a, const 
   return inside && unmasked && out_vectorizable(a, out);
 }
 
+// Accumulators of a wavefront's sub-tile come in two register layouts.  32x32x16 MFMA
+// (float16_t acc[TM][TN]): see above.  16x16x32 MFMA (float4_t acc[2*TM][2*TN], transposed the
+// same way): acc[i][j] is the 16 x 16 block of rows 16*i.., columns 16*j..; lane l holds output
+// row l % 16 and, in element e, column 4*(l/16) + e.  The epilogues see both through these two
+// helpers, which put 32-row block i of the sub-tile into the wavefront's LDS slot.
+template <class T> struct is_mi16 { static constexpr bool value = false; };
+template <int A, int B> struct is_mi16<float4_t[A][B]> { static constexpr bool value = true; };
+
+// [32 rows][TN*32 halves], PITCH bytes per row; `mul` multiplies when `scaled`
+template <int TM, int TN, class Acc>
+__device__ __forceinline__ void stage_block_f16(Acc& acc, int i, unsigned char* slot, int lane,
+                                                bool scaled, half_t mul) {
+  constexpr int PITCH = TN * 64 + 16;
+  if constexpr (is_mi16<Acc>::value) {
+    const int lrow = lane & 15, g = lane >> 4;
+#pragma unroll
+    for (int h2 = 0; h2 < 2; h2++)
+#pragma unroll
+      for (int j = 0; j < 2 * TN; j++) {
+        half4_t h;
+#pragma unroll
+        for (int e = 0; e < 4; e++) h[e] = (half_t)acc[2 * i + h2][j][e];
+        *(half4_t*)(slot + (h2 * 16 + lrow) * PITCH + (j * 16 + 4 * g) * 2) = scaled ? h * mul : h;
+      }
+  } else {
+    const int lrow = lane & 31, g = lane >> 5;
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        half4_t h;
+#pragma unroll
+        for (int e = 0; e < 4; e++) h[e] = (half_t)acc[i][j][4 * q + e];
+        *(half4_t*)(slot + lrow * PITCH + (j * 32 + 8 * q + 4 * g) * 2) = scaled ? h * mul : h;
+      }
+  }
+}
+
+// fp32: columns [qh*8*QN, +8*QN) of 32 x 32 block (i, j) as [32 rows][8*QN floats], FP bytes per row
+template <int QN, class Acc>
+__device__ __forceinline__ void stage_block_f32(Acc& acc, int i, int j, int qh, unsigned char* slot,
+                                                int lane) {
+  constexpr int FP = QN * 32 + 16;
+  if constexpr (is_mi16<Acc>::value) {
+    const int lrow = lane & 15, g = lane >> 4;
+#pragma unroll
+    for (int h2 = 0; h2 < 2; h2++)
+#pragma unroll
+      for (int jj = 0; jj < QN / 2; jj++)   // 16-column blocks staged at once: 2 (QN 4) or 1 (QN 2)
+        *(float4_t*)(slot + (h2 * 16 + lrow) * FP + (jj * 16 + 4 * g) * 4) =
+            acc[2 * i + h2][2 * j + (QN == 4 ? jj : qh)];
+  } else {
+    const int lrow = lane & 31, g = lane >> 5;
+#pragma unroll
+    for (int qq = 0; qq < QN; qq++) {
+      const int q = qh * QN + qq;
+      const float4_t v = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2],
+                          acc[i][j][4 * q + 3]};
+      *(float4_t*)(slot + lrow * FP + (qq * 8 + 4 * g) * 4) = v;
+    }
+  }
+}
+
 // The straight-line epilogue for ONE store operator (OP is a compile-time constant: every
 // operator gets its own compact instruction stream; with the operator switch inside the chunk
 // loop the code of all of them, exp and tanh included, sat between any two stores, and the
 // operators that are not Identity paid for it in instruction fetch).
-template <int TM, int TN, uint32_t OP>
-__device__ __forceinline__ void straight_epilogue(const MatmulArgs& a, half_t* out,
-                                                  float16_t (&acc)[TM][TN], int y0, int x0,
-                                                  unsigned char* slot, half_t hscale, int lane) {
+template <int TM, int TN, uint32_t OP, class Acc>
+__device__ __forceinline__ void straight_epilogue(const MatmulArgs& a, half_t* out, Acc& acc, int y0,
+                                                  int x0, unsigned char* slot, half_t hscale,
+                                                  int lane) {
   constexpr bool plain_op = OP == ADR_STORE_IDENTITY || OP == ADR_STORE_SCALE;
   constexpr bool np = OP == ADR_STORE_ADD || OP == ADR_STORE_BETA_BIAS ||
                       OP == ADR_STORE_BETA_GELU_BIAS || OP == STORE_ACC_BETA;
   constexpr bool nb = OP == ADR_STORE_BETA_BIAS || OP == ADR_STORE_BETA_GELU_BIAS ||
                       OP == ADR_STORE_QUICK_GELU_BIAS;
   const Epilogue ep{a.bias, a.beta, hscale, OP, true};
-  const int lrow = lane & 31, g = lane >> 5;
   constexpr int PITCH = TN * 64 + 16;  // bytes per staged row (TN*32 halves + pad)
   constexpr int CPW = TN * 4;          // 16-byte chunks per staged row
   const half_t mul = OP == ADR_STORE_SCALE ? hscale : (half_t)1.0f;
@@ -226,17 +288,9 @@ __device__ __forceinline__ void straight_epilogue(const MatmulArgs& a, half_t* o
   }
 #pragma unroll
   for (int i = 0; i < TM; i++) {
-#pragma unroll
-    for (int j = 0; j < TN; j++)
-#pragma unroll
-      for (int q = 0; q < 4; q++) {
-        half4_t h;
-#pragma unroll
-        for (int e = 0; e < 4; e++) h[e] = (half_t)acc[i][j][4 * q + e];
-        // x * 1 is exact, so one multiply serves Identity and Scale (matmul.cu Scale: fp16
-        // product); the other operators take the narrowed sum as it is
-        *(half4_t*)(slot + lrow * PITCH + (j * 32 + 8 * q + 4 * g) * 2) = plain_op ? h * mul : h;
-      }
+    // x * 1 is exact, so one multiply serves Identity and Scale (matmul.cu Scale: fp16
+    // product); the other operators take the narrowed sum as it is
+    stage_block_f16<TM, TN>(acc, i, slot, lane, plain_op, mul);
 #pragma unroll
     for (int it = 0; it < TN * 2; it++) {
       half8_t v = *(const half8_t*)(slot + rd[it]);
@@ -262,12 +316,10 @@ __device__ __forceinline__ void straight_epilogue(const MatmulArgs& a, half_t* o
   }
 }
 
-template <int TM, int TN>
-__device__ __forceinline__ void wave_epilogue(const MatmulArgs& a, half_t* out,
-                                              float16_t (&acc)[TM][TN], int y0, int x0,
-                                              unsigned char* slot, half_t hscale, int lane) {
+template <int TM, int TN, class Acc>
+__device__ __forceinline__ void wave_epilogue(const MatmulArgs& a, half_t* out, Acc& acc, int y0,
+                                              int x0, unsigned char* slot, half_t hscale, int lane) {
   Epilogue ep{a.bias, a.beta, hscale, a.store, true};
-  const int lrow = lane & 31, g = lane >> 5;
   constexpr int PITCH = TN * 64 + 16;  // bytes per staged row (TN*32 halves + pad)
   constexpr int CPW = TN * 4;          // 16-byte chunks per staged row
   // Common case, straight-line: the sub-tile's columns lie inside the matrix, it is (for a
@@ -293,15 +345,7 @@ __device__ __forceinline__ void wave_epilogue(const MatmulArgs& a, half_t* out,
   if (out_vectorizable(a, out)) {
 #pragma unroll
     for (int i = 0; i < TM; i++) {
-#pragma unroll
-      for (int j = 0; j < TN; j++)
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-          half4_t h;
-#pragma unroll
-          for (int e = 0; e < 4; e++) h[e] = (half_t)acc[i][j][4 * q + e];
-          *(half4_t*)(slot + lrow * PITCH + (j * 32 + 8 * q + 4 * g) * 2) = h;
-        }
+      stage_block_f16<TM, TN>(acc, i, slot, lane, false, (half_t)1.0f);
 #pragma unroll 1
       for (int it = 0; it < TN * 2; it++) {
         const int idx = it * 64 + lane;
@@ -312,29 +356,40 @@ __device__ __forceinline__ void wave_epilogue(const MatmulArgs& a, half_t* out,
       }
     }
   } else {
+    // Element by element (unaligned or strided rows, or the fp32 form of acc + beta * out): the
+    // fp32 accumulators pass through the wavefront's LDS slot, QN groups of eight columns of a
+    // 32 x 32 block at a time, so that consecutive lanes store consecutive columns and the loop
+    // over the elements needs no unrolling (a run-time index into the accumulator registers
+    // would put them in scratch memory).
     const bool need_prev = Epilogue::needs_prev(a.store);
     const bool need_bias = Epilogue::needs_bias(a.store);
     const bool causal = a.mask == ADR_MASK_CAUSAL;
+    constexpr int QN = TN >= 2 ? 4 : 2;     // 32 rows x (QN * 32 + 16) bytes fit the slot
+    constexpr int FP = QN * 32 + 16;        // bytes per staged row
+    static_assert(32 * FP <= 32 * PITCH, "fp32 staging must fit the wavefront's slot");
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
-      const int y = y0 + i * 32 + lrow;
-      if (y >= a.m) continue;
+    for (int i = 0; i < TM; i++)
 #pragma unroll
       for (int j = 0; j < TN; j++)
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-          const int x = x0 + j * 32 + 8 * (r / 4) + 4 * g + (r % 4);
-          if (x >= a.n) continue;
-          half_t* p = out + (int64_t)y * a.stride_oy + x;
-          if (causal && x > y) {
-            *p = neg_inf_half();
-          } else {
-            half_t prev = need_prev ? *p : (half_t)0;
-            half_t bias = need_bias ? a.bias[x] : (half_t)0;
-            *p = ep.apply(acc[i][j][r], prev, bias);
+        for (int qh = 0; qh < 4 / QN; qh++) {
+          stage_block_f32<QN>(acc, i, j, qh, slot, lane);
+#pragma unroll 1
+          for (int e = lane; e < 32 * 8 * QN; e += 64) {
+            const int row = e / (8 * QN), c = e % (8 * QN);
+            const int y = y0 + i * 32 + row, x = x0 + j * 32 + qh * QN * 8 + c;
+            if (y >= a.m || x >= a.n) continue;
+            const float sum = *(const float*)(slot + row * FP + c * 4);
+            half_t* p = out + (int64_t)y * a.stride_oy + x;
+            if (causal && x > y) {
+              *p = neg_inf_half();
+            } else {
+              half_t prev = need_prev ? *p : (half_t)0;
+              half_t bias = need_bias ? a.bias[x] : (half_t)0;
+              *p = ep.apply(sum, prev, bias);
+            }
           }
         }
-    }
   }
 }
 
@@ -371,12 +426,18 @@ __device__ __forceinline__ void fill_masked_tile(const MatmulArgs& a, half_t* ou
 // leaving the fp32 accumulators in a.workspace ([piece][tile][register chunk][thread] float4, so
 // that consecutive threads store consecutive 16 bytes); splitk_reduce_kernel sums the pieces in
 // a fixed order and runs the epilogue.
-template <int BM, int BN, int WM, int WN, int NSTAGE, int MINB, bool NN, int BK = 64, bool SPLIT = false>
+// MI16: v_mfma_f32_16x16x32_f16 instead of 32x32x16.  Same flops per clock, but on data that is
+// not constant the part sustains 16 % more of them within its power limit (a bare loop on a
+// 128 x 128 wavefront tile: 2070 against 1780 TFLOP/s; both 2460 on zeros).
+template <int BM, int BN, int WM, int WN, int NSTAGE, int MINB, bool NN, int BK = 64, bool SPLIT = false,
+          bool MI16 = false>
 __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulArgs a,
                                                                          TileMap map) {
   // K slices of 64 (128 bytes of a row per slice and DMA request), or of 128 for the small tiles
   // of few-row products, which are bound by how DRAM serves those requests
-  constexpr int CPR = BK / 8, KK = BK / 16;
+  constexpr int MI = MI16 ? 16 : 32;           // rows (and columns) of one MFMA block
+  constexpr int KG = 64 / MI;                  // 16-byte k-groups per k-step: lane / MI
+  constexpr int CPR = BK / 8, KK = CPR / KG;   // k-steps per slice: of 16 k (32x32x16) or 32 k
   static_assert(BK == 64 || (BK == 128 && !NN && NSTAGE == 3), "slices of 64, or 128 with three stages");
   constexpr int NW = WM * WN, NT = NW * 64;
   // DMA instructions per thread and slice.  NSTAGE == 6: the first half of the wavefronts issues
@@ -384,18 +445,16 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   constexpr int NWD = NSTAGE == 6 ? NW / 2 : NW;
   constexpr int IA = BM * CPR / (NWD * 64), IB = BN * CPR / (NWD * 64);
   constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
+  constexpr int FM = WTM / MI, FN = WTN / MI;  // MFMA blocks of the wavefront's sub-tile
   constexpr int SLOT = 32 * (TN * 64 + 16);
+  static_assert(!MI16 || (!NN && !SPLIT), "16x16x32: plain NT products");
   static_assert(BM * CPR % (NWD * 64) == 0 && BN * CPR % (NWD * 64) == 0,
                 "slices must split evenly over lanes");
   static_assert(WTM % 32 == 0 && WTN % 32 == 0, "MFMA 32x32x16 tiling");
-  // epilogue slots: half of the wavefronts in each A stage, or (256 x 256) as many as fit per
-  // stage buffer over the A and then the B stages
-  constexpr bool SLOTS_IN_A = (NW / 2) * SLOT <= BM * BK * 2;
-  constexpr int SLOTS_PER_BUF = (BM * BK * 2) / SLOT;
-  static_assert(SLOTS_IN_A || (BN >= BM && NSTAGE == 5 && 5 * SLOTS_PER_BUF >= NW),
-                "epilogue slots must fit in the stage buffers");
-  static_assert(NSTAGE == 2 || NSTAGE == 3 || NSTAGE == 5 || NSTAGE == 6,
-                "2 or 3 LDS stages, or 5 / 6: two stages of the left and three / four of the right operand");
+  // epilogue slots: half of the wavefronts in each of the first two A stages
+  static_assert((NW / 2) * SLOT <= BM * BK * 2, "epilogue slots must fit in the stage buffers");
+  static_assert(NSTAGE == 2 || NSTAGE == 3 || NSTAGE == 6,
+                "2 or 3 LDS stages, or 6: two stages of the left and four of the right operand");
   static_assert(NSTAGE != 6 || (!NN && !SPLIT && NW % 2 == 0), "role split: plain NT products");
   static_assert(!NN || BN == 128, "the N-contiguous right operand is staged as [64][128] tiles");
   // Separate objects per stage: the compiler's alias analysis then knows that the asynchronous
@@ -480,24 +539,26 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
     dmaB(ks, dB);
   };
 
-  float16_t acc[TM][TN];
+  typedef typename std::conditional<MI16, float4_t, float16_t>::type acc_t;
+  acc_t acc[FM][FN];
 #pragma unroll
-  for (int i = 0; i < TM; i++)
+  for (int i = 0; i < FM; i++)
 #pragma unroll
-    for (int j = 0; j < TN; j++)
+    for (int j = 0; j < FN; j++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+      for (int r = 0; r < (MI16 ? 4 : 16); r++) acc[i][j][r] = 0.0f;
 
-  // fragment addressing: lane -> (row = lane % 32, k-group = lane / 32), 8 halves = one chunk
-  const int frow = lane & 31, fkg = lane >> 5;
-  int offA[TM][KK], offB[TN][KK];
+  // fragment addressing: lane -> (row = lane % MI, k-group = lane / MI), 8 halves = one chunk.
+  // MI rows further down the chunk sits MI * CPR * 16 bytes further (a whole number of 256-byte
+  // lines times 8: the swizzle does not change), so one offset per k-step serves all blocks.
+  const int frow = lane & (MI - 1), fkg = lane / MI;
+  constexpr int FSTEP = MI * CPR * 16;
+  int offA[KK], offB[NN ? TN : 1][KK];
 #pragma unroll
   for (int kk = 0; kk < KK; kk++) {
+    offA[kk] = lds_chunk_off<CPR>(wm * WTM + frow, kk * KG + fkg);
 #pragma unroll
-    for (int i = 0; i < TM; i++)
-      offA[i][kk] = lds_chunk_off<CPR>(wm * WTM + i * 32 + frow, kk * 2 + fkg);
-#pragma unroll
-    for (int j = 0; j < TN; j++) {
+    for (int j = 0; j < (NN ? TN : 1); j++) {
       if (NN) {
         // transposing read (ds_read_b64_tr_b16): inside each group of 16 lanes, lanes 4r..4r+3
         // address 16 consecutive halves of k-row r and lane i receives column i of that 4 x 16
@@ -509,17 +570,17 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
         const int col = wn * WTN + j * 32 + 16 * (q & 1) + 4 * jj;
         offB[j][kk] = krow * 256 + ((((col >> 3) ^ ((krow & 3) << 2))) << 4) + (jj & 1) * 8;
       } else {
-        offB[j][kk] = lds_chunk_off<CPR>(wn * WTN + j * 32 + frow, kk * 2 + fkg);
+        offB[0][kk] = lds_chunk_off<CPR>(wn * WTN + frow, kk * KG + fkg);
       }
     }
   }
 
-  half8_t fa[2][TM], fb[2][TN];
+  half8_t fa[2][FM], fb[2][FN];
   auto load_frags = [&](int slot, const unsigned char* cA, const unsigned char* cB, int kk) {
 #pragma unroll
-    for (int i = 0; i < TM; i++) fa[slot][i] = *(const half8_t*)(cA + offA[i][kk]);
+    for (int i = 0; i < FM; i++) fa[slot][i] = *(const half8_t*)(cA + offA[kk] + i * FSTEP);
 #pragma unroll
-    for (int j = 0; j < TN; j++) {
+    for (int j = 0; j < FN; j++) {
       if (NN) {
         typedef short short4_t __attribute__((ext_vector_type(4)));
         typedef __attribute__((address_space(3))) short4_t lds_short4_t;
@@ -530,17 +591,22 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
         fb[slot][j] = __builtin_shufflevector(__builtin_bit_cast(half4_t, lo),
                                               __builtin_bit_cast(half4_t, hi), 0, 1, 2, 3, 4, 5, 6, 7);
       } else {
-        fb[slot][j] = *(const half8_t*)(cB + offB[j][kk]);
+        fb[slot][j] = *(const half8_t*)(cB + offB[0][kk] + j * FSTEP);
       }
     }
   };
   auto mfmas = [&](int slot) {
 #pragma unroll
-    for (int i = 0; i < TM; i++)
+    for (int i = 0; i < FM; i++)
 #pragma unroll
-      for (int j = 0; j < TN; j++)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[slot][j], fa[slot][i], acc[i][j],
-                                                           0, 0, 0);
+      for (int j = 0; j < FN; j++) {
+        if constexpr (MI16)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[slot][j], fa[slot][i], acc[i][j],
+                                                             0, 0, 0);
+        else
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[slot][j], fa[slot][i], acc[i][j],
+                                                             0, 0, 0);
+      }
   };
   // s_waitcnt vmcnt(n) lgkmcnt(0): n outstanding DMA instructions may remain in flight
   auto wait_dma_barrier = [&](auto n_tag) {
@@ -563,13 +629,13 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
         load_frags((kk + 1) & 1, cA, cB, kk + 1);
         mfmas(kk & 1);
         // interleave: LDS reads behind the first MFMAs of this k-step
-        constexpr int READS = TM + (NN ? 2 * TN : TN);
-        constexpr int PER = (READS + TM * TN - 1) / (TM * TN);
+        constexpr int READS = FM + (NN ? 2 * FN : FN);
+        constexpr int PER = (READS + FM * FN - 1) / (FM * FN);
 #pragma unroll
-        for (int q = 0; q < TM * TN; q++) {
+        for (int q = 0; q < FM * FN; q++) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x100, PER, 0);
-          if (kk * TM * TN + q < IA + IB) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+          if (kk * FM * FN + q < IA + IB) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
         }
       } else {
         mfmas(kk & 1);
@@ -603,10 +669,10 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
             load_frags((kk + 1) & 1, cA, cB, kk + 1);
             mfmas(kk & 1);
 #pragma unroll
-            for (int q = 0; q < TM * TN; q++) {
+            for (int q = 0; q < FM * FN; q++) {
               __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
               __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-              if (kk * TM * TN + q < (LEFT ? IA : IB)) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+              if (kk * FM * FN + q < (LEFT ? IA : IB)) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
             }
           } else {
             mfmas(kk & 1);
@@ -637,55 +703,6 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
       if (kt < KT) { slice6(sA0, sB2, sA1, sB3, sA1, sB1); kt++; }
     };
     if (__builtin_amdgcn_readfirstlane(wave) < NW / 2) run(std::true_type{}); else run(std::false_type{});
-  } else if (NSTAGE == 5) {
-    // Two stages of the left and three of the right operand: slice kt reads A stage kt % 2 and
-    // B stage kt % 3; at its head the DMA of A(kt+1) and then of B(kt+2) is issued, and at its
-    // end everything but B(kt+2) has to have landed.  The right operand (weights that no cache
-    // holds between launches of a model) gets two slices to arrive, the left one (activations
-    // just written, resident in L2) one.
-    int kA = 0, kB = 0;
-    auto slice5 = [&](const unsigned char* cA, const unsigned char* cB, const unsigned char* nA,
-                      const unsigned char* nB, unsigned char* dA, unsigned char* dB) {
-      dmaA(min(kA++, KT - 1), dA);
-      dmaB(min(kB++, KT - 1), dB);
-#pragma unroll
-      for (int kk = 0; kk < KK; kk++) {
-        if (kk + 1 < KK) {
-          load_frags((kk + 1) & 1, cA, cB, kk + 1);
-          mfmas(kk & 1);
-#pragma unroll
-          for (int q = 0; q < TM * TN; q++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            if (kk < 2) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
-          }
-        } else {
-          mfmas(kk & 1);
-        }
-      }
-      wait_dma_barrier(std::integral_constant<int, IB>{});
-      load_frags(0, nA, nB, 0);
-      __builtin_amdgcn_sched_barrier(0);
-    };
-    dmaB(min(kB++, KT - 1), sB0);
-    dmaA(min(kA++, KT - 1), sA0);
-    dmaB(min(kB++, KT - 1), sB1);
-    wait_dma_barrier(std::integral_constant<int, IB>{});
-    load_frags(0, sA0, sB0, 0);
-    int kt = 0;
-    for (; kt + 6 <= KT; kt += 6) {
-      slice5(sA0, sB0, sA1, sB1, sA1, sB2);
-      slice5(sA1, sB1, sA0, sB2, sA0, sB0);
-      slice5(sA0, sB2, sA1, sB0, sA1, sB1);
-      slice5(sA1, sB0, sA0, sB1, sA0, sB2);
-      slice5(sA0, sB1, sA1, sB2, sA1, sB0);
-      slice5(sA1, sB2, sA0, sB0, sA0, sB1);
-    }
-    if (kt < KT) { slice5(sA0, sB0, sA1, sB1, sA1, sB2); kt++; }
-    if (kt < KT) { slice5(sA1, sB1, sA0, sB2, sA0, sB0); kt++; }
-    if (kt < KT) { slice5(sA0, sB2, sA1, sB0, sA1, sB1); kt++; }
-    if (kt < KT) { slice5(sA1, sB0, sA0, sB1, sA0, sB2); kt++; }
-    if (kt < KT) { slice5(sA0, sB1, sA1, sB2, sA1, sB0); kt++; }
   } else if (NSTAGE == 3) {
     dma(sA0, sB0);
     dma(sA1, sB1);
@@ -713,7 +730,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   // drain the trailing (redundant) DMA before the stages are reused by the epilogue
   wait_dma_barrier(std::integral_constant<int, 0>{});
 
-  if (SPLIT) {
+  if constexpr (SPLIT) {
     float4_t* const ws = (float4_t*)a.workspace +
                          ((int64_t)piece * map.total + tile_id) * (TM * TN * 4) * NT + tid;
 #pragma unroll
@@ -728,14 +745,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
         }
     return;
   }
-  unsigned char* slot;
-  if (SLOTS_IN_A) {
-    slot = (wave < NW / 2 ? sA0 : sA1) + (wave % (NW / 2)) * SLOT;
-  } else {
-    const int buf = wave / SLOTS_PER_BUF;
-    slot = (buf == 0 ? sA0 : buf == 1 ? sA1 : buf == 2 ? sB0 : buf == 3 ? sB1 : sB2) +
-           (wave % SLOTS_PER_BUF) * SLOT;
-  }
+  unsigned char* const slot = (wave < NW / 2 ? sA0 : sA1) + (wave % (NW / 2)) * SLOT;
   wave_epilogue<TM, TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, slot, (half_t)a.scale, lane);
 }
 
@@ -1434,11 +1444,11 @@ TileMap make_map(const MatmulArgs& a, int bm, int bn) {
   return map;
 }
 
-template <int BM, int BN, int WM, int WN, int NSTAGE, int MINB, bool NN = false, int BK = 64>
+template <int BM, int BN, int WM, int WN, int NSTAGE, int MINB, bool NN = false, int BK = 64, bool MI16 = false>
 hipError_t launch_dma(hipStream_t stream, const MatmulArgs& a) {
   TileMap map = make_map(a, BM, BN);
   if (map.total < 0) return hipErrorInvalidConfiguration;
-  hipLaunchKernelGGL((gemm_nt_dma_kernel<BM, BN, WM, WN, NSTAGE, MINB, NN, BK>),
+  hipLaunchKernelGGL((gemm_nt_dma_kernel<BM, BN, WM, WN, NSTAGE, MINB, NN, BK, false, MI16>),
                      dim3((unsigned)map.total), dim3(WM * WN * 64), 0, stream, a, map);
   return hipGetLastError();
 }
@@ -1520,7 +1530,7 @@ enum GemmChoice {
   GEMM_NONE = 0,
   SHORTK_64, SHORTK_128,
   U8_256x192, U8_256x128,
-  DMA_256x256, DMA_256x192, DMA_256x128, DMA_128x128, DMA_128x64, DMA_64x64, DMA_64x64_K128, DMA_128x64_K128,
+  DMA_256x192, DMA_256x128, DMA_128x128, DMA_128x64, DMA_64x64, DMA_64x64_K128, DMA_128x64_K128,
   DMA_NN_256x128, DMA_NN_128x128,
   STAGE_256x128, STAGE_128x128, STAGE_64x64,
 };
@@ -1553,8 +1563,11 @@ GemmChoice pick(const MatmulArgs& a, const Candidate* c, int n, double* cost_out
   return best;
 }
 
+// (the two large tiles run on 16x16x32 MFMAs: 9-16 % faster than on 32x32x16 on data that is not
+// constant -- qkv 170 -> 156 us, o 68 -> 58, down 162 -> 144 -- while the smaller tiles, which are
+// not bound by the power limit, gain nothing from it and stay on 32x32x16)
 const Candidate DMA_TILES[] = {
-    {DMA_256x192, 256, 192, 1, 1.10f}, {DMA_256x128, 256, 128, 1, 1.00f},
+    {DMA_256x192, 256, 192, 1, 1.24f}, {DMA_256x128, 256, 128, 1, 1.13f},
     {DMA_128x128, 128, 128, 2, 0.80f}, {DMA_128x64, 128, 64, 2, 0.60f},
     {DMA_64x64, 64, 64, 4, 0.40f}};
 
@@ -1588,19 +1601,7 @@ GemmChoice choose(const MatmulArgs& a) {
                                          {DMA_64x64, 64, 64, 4, 0.50f}};
       return pick(a, shortk, 2);
     }
-    double cost;
-    GemmChoice c = pick(a, DMA_TILES, 5, &cost);
-    // 256 x 256 tiles move 14 % fewer bytes into LDS per flop than 256 x 192 (2 % faster per
-    // tile area) but are too coarse for most shapes; they win where they fill whole rounds and
-    // the smaller tiles do not (M2048 K4096 N8192: 137 -> 124 us, M4096 N4096: 134 -> 122 us).
-    // Long K only: with few slices one large tile per CU has nothing to overlap its prologue
-    // and epilogue with.
-    if (a.k >= 2048) {
-      static const Candidate big = {DMA_256x256, 256, 256, 1, 1.12f};
-      double cost_big;
-      pick(a, &big, 1, &cost_big);
-      if (cost_big < cost) c = DMA_256x256;
-    }
+    GemmChoice c = pick(a, DMA_TILES, 5);
     // At most one 64 x 64 tile per CU (a few dozen to a few hundred rows against a weight
     // matrix): the product is bound by how DRAM serves the weight requests -- one piece of every
     // tile row per slice, a whole weight row apart -- and pieces of 256 bytes (slices of 128)
@@ -1720,7 +1721,6 @@ static bool choice_name(GemmChoice c, const char** name, bool u8 = false) {
     case SHORTK_128: *name = "gemm_nt_mfma_persistent_128x128_k128"; return true;
     case U8_256x192: *name = "gemm_nt_u8_mfma_256x192x64"; return true;
     case U8_256x128: *name = "gemm_nt_u8_mfma_256x128x64"; return true;
-    case DMA_256x256: *name = "gemm_nt_mfma_dma_256x256x64"; return true;
     case DMA_256x192: *name = "gemm_nt_mfma_dma_256x192x64"; return true;
     case DMA_256x128: *name = "gemm_nt_mfma_dma_256x128x64"; return true;
     case DMA_128x128: *name = "gemm_nt_mfma_dma_128x128x64"; return true;
@@ -1743,9 +1743,8 @@ static hipError_t launch_choice(hipStream_t stream, const MatmulArgs& a, GemmCho
     case SHORTK_128: return launch_shortk<16>(stream, a);
     case U8_256x192: return launch_u8<256, 192, 4, 2>(stream, a);
     case U8_256x128: return launch_u8<256, 128, 4, 2>(stream, a);
-    case DMA_256x256: return launch_dma<256, 256, 4, 2, 5, 1>(stream, a);
-    case DMA_256x192: return launch_dma<256, 192, 4, 2, 6, 1>(stream, a);
-    case DMA_256x128: return launch_dma<256, 128, 4, 2, 3, 1>(stream, a);
+    case DMA_256x192: return launch_dma<256, 192, 4, 2, 6, 1, false, 64, true>(stream, a);
+    case DMA_256x128: return launch_dma<256, 128, 4, 2, 3, 1, false, 64, true>(stream, a);
     case DMA_128x128: return launch_dma<128, 128, 2, 2, 3, 1>(stream, a);
     case DMA_128x64: return launch_dma<128, 64, 2, 2, 3, 2>(stream, a);
     case DMA_64x64: return launch_dma<64, 64, 2, 2, 3, 3>(stream, a);

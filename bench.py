@@ -221,10 +221,10 @@ def main():
             del ws
         return rows
 
-    def decode_set():
+    def decode_set(ms=(1, 4, 16)):
         gemv = []
         for K, N in DECODE_SET:
-            for m in (1, 4, 16):
+            for m in ms:
                 t, byts, tp = u8_case(m, K, N, 200, probe=(m == 1))
                 row = {"M": m, "K": K, "N": N, "us": round(t * 1e6, 2),
                        "gbs": round(byts / t / 1e9, 1),
@@ -396,7 +396,10 @@ def main():
         return
 
     if args.decode_only:
-        print(json.dumps({"u8_decode_gemv": decode_set(), "f16_decode_gemv": f16_decode_set()}))
+        # (with the row counts of a short prompt: the reference's LLaMA re-runs the whole sequence
+        # for every token, llama.rs:456-483, so these are calls it makes too)
+        print(json.dumps({"u8_decode_gemv": decode_set(), "f16_decode_gemv": f16_decode_set(),
+                          "u8_17_to_128_rows": decode_set((32, 64, 128))}))
         return
 
     def u8_prefill_set():

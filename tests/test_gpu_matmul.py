@@ -479,14 +479,13 @@ def test_large_tile_kernel_every_k_tail_exact(K):
 
 
 @pytest.mark.parametrize("K", [2048, 2112, 2176, 2240, 2304, 2368])
-def test_256x256_tile_every_k_tail_exact(K):
-    """The 256 x 256 kernel (long K, whole rounds of 256 tiles) rotates two left and three right
-    LDS stages with a period of six slices; its epilogue slots spill over into the right
-    operand's stages.  Every remainder of the loop on inputs whose fp32 sums are exact, ragged
-    last tile row and column."""
+def test_256x128_tile_every_k_tail_exact(K):
+    """The 256 x 128 kernel (16x16x32 MFMAs, three LDS stages) on two whole rounds of tiles:
+    every remainder of its three-slice loop on inputs whose fp32 sums are exact, ragged last
+    tile row and column."""
     M, N = 2000, 8184
     so, sl, sr = nt_strides(M, K, N)
-    assert plan(1, M, K, N, so, sl, sr) == "gemm_nt_mfma_dma_256x256x64"
+    assert plan(1, M, K, N, so, sl, sr) == "gemm_nt_mfma_dma_256x128x64"
     gen = torch.Generator(device="cuda").manual_seed(K)
     a = (torch.randint(-4, 5, (M, K), generator=gen, device="cuda").float() / 64).half()
     w = (torch.randint(-4, 5, (N, K), generator=gen, device="cuda").float() / 64).half()
@@ -498,13 +497,13 @@ def test_256x256_tile_every_k_tail_exact(K):
 
 @pytest.mark.parametrize("store", STORES_EXACT + STORES_F32)
 @pytest.mark.parametrize("mask", [oracle.MASK_NONE, oracle.MASK_CAUSAL])
-def test_256x256_tile_epilogues_against_the_slow_kernel(store, mask):
-    """Every store operator and the causal mask through the 256 x 256 tile's epilogue, compared
-    with the step-for-step kernel on bands of rows (first tile row, a diagonal tile, the ragged
-    last rows)."""
+def test_256x128_tile_epilogues_against_the_slow_kernel(store, mask):
+    """Every store operator and the causal mask through the epilogue of the 256 x 128 tile (its
+    accumulators are 16 x 16 blocks), compared with the step-for-step kernel on bands of rows
+    (first tile row, a diagonal tile, the ragged last rows)."""
     M, K, N = 4000, 2048, 4090 - 2
     so, sl, sr = nt_strides(M, K, N)
-    assert plan(1, M, K, N, so, sl, sr, store=store, mask=mask) == "gemm_nt_mfma_dma_256x256x64"
+    assert plan(1, M, K, N, so, sl, sr, store=store, mask=mask) == "gemm_nt_mfma_dma_256x128x64"
     gen = torch.Generator(device="cuda").manual_seed(900 + store * 2 + mask)
     a = torch.randn(M, K, generator=gen, device="cuda").half()
     w = (torch.randn(N, K, generator=gen, device="cuda") * K ** -0.5).half()
