@@ -1084,18 +1084,22 @@ __global__ __launch_bounds__(1024, 1) void gemm_nt_shortk_kernel(MatmulArgs a, S
 // chunks of slice kt+1 are dequantised (bit-identical to quantize.cu:53-54) and written to one
 // of two fp16 LDS stages in the same swizzled layout the DMA produces, so that every weight is
 // dequantised once per workgroup and the MFMA loop is the one of the fp16 kernel.
-template <int BM, int BN, int WM, int WN>
+// MI16: 16x16x32 MFMAs, two k-steps per slice, all chunks dequantised in the first (the 256 x 128
+// tile: 5-6 % faster; the 256 x 192 tile has no registers for the second set of fragments)
+template <int BM, int BN, int WM, int WN, bool MI16>
 __global__ __launch_bounds__(WM* WN * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a, TileMap map,
                                                                    int block_shift) {
-  constexpr int BK = 64, CPR = 8, KK = 4;
+  constexpr int BK = 64, CPR = 8, MI = MI16 ? 16 : 32, KG = 64 / MI, KK = CPR / KG;
   constexpr int NW = WM * WN, NT = NW * 64;
   constexpr int IA = BM * CPR / NT;   // DMA instructions per lane and slice
   constexpr int LB = BN * CPR / NT;   // 8-weight chunks per lane and slice
   constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
+  constexpr int FM = WTM / MI, FN = WTN / MI;  // MFMA blocks of the wavefront's sub-tile
+  constexpr int FSTEP = MI * CPR * 16;         // bytes between the fragments of consecutive blocks
   constexpr int SLOT = 32 * (TN * 64 + 16);
   static_assert(BM * CPR % NT == 0 && BN * CPR % NT == 0, "slices must split evenly over lanes");
   static_assert((NW / 2) * SLOT <= BM * BK * 2, "epilogue slots must fit in two A stages");
-  static_assert(LB < KK, "one chunk per k-step, none in the last");
+  static_assert(MI16 ? LB <= 3 : LB < KK, "no chunk is dequantised in the last k-step");
   __shared__ __attribute__((aligned(1024))) unsigned char sA0[BM * BK * 2];
   __shared__ __attribute__((aligned(1024))) unsigned char sA1[BM * BK * 2];
   __shared__ __attribute__((aligned(1024))) unsigned char sA2[BM * BK * 2];
@@ -1163,39 +1167,42 @@ __global__ __launch_bounds__(WM* WN * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a
     for (int i = 0; i < LB; i++) dequant_store1(set, dB, i);
   };
 
-  float16_t acc[TM][TN];
+  typedef typename std::conditional<MI16, float4_t, float16_t>::type acc_t;
+  acc_t acc[FM][FN];
 #pragma unroll
-  for (int i = 0; i < TM; i++)
+  for (int i = 0; i < FM; i++)
 #pragma unroll
-    for (int j = 0; j < TN; j++)
+    for (int j = 0; j < FN; j++)
 #pragma unroll
-      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+      for (int r = 0; r < (MI16 ? 4 : 16); r++) acc[i][j][r] = 0.0f;
 
-  const int frow = lane & 31, fkg = lane >> 5;
-  int offFA[TM][KK], offFB[TN][KK];
+  // fragment of block i: FSTEP bytes per block beyond the first one's (see gemm_nt_dma_kernel)
+  const int frow = lane & (MI - 1), fkg = lane / MI;
+  int offFA[KK], offFB[KK];
 #pragma unroll
   for (int kk = 0; kk < KK; kk++) {
-#pragma unroll
-    for (int i = 0; i < TM; i++)
-      offFA[i][kk] = lds_chunk_off<CPR>(wm * WTM + i * 32 + frow, kk * 2 + fkg);
-#pragma unroll
-    for (int j = 0; j < TN; j++)
-      offFB[j][kk] = lds_chunk_off<CPR>(wn * WTN + j * 32 + frow, kk * 2 + fkg);
+    offFA[kk] = lds_chunk_off<CPR>(wm * WTM + frow, kk * KG + fkg);
+    offFB[kk] = lds_chunk_off<CPR>(wn * WTN + frow, kk * KG + fkg);
   }
-  half8_t fa[2][TM], fb[2][TN];
+  half8_t fa[2][FM], fb[2][FN];
   auto load_frags = [&](int slot, const unsigned char* cA, const unsigned char* cB, int kk) {
 #pragma unroll
-    for (int i = 0; i < TM; i++) fa[slot][i] = *(const half8_t*)(cA + offFA[i][kk]);
+    for (int i = 0; i < FM; i++) fa[slot][i] = *(const half8_t*)(cA + offFA[kk] + i * FSTEP);
 #pragma unroll
-    for (int j = 0; j < TN; j++) fb[slot][j] = *(const half8_t*)(cB + offFB[j][kk]);
+    for (int j = 0; j < FN; j++) fb[slot][j] = *(const half8_t*)(cB + offFB[kk] + j * FSTEP);
   };
   auto mfmas = [&](int slot) {
 #pragma unroll
-    for (int i = 0; i < TM; i++)
+    for (int i = 0; i < FM; i++)
 #pragma unroll
-      for (int j = 0; j < TN; j++)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[slot][j], fa[slot][i], acc[i][j],
-                                                           0, 0, 0);
+      for (int j = 0; j < FN; j++) {
+        if constexpr (MI16)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[slot][j], fa[slot][i], acc[i][j],
+                                                             0, 0, 0);
+        else
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[slot][j], fa[slot][i], acc[i][j],
+                                                             0, 0, 0);
+      }
   };
   // Slice kt.  (cA, cB): its stages; (nA, nB): those of slice kt+1 -- nB is filled here from
   // register set `nset`; dA: the A stage refilled with slice kt+2; `fset`: the register set
@@ -1205,21 +1212,27 @@ __global__ __launch_bounds__(WM* WN * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a
     fetchQ(fset);
     dmaA(dA);
     __builtin_amdgcn_sched_barrier(0);
+    // first k-step: the fragments of the second are read and the slice's LB 8-weight chunks are
+    // dequantised, their VALU work and LDS writes filling the gaps between its MFMAs
 #pragma unroll
     for (int kk = 0; kk < KK; kk++) {
       if (kk + 1 < KK) load_frags((kk + 1) & 1, cA, cB, kk + 1);
-      // one 8-weight chunk is dequantised per k-step: its VALU work and its LDS write fill the
-      // gaps between the MFMAs of that step
-      if (kk < LB) dequant_store1(nset, nB, kk);
+      // the slice's LB 8-weight chunks are dequantised one per k-step (32x32x16) or all in the
+      // first (16x16x32): their VALU work and LDS writes fill the gaps between that step's MFMAs
+      constexpr int PER_CHUNK = MI16 ? FM * FN / LB : FM * FN;  // MFMAs per chunk
+      const bool chunks_here = MI16 ? kk == 0 : kk < LB;
+      if (chunks_here) {
+        if constexpr (MI16) dequant_store(nset, nB); else dequant_store1(nset, nB, kk);
+      }
       mfmas(kk & 1);
       if (kk + 1 < KK) {
 #pragma unroll
-        for (int q = 0; q < TM * TN; q++) {
+        for (int q = 0; q < FM * FN; q++) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-          if (kk < LB) {
-            __builtin_amdgcn_sched_group_barrier(0x002, 20 / (TM * TN) + 1, 0);
-            if (q == TM * TN - 1) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+          if (chunks_here) {
+            __builtin_amdgcn_sched_group_barrier(0x002, 20 / PER_CHUNK + 1, 0);
+            if (q % PER_CHUNK == PER_CHUNK - 1) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
           }
         }
       }
@@ -1493,11 +1506,11 @@ hipError_t launch_stage(hipStream_t stream, const MatmulArgs& a) {
   return hipGetLastError();
 }
 
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, bool MI16>
 hipError_t launch_u8(hipStream_t stream, const MatmulArgs& a) {
   TileMap map = make_map(a, BM, BN);
   if (map.total < 0) return hipErrorInvalidConfiguration;
-  hipLaunchKernelGGL((gemm_nt_u8_kernel<BM, BN, WM, WN>), dim3((unsigned)map.total),
+  hipLaunchKernelGGL((gemm_nt_u8_kernel<BM, BN, WM, WN, MI16>), dim3((unsigned)map.total),
                      dim3(WM * WN * 64), 0, stream, a, map, __builtin_ctz(a.block_size));
   return hipGetLastError();
 }
@@ -1637,7 +1650,7 @@ GemmChoice choose(const MatmulArgs& a) {
       // N4096 m=129..512, K4096 59..65 -> 43..50 us, K11008 171..187 -> 129..141; with 96 tiles and
       // more, N12288, they lose: 69..76 -> 91..126)
       (int64_t)((a.m + 255) / 256) * ((a.n + 127) / 128) > 64) {
-    static const Candidate u8[] = {{U8_256x192, 256, 192, 1, 1.10f}, {U8_256x128, 256, 128, 1, 1.00f}};
+    static const Candidate u8[] = {{U8_256x192, 256, 192, 1, 1.10f}, {U8_256x128, 256, 128, 1, 1.05f}};
     return pick(a, u8, 2);
   }
   static const Candidate stage[] = {{STAGE_256x128, 256, 128, 2, 1.00f},
@@ -1741,8 +1754,8 @@ static hipError_t launch_choice(hipStream_t stream, const MatmulArgs& a, GemmCho
   switch (c) {
     case SHORTK_64: return launch_shortk<8>(stream, a);
     case SHORTK_128: return launch_shortk<16>(stream, a);
-    case U8_256x192: return launch_u8<256, 192, 4, 2>(stream, a);
-    case U8_256x128: return launch_u8<256, 128, 4, 2>(stream, a);
+    case U8_256x192: return launch_u8<256, 192, 4, 2, false>(stream, a);
+    case U8_256x128: return launch_u8<256, 128, 4, 2, true>(stream, a);
     case DMA_256x192: return launch_dma<256, 192, 4, 2, 6, 1, false, 64, true>(stream, a);
     case DMA_256x128: return launch_dma<256, 128, 4, 2, 3, 1, false, 64, true>(stream, a);
     case DMA_128x128: return launch_dma<128, 128, 2, 2, 3, 1>(stream, a);
