@@ -478,14 +478,18 @@ def test_large_tile_kernel_every_k_tail_exact(K):
     assert torch.equal(out.view(torch.int16), want.view(torch.int16))
 
 
+# (M, N, the tile the choice model gives the shape at K >= 2048)
+TILE_SHAPES = [(2000, 8184, "256x128"), (630, 12280, "128x256"), (380, 12280, "128x192")]
+
+
 @pytest.mark.parametrize("K", [2048, 2112, 2176, 2240, 2304, 2368])
-def test_256x128_tile_every_k_tail_exact(K):
-    """The 256 x 128 kernel (16x16x32 MFMAs, three LDS stages) on two whole rounds of tiles:
-    every remainder of its three-slice loop on inputs whose fp32 sums are exact, ragged last
-    tile row and column."""
-    M, N = 2000, 8184
+@pytest.mark.parametrize("M,N,tile", TILE_SHAPES)
+def test_large_tiles_every_k_tail_exact(K, M, N, tile):
+    """The 256 x 128 and 128 x 256 kernels (16x16x32 MFMAs) and the 128 x 192 kernel (32x32x16),
+    three LDS stages each: every remainder of the three-slice loop on inputs whose fp32 sums are
+    exact, ragged last tile row and column."""
     so, sl, sr = nt_strides(M, K, N)
-    assert plan(1, M, K, N, so, sl, sr) == "gemm_nt_mfma_dma_256x128x64"
+    assert plan(1, M, K, N, so, sl, sr) == f"gemm_nt_mfma_dma_{tile}x64"
     gen = torch.Generator(device="cuda").manual_seed(K)
     a = (torch.randint(-4, 5, (M, K), generator=gen, device="cuda").float() / 64).half()
     w = (torch.randint(-4, 5, (N, K), generator=gen, device="cuda").float() / 64).half()
@@ -497,13 +501,15 @@ def test_256x128_tile_every_k_tail_exact(K):
 
 @pytest.mark.parametrize("store", STORES_EXACT + STORES_F32)
 @pytest.mark.parametrize("mask", [oracle.MASK_NONE, oracle.MASK_CAUSAL])
-def test_256x128_tile_epilogues_against_the_slow_kernel(store, mask):
-    """Every store operator and the causal mask through the epilogue of the 256 x 128 tile (its
-    accumulators are 16 x 16 blocks), compared with the step-for-step kernel on bands of rows
-    (first tile row, a diagonal tile, the ragged last rows)."""
-    M, K, N = 4000, 2048, 4090 - 2
+@pytest.mark.parametrize("M,N,tile", [(4000, 4088, "256x128"), (630, 12280, "128x256"), (380, 12280, "128x192")])
+def test_large_tile_epilogues_against_the_slow_kernel(store, mask, M, N, tile):
+    """Every store operator and the causal mask through the epilogues of the 256 x 128 and
+    128 x 256 tiles (accumulators in 16 x 16 blocks, the latter's staging slots in the right
+    operand's LDS stages) and of the 128 x 192 tile, compared with the step-for-step kernel on
+    bands of rows (first tile row, a diagonal tile, the ragged last rows)."""
+    K = 2048
     so, sl, sr = nt_strides(M, K, N)
-    assert plan(1, M, K, N, so, sl, sr, store=store, mask=mask) == "gemm_nt_mfma_dma_256x128x64"
+    assert plan(1, M, K, N, so, sl, sr, store=store, mask=mask) == f"gemm_nt_mfma_dma_{tile}x64"
     gen = torch.Generator(device="cuda").manual_seed(900 + store * 2 + mask)
     a = torch.randn(M, K, generator=gen, device="cuda").half()
     w = (torch.randn(N, K, generator=gen, device="cuda") * K ** -0.5).half()
@@ -512,7 +518,7 @@ def test_256x128_tile_epilogues_against_the_slow_kernel(store, mask):
     kw = dict(bias_t=bias, beta=0.7, scale=0.2, store=store, mask=mask)
     out = prev.clone()
     assert raw_matmul("adr_matmul_f16", out, a, w, 1, M, K, N, so, sl, sr, **kw) == 0
-    for r0, rows in ((0, 40), (1500, 72), (M - 30, 30)):
+    for r0, rows in ((0, 40), (M * 3 // 8, 72), (M - 30, 30)):
         # the causal mask compares absolute row numbers: run the band as a product of its own
         # with the columns it may see shifted accordingly (a band of the full problem on the
         # slow kernel = rows r0.. of a, previous output rows r0..)
