@@ -469,7 +469,7 @@ int adr_microbench_empty(adr_stream_t stream) {
 }
 
 int adr_microbench_mfma_f16(adr_stream_t stream, int blocks, int times, int pattern, float* sink) {
-  if (blocks <= 0 || times < 0 || pattern < 0 || pattern > 2) return ADR_EINVAL_SHAPE;
+  if (blocks <= 0 || times < 0 || pattern < 0 || pattern > 4) return ADR_EINVAL_SHAPE;
   if (!sink) return ADR_ENULL;
   if (int rc = check_device()) return rc;
   return (int)launch_microbench_mfma((hipStream_t)stream, blocks, times, pattern, sink);

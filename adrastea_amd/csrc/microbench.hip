@@ -86,6 +86,61 @@ __global__ __launch_bounds__(256) void mfma_rotating_kernel(int times, float* si
   sink[id] = s;
 }
 
+// The two MFMA shapes on a wavefront's 128 x 128 tile, as a GEMM's k-steps issue them: every
+// block (row fragment i, column fragment j) of the tile once per k-step, fragments alternating
+// between two register sets from one k-step to the next, random data, no memory traffic.
+// WIDE: 4 x 4 blocks of v_mfma_f32_32x32x16_f16 (2 k-steps = 32 instructions = 2^20 flop per
+// iteration); otherwise 8 x 8 blocks of v_mfma_f32_16x16x32_f16 (2 k-steps = 128 instructions =
+// 2^21 flop).  Same flops per clock, but not the same power: the kernels choose between the
+// two by this measurement.  (Inline assembly ties every accumulator to its registers; the
+// builtins let the compiler move the 256 of them around between instructions.)
+template <bool WIDE>
+__global__ __launch_bounds__(256) void mfma_tile_kernel(int times, float* sink) {
+  constexpr int F = WIDE ? 4 : 8;
+  const uint32_t id = blockIdx.x * 256 + threadIdx.x;
+  half8_t a[2][F], b[2][F];
+#pragma unroll
+  for (int q = 0; q < 2; q++)
+#pragma unroll
+    for (int i = 0; i < F; i++)
+#pragma unroll
+      for (int e = 0; e < 8; e++) {
+        uint32_t h = ((id * 2 + q) * 64 + i * 8 + e) * 2654435761u;
+        h ^= h >> 15; h *= 2246822519u; h ^= h >> 13;
+        a[q][i][e] = bits_to_half((uint16_t)((h & 0x83ffu) | 0x3800u));
+        b[q][i][e] = bits_to_half((uint16_t)(((h >> 16) & 0x83ffu) | 0x3800u));
+      }
+  typedef typename std::conditional<WIDE, float16_t, float4_t>::type acc_t;
+  acc_t acc[F][F];
+#pragma unroll
+  for (int i = 0; i < F; i++)
+#pragma unroll
+    for (int j = 0; j < F; j++)
+#pragma unroll
+      for (int r = 0; r < (WIDE ? 16 : 4); r++) acc[i][j][r] = 0.0f;
+  for (int t = 0; t < times; t++) {
+#pragma unroll
+    for (int q = 0; q < 2; q++)
+#pragma unroll
+      for (int i = 0; i < F; i++)
+#pragma unroll
+        for (int j = 0; j < F; j++) {
+          if constexpr (WIDE)
+            asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(b[q][j]), "v"(a[q][i]));
+          else
+            asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(b[q][j]), "v"(a[q][i]));
+        }
+  }
+  float s = 0.0f;
+#pragma unroll
+  for (int i = 0; i < F; i++)
+#pragma unroll
+    for (int j = 0; j < F; j++)
+#pragma unroll
+      for (int r = 0; r < (WIDE ? 16 : 4); r++) s += acc[i][j][r];
+  sink[id] = s;
+}
+
 // Every workgroup reads one contiguous piece with 16-byte streaming loads (the access shape
 // that reads fastest on this part), four loads in flight per lane.
 __global__ __launch_bounds__(256) void stream_read_kernel(const u32x4_t* p, int64_t n16,
@@ -114,7 +169,11 @@ hipError_t launch_microbench_empty(hipStream_t stream) {
 }
 
 hipError_t launch_microbench_mfma(hipStream_t stream, int blocks, int times, int pattern, float* sink) {
-  if (pattern == 2)
+  if (pattern == 4)
+    hipLaunchKernelGGL(mfma_tile_kernel<false>, dim3(blocks), dim3(256), 0, stream, times, sink);
+  else if (pattern == 3)
+    hipLaunchKernelGGL(mfma_tile_kernel<true>, dim3(blocks), dim3(256), 0, stream, times, sink);
+  else if (pattern == 2)
     hipLaunchKernelGGL(mfma_rotating_kernel, dim3(blocks), dim3(256), 0, stream, times, sink);
   else
     hipLaunchKernelGGL(mfma_loop_kernel, dim3(blocks), dim3(256), 0, stream, times, pattern, sink);

@@ -361,6 +361,13 @@ def main():
                             (2, "mfma_loop_f32_f16 (random operands, changing with every instruction)")):
             rows.append(run(nm, flop, lambda: ok(lib.adr_microbench_mfma_f16(
                 stream(), blocks, times_, pattern, sink.data_ptr())), "TFLOP/s"))
+        # the two MFMA shapes on a 128 x 128 wavefront tile, random operands: what decides which
+        # one the GEMM kernels issue
+        for pattern, nm, per in ((3, "mfma 32x32x16 on a 128x128 wavefront tile (random operands)", 1 << 20),
+                                 (4, "mfma 16x16x32 on a 128x128 wavefront tile (random operands)", 1 << 21)):
+            t_ = 4000 if pattern == 3 else 2000
+            rows.append(run(nm, blocks * 4 * t_ * per, lambda: ok(lib.adr_microbench_mfma_f16(
+                stream(), blocks, t_, pattern, sink.data_ptr())), "TFLOP/s"))
         nbytes = 1 << 30
         src = torch.ones(nbytes, dtype=torch.uint8, device=dev)
         sink32 = torch.zeros(1, dtype=torch.int32, device=dev)

@@ -329,6 +329,11 @@ int adr_matmul_f16_ws_plan(char* name, int32_t cap, int32_t batches, int32_t m, 
  *                            zero operands, 1: pseudo-random fp16 operands, 2: pseudo-random
  *                            operands that change with every instruction as in a product's
  *                            inner loop (2 x 2 sub-tiles, fragments rotated in registers).
+ *                            Patterns 3 and 4 compare the two MFMA shapes on a wavefront's
+ *                            128 x 128 tile, random operands alternating between two register
+ *                            sets per k-step: 3: times x 32 v_mfma_f32_32x32x16_f16 (2^20 flop
+ *                            per wavefront and unit of `times`), 4: times x 128
+ *                            v_mfma_f32_16x16x32_f16 (2^21 flop).
  *                            `sink` receives blocks * 256 floats.
  *   adr_microbench_stream_read  reads `bytes` (a multiple of 16 * blocks) from `src` with
  *                            `blocks` workgroups, one contiguous piece each; `sink`: 4 bytes.

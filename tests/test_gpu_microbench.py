@@ -18,7 +18,7 @@ def test_empty_and_argument_checks():
     assert L.adr_microbench_empty(stream()) == 0
     sink = torch.zeros(256, device="cuda")
     assert L.adr_microbench_mfma_f16(stream(), 0, 1, 0, sink.data_ptr()) == _ffi.ADR_EINVAL_SHAPE
-    assert L.adr_microbench_mfma_f16(stream(), 1, 1, 3, sink.data_ptr()) == _ffi.ADR_EINVAL_SHAPE
+    assert L.adr_microbench_mfma_f16(stream(), 1, 1, 5, sink.data_ptr()) == _ffi.ADR_EINVAL_SHAPE
     assert L.adr_microbench_mfma_f16(stream(), 1, 1, 0, None) == _ffi.ADR_ENULL
     buf = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda")
     s32 = torch.zeros(1, dtype=torch.int32, device="cuda")
@@ -53,3 +53,12 @@ def test_mfma_loop_multiplies():
     torch.cuda.synchronize()
     assert torch.isfinite(r4).all() and (r4 != 0).any()
     assert torch.allclose(r8, 2 * r4, rtol=1e-4, atol=1e-3)
+    # the two MFMA shapes on a 128 x 128 wavefront tile: an iteration sums the same products again
+    for pattern in (3, 4):
+        t1 = torch.full((blocks * 256,), -1.0, device="cuda")
+        t2 = torch.full((blocks * 256,), -1.0, device="cuda")
+        assert L.adr_microbench_mfma_f16(stream(), blocks, 1, pattern, t1.data_ptr()) == 0
+        assert L.adr_microbench_mfma_f16(stream(), blocks, 2, pattern, t2.data_ptr()) == 0
+        torch.cuda.synchronize()
+        assert torch.isfinite(t1).all() and (t1 != 0).any()
+        assert torch.allclose(t2, 2 * t1, rtol=1e-4, atol=1e-2)
