@@ -274,6 +274,9 @@ static bool skinny_ok(const MatmulArgs& a) {
   // kernels are ahead (K4096 N12288 m=64: 38.8 against 29 us; N8192 and narrower: 38.7 against
   // 42.4, 14.0 against 14.4, K11008 N4096 31.9 against 53)
   if (a.m > 48 && a.n >= 40 * device_info_for_plan().cus) return false;
+  // the same from 33 rows on where K is short of 8192 (K5120 N13824 m=48: 31.4 against 42.9 us,
+  // K4096 N32000: 57.5 against 66.1; K8192 N22016 stays: 78.2 against 82.1)
+  if (a.m > 32 && a.n >= 40 * device_info_for_plan().cus && a.k < 8192) return false;
   // (one to four rows: only where the dot-product kernel does not reach, K > 12288 --
   // K13824 N5120 m=4: 53 us on the tiled kernels, 33 here)
   return a.m >= 1 && a.m <= 64;
@@ -306,11 +309,28 @@ bool gemv_f16_supported(const MatmulArgs& a, const char** name) {
 
 hipError_t launch_gemv_f16(hipStream_t stream, const MatmulArgs& a) {
   if (choose_skinny(a) == SKINNY_MFMA) {
-    // weight rows per workgroup: as few as still give (nearly) every CU a workgroup (N4096: 16
-    // rows, 256 workgroups, K11008 m=16 27.2 us against 39.5 with 32 rows; N12288: 48 rows,
-    // 25.7 against 28.7 with 16; N11008: 48 rows 25.2 against 31.7 with 32)
+    // Groups of 16 weight rows per workgroup (measured over K 4096 .. 22016, N 4096 .. 32000):
+    // one where that gives at most one workgroup per CU (N4096: K11008 m=16 27.2 us against 39.5
+    // with two); two where one would leave a second, mostly empty round (N5120: K13824 m=64 52
+    // against 68 us); beyond that, with up to 16 activation rows, one again -- two workgroups fit a
+    // CU then and many short ones balance best (N8192 m=16 27 against 34 us, N17920 m=8 44
+    // against 52); with more activation rows a workgroup re-reads more activations than it
+    // reads weights unless it owns three groups (N12288 m=32: 23.2 against 25.1 with one), or
+    // two where three would leave a nearly empty last round (N13824: 288 workgroups).
     const int cus = device_info_for_plan().cus;  // MI355X: 256
-    const int rg = a.n >= 40 * cus ? 3 : a.n >= 24 * cus ? 2 : 1;
+    const int groups = (a.n + 15) / 16;
+    int rg;
+    if (groups <= cus) {
+      rg = 1;
+    } else if (groups <= 28 * cus / 16) {
+      rg = 2;
+    } else if (a.m <= 16) {
+      rg = 1;
+    } else {
+      rg = a.n >= 40 * cus ? 3 : 2;
+      const int w3 = (a.n + 47) / 48;
+      if (rg == 3 && w3 > cus && w3 <= 2 * cus && w3 % cus <= cus / 4) rg = 2;
+    }
     switch ((a.m + 15) / 16) {  // blocks of sixteen activation rows
 #define ADR_REG_CASE(MB, RG3)                                            \
       case MB:                                                           \
