@@ -547,11 +547,16 @@ hipError_t launch_regstream(hipStream_t stream, half_t* out, const half_t* lhs, 
 }
 
 // groups of sixteen weight rows per workgroup: as many as still give every compute unit a
-// workgroup (at most three: 48 rows share one fetch of the activations)
+// workgroup (at most three: 48 rows share one fetch of the activations), but never a count that
+// leaves a second, nearly empty round of workgroups (N5120, 320 groups: two per workgroup, K13824
+// m=32 39.3 -> 31.4 us; N13824, 288 workgroups of three: two, K5120 m=32 39.0 -> 29.7)
 int regstream_row_groups(int n) {
   const int cus = device_info_for_plan().cus;
   const int groups = (n + ROWS - 1) / ROWS;
-  return groups >= 3 * cus - cus / 2 ? 3 : groups >= 2 * cus - cus / 2 ? 2 : 1;
+  if (groups <= cus) return 1;
+  if (groups < 3 * cus - cus / 2) return 2;
+  const int w3 = (groups + 2) / 3;
+  return w3 > cus && w3 <= 2 * cus && w3 % cus <= cus / 4 ? 2 : 3;
 }
 
 // MR activation rows, NW wavefronts, RPB weight rows per workgroup, SEGW 1 KiB K segments per
