@@ -94,7 +94,9 @@ __global__ __launch_bounds__(256, 2) void attention_fwd_kernel(AttnArgs a) {
   __shared__ __attribute__((aligned(1024))) unsigned char sV0[TILE];
   __shared__ __attribute__((aligned(1024))) unsigned char sV1[TILE];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // (the wavefront index as a scalar: everything derived from it -- LDS stage addresses of the
+  // transfers, role branches -- then stays out of the vector registers and the vector ALU)
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int frow = lane & 31, g = lane >> 5;
   const bool causal = a.mask == ADR_MASK_CAUSAL;
 

@@ -474,7 +474,9 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   const int piece = SPLIT ? (int)(blockIdx.x / (unsigned)map.total) : 0;
   map_tile(map, batch, tile_m, tile_n, tile_id);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  // (the wavefront index as a scalar: everything derived from it -- LDS stage addresses of the
+  // transfers, role branches -- then stays out of the vector registers and the vector ALU)
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WN, wn = wave % WN;
   half_t* const out = a.output + (int64_t)batch * a.stride_oz;
 
@@ -765,7 +767,7 @@ __global__ __launch_bounds__(WM* WN * 64) void splitk_reduce_kernel(MatmulArgs a
   int batch, tile_m, tile_n;
   map_tile(map, batch, tile_m, tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WN, wn = wave % WN;
   half_t* const out = a.output + (int64_t)batch * a.stride_oz;
   if (a.mask == ADR_MASK_CAUSAL && n0 > m0 + BM - 1) {
@@ -832,7 +834,7 @@ __global__ __launch_bounds__(1024, 1) void gemm_nt_shortk_kernel(MatmulArgs a, S
   // staging tile: row r = 256 bytes, 16-byte chunk c at position c ^ (r & 15)
   __shared__ __attribute__((aligned(1024))) unsigned char sC[BM * BN * 2];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int G = gridDim.x;
   // Workgroup g runs on die g % 8: the workgroups of a die take neighbouring units (they share
   // right panels in the die's L2).  Odd rounds walk the workgroups backwards, which pairs long
@@ -1112,7 +1114,7 @@ __global__ __launch_bounds__(WM* WN * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a
   int batch, tile_m, tile_n;
   map_tile(map, batch, tile_m, tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WN, wn = wave % WN;
   half_t* const out = a.output;
 
@@ -1303,7 +1305,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_stage_kernel(Matmul
   int batch, tile_m, tile_n;
   map_tile(map, batch, tile_m, tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WN, wn = wave % WN;
   half_t* const out = a.output + (int64_t)batch * a.stride_oz;
 
