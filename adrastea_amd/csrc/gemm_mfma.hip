@@ -5,26 +5,32 @@
 // and the attention score product Q.K^T on the interleaved-head views of llama.rs:534-550.
 // Row strides (stride_ly, stride_rx, stride_oy) and batch strides are free.
 //
-// Two kernels share the tiling, the LDS layout and the epilogue:
+// The kernels share the tiling, the LDS layout and the epilogue:
 //
 //  gemm_nt_dma_kernel   K % 64 == 0, plain fp16 operands.  K slices of depth 64 go from global
 //                       memory straight into LDS (global_load_lds_dwordx4, no register round
-//                       trip) into 2 or 3 statically separate LDS stages, so the loads of the
-//                       next one or two slices are in flight while the current slice feeds the
-//                       MFMAs; one barrier per slice.  MFMA fragments are prefetched one k-step
-//                       ahead and interleaved with the MFMAs by scheduling-group barriers.
+//                       trip) into statically separate LDS stages (three per operand, or two of
+//                       the left and four of the right operand with the transfers split by
+//                       wavefront role), so the loads of the next slices are in flight while
+//                       the current slice feeds the MFMAs; one barrier per slice.  MFMA
+//                       fragments are prefetched one k-step ahead and interleaved with the
+//                       MFMAs by scheduling-group barriers.
+//  gemm_nt_u8_kernel    the same with u8 weights dequantised on their way into LDS.
+//  gemm_nt_shortk_kernel  K = 64 / 128 (the attention score product): persistent workgroups.
 //  gemm_nt_stage_kernel any K % 8 == 0, and the variants that must touch the data on the way
 //                       in: u8 weights dequantised while staging (adr_matmul_nt_fp16u8), and
 //                       the Load Scale operator.  Global -> registers -> LDS, two LDS stages.
 //
 // One workgroup owns a BM x BN output tile, WM x WN wavefronts each own a (BM/WM) x (BN/WN)
-// sub-tile as 32x32 fp32 accumulators of v_mfma_f32_32x32x16_f16.  LDS rows are XOR-swizzled
-// at 16-byte granularity over 256-byte lines (64 banks) so that the 128-bit fragment reads of
-// 16 consecutive rows are conflict-free (SQ_LDS_BANK_CONFLICT reads 0).  Accumulators are kept
-// TRANSPOSED (the weight fragment is the first MFMA operand) so that a lane owns 4 consecutive
-// output columns; the epilogue narrows them to fp16, transposes through a per-wavefront LDS
-// slot and writes whole 16-byte chunks of output rows, applying the store operator, the bias
-// and the causal mask on the way.
+// sub-tile as fp32 accumulator blocks: 16 x 16 blocks of v_mfma_f32_16x16x32_f16 in the tiles
+// with 256 rows or columns (more flops within the part's power limit), 32 x 32 blocks of
+// v_mfma_f32_32x32x16_f16 in the smaller ones.  LDS rows are XOR-swizzled at 16-byte granularity
+// over 256-byte lines (64 banks) so that the 128-bit fragment reads of 16 consecutive rows are
+// conflict-free (SQ_LDS_BANK_CONFLICT reads 0).  Accumulators are kept TRANSPOSED (the weight
+// fragment is the first MFMA operand) so that a lane owns 4 consecutive output columns; the
+// epilogue narrows them to fp16, transposes through a per-wavefront LDS slot and writes whole
+// 16-byte chunks of output rows, applying the store operator, the bias and the causal mask on
+// the way.
 #include <stdint.h>
 #include <type_traits>
 
