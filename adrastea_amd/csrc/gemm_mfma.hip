@@ -1462,7 +1462,12 @@ TileMap make_map(const MatmulArgs& a, int bm, int bn) {
   map.tiles_per_batch = map.tiles_m * map.tiles_n;
   const int64_t total = (int64_t)map.tiles_per_batch * a.batches;
   map.total = total > 0x7fffffffLL ? -1 : (int)total;
-  map.group_m = map.tiles_m < 8 ? map.tiles_m : 8;
+  // tile rows per group: a die holds 32 tiles of 256 rows at a time (64 of the smaller ones); g
+  // rows x 32/g columns of them fetch g * bm + 32/g * bn operand rows per K slice, least near
+  // g = sqrt(32 bn / bm): 4 for the 256-row tiles (qkv: 21.0 instead of 23.1 MB per die and
+  // round), 8 for the others
+  const int g = bm >= 256 ? 4 : 8;
+  map.group_m = map.tiles_m < g ? map.tiles_m : g;
   map.xcds = device_info_for_plan().xcds;
   map.splits = 1;
   return map;
