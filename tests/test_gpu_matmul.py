@@ -344,6 +344,29 @@ def test_row_and_batch_strides_with_padding_on_the_fast_path():
     assert np.array_equal(to_np(o_t).view(np.uint16), want.view(np.uint16))  # gaps untouched too
 
 
+@pytest.mark.parametrize("B,M,K,N,tile", [(2, 600, 1088, 6136, "128x256"), (2, 380, 1088, 6136, "128x192"),
+                                          (2, 1000, 1088, 4088, "256x128"), (3, 1000, 1088, 3064, "256x192")])
+def test_batched_padded_operands_on_the_large_tiles(B, M, K, N, tile):
+    """Batches with row pitches wider than the rows and batch strides wider than the matrices on
+    every large tile (16 x 16 and 32 x 32 accumulator blocks), exact inputs; whatever lies between
+    the rows and after the last batch of the output must stay as it was."""
+    ly, rx, oy = K + 8, K + 16, N + 8
+    lz, rz, oz = M * ly + 64, N * rx + 24, M * oy + 16
+    so, sl, sr = (1, oy, oz), (1, ly, lz), (rx, 1, rz)
+    assert plan(B, M, K, N, so, sl, sr) == f"gemm_nt_mfma_dma_{tile}x64"
+    gen = torch.Generator(device="cuda").manual_seed(B * M + N)
+    lbuf = (torch.randint(-4, 5, (B * lz + 8,), generator=gen, device="cuda").float() / 64).half()
+    rbuf = (torch.randint(-4, 5, (B * rz + 8,), generator=gen, device="cuda").float() / 64).half()
+    obuf = torch.full((B * oz + 8,), 5.0, dtype=torch.float16, device="cuda")
+    assert raw_matmul("adr_matmul_f16", obuf, lbuf, rbuf, B, M, K, N, so, sl, sr) == 0
+    want = torch.full_like(obuf, 5.0)
+    for b in range(B):
+        a = torch.as_strided(lbuf, (M, K), (ly, 1), b * lz).double()
+        w = torch.as_strided(rbuf, (N, K), (rx, 1), b * rz).double()
+        torch.as_strided(want, (M, N), (oy, 1), b * oz).copy_((a @ w.t()).half())
+    assert torch.equal(obuf.view(torch.int16), want.view(torch.int16))
+
+
 def test_unsupported_layouts_fall_back_and_stay_correct():
     g = rng(550)
     B, M, K, N = 1, 40, 50, 30   # K % 8 != 0
