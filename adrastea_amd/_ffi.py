@@ -12,6 +12,7 @@ SYMBOLS = (
     "adr_matmul_f16", "adr_matmul_f16_slow", "adr_matmul_f16_raw", "adr_matmul_nt_f16",
     "adr_matmul_f16_ws", "adr_matmul_f16_workspace_bytes", "adr_matmul_f16_ws_plan",
     "adr_matmul_f16_noalloc",
+    "adr_set_held_workspace_limit", "adr_held_workspace_limit", "adr_held_workspace_bytes",
     "adr_matmul_nt_fp16u8", "adr_matmul_nt_fp16u8_ws", "adr_matmul_nt_fp16u8_workspace_bytes",
     "adr_dequantize_absmax_u8", "adr_quantize_absmax_u8",
     "adr_dequantize_absmax_uint8", "adr_quantize_absmax_uint8", "adr_matmul_f16_plan",
@@ -24,6 +25,7 @@ ADR_OK, ADR_EINVAL_SHAPE, ADR_EINVAL_ENUM, ADR_ENOTIMPL, ADR_ENULL, ADR_EDIVISIB
     0, -1, -2, -3, -4, -5)
 ADR_EUNSUPPORTED_DEVICE, ADR_EUNSUPPORTED_LAYOUT, ADR_ESCRATCH = -6, -7, -8
 NOALLOC_SCRATCH_BYTES = 16 * 1024 * 1024
+HELD_WORKSPACE_DEFAULT_BYTES = 128 * 1024 * 1024
 
 
 class TensorDesc(C.Structure):
@@ -56,6 +58,11 @@ def lib():
     L.adr_matmul_f16_slow.argtypes = mm
     L.adr_matmul_f16_ws.argtypes = mm + [vp, C.c_int64]
     L.adr_matmul_f16_noalloc.argtypes = mm
+    L.adr_set_held_workspace_limit.argtypes = [C.c_int64]
+    L.adr_held_workspace_limit.argtypes = []
+    L.adr_held_workspace_limit.restype = C.c_int64
+    L.adr_held_workspace_bytes.argtypes = []
+    L.adr_held_workspace_bytes.restype = C.c_int64
     L.adr_matmul_f16_workspace_bytes.argtypes = [i32] * 13 + [u32, u32, u32]
     L.adr_matmul_f16_ws_plan.argtypes = [C.c_char_p, i32] + [i32] * 13 + [u32, u32, u32, C.c_int64]
     L.adr_matmul_f16_raw.argtypes = [vp, vp, vp, vp] + [i32] * 13

@@ -214,9 +214,10 @@ hipError_t launch_matmul_general(hipStream_t stream, const MatmulArgs& a);
 // Returns true and fills `name` when the MFMA kernel family covers these arguments.
 bool mfma_gemm_supported(const MatmulArgs& a, const char** name);
 hipError_t launch_mfma_gemm(hipStream_t stream, const MatmulArgs& a);
-// Scratch bytes the split-K form of these arguments would use (0: no split pays here); the
-// kernel family splits only when a.workspace holds at least this much.
-int64_t mfma_gemm_workspace_bytes(const MatmulArgs& a);
+// Scratch bytes the split-K form of these arguments would use when at most `avail` bytes can be
+// had (0: no split pays here, or none fits); the kernel family splits that way when a.workspace
+// holds at least this much.
+int64_t mfma_gemm_workspace_bytes(const MatmulArgs& a, int64_t avail = INT64_MAX);
 // fp16 skinny matmul (m <= 32, K-contiguous operands): true when a streaming kernel covers it.
 bool gemv_f16_supported(const MatmulArgs& a, const char** name);
 hipError_t launch_gemv_f16(hipStream_t stream, const MatmulArgs& a);

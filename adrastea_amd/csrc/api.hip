@@ -3,6 +3,7 @@
 #include <string.h>
 
 #include <atomic>
+#include <mutex>
 
 #include "adr_common.hpp"
 
@@ -130,6 +131,104 @@ void* scratch_on_current_device(hipError_t* err) {
   return p;
 }
 
+// ---- workspace the plain entry points hold themselves -------------------------------------------
+// adr_matmul_f16, adr_matmul_nt_f16 and adr_matmul_nt_fp16u8 have the reference's argument tuples
+// and therefore no workspace argument.  Where a workspace pays (K split over workgroups; the u8
+// matrix dequantised once) they take it from a cache that grows on demand: one buffer per
+// (device, stream), since launches on one stream run in order and launches on different streams
+// may overlap.  A buffer that has become too small is replaced and not freed (kernels in flight
+// may still use it, and freeing would synchronise the device); sizes double from 16 MiB up to the
+// limit, so the memory given up that way stays below the size of the buffer in use.
+constexpr int MAX_HELD = 64;
+constexpr int64_t HELD_FLOOR = (int64_t)16 << 20;
+struct Held {
+  int device;
+  hipStream_t stream;
+  void* ptr;
+  int64_t bytes;
+};
+std::mutex held_mutex;
+Held held[MAX_HELD];
+int held_count = 0;
+int64_t held_total = 0;  // bytes allocated so far, replaced buffers included
+std::atomic<int64_t> held_limit{ADR_HELD_WORKSPACE_DEFAULT_BYTES};
+
+// May this call use (and if need be allocate) a held buffer on `stream`?  Not while the stream is
+// being captured: the launches would tie the buffer into a graph that can be replayed on any stream
+// at any time.  Not on the per-thread default stream, whose handle names a different stream in
+// every thread.
+bool held_allowed(hipStream_t stream) {
+  if (stream == hipStreamPerThread) return false;
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &st) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return st == hipStreamCaptureStatusNone;
+}
+
+// A buffer of at least `want` bytes for (current device, stream), or null (then the caller runs
+// without one).  held_mutex is held by the caller, and stays held over the launches that use the
+// buffer, so that two threads launching on one stream cannot interleave their pairs of launches.
+void* held_buffer(hipStream_t stream, int64_t want, int64_t* bytes) {
+  const int64_t limit = held_limit.load(std::memory_order_relaxed);
+  if (want <= 0 || want > limit) return nullptr;
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+  Held* h = nullptr;
+  for (int i = 0; i < held_count; i++)
+    if (held[i].device == dev && held[i].stream == stream) h = &held[i];
+  if (h && h->bytes >= want) {
+    *bytes = h->bytes;
+    return h->ptr;
+  }
+  if (!h && held_count == MAX_HELD) return nullptr;
+  int64_t size = HELD_FLOOR;
+  while (size < want) size *= 2;
+  if (size > limit) size = limit;
+  // (an allocation is an "unsafe" call for a capture in global mode that some other stream of the
+  // process may be in; it touches no stream, so it is made in relaxed mode)
+  hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+  (void)hipThreadExchangeStreamCaptureMode(&mode);
+  void* p = nullptr;
+  const hipError_t e = hipMalloc(&p, (size_t)size);
+  (void)hipThreadExchangeStreamCaptureMode(&mode);
+  if (e != hipSuccess || !p) {
+    (void)hipGetLastError();  // out of memory: the product runs without a workspace
+    return nullptr;
+  }
+  if (!h) {
+    h = &held[held_count++];
+    h->device = dev;
+    h->stream = stream;
+  }
+  h->ptr = p;
+  h->bytes = size;
+  held_total += size;
+  *bytes = size;
+  return p;
+}
+
+// run_matmul for the entry points without a workspace argument.
+int run_matmul_held(hipStream_t stream, MatmulArgs& a) {
+  if (empty(a)) return ADR_OK;
+  if (int rc = check_device()) return rc;
+  const char* name;
+  const int64_t limit = held_limit.load(std::memory_order_relaxed);
+  // (a product that would like more than the limit is cut into fewer pieces, or not at all)
+  const int64_t need = limit > 0 && !gemv_f16_supported(a, &name) ? mfma_gemm_workspace_bytes(a, limit) : 0;
+  if (need > 0 && held_allowed(stream)) {
+    std::lock_guard<std::mutex> lock(held_mutex);
+    int64_t bytes = 0;
+    if (void* p = held_buffer(stream, need, &bytes)) {
+      a.workspace = (float*)p;
+      a.workspace_bytes = bytes;
+      return run_matmul(stream, a, true);
+    }
+  }
+  return run_matmul(stream, a, true);
+}
+
 }  // namespace
 
 extern "C" {
@@ -165,7 +264,20 @@ int adr_matmul_f16(adr_stream_t stream, uint16_t* output, const uint16_t* lhs, c
                       stride_lx, stride_ly, stride_lz, stride_rx, stride_ry, stride_rz, bias, beta,
                       scale, store, load, mask);
   if (int rc = validate_matmul(a, true)) return rc;
-  return run_matmul((hipStream_t)stream, a, true);
+  return run_matmul_held((hipStream_t)stream, a);
+}
+
+int adr_set_held_workspace_limit(int64_t bytes) {
+  if (bytes < 0) return ADR_EINVAL_SHAPE;
+  held_limit.store(bytes, std::memory_order_relaxed);
+  return ADR_OK;
+}
+
+int64_t adr_held_workspace_limit(void) { return held_limit.load(std::memory_order_relaxed); }
+
+int64_t adr_held_workspace_bytes(void) {
+  std::lock_guard<std::mutex> lock(held_mutex);
+  return held_total;
 }
 
 int adr_matmul_f16_ws(adr_stream_t stream, uint16_t* output, const uint16_t* lhs, const uint16_t* rhs,
@@ -287,8 +399,9 @@ int adr_matmul_f16_ws_plan(char* name, int32_t cap, int32_t batches, int32_t m, 
   return ADR_OK;
 }
 
-int adr_matmul_nt_f16(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
-                      const uint16_t* rhs, int32_t m, int32_t p, int32_t n, float beta) {
+// adr_matmul_nt_f16; `held`: may take the split-K workspace from the library's own cache
+static int nt_f16(adr_stream_t stream, uint16_t* output, const uint16_t* lhs, const uint16_t* rhs,
+                  int32_t m, int32_t p, int32_t n, float beta, bool held) {
   if (m < 0 || p < 0 || n < 0) return ADR_EINVAL_SHAPE;
   if (m == 0 || n == 0) return ADR_OK;
   if (!output || (p && (!lhs || !rhs))) return ADR_ENULL;
@@ -297,22 +410,12 @@ int adr_matmul_nt_f16(adr_stream_t stream, uint16_t* output, const uint16_t* lhs
     return ADR_EINVAL_SHAPE;  // (32-bit element offsets, as in adr_matmul_f16)
   MatmulArgs a = pack(output, lhs, rhs, 1, m, p, n, 1, n, 0, 1, p, 0, p, 1, 0, nullptr, beta, 1.0f,
                       STORE_ACC_BETA, ADR_LOAD_IDENTITY, ADR_MASK_NONE);
-  return run_matmul((hipStream_t)stream, a, true);
+  return held ? run_matmul_held((hipStream_t)stream, a) : run_matmul((hipStream_t)stream, a, true);
 }
 
-int adr_matmul_nt_fp16u8(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
-                         const uint8_t* rhs, const uint16_t* scales, int32_t m, int32_t p,
-                         int32_t n, int32_t block_size, float beta) {
-  if (m < 0 || p < 0 || n < 0 || block_size <= 0) return ADR_EINVAL_SHAPE;
-  if (p % block_size != 0) return ADR_EDIVISIBILITY;
-  if (m == 0 || n == 0) return ADR_OK;
-  if (!output || (p && (!lhs || !rhs || !scales))) return ADR_ENULL;
-  if ((int64_t)m * n >= ((int64_t)1 << 31) || (int64_t)m * p >= ((int64_t)1 << 31) ||
-      (int64_t)n * p >= ((int64_t)1 << 31))
-    return ADR_EINVAL_SHAPE;  // (32-bit element offsets, as in adr_matmul_f16)
-  if (int rc = check_device()) return rc;
-  return (int)launch_gemm_u8((hipStream_t)stream, (half_t*)output, (const half_t*)lhs, rhs,
-                             (const half_t*)scales, m, p, n, block_size, beta);
+int adr_matmul_nt_f16(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
+                      const uint16_t* rhs, int32_t m, int32_t p, int32_t n, float beta) {
+  return nt_f16(stream, output, lhs, rhs, m, p, n, beta, true);
 }
 
 // Where dequantising the matrix once and running the fp16 kernels beats the fused kernels
@@ -329,6 +432,56 @@ static bool u8_dequantise_first(int m, int p, int n) {
   return m <= 512 ? n <= 10240 : n < 8192;
 }
 
+static int validate_u8(const uint16_t* output, const uint16_t* lhs, const uint8_t* rhs,
+                       const uint16_t* scales, int32_t m, int32_t p, int32_t n, int32_t block_size,
+                       bool* nothing_to_do) {
+  *nothing_to_do = false;
+  if (m < 0 || p < 0 || n < 0 || block_size <= 0) return ADR_EINVAL_SHAPE;
+  if (p % block_size != 0) return ADR_EDIVISIBILITY;
+  if (m == 0 || n == 0) {
+    *nothing_to_do = true;
+    return ADR_OK;
+  }
+  if (!output || (p && (!lhs || !rhs || !scales))) return ADR_ENULL;
+  if ((int64_t)m * n >= ((int64_t)1 << 31) || (int64_t)m * p >= ((int64_t)1 << 31) ||
+      (int64_t)n * p >= ((int64_t)1 << 31))
+    return ADR_EINVAL_SHAPE;  // (32-bit element offsets, as in adr_matmul_f16)
+  return ADR_OK;
+}
+
+// the matrix dequantised into `workspace` (n * p halves), then the fp16 kernels on it
+static int u8_by_way_of_fp16(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
+                             const uint8_t* rhs, const uint16_t* scales, int32_t m, int32_t p,
+                             int32_t n, int32_t block_size, float beta, void* workspace) {
+  if (int rc = adr_dequantize_absmax_u8(stream, (uint16_t*)workspace, rhs, scales, n, p, block_size)) return rc;
+  return nt_f16(stream, output, lhs, (const uint16_t*)workspace, m, p, n, beta, false);
+}
+
+static int u8_fused(adr_stream_t stream, uint16_t* output, const uint16_t* lhs, const uint8_t* rhs,
+                    const uint16_t* scales, int32_t m, int32_t p, int32_t n, int32_t block_size,
+                    float beta) {
+  if (int rc = check_device()) return rc;
+  return (int)launch_gemm_u8((hipStream_t)stream, (half_t*)output, (const half_t*)lhs, rhs,
+                             (const half_t*)scales, m, p, n, block_size, beta);
+}
+
+int adr_matmul_nt_fp16u8(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
+                         const uint8_t* rhs, const uint16_t* scales, int32_t m, int32_t p,
+                         int32_t n, int32_t block_size, float beta) {
+  bool nothing;
+  if (int rc = validate_u8(output, lhs, rhs, scales, m, p, n, block_size, &nothing)) return rc;
+  if (nothing) return ADR_OK;
+  const int64_t need = u8_dequantise_first(m, p, n) ? (int64_t)n * p * 2 : 0;
+  if (need > 0 && need <= held_limit.load(std::memory_order_relaxed) && held_allowed((hipStream_t)stream)) {
+    if (int rc = check_device()) return rc;
+    std::lock_guard<std::mutex> lock(held_mutex);
+    int64_t bytes = 0;
+    if (void* ws = held_buffer((hipStream_t)stream, need, &bytes))
+      return u8_by_way_of_fp16(stream, output, lhs, rhs, scales, m, p, n, block_size, beta, ws);
+  }
+  return u8_fused(stream, output, lhs, rhs, scales, m, p, n, block_size, beta);
+}
+
 int64_t adr_matmul_nt_fp16u8_workspace_bytes(int32_t m, int32_t p, int32_t n, int32_t block_size) {
   if (m < 0 || p < 0 || n < 0 || block_size <= 0) return ADR_EINVAL_SHAPE;
   if (p % block_size != 0) return ADR_EDIVISIBILITY;
@@ -341,13 +494,13 @@ int adr_matmul_nt_fp16u8_ws(adr_stream_t stream, uint16_t* output, const uint16_
                             int64_t workspace_bytes) {
   if (workspace_bytes < 0 || (workspace_bytes > 0 && !workspace)) return ADR_ENULL;
   if ((uintptr_t)workspace % 16 != 0) return ADR_EINVAL_SHAPE;
-  if (m < 0 || p < 0 || n < 0 || block_size <= 0) return ADR_EINVAL_SHAPE;
-  if (p % block_size != 0) return ADR_EDIVISIBILITY;
+  bool nothing;
+  if (int rc = validate_u8(output, lhs, rhs, scales, m, p, n, block_size, &nothing)) return rc;
+  if (nothing) return ADR_OK;
+  // (only the caller's buffer is ever used here, never the library's own)
   if (!u8_dequantise_first(m, p, n) || workspace_bytes < (int64_t)n * p * 2)
-    return adr_matmul_nt_fp16u8(stream, output, lhs, rhs, scales, m, p, n, block_size, beta);
-  if (!output || !lhs || !rhs || !scales) return ADR_ENULL;
-  if (int rc = adr_dequantize_absmax_u8(stream, (uint16_t*)workspace, rhs, scales, n, p, block_size)) return rc;
-  return adr_matmul_nt_f16(stream, output, lhs, (const uint16_t*)workspace, m, p, n, beta);
+    return u8_fused(stream, output, lhs, rhs, scales, m, p, n, block_size, beta);
+  return u8_by_way_of_fp16(stream, output, lhs, rhs, scales, m, p, n, block_size, beta, workspace);
 }
 
 int adr_matmul_nt_fp16u8_plan(char* name, int32_t cap, int32_t m, int32_t p, int32_t n,

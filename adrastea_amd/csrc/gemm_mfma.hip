@@ -1849,8 +1849,8 @@ static const char* split_name(const SplitChoice& sc) {
   return names[t][sc.splits - 2];
 }
 
-int64_t mfma_gemm_workspace_bytes(const MatmulArgs& a) {
-  const SplitChoice sc = choose_split(a, INT64_MAX);
+int64_t mfma_gemm_workspace_bytes(const MatmulArgs& a, int64_t avail) {
+  const SplitChoice sc = choose_split(a, avail);
   return sc.tile == GEMM_NONE ? 0 : split_workspace_bytes(a, sc.bm, sc.bn, sc.splits);
 }
 

@@ -221,6 +221,36 @@ def main():
             del ws
         return rows
 
+    def short_prompt_set():
+        """fp16 products with the row counts of a short prompt (the reference's LLaMA issues them
+        for every generated token, llama.rs:456-483), as a caller without graphs makes them: eager
+        launches timed with events, weights rotated through > 600 MB.  `us`: the entry point as it
+        comes (K split over workgroups where that pays, through a buffer the library holds per
+        stream); `unsplit_us`: with adr_set_held_workspace_limit(0)."""
+        rows = []
+        for K, N in DECODE_SET:
+            per = N * K * 2
+            nbuf = max(2, int(600e6 // per) + 1)
+            ws = [randn_h(N, K, std=K ** -0.5) for _ in range(nbuf)]
+            for m in (96, 128, 256, 512):
+                a = randn_h(m, K)
+                o = torch.zeros(m, N, dtype=torch.float16, device=dev)
+                i = [0]
+
+                def f():
+                    j = i[0] % nbuf
+                    i[0] += 1
+                    mm(o, a, ws[j], m, K, N)
+                t = timed(f, 4 * nbuf, nbuf)
+                lib.adr_set_held_workspace_limit(0)
+                t0 = timed(f, 4 * nbuf, nbuf)
+                lib.adr_set_held_workspace_limit(_ffi.HELD_WORKSPACE_DEFAULT_BYTES)
+                rows.append({"M": m, "K": K, "N": N, "us": round(t * 1e6, 1),
+                             "unsplit_us": round(t0 * 1e6, 1),
+                             "tflops": round(2.0 * m * K * N / t / 1e12, 1)})
+            del ws
+        return rows
+
     def decode_set(ms=(1, 4, 16)):
         gemv = []
         for K, N in DECODE_SET:
@@ -406,7 +436,8 @@ def main():
         # (with the row counts of a short prompt: the reference's LLaMA re-runs the whole sequence
         # for every token, llama.rs:456-483, so these are calls it makes too)
         print(json.dumps({"u8_decode_gemv": decode_set(), "f16_decode_gemv": f16_decode_set(),
-                          "u8_17_to_128_rows": decode_set((32, 64, 128))}))
+                          "u8_17_to_128_rows": decode_set((32, 64, 128)),
+                          "f16_short_prompt_rows": short_prompt_set()}))
         return
 
     def u8_prefill_set():
@@ -426,9 +457,16 @@ def main():
                                               q.data_ptr(), s.data_ptr(), M, K, N, 32, 0.0)
                 if rc != 0:
                     raise RuntimeError(_ffi.strerror(rc))
+            # the entry point as it comes: from 96 rows on it dequantises the matrix once per call
+            # into a buffer the library holds per stream (adr_set_held_workspace_limit, 128 MiB by
+            # default) and runs the fp16 kernels on it; same bits as the fused kernels
+            timed(f, 30, 5)  # (discarded: the first calls allocate the buffer and find the clocks low)
             t = timed(f, 50, 5)
-            # the same product through adr_matmul_nt_fp16u8_ws with a workspace for the dequantised
-            # matrix (dequantised once per call, then the fp16 kernels; same bits)
+            # the fused kernels alone (dequantisation inside the GEMM's K loop, no buffer)
+            lib.adr_set_held_workspace_limit(0)
+            t_fused = timed(f, 50, 5)
+            lib.adr_set_held_workspace_limit(_ffi.HELD_WORKSPACE_DEFAULT_BYTES)
+            # the same product through adr_matmul_nt_fp16u8_ws with the caller's workspace
             ws = torch.empty(N * K * 2, dtype=torch.uint8, device=dev)
 
             def f_ws():
@@ -441,6 +479,8 @@ def main():
             u8p[name] = {"M": M, "K": K, "N": N, "us": round(t * 1e6, 1),
                          "tflops": round(2.0 * M * K * N / t / 1e12, 1),
                          "frac_mfma_peak": round(2.0 * M * K * N / t / 1e12 / PEAK_F16_TFLOPS, 4),
+                         "fused_kernel_us": round(t_fused * 1e6, 1),
+                         "fused_kernel_tflops": round(2.0 * M * K * N / t_fused / 1e12, 1),
                          "with_workspace_us": round(t_ws * 1e6, 1),
                          "with_workspace_tflops": round(2.0 * M * K * N / t_ws / 1e12, 1)}
             del q, s, ws

@@ -100,7 +100,8 @@ int adr_matmul_f16_slow(adr_stream_t stream, uint16_t* output, const uint16_t* l
  * workspace, and a second kernel sums them in a fixed order and applies the store operator.
  * adr_matmul_f16_workspace_bytes tells how much such a product would use at best (0: it would
  * not be split); with less, K is cut into fewer pieces or not at all, and with
- * workspace_bytes == 0 the call is adr_matmul_f16.
+ * workspace_bytes == 0 the product runs unsplit.  Only the caller's buffer is used, never the
+ * library's own (adr_set_held_workspace_limit below).
  * The workspace is written and read by the two launches only; it carries nothing from one call
  * to the next, so one buffer serves all calls on a stream.  Calls that may overlap (different
  * streams) need different buffers.
@@ -142,6 +143,34 @@ int adr_matmul_f16_noalloc(adr_stream_t stream, uint16_t* output, const uint16_t
                            int32_t stride_rx, int32_t stride_ry, int32_t stride_rz,
                            const uint16_t* bias, float beta, float scale, uint32_t store,
                            uint32_t load, uint32_t mask);
+
+/*
+ * The workspace that adr_matmul_f16, adr_matmul_nt_f16 and adr_matmul_nt_fp16u8 hold themselves
+ * (no counterpart in the reference).  Those entry points keep the reference's argument tuples and
+ * so have no workspace argument; where a workspace pays -- the products adr_matmul_f16_ws splits
+ * along K, and the u8 products adr_matmul_nt_fp16u8_ws runs on a matrix dequantised once -- they
+ * take one from a cache inside the library: one buffer per (device, stream), allocated with
+ * hipMalloc at the first call that wants it, replaced by a larger one when a later call wants more
+ * (16 MiB doubling up to the limit; a replaced buffer is not freed, kernels in flight may still use
+ * it), kept until the process ends.  Calls on one stream share a buffer and run in stream order;
+ * the cache is locked while a call that uses it launches, so any thread may call on any stream.
+ * No buffer is used or allocated -- and the call runs exactly as with a limit of 0 -- while the
+ * stream is being captured into a graph (the launches would tie the buffer to a graph that may be
+ * replayed on another stream), on hipStreamPerThread, when a product wants more than the limit
+ * (adr_matmul_f16: it is split into fewer pieces instead), or when the allocation fails.
+ * Results: the split products sum K in pieces, so on inexact data the last bits may differ from
+ * the unsplit launch (both within the stated tolerance); the u8 products from 257 rows on give
+ * the same bits either way.
+ * adr_set_held_workspace_limit: bytes per buffer (default ADR_HELD_WORKSPACE_DEFAULT_BYTES =
+ * 128 MiB: the LLaMA-7B qkv matrix dequantised, 100.7 MB, fits); 0 switches the cache off for
+ * later calls (buffers already allocated stay).  adr_held_workspace_bytes: bytes allocated so
+ * far in this process, replaced buffers included.  Callers that must not allocate at all use
+ * adr_matmul_f16_noalloc or the _ws forms, which never touch the cache.
+ */
+#define ADR_HELD_WORKSPACE_DEFAULT_BYTES ((int64_t)128 * 1024 * 1024)
+int adr_set_held_workspace_limit(int64_t bytes);
+int64_t adr_held_workspace_limit(void);
+int64_t adr_held_workspace_bytes(void);
 
 /* `matmul_f16_raw` (matmul.cu:515-517): identity operators, the 16 common arguments. */
 int adr_matmul_f16_raw(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,

@@ -26,3 +26,17 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture(autouse=True)
+def held_workspace_off():
+    """The plain entry points take a workspace from the library's own cache where that pays
+    (adr_set_held_workspace_limit).  Most tests here name the kernel a product runs on
+    (adr_matmul_f16_plan) and then call the plain entry point to test THAT kernel, so the cache is
+    off unless a test switches it on (tests/test_gpu_held_workspace.py and the randomised tests do)."""
+    from adrastea_amd import _ffi
+    lib = _ffi.lib()
+    before = lib.adr_held_workspace_limit()
+    lib.adr_set_held_workspace_limit(0)
+    yield
+    lib.adr_set_held_workspace_limit(before)

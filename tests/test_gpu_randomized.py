@@ -39,7 +39,7 @@ def _layout(g, rows, cols, contiguous, pads):
     return rows + pad, 1, cols * (rows + pad)
 
 
-def _f16_case(g):
+def _f16_case(g, long_k=False):
     pick = lambda xs: xs[int(g.integers(0, len(xs)))]
     aligned = g.random() < 0.85
     B = int(pick([1, 1, 1, 1, 2, 3, 5]))
@@ -55,6 +55,10 @@ def _f16_case(g):
             else 8 * int(g.integers(1, 300))
     else:
         K = 8 * int(g.integers(1, 200)) if km < 0.5 else int(g.integers(1, 700))
+    if long_k and g.random() < 0.6:   # few tiles, long K: what a workspace splits
+        M = int(g.integers(1, 400))
+        N = int(pick([256, 512, 1024, 2048, 4096, 5120])) + int(pick([0, 0, 8, -8, 1]))
+        K = int(pick([1024, 2048, 4096, 5120, 8192, 11008, 13824]))
     if M * N * B > 40e6 or M * N * K * B > 1.2e11:
         return None
     pads = [0, 0, 0, 8, 16, 64] if aligned else [0, 0, 8, 1, 3]
@@ -86,13 +90,23 @@ def _plan(c):
     return buf.value.decode()
 
 
-@pytest.mark.parametrize("seed", [11, 12, 13])
-def test_random_products_match_the_slow_kernel(seed):
+@pytest.fixture
+def held(request):
+    """The library's own workspace cache switched on (default size) or left off for the test."""
+    L = _ffi.lib()
+    L.adr_set_held_workspace_limit(_ffi.HELD_WORKSPACE_DEFAULT_BYTES if request.param else 0)
+    yield request.param
+    L.adr_set_held_workspace_limit(0)
+
+
+@pytest.mark.parametrize("seed,held", [(11, False), (12, False), (13, False), (14, True), (15, True)],
+                         indirect=["held"])
+def test_random_products_match_the_slow_kernel(seed, held):
     g = np.random.default_rng(seed)
     L = _ffi.lib()
     plans, failures = {}, []
     for it in range(110):
-        c = _f16_case(g)
+        c = _f16_case(g, long_k=held)
         if c is None:
             continue
         B, M, K, N = c["B"], c["M"], c["K"], c["N"]
@@ -147,8 +161,8 @@ def _u8_case(g):
     return dict(m=m, p=p, n=n, bs=bs, beta=float(pick([0.0, 0.0, 1.0, 0.5])))
 
 
-@pytest.mark.parametrize("seed", [21, 22])
-def test_random_u8_products_match_float64(seed):
+@pytest.mark.parametrize("seed,held", [(21, False), (22, False), (23, True)], indirect=["held"])
+def test_random_u8_products_match_float64(seed, held):
     g = np.random.default_rng(seed)
     L = _ffi.lib()
     plans, failures = {}, []
