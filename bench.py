@@ -545,8 +545,8 @@ def main():
         for name, K, N in LAYER_SET:
             mm(outs[name], acts[K], weights[name], M, K, N)
 
-    # The five launches of a step are recorded once into a HIP graph (the entry points neither
-    # allocate nor synchronise, so they can be captured) and the step is replayed: the timed
+    # The five launches of a step are recorded once into a HIP graph (under capture the entry
+    # points neither allocate nor synchronise) and the step is replayed: the timed
     # region then holds the device work of K steps, not the rate at which Python can call.
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())

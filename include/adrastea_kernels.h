@@ -4,12 +4,14 @@
  * This is the boundary a Rust `extern "C"` block in adrastea_kernels binds.  Every entry
  * point takes plain pointers and scalars, launches asynchronously on the given HIP stream
  * (NULL = the null stream, which is what the reference uses: `stream: None`,
- * adrastea_models/src/kernels.rs:862), never synchronises, never allocates, and returns
- * 0 on success, a positive hipError_t, or a negative ADR_E* code.  Invalid requests are
+ * adrastea_models/src/kernels.rs:862), never synchronises, allocates nothing per call, and
+ * returns 0 on success, a positive hipError_t, or a negative ADR_E* code.  Invalid requests are
  * rejected on the host; no entry point traps on the device.  The kernels exist for gfx950 only:
  * with any other device current, every launching entry point returns ADR_EUNSUPPORTED_DEVICE
  * (the device's architecture, compute-unit and die counts are queried once per device and
- * cached; that cache is the only state the library keeps).
+ * cached).  Beside that cache the library keeps one piece of state: the workspace that
+ * adr_matmul_f16, adr_matmul_nt_f16 and adr_matmul_nt_fp16u8 hold per stream, grown on demand
+ * (adr_set_held_workspace_limit below; 0 switches it off).
  *
  * fp16 data is passed as uint16_t bit patterns (Rust `half::f16` is repr(transparent) u16).
  * All strides are in ELEMENTS.  `x` is the last tensor dimension, `y` the second to last,
