@@ -10,5 +10,5 @@ without a GPU, calls raise.
 from .tensor import TensorLayout, TensorView  # noqa: F401
 from .kernels import (  # noqa: F401
     CommonKernels, GpuKernels, MatmulLoad, MatmulMask, MatmulOptions, MatmulStore, MatmulTracer,
-    AdrasteaError,
+    AdrasteaError, set_held_workspace_limit, held_workspace_limit, held_workspace_bytes,
 )

@@ -181,7 +181,8 @@ class GpuKernels(CommonKernels):
     tensor of the host (in the reference: one more GpuBuffer held by GpuKernels); matmul_f16 then
     goes through adr_matmul_f16_ws, which may split K over workgroups for products with few
     output tiles and a long K.  The buffer carries nothing between calls; one instance must not
-    be used from streams that run concurrently."""
+    be used from streams that run concurrently.  Without it (the default) the library takes such
+    a buffer from its own per-stream cache (set_held_workspace_limit)."""
 
     def __init__(self, workspace_bytes: int = 0):
         self._lib = _ffi.lib()
@@ -361,6 +362,23 @@ def matmul_workspace_bytes(output: TensorLayout, left: TensorLayout, right: Tens
     if n < 0:
         raise AdrasteaError(int(n), "matmul_f16_workspace_bytes")
     return int(n)
+
+
+def set_held_workspace_limit(nbytes: int) -> None:
+    """Bytes per buffer of the workspace cache that adr_matmul_f16, adr_matmul_nt_f16 and
+    adr_matmul_nt_fp16u8 keep per (device, stream); 0 switches the cache off."""
+    rc = _ffi.lib().adr_set_held_workspace_limit(int(nbytes))
+    if rc != 0:
+        raise AdrasteaError(int(rc), "set_held_workspace_limit")
+
+
+def held_workspace_limit() -> int:
+    return int(_ffi.lib().adr_held_workspace_limit())
+
+
+def held_workspace_bytes() -> int:
+    """Bytes the cache has allocated in this process so far (replaced buffers included)."""
+    return int(_ffi.lib().adr_held_workspace_bytes())
 
 
 class MatmulTracer(CommonKernels):

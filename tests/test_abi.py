@@ -194,3 +194,21 @@ def test_u8_workspace_size_and_validation():
     assert ws(None, 8, 8, 8, 8, 256, 64, 64, 32, 0.0, None, 1 << 20) == _ffi.ADR_ENULL
     assert ws(None, 8, 8, 8, 8, 256, 64, 64, 32, 0.0, 24, 1 << 20) == _ffi.ADR_EINVAL_SHAPE   # unaligned
     assert ws(None, 8, 8, 8, 8, 0, 64, 64, 32, 0.0, None, 0) == 0                              # empty
+
+
+def test_held_workspace_controls():
+    import adrastea_amd as A
+    lib = _ffi.lib()
+    assert _ffi.HELD_WORKSPACE_DEFAULT_BYTES == 128 << 20
+    before = lib.adr_held_workspace_limit()
+    try:
+        A.set_held_workspace_limit(3 << 20)
+        assert A.held_workspace_limit() == lib.adr_held_workspace_limit() == 3 << 20
+        assert lib.adr_set_held_workspace_limit(-1) == _ffi.ADR_EINVAL_SHAPE
+        assert A.held_workspace_limit() == 3 << 20
+        with pytest.raises(A.AdrasteaError):
+            A.set_held_workspace_limit(-1)
+        # nothing is allocated by asking
+        assert A.held_workspace_bytes() == lib.adr_held_workspace_bytes() >= 0
+    finally:
+        lib.adr_set_held_workspace_limit(before)
