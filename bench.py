@@ -251,6 +251,40 @@ def main():
             del ws
         return rows
 
+    def u8_short_prompt_set():
+        """The same row counts against u8 weights: `us` as the entry point comes (from 96 rows on
+        wide and 160 rows on narrow matrices the matrix is dequantised once into the buffer the
+        library holds and the fp16 kernels run on it), `fused_us` with the cache switched off (the
+        streaming kernels in passes of 64 rows, or the tiled u8 kernels)."""
+        rows = []
+        for K, N in DECODE_SET:
+            per = N * K + N * (K // 32) * 2
+            nbuf = max(2, int(600e6 // per) + 1)
+            qs = [torch.randint(0, 256, (N, K), generator=gen, device=dev, dtype=torch.uint8)
+                  for _ in range(nbuf)]
+            ss = [(torch.rand(N, K // 32, generator=gen, device=dev) * 0.019 + 0.001).half()
+                  for _ in range(nbuf)]
+            for m in (96, 128, 256, 512):
+                a = randn_h(m, K)
+                o = torch.zeros(m, N, dtype=torch.float16, device=dev)
+                i = [0]
+
+                def f():
+                    j = i[0] % nbuf
+                    i[0] += 1
+                    rc = lib.adr_matmul_nt_fp16u8(stream(), o.data_ptr(), a.data_ptr(), qs[j].data_ptr(),
+                                                  ss[j].data_ptr(), m, K, N, 32, 0.0)
+                    if rc != 0:
+                        raise RuntimeError(_ffi.strerror(rc))
+                t = timed(f, 4 * nbuf, nbuf)
+                lib.adr_set_held_workspace_limit(0)
+                t0 = timed(f, 4 * nbuf, nbuf)
+                lib.adr_set_held_workspace_limit(_ffi.HELD_WORKSPACE_DEFAULT_BYTES)
+                rows.append({"M": m, "K": K, "N": N, "us": round(t * 1e6, 1),
+                             "fused_us": round(t0 * 1e6, 1)})
+            del qs, ss
+        return rows
+
     def decode_set(ms=(1, 4, 16)):
         gemv = []
         for K, N in DECODE_SET:
@@ -437,7 +471,8 @@ def main():
         # for every token, llama.rs:456-483, so these are calls it makes too)
         print(json.dumps({"u8_decode_gemv": decode_set(), "f16_decode_gemv": f16_decode_set(),
                           "u8_17_to_128_rows": decode_set((32, 64, 128)),
-                          "f16_short_prompt_rows": short_prompt_set()}))
+                          "f16_short_prompt_rows": short_prompt_set(),
+                          "u8_short_prompt_rows": u8_short_prompt_set()}))
         return
 
     def u8_prefill_set():

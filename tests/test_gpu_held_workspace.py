@@ -167,7 +167,8 @@ def test_u8_products_by_way_of_the_held_workspace(held_on):
     lib = held_on
     g = rng(10)
     main = torch.cuda.current_stream().cuda_stream
-    for m, p, n, bs in [(300, 4096, 4096, 32), (2048, 4096, 4096, 32), (128, 4096, 8192, 32), (1100, 1024, 5120, 64)]:
+    for m, p, n, bs in [(300, 4096, 4096, 32), (2048, 4096, 4096, 32), (128, 4096, 8192, 32), (1100, 1024, 5120, 64),
+                        (256, 11008, 4096, 32)]:
         need = lib.adr_matmul_nt_fp16u8_workspace_bytes(m, p, n, bs)
         assert need == n * p * 2
         q = torch.from_numpy(g.integers(0, 256, size=(n, p), dtype=np.uint8)).cuda()
@@ -178,9 +179,10 @@ def test_u8_products_by_way_of_the_held_workspace(held_on):
         o_fused = torch.zeros_like(o_held)
         rc = lib.adr_matmul_nt_fp16u8(main, o_held.data_ptr(), x.data_ptr(), q.data_ptr(), sc.data_ptr(), m, p, n, bs, 0.0)
         assert rc == 0
-        ws = torch.empty(need, dtype=torch.uint8, device="cuda")
+        # (a caller's buffer of the cache's limit; only the matrix's n * p * 2 bytes are used)
+        ws = torch.empty(_ffi.HELD_WORKSPACE_DEFAULT_BYTES, dtype=torch.uint8, device="cuda")
         rc = lib.adr_matmul_nt_fp16u8_ws(main, o_ws.data_ptr(), x.data_ptr(), q.data_ptr(), sc.data_ptr(), m, p, n, bs, 0.0,
-                                         ws.data_ptr(), need)
+                                         ws.data_ptr(), ws.numel())
         assert rc == 0
         lib.adr_set_held_workspace_limit(0)
         rc = lib.adr_matmul_nt_fp16u8(main, o_fused.data_ptr(), x.data_ptr(), q.data_ptr(), sc.data_ptr(), m, p, n, bs, 0.0)
