@@ -171,13 +171,14 @@ __device__ __forceinline__ void store_chunk(const MatmulArgs& a, const Epilogue&
 // column block j: lane l holds output row l % 32 and, in element r, column
 // 8*(r/4) + 4*(l/32) + r%4.  (y0, x0) is the origin of the wavefront's sub-tile; `slot` is an
 // LDS region private to this wavefront of at least 32 * (TN*64 + 16) bytes.
-// The straight-line epilogue applies: the sub-tile's columns lie inside the matrix (rows may run
-// past the last one: those are read from the last row and not stored), it is on or below the
-// diagonal of a causal product, rows are 16-byte aligned.
+// The straight-line epilogue applies: the sub-tile begins inside the matrix and every 16-byte chunk
+// of its rows lies wholly inside or wholly outside (all of them inside, or n a multiple of 8; rows
+// and chunks past the matrix are read from the last row / chunk and not stored), it is on or below
+// the diagonal of a causal product, rows are 16-byte aligned.
 template <int TM, int TN>
 __device__ __forceinline__ bool epilogue_is_straight(const MatmulArgs& a, const half_t* out, int y0,
                                                      int x0) {
-  const bool inside = y0 < a.m && x0 + TN * 32 <= a.n;
+  const bool inside = y0 < a.m && x0 < a.n && (x0 + TN * 32 <= a.n || (a.n & 7) == 0);
   const bool unmasked = a.mask != ADR_MASK_CAUSAL || x0 + TN * 32 - 1 <= y0;
   return inside && unmasked && out_vectorizable(a, out);
 }
@@ -263,13 +264,18 @@ __device__ __forceinline__ void straight_epilogue(const MatmulArgs& a, half_t* o
   constexpr int CPW = TN * 4;          // 16-byte chunks per staged row
   const half_t mul = OP == ADR_STORE_SCALE ? hscale : (half_t)1.0f;
   // store round `it` of a 32-row block: lane -> 16-byte chunk it*64 + lane of the staged block
+  // (scol: the chunk's first column, clamped to the last chunk of the matrix for the loads;
+  // colin: the chunk lies inside the matrix)
   int rd[TN * 2], srow[TN * 2], scol[TN * 2];
+  bool colin[TN * 2];
+  const int cmax = a.n - 8 - x0;  // first column of the matrix's last chunk, relative to the sub-tile
 #pragma unroll
   for (int it = 0; it < TN * 2; it++) {
     const int idx = it * 64 + lane, row = idx / CPW, c = idx % CPW;
     rd[it] = row * PITCH + c * 16;
     srow[it] = row;
-    scol[it] = c * 8;
+    colin[it] = c * 8 <= cmax;
+    scol[it] = min(c * 8, cmax);
   }
   half8_t bias[TN * 2];
   if (nb) {
@@ -278,8 +284,8 @@ __device__ __forceinline__ void straight_epilogue(const MatmulArgs& a, half_t* o
   }
   half_t* const p0 = out + (int64_t)y0 * a.stride_oy + x0;
   const int last = a.m - y0 - 1;  // last row of the matrix, relative to the sub-tile
-  // rows past the matrix are clamped for loads (so that no load sits under a lane mask) and
-  // skipped for stores
+  // rows and chunks past the matrix are clamped for loads (so that no load sits under a lane
+  // mask) and skipped for stores
   auto at = [&](int i, int it) {
     return p0 + (int64_t)min(i * 32 + srow[it], last) * a.stride_oy + scol[it];
   };
@@ -317,7 +323,7 @@ __device__ __forceinline__ void straight_epilogue(const MatmulArgs& a, half_t* o
       }
       // streaming store: the output is not read again by this launch and should not evict
       // operand panels from L2
-      if (i * 32 + srow[it] <= last) __builtin_nontemporal_store(v, (half8_t*)at(i, it));
+      if (i * 32 + srow[it] <= last && colin[it]) __builtin_nontemporal_store(v, (half8_t*)at(i, it));
     }
   }
 }
@@ -1648,20 +1654,11 @@ GemmChoice choose(const MatmulArgs& a) {
     if (c == DMA_128x64 && a.k % 128 == 0 && a.k >= 1024 &&
         (int64_t)((a.m + 127) / 128) * ((a.n + 63) / 64) * a.batches <= NUM_CU)
       return DMA_128x64_K128;
-    // Short K with one large tile on (nearly) every CU: every workgroup then runs its prologue,
-    // its few slices and its epilogue in step with all the others.  Twice as many tiles of half
-    // the size, two resident per CU, overlap those phases (measured over a sweep of forced
-    // tiles: up to 38 % faster for K <= 1024, e.g. M1024 K320 N8192 17.3 -> 12.6 us).
-    if (a.k <= 1024 && (c == DMA_256x192 || c == DMA_256x128 || c == DMA_128x128)) {
-      auto tiles = [&](int bm, int bn) {
-        return (int64_t)((a.m + bm - 1) / bm) * ((a.n + bn - 1) / bn) * a.batches;
-      };
-      const int64_t now = c == DMA_256x192 ? tiles(256, 192) : c == DMA_256x128 ? tiles(256, 128)
-                                                                                 : tiles(128, 128);
-      const bool to_64 = c == DMA_128x128;
-      const int64_t then = to_64 ? tiles(128, 64) : tiles(128, 128);
-      if (now >= NUM_CU - 32 && now <= NUM_CU && then <= 2 * NUM_CU) return to_64 ? DMA_128x64 : DMA_128x128;
-    }
+    // (One large tile on nearly every CU with a short K used to be replaced by twice as many tiles
+    // of half the size, two resident per CU, whose prologues and epilogues overlap.  With the
+    // 256-row tiles on 16x16x32 MFMAs that no longer pays: over K 320 .. 1280 the 256 x 128 tile is
+    // 15-28 % ahead of two 128 x 128 per CU (M2048 K1024 N4096 17.9 against 21.0 us), and 128 x 64
+    // instead of 128 x 128 is within +-4 % up to K 512 and 4-12 % behind above.)
     return c;
   }
   if (a.rhs_q && a.k % 64 == 0 && a.block_size >= 8 && (a.block_size & (a.block_size - 1)) == 0 &&
