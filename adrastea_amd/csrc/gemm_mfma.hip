@@ -328,12 +328,83 @@ __device__ __forceinline__ void straight_epilogue(const MatmulArgs& a, half_t* o
   }
 }
 
+// acc + beta * out with beta != 0 (matmul_nt_wmma_16x128x256.cu:8-68 and its u8 twin: one rounding,
+// of the fp32 sum): the straight-line form.  The fp32 accumulators pass through the wavefront's
+// LDS slot, QN groups of eight columns of a 32 x 32 block at a time; a lane then owns whole
+// 16-byte chunks of the output, whose previous values were all requested up front.  Same
+// conditions as epilogue_is_straight, minus the restriction to beta == 0.
+template <int TM, int TN>
+__device__ __forceinline__ bool acc_beta_is_straight(const MatmulArgs& a, const half_t* out, int y0,
+                                                     int x0) {
+  return a.store == STORE_ACC_BETA && a.beta != 0.0f && a.mask == ADR_MASK_NONE && y0 < a.m &&
+         x0 < a.n && (x0 + TN * 32 <= a.n || (a.n & 7) == 0) && !(a.stride_oy & 7) &&
+         !((uintptr_t)out & 15);
+}
+
+template <int TM, int TN, class Acc>
+__device__ __forceinline__ void straight_epilogue_acc_beta(const MatmulArgs& a, half_t* out, Acc& acc,
+                                                           int y0, int x0, unsigned char* slot,
+                                                           int lane) {
+  constexpr int QN = TN >= 2 ? 4 : 2;     // 32 rows x (QN * 32 + 16) bytes fit the slot
+  constexpr int FP = QN * 32 + 16;        // bytes per staged row
+  constexpr int QH = 4 / QN;              // column groups per 32 x 32 block
+  constexpr int H = QN * 32 / 64;         // chunks per lane and group
+  static_assert(32 * FP <= 32 * (TN * 64 + 16), "fp32 staging must fit the wavefront's slot");
+  const int cmax = a.n - 8 - x0;          // first column of the matrix's last chunk, relative to the sub-tile
+  const int last = a.m - y0 - 1;          // last row of the matrix, relative to the sub-tile
+  half_t* const p0 = out + (int64_t)y0 * a.stride_oy + x0;
+  int rrow[H], rcol[H];
+#pragma unroll
+  for (int h = 0; h < H; h++) {
+    const int idx = h * 64 + lane;
+    rrow[h] = idx / QN;
+    rcol[h] = (idx % QN) * 8;
+  }
+  // rows and chunks past the matrix are clamped for the loads and skipped for the stores
+  auto at = [&](int i, int j, int qh, int h) {
+    return p0 + (int64_t)min(i * 32 + rrow[h], last) * a.stride_oy + min(j * 32 + qh * QN * 8 + rcol[h], cmax);
+  };
+  half8_t prev[TM][TN][QH][H];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int qh = 0; qh < QH; qh++)
+#pragma unroll
+        for (int h = 0; h < H; h++) prev[i][j][qh][h] = *(const half8_t*)at(i, j, qh, h);
+  const float beta = a.beta;
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int qh = 0; qh < QH; qh++) {
+        stage_block_f32<QN>(acc, i, j, qh, slot, lane);
+#pragma unroll
+        for (int h = 0; h < H; h++) {
+          const float4_t lo = *(const float4_t*)(slot + rrow[h] * FP + rcol[h] * 4);
+          const float4_t hi = *(const float4_t*)(slot + rrow[h] * FP + rcol[h] * 4 + 16);
+          half8_t v;
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            v[e] = (half_t)(lo[e] + beta * (float)prev[i][j][qh][h][e]);
+            v[4 + e] = (half_t)(hi[e] + beta * (float)prev[i][j][qh][h][4 + e]);
+          }
+          if (i * 32 + rrow[h] <= last && j * 32 + qh * QN * 8 + rcol[h] <= cmax)
+            __builtin_nontemporal_store(v, (half8_t*)at(i, j, qh, h));
+        }
+      }
+}
+
 template <int TM, int TN, class Acc>
 __device__ __forceinline__ void wave_epilogue(const MatmulArgs& a, half_t* out, Acc& acc, int y0,
                                               int x0, unsigned char* slot, half_t hscale, int lane) {
   Epilogue ep{a.bias, a.beta, hscale, a.store, true};
   constexpr int PITCH = TN * 64 + 16;  // bytes per staged row (TN*32 halves + pad)
   constexpr int CPW = TN * 4;          // 16-byte chunks per staged row
+  if (acc_beta_is_straight<TM, TN>(a, out, y0, x0))
+    return straight_epilogue_acc_beta<TM, TN>(a, out, acc, y0, x0, slot, lane);
   // Common case, straight-line: the sub-tile's columns lie inside the matrix, it is (for a
   // causal product) on or below the diagonal, rows are 16-byte aligned.
   if (epilogue_is_straight<TM, TN>(a, out, y0, x0)) {

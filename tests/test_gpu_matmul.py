@@ -406,25 +406,28 @@ def test_matmul_nt_f16_entry_point():
 @pytest.mark.parametrize("M,K,N,tile", [(2000, 2048, 8184, "256x128"), (630, 2048, 12280, "128x256"),
                                         (380, 2048, 12280, "128x192"), (2048, 1024, 12288, "256x192"),
                                         (2000, 2048, 8186, "256x128"), (1000, 2048, 4090, "128x128")])
-def test_elementwise_epilogue_of_the_large_tiles(M, K, N, tile):
-    """out = acc + beta * out on the unrounded fp32 accumulator (adr_matmul_nt_f16 with beta != 0)
-    and rows that are not 16-byte aligned (N = 8186, 4090) leave the vector epilogue: the accumulators
-    -- 16 x 16 blocks in the 256-row and 256-column tiles, 32 x 32 blocks in 128 x 192 -- pass
-    through LDS as fp32 and are stored element by element.  Exact on inputs whose sums are exact
-    (beta = 1: the sum of two exact terms rounded once), ragged last tiles."""
+@pytest.mark.parametrize("beta", [1.0, 0.5])
+def test_fp32_epilogues_of_the_large_tiles(M, K, N, tile, beta):
+    """out = acc + beta * out on the unrounded fp32 accumulator (adr_matmul_nt_f16 with beta != 0):
+    the accumulators -- 16 x 16 blocks in the 256-row and 256-column tiles, 32 x 32 blocks in
+    128 x 192 -- pass through LDS as fp32; with 16-byte aligned rows a lane then owns whole chunks
+    whose previous values were requested up front (N = 8184, 12280: the last tile column runs past
+    the matrix; M = 2000 ...: so does the last tile row), with unaligned rows (N = 8186, 4090) the
+    elements are stored one by one.  Exact on inputs whose sums are exact (the sum of two exact
+    terms rounded once)."""
     so, sl, sr = nt_strides(M, K, N)
     assert plan(1, M, K, N, so, sl, sr, store=0) == f"gemm_nt_mfma_dma_{tile}x64"
     gen = torch.Generator(device="cuda").manual_seed(M + N)
     a = (torch.randint(-4, 5, (M, K), generator=gen, device="cuda").float() / 64).half()
     w = (torch.randint(-4, 5, (N, K), generator=gen, device="cuda").float() / 64).half()
     prev = (torch.randint(-64, 65, (M, N), generator=gen, device="cuda").float() / 16).half()
-    want = (a.double() @ w.double().t() + prev.double()).half()
+    want = (a.double() @ w.double().t() + beta * prev.double()).half()
     out = prev.clone()
     stream = torch.cuda.current_stream().cuda_stream
     assert _ffi.lib().adr_matmul_nt_f16(stream, out.data_ptr(), a.data_ptr(), w.data_ptr(), M, K, N,
-                                        1.0) == 0
+                                        beta) == 0
     assert torch.equal(out.view(torch.int16), want.view(torch.int16))
-    if N % 8:
+    if N % 8 and beta == 1.0:
         # unaligned rows through the plain entry point too (Identity)
         out = torch.full((M, N), 9.0, dtype=torch.float16, device="cuda")
         assert raw_matmul("adr_matmul_f16", out, a, w, 1, M, K, N, so, sl, sr) == 0
