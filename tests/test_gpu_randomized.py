@@ -192,3 +192,37 @@ def test_random_u8_products_match_float64(seed, held):
             failures.append((c, name, int((want.view(torch.int16) != o_t.view(torch.int16)).sum())))
     assert not failures, failures
     assert len(plans) >= 4, plans
+
+
+@pytest.mark.parametrize("seed,held", [(31, False), (32, True)], indirect=["held"])
+def test_random_nt_f16_products_match_float64(seed, held):
+    """adr_matmul_nt_f16 (matmul_nt_wmma_16x128x256.cu:8-68: O = A B^T + beta O on the fp32 sum,
+    rounded once) on random sizes; exact data, so every kernel and epilogue it may take -- streaming
+    kernels, tiles with rows or columns past the matrix, aligned and unaligned rows -- has to give
+    the bits of a float64 evaluation."""
+    g = np.random.default_rng(seed)
+    L = _ffi.lib()
+    pick = lambda xs: xs[int(g.integers(0, len(xs)))]
+    failures = []
+    for it in range(70):
+        r = g.random()
+        m = int(g.integers(1, 65)) if r < 0.3 else int(g.integers(65, 700)) if r < 0.6 else \
+            int(pick([1024, 2048, 2056, 4096])) + int(pick([0, 0, 1, -1, 8, -100]))
+        n = int(g.integers(1, 600)) if g.random() < 0.25 else \
+            int(pick([1024, 4096, 8192, 11008, 12288])) + int(pick([0, 0, 0, 1, -1, 8, -8, 24, -200]))
+        p = int(pick([64, 128, 256, 320, 512, 1024, 2048, 4096, 11008])) if g.random() < 0.8 else 8 * int(g.integers(1, 300))
+        if m * n > 40e6 or m * n * p > 1.2e11:
+            continue
+        beta = float(pick([0.0, 1.0, 1.0, 0.5, -2.0]))
+        a = torch.from_numpy(g.integers(-3, 4, size=(m, p)).astype(np.float16)).cuda()
+        w = torch.from_numpy(g.integers(-2, 3, size=(n, p)).astype(np.float16)).cuda()
+        prev = torch.from_numpy((g.integers(-8, 9, size=(m, n)) / 4.0).astype(np.float16)).cuda()
+        out = prev.clone()
+        print(f"seed {seed} case {it}: m={m} p={p} n={n} beta={beta}", flush=True)
+        rc = L.adr_matmul_nt_f16(_stream(), out.data_ptr(), a.data_ptr(), w.data_ptr(), m, p, n, beta)
+        torch.cuda.synchronize()
+        assert rc == 0
+        want = (a.double() @ w.double().t() + beta * prev.double()).half()
+        if not torch.equal(want.view(torch.int16), out.view(torch.int16)):
+            failures.append((m, p, n, beta, int((want.view(torch.int16) != out.view(torch.int16)).sum())))
+    assert not failures, failures
