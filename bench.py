@@ -495,7 +495,9 @@ def main():
             # the entry point as it comes: from 96 rows on it dequantises the matrix once per call
             # into a buffer the library holds per stream (adr_set_held_workspace_limit, 128 MiB by
             # default) and runs the fp16 kernels on it; same bits as the fused kernels
-            timed(f, 30, 5)  # (discarded: the first calls allocate the buffer and find the clocks low)
+            # (discarded: the first calls allocate the buffer, and the clocks need tens of
+            # milliseconds of load to settle)
+            timed(f, 200 if not u8p else 30, 5)
             t = timed(f, 50, 5)
             # the fused kernels alone (dequantisation inside the GEMM's K loop, no buffer)
             lib.adr_set_held_workspace_limit(0)
