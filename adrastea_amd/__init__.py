@@ -11,4 +11,5 @@ from .tensor import TensorLayout, TensorView  # noqa: F401
 from .kernels import (  # noqa: F401
     CommonKernels, GpuKernels, MatmulLoad, MatmulMask, MatmulOptions, MatmulStore, MatmulTracer,
     AdrasteaError, set_held_workspace_limit, held_workspace_limit, held_workspace_bytes,
+    held_workspace_declined, release_held_workspace, set_u8_dequantise_first,
 )

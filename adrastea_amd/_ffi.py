@@ -13,6 +13,8 @@ SYMBOLS = (
     "adr_matmul_f16_ws", "adr_matmul_f16_workspace_bytes", "adr_matmul_f16_ws_plan",
     "adr_matmul_f16_noalloc",
     "adr_set_held_workspace_limit", "adr_held_workspace_limit", "adr_held_workspace_bytes",
+    "adr_held_workspace_declined", "adr_release_held_workspace", "adr_release_held_workspace_all",
+    "adr_set_u8_dequantise_first", "adr_u8_dequantise_first",
     "adr_matmul_nt_fp16u8", "adr_matmul_nt_fp16u8_ws", "adr_matmul_nt_fp16u8_workspace_bytes",
     "adr_dequantize_absmax_u8", "adr_quantize_absmax_u8",
     "adr_dequantize_absmax_uint8", "adr_quantize_absmax_uint8", "adr_matmul_f16_plan",
@@ -63,6 +65,11 @@ def lib():
     L.adr_held_workspace_limit.restype = C.c_int64
     L.adr_held_workspace_bytes.argtypes = []
     L.adr_held_workspace_bytes.restype = C.c_int64
+    L.adr_held_workspace_declined.argtypes = []
+    L.adr_release_held_workspace.argtypes = [vp]
+    L.adr_release_held_workspace_all.argtypes = []
+    L.adr_set_u8_dequantise_first.argtypes = [C.c_int]
+    L.adr_u8_dequantise_first.argtypes = []
     L.adr_matmul_f16_workspace_bytes.argtypes = [i32] * 13 + [u32, u32, u32]
     L.adr_matmul_f16_ws_plan.argtypes = [C.c_char_p, i32] + [i32] * 13 + [u32, u32, u32, C.c_int64]
     L.adr_matmul_f16_raw.argtypes = [vp, vp, vp, vp] + [i32] * 13
@@ -92,6 +99,10 @@ def lib():
         if name not in ("adr_strerror",):
             getattr(L, name).restype = C.c_int
     L.adr_matmul_f16_workspace_bytes.restype = C.c_int64
+    L.adr_held_workspace_limit.restype = C.c_int64
+    L.adr_held_workspace_bytes.restype = C.c_int64
+    L.adr_held_workspace_declined.restype = C.c_int64
+    L.adr_matmul_nt_fp16u8_workspace_bytes.restype = C.c_int64
     _lib = L
     return L
 

@@ -133,25 +133,33 @@ void* scratch_on_current_device(hipError_t* err) {
 
 // ---- workspace the plain entry points hold themselves -------------------------------------------
 // adr_matmul_f16, adr_matmul_nt_f16 and adr_matmul_nt_fp16u8 have the reference's argument tuples
-// and therefore no workspace argument.  Where a workspace pays (K split over workgroups; the u8
-// matrix dequantised once) they take it from a cache that grows on demand: one buffer per
-// (device, stream), since launches on one stream run in order and launches on different streams
-// may overlap.  A buffer that has become too small is replaced and not freed (kernels in flight
-// may still use it, and freeing would synchronise the device); sizes double from 16 MiB up to the
-// limit, so the memory given up that way stays below the size of the buffer in use.
-constexpr int MAX_HELD = 64;
+// and therefore no workspace argument.  Where a workspace pays (K split over workgroups; on request
+// the u8 matrix dequantised once) they take it from a pool that grows on demand.  A buffer has an
+// owner, (device, stream) -- launches on one stream run in order, launches on different streams may
+// overlap -- and an event recorded behind the last launches that used it.  A buffer changes hands
+// (a buffer its owner outgrew, or the least recently used one when all MAX_HELD entries are
+// taken) by making the new owner's stream wait for that event: no host synchronisation, no free
+// and no allocation inside a matmul call beyond the first ones.  Memory goes back to the device
+// only through adr_release_held_workspace*, which wait for the event first.
+constexpr int MAX_HELD = 16;
 constexpr int64_t HELD_FLOOR = (int64_t)16 << 20;
 struct Held {
   int device;
-  hipStream_t stream;
+  hipStream_t stream;  // owner; `owned` false: outgrown by its owner, free to be taken over
+  bool owned;
   void* ptr;
   int64_t bytes;
+  hipEvent_t last_use;  // recorded on the owner's stream behind the last launches that used ptr
+  uint64_t tick;        // value of held_clock at the last use
 };
 std::mutex held_mutex;
 Held held[MAX_HELD];
 int held_count = 0;
-int64_t held_total = 0;  // bytes allocated so far, replaced buffers included
+int64_t held_total = 0;     // bytes allocated and not yet released
+uint64_t held_clock = 0;
+std::atomic<int64_t> held_declined{0};  // calls that wanted a buffer and ran without
 std::atomic<int64_t> held_limit{ADR_HELD_WORKSPACE_DEFAULT_BYTES};
+std::atomic<int> u8_dequantise_first_enabled{0};
 
 // May this call use (and if need be allocate) a held buffer on `stream`?  Not while the stream is
 // being captured: the launches would tie the buffer into a graph that can be replayed on any stream
@@ -167,46 +175,95 @@ bool held_allowed(hipStream_t stream) {
   return st == hipStreamCaptureStatusNone;
 }
 
+// `stream` takes over entry h: everything the previous owner launched on the buffer is ordered
+// before whatever `stream` launches next.
+bool held_take_over(Held* h, hipStream_t stream) {
+  if (hipStreamWaitEvent(stream, h->last_use, 0) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  h->stream = stream;
+  h->owned = true;
+  return true;
+}
+
 // A buffer of at least `want` bytes for (current device, stream), or null (then the caller runs
-// without one).  held_mutex is held by the caller, and stays held over the launches that use the
-// buffer, so that two threads launching on one stream cannot interleave their pairs of launches.
-void* held_buffer(hipStream_t stream, int64_t want, int64_t* bytes) {
+// without one, and the call is counted in held_declined).  held_mutex is held by the caller, and
+// stays held over the launches that use the buffer and the held_used() behind them, so that two
+// threads launching on one stream cannot interleave their pairs of launches.
+Held* held_buffer(hipStream_t stream, int64_t want) {
   const int64_t limit = held_limit.load(std::memory_order_relaxed);
-  if (want <= 0 || want > limit) return nullptr;
-  int dev = -1;
-  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
-  Held* h = nullptr;
-  for (int i = 0; i < held_count; i++)
-    if (held[i].device == dev && held[i].stream == stream) h = &held[i];
-  if (h && h->bytes >= want) {
-    *bytes = h->bytes;
-    return h->ptr;
-  }
-  if (!h && held_count == MAX_HELD) return nullptr;
-  int64_t size = HELD_FLOOR;
-  while (size < want) size *= 2;
-  if (size > limit) size = limit;
-  // (an allocation is an "unsafe" call for a capture in global mode that some other stream of the
-  // process may be in; it touches no stream, so it is made in relaxed mode)
-  hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
-  (void)hipThreadExchangeStreamCaptureMode(&mode);
-  void* p = nullptr;
-  const hipError_t e = hipMalloc(&p, (size_t)size);
-  (void)hipThreadExchangeStreamCaptureMode(&mode);
-  if (e != hipSuccess || !p) {
-    (void)hipGetLastError();  // out of memory: the product runs without a workspace
+  if (want <= 0) return nullptr;
+  auto declined = [&]() -> Held* {
+    held_declined.fetch_add(1, std::memory_order_relaxed);
     return nullptr;
+  };
+  if (want > limit) return declined();
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) return declined();
+  Held* mine = nullptr;
+  for (int i = 0; i < held_count; i++)
+    if (held[i].owned && held[i].device == dev && held[i].stream == stream) mine = &held[i];
+  if (mine && mine->bytes >= want) return mine;
+  // a buffer some stream outgrew that is large enough
+  for (int i = 0; i < held_count; i++)
+    if (!held[i].owned && held[i].device == dev && held[i].bytes >= want && held_take_over(&held[i], stream)) {
+      if (mine) mine->owned = false;
+      return &held[i];
+    }
+  if (held_count < MAX_HELD) {
+    int64_t size = HELD_FLOOR;
+    while (size < want) size *= 2;
+    if (size > limit) size = limit;
+    // (an allocation is an "unsafe" call for a capture in global mode that some other stream of the
+    // process may be in; it touches no stream, so it is made in relaxed mode)
+    hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+    (void)hipThreadExchangeStreamCaptureMode(&mode);
+    void* p = nullptr;
+    hipEvent_t ev = nullptr;
+    hipError_t e = hipMalloc(&p, (size_t)size);
+    if (e == hipSuccess && p) {
+      e = hipEventCreateWithFlags(&ev, hipEventDisableTiming);
+      if (e != hipSuccess) (void)hipFree(p);
+    }
+    (void)hipThreadExchangeStreamCaptureMode(&mode);
+    if (e != hipSuccess || !p) {
+      (void)hipGetLastError();  // out of memory: the product runs without a workspace
+      return declined();
+    }
+    if (mine) mine->owned = false;  // outgrown: stays in the pool for a stream that wants less
+    Held* h = &held[held_count++];
+    *h = Held{dev, stream, true, p, size, ev, 0};
+    held_total += size;
+    return h;
   }
-  if (!h) {
-    h = &held[held_count++];
-    h->device = dev;
-    h->stream = stream;
+  // every entry is taken: the least recently used buffer of this device that is large enough
+  Held* lru = nullptr;
+  for (int i = 0; i < held_count; i++)
+    if (held[i].device == dev && held[i].bytes >= want && &held[i] != mine &&
+        (!lru || held[i].tick < lru->tick))
+      lru = &held[i];
+  if (lru && held_take_over(lru, stream)) {
+    if (mine) mine->owned = false;
+    return lru;
   }
-  h->ptr = p;
-  h->bytes = size;
-  held_total += size;
-  *bytes = size;
-  return p;
+  return declined();
+}
+
+// behind the launches that used h->ptr on its owner's stream
+void held_used(Held* h) {
+  h->tick = ++held_clock;
+  if (hipEventRecord(h->last_use, h->stream) != hipSuccess) (void)hipGetLastError();
+}
+
+// Frees entry i (waits for its last use first) and closes the gap.  held_mutex is held.
+void held_free(int i) {
+  (void)hipEventSynchronize(held[i].last_use);
+  (void)hipEventDestroy(held[i].last_use);
+  (void)hipFree(held[i].ptr);
+  (void)hipGetLastError();
+  held_total -= held[i].bytes;
+  held[i] = held[--held_count];
 }
 
 // run_matmul for the entry points without a workspace argument.
@@ -219,11 +276,12 @@ int run_matmul_held(hipStream_t stream, MatmulArgs& a) {
   const int64_t need = limit > 0 && !gemv_f16_supported(a, &name) ? mfma_gemm_workspace_bytes(a, limit) : 0;
   if (need > 0 && held_allowed(stream)) {
     std::lock_guard<std::mutex> lock(held_mutex);
-    int64_t bytes = 0;
-    if (void* p = held_buffer(stream, need, &bytes)) {
-      a.workspace = (float*)p;
-      a.workspace_bytes = bytes;
-      return run_matmul(stream, a, true);
+    if (Held* h = held_buffer(stream, need)) {
+      a.workspace = (float*)h->ptr;
+      a.workspace_bytes = h->bytes;
+      const int rc = run_matmul(stream, a, true);
+      held_used(h);
+      return rc;
     }
   }
   return run_matmul(stream, a, true);
@@ -280,6 +338,30 @@ int64_t adr_held_workspace_bytes(void) {
   return held_total;
 }
 
+int64_t adr_held_workspace_declined(void) { return held_declined.load(std::memory_order_relaxed); }
+
+int adr_release_held_workspace(adr_stream_t stream) {
+  int dev = -1;
+  if (hipError_t e = hipGetDevice(&dev)) return (int)e;
+  std::lock_guard<std::mutex> lock(held_mutex);
+  for (int i = held_count - 1; i >= 0; i--)
+    if (held[i].device == dev && (!held[i].owned || held[i].stream == (hipStream_t)stream)) held_free(i);
+  return ADR_OK;
+}
+
+int adr_release_held_workspace_all(void) {
+  std::lock_guard<std::mutex> lock(held_mutex);
+  while (held_count > 0) held_free(held_count - 1);
+  return ADR_OK;
+}
+
+int adr_set_u8_dequantise_first(int enabled) {
+  u8_dequantise_first_enabled.store(enabled != 0, std::memory_order_relaxed);
+  return ADR_OK;
+}
+
+int adr_u8_dequantise_first(void) { return u8_dequantise_first_enabled.load(std::memory_order_relaxed); }
+
 int adr_matmul_f16_ws(adr_stream_t stream, uint16_t* output, const uint16_t* lhs, const uint16_t* rhs,
                       int32_t batches, int32_t m, int32_t k, int32_t n, int32_t stride_ox,
                       int32_t stride_oy, int32_t stride_oz, int32_t stride_lx, int32_t stride_ly,
@@ -309,10 +391,12 @@ int adr_matmul_f16_noalloc(adr_stream_t stream, uint16_t* output, const uint16_t
   if (int rc = validate_matmul(a, true)) return rc;
   if (empty(a)) return ADR_OK;
   if (int rc = check_device()) return rc;
-  // what the product would use with a workspace of any size: it has to fit the built-in one
+  // what the product uses of the built-in scratch: a product that would like more is cut into
+  // fewer pieces, or not at all (the launcher makes the same choice from a.workspace_bytes)
   const char* name;
-  const int64_t need = gemv_f16_supported(a, &name) ? 0 : mfma_gemm_workspace_bytes(a);
-  if (need > ADR_NOALLOC_SCRATCH_BYTES) return ADR_ESCRATCH;
+  const int64_t need =
+      gemv_f16_supported(a, &name) ? 0 : mfma_gemm_workspace_bytes(a, ADR_NOALLOC_SCRATCH_BYTES);
+  if (need > ADR_NOALLOC_SCRATCH_BYTES) return ADR_ESCRATCH;  // (cannot happen: the choice is bounded)
   if (need > 0) {
     hipError_t e;
     void* p = scratch_on_current_device(&e);
@@ -368,6 +452,9 @@ int adr_matmul_f16_plan(char* name, int32_t cap, int32_t batches, int32_t m, int
                       stride_lx, stride_ly, stride_lz, stride_rx, stride_ry, stride_rz, nullptr,
                       0.0f, 1.0f, store, load, mask);
   if (int rc = validate_matmul(a, false)) return rc;
+  // what run_matmul_held does on a stream that is not being captured: a workspace of up to the
+  // current limit from the library's own pool
+  a.workspace_bytes = held_limit.load(std::memory_order_relaxed);
   const char* chosen = "none (empty)";
   if (!empty(a) && !gemv_f16_supported(a, &chosen) && !mfma_gemm_supported(a, &chosen))
     chosen = "matmul_general";
@@ -465,19 +552,27 @@ static int u8_fused(adr_stream_t stream, uint16_t* output, const uint16_t* lhs, 
                              (const half_t*)scales, m, p, n, block_size, beta);
 }
 
+// Does the plain u8 entry point dequantise first?  Only on request (adr_set_u8_dequantise_first),
+// where that is the faster route and the matrix fits the held-workspace limit.
+static bool u8_held_route(int m, int p, int n) {
+  return u8_dequantise_first_enabled.load(std::memory_order_relaxed) && u8_dequantise_first(m, p, n) &&
+         (int64_t)n * p * 2 <= held_limit.load(std::memory_order_relaxed);
+}
+
 int adr_matmul_nt_fp16u8(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
                          const uint8_t* rhs, const uint16_t* scales, int32_t m, int32_t p,
                          int32_t n, int32_t block_size, float beta) {
   bool nothing;
   if (int rc = validate_u8(output, lhs, rhs, scales, m, p, n, block_size, &nothing)) return rc;
   if (nothing) return ADR_OK;
-  const int64_t need = u8_dequantise_first(m, p, n) ? (int64_t)n * p * 2 : 0;
-  if (need > 0 && need <= held_limit.load(std::memory_order_relaxed) && held_allowed((hipStream_t)stream)) {
+  if (u8_held_route(m, p, n) && held_allowed((hipStream_t)stream)) {
     if (int rc = check_device()) return rc;
     std::lock_guard<std::mutex> lock(held_mutex);
-    int64_t bytes = 0;
-    if (void* ws = held_buffer((hipStream_t)stream, need, &bytes))
-      return u8_by_way_of_fp16(stream, output, lhs, rhs, scales, m, p, n, block_size, beta, ws);
+    if (Held* h = held_buffer((hipStream_t)stream, (int64_t)n * p * 2)) {
+      const int rc = u8_by_way_of_fp16(stream, output, lhs, rhs, scales, m, p, n, block_size, beta, h->ptr);
+      held_used(h);
+      return rc;
+    }
   }
   return u8_fused(stream, output, lhs, rhs, scales, m, p, n, block_size, beta);
 }
@@ -508,6 +603,8 @@ int adr_matmul_nt_fp16u8_plan(char* name, int32_t cap, int32_t m, int32_t p, int
   if (m < 0 || p < 0 || n < 0 || block_size <= 0) return ADR_EINVAL_SHAPE;
   if (p % block_size != 0) return ADR_EDIVISIBILITY;
   const char* chosen = (m == 0 || n == 0) ? "none (empty)" : gemm_u8_plan(m, p, n, block_size);
+  // (the opt-in route of the plain entry point on a stream that is not being captured)
+  if (m != 0 && n != 0 && u8_held_route(m, p, n)) chosen = "dequantize_absmax_u8 + fp16 gemm";
   if (name && cap > 0) {
     strncpy(name, chosen, (size_t)cap - 1);
     name[cap - 1] = 0;

@@ -55,6 +55,11 @@ DeviceInfo device_info() {
   Slot& s = slots[dev];
   if (s.ready.load(std::memory_order_acquire) == 2) return s.info;
   const DeviceInfo d = query(dev);
+  // a failed query (a positive hipError_t) may be transient: reported, not remembered
+  if (d.status > 0) {
+    (void)hipGetLastError();
+    return d;
+  }
   int expect = 0;
   if (s.ready.compare_exchange_strong(expect, 1, std::memory_order_acq_rel)) {
     s.info = d;

@@ -784,7 +784,15 @@ hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, co
       half_t* o = out + (int64_t)r0 * n;
       const half_t* l = lhs + (int64_t)r0 * p;
       hipError_t e;
-      if (mb <= 16) {
+      if (mb <= 16 && r0 > 0) {
+        // The last pass of a product of more than 64 rows: on the kernels of the other passes
+        // (weights rounded to fp16 as dequantize_absmax_uint8 does), so that every row of one
+        // product sees the same arithmetic; the sixteen-row kernels evaluate the naive kernel's
+        // formula on unrounded weights.
+        e = rg == 3 ? launch_blocks<3, 1>(stream, o, l, rhs, scales, mb, p, n, beta)
+          : rg == 2 ? launch_blocks<2, 1>(stream, o, l, rhs, scales, mb, p, n, beta)
+                    : launch_blocks<1, 2>(stream, o, l, rhs, scales, mb, p, n, beta);
+      } else if (mb <= 16) {
         e = launch_gemm_u8(stream, o, l, rhs, scales, mb, p, n, block_size, beta);
       } else if (mb <= 32 && p == 16 * MACRO_K) {
         // K 4096, up to 32 rows: the DMA-ring kernel with two blocks is 4-10 % ahead (m=32: N4096

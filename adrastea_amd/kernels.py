@@ -365,8 +365,8 @@ def matmul_workspace_bytes(output: TensorLayout, left: TensorLayout, right: Tens
 
 
 def set_held_workspace_limit(nbytes: int) -> None:
-    """Bytes per buffer of the workspace cache that adr_matmul_f16, adr_matmul_nt_f16 and
-    adr_matmul_nt_fp16u8 keep per (device, stream); 0 switches the cache off."""
+    """Bytes per buffer of the workspace pool that adr_matmul_f16 and adr_matmul_nt_f16 (and, on
+    request, adr_matmul_nt_fp16u8) draw from, one buffer per (device, stream); 0 switches it off."""
     rc = _ffi.lib().adr_set_held_workspace_limit(int(nbytes))
     if rc != 0:
         raise AdrasteaError(int(rc), "set_held_workspace_limit")
@@ -377,8 +377,30 @@ def held_workspace_limit() -> int:
 
 
 def held_workspace_bytes() -> int:
-    """Bytes the cache has allocated in this process so far (replaced buffers included)."""
+    """Bytes the pool holds now."""
     return int(_ffi.lib().adr_held_workspace_bytes())
+
+
+def held_workspace_declined() -> int:
+    """Calls so far that wanted a buffer of the pool and ran without one."""
+    return int(_ffi.lib().adr_held_workspace_declined())
+
+
+def release_held_workspace(stream=None) -> None:
+    """Frees the pool's buffers of `stream` (a raw stream handle; default: torch's current stream)
+    and those no stream owns any more, after waiting for the last launches that used them.  Call it
+    before destroying a stream.  `stream="all"`: every buffer on every device."""
+    L = _ffi.lib()
+    rc = (L.adr_release_held_workspace_all() if stream == "all" else
+          L.adr_release_held_workspace(_current_stream() if stream is None else stream))
+    if rc != 0:
+        raise AdrasteaError(int(rc), "release_held_workspace")
+
+
+def set_u8_dequantise_first(enabled: bool) -> None:
+    """Lets adr_matmul_nt_fp16u8 dequantise the weight matrix once into a buffer of the pool and
+    run the fp16 kernels on it where that is faster (off by default: always the fused kernels)."""
+    _ffi.lib().adr_set_u8_dequantise_first(1 if enabled else 0)
 
 
 class MatmulTracer(CommonKernels):

@@ -77,6 +77,12 @@ def main():
     ap.add_argument("--microbenchmark", action="store_true",
                     help="launch overhead, matrix-core issue peak, streaming-read peak and the "
                          "2048x4096x4096 products of the reference's microbenchmark()")
+    ap.add_argument("--settle-ms", type=float, default=300.0,
+                    help="untimed replays of the step for this many milliseconds before the declared "
+                         "warm-up (the clocks of a cold device settle under load); reported as settle_ms")
+    ap.add_argument("--step-trace", action="store_true",
+                    help="time each of the first 300 replays of the step graph on its own (HIP events), "
+                         "from a cold start, and print them: shows how long the device takes to settle")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain 256 MiB device copy (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters of rocprofv3 --pmc)")
@@ -252,10 +258,11 @@ def main():
         return rows
 
     def u8_short_prompt_set():
-        """The same row counts against u8 weights: `us` as the entry point comes (from 96 rows on
-        wide and 160 rows on narrow matrices the matrix is dequantised once into the buffer the
-        library holds and the fp16 kernels run on it), `fused_us` with the cache switched off (the
-        streaming kernels in passes of 64 rows, or the tiled u8 kernels)."""
+        """The same row counts against u8 weights: `us` as the entry point comes (the streaming
+        kernels in passes of 64 rows, or the tiled u8 kernels), `dequantise_first_us` after
+        adr_set_u8_dequantise_first(1) (from 96 rows on wide and 160 rows on narrow matrices the
+        matrix is dequantised once into a buffer of the library's pool and the fp16 kernels run
+        on it)."""
         rows = []
         for K, N in DECODE_SET:
             per = N * K + N * (K // 32) * 2
@@ -277,11 +284,11 @@ def main():
                     if rc != 0:
                         raise RuntimeError(_ffi.strerror(rc))
                 t = timed(f, 4 * nbuf, nbuf)
-                lib.adr_set_held_workspace_limit(0)
-                t0 = timed(f, 4 * nbuf, nbuf)
-                lib.adr_set_held_workspace_limit(_ffi.HELD_WORKSPACE_DEFAULT_BYTES)
+                lib.adr_set_u8_dequantise_first(1)
+                t1 = timed(f, 4 * nbuf, nbuf)
+                lib.adr_set_u8_dequantise_first(0)
                 rows.append({"M": m, "K": K, "N": N, "us": round(t * 1e6, 1),
-                             "fused_us": round(t0 * 1e6, 1)})
+                             "dequantise_first_us": round(t1 * 1e6, 1)})
             del qs, ss
         return rows
 
@@ -492,17 +499,17 @@ def main():
                                               q.data_ptr(), s.data_ptr(), M, K, N, 32, 0.0)
                 if rc != 0:
                     raise RuntimeError(_ffi.strerror(rc))
-            # the entry point as it comes: from 96 rows on it dequantises the matrix once per call
-            # into a buffer the library holds per stream (adr_set_held_workspace_limit, 128 MiB by
-            # default) and runs the fp16 kernels on it; same bits as the fused kernels
-            # (discarded: the first calls allocate the buffer, and the clocks need tens of
-            # milliseconds of load to settle)
+            # the entry point as it comes: the fused kernels (dequantisation inside the GEMM's K
+            # loop, nothing written back), eagerly and under capture alike
+            # (discarded: the clocks need tens of milliseconds of load to settle)
             timed(f, 200 if not u8p else 30, 5)
             t = timed(f, 50, 5)
-            # the fused kernels alone (dequantisation inside the GEMM's K loop, no buffer)
-            lib.adr_set_held_workspace_limit(0)
-            t_fused = timed(f, 50, 5)
-            lib.adr_set_held_workspace_limit(_ffi.HELD_WORKSPACE_DEFAULT_BYTES)
+            # on request (adr_set_u8_dequantise_first): the matrix dequantised once per call into a
+            # buffer of the library's pool, then the fp16 kernels; same bits
+            lib.adr_set_u8_dequantise_first(1)
+            timed(f, 5, 2)   # (allocates the buffer)
+            t_pool = timed(f, 50, 5)
+            lib.adr_set_u8_dequantise_first(0)
             # the same product through adr_matmul_nt_fp16u8_ws with the caller's workspace
             ws = torch.empty(N * K * 2, dtype=torch.uint8, device=dev)
 
@@ -516,8 +523,8 @@ def main():
             u8p[name] = {"M": M, "K": K, "N": N, "us": round(t * 1e6, 1),
                          "tflops": round(2.0 * M * K * N / t / 1e12, 1),
                          "frac_mfma_peak": round(2.0 * M * K * N / t / 1e12 / PEAK_F16_TFLOPS, 4),
-                         "fused_kernel_us": round(t_fused * 1e6, 1),
-                         "fused_kernel_tflops": round(2.0 * M * K * N / t_fused / 1e12, 1),
+                         "dequantise_first_us": round(t_pool * 1e6, 1),
+                         "dequantise_first_tflops": round(2.0 * M * K * N / t_pool / 1e12, 1),
                          "with_workspace_us": round(t_ws * 1e6, 1),
                          "with_workspace_tflops": round(2.0 * M * K * N / t_ws / 1e12, 1)}
             del q, s, ws
@@ -594,6 +601,34 @@ def main():
     step_graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(step_graph):
         step()
+    step_flops = sum(2.0 * M * K * N for _, K, N in LAYER_SET)
+    if args.step_trace:
+        # every replay between its own pair of events, starting cold (nothing has run but the
+        # capture): replay i's time and the running mean of ten
+        n_tr = 300
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(n_tr + 1)]
+        ev[0].record()
+        for i in range(n_tr):
+            step_graph.replay()
+            ev[i + 1].record()
+        torch.cuda.synchronize()
+        us = [round(ev[i].elapsed_time(ev[i + 1]) * 1e3, 1) for i in range(n_tr)]
+        tail = sorted(us[200:])
+        print(json.dumps({"step_trace_us": us, "median_of_replays_200_to_299_us": tail[len(tail) // 2],
+                          "mean_of_replays_0_to_24_us": round(sum(us[:25]) / 25, 1),
+                          "gflop_per_step": round(step_flops / 1e9, 1)}))
+        return
+    # Settle phase, untimed and reported: the clocks of a device that has been idle need some
+    # hundred milliseconds of this load to reach their steady state (--step-trace shows it), the
+    # reference's own harness runs every entry for up to five seconds for the same reason
+    # (adrastea/src/main.rs:409-454).  The declared warm-up follows it.
+    settle_t0 = time.perf_counter()
+    settle_steps = 0
+    while (time.perf_counter() - settle_t0) * 1e3 < args.settle_ms:
+        for _ in range(10):
+            step_graph.replay()
+        torch.cuda.synchronize()
+        settle_steps += 10
     for _ in range(args.warmup):
         step_graph.replay()
     torch.cuda.synchronize()
@@ -602,7 +637,6 @@ def main():
         step_graph.replay()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    step_flops = sum(2.0 * M * K * N for _, K, N in LAYER_SET)
     ms_per_step = elapsed / args.steps * 1e3
     value = step_flops / (elapsed / args.steps) / 1e12
 
@@ -795,7 +829,8 @@ def main():
 
     line = {
         "metric": METRIC, "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "steps": args.steps, "warmup": args.warmup, "settle_ms": args.settle_ms,
+        "settle_steps": settle_steps, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16",
         "data": "synthetic",
         "config": {"workload": "llama7b_layer_gemm_set_fp16_prefill_M2048 (configs[4] of the benchmark definition, "

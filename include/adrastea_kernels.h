@@ -9,9 +9,10 @@
  * rejected on the host; no entry point traps on the device.  The kernels exist for gfx950 only:
  * with any other device current, every launching entry point returns ADR_EUNSUPPORTED_DEVICE
  * (the device's architecture, compute-unit and die counts are queried once per device and
- * cached).  Beside that cache the library keeps one piece of state: the workspace that
- * adr_matmul_f16, adr_matmul_nt_f16 and adr_matmul_nt_fp16u8 hold per stream, grown on demand
- * (adr_set_held_workspace_limit below; 0 switches it off).
+ * cached).  Beside that cache the library keeps one piece of state: the pool of workspaces that
+ * adr_matmul_f16, adr_matmul_nt_f16 and (on request) adr_matmul_nt_fp16u8 draw from, grown on
+ * demand and given back through adr_release_held_workspace* (adr_set_held_workspace_limit below;
+ * 0 switches it off).
  *
  * fp16 data is passed as uint16_t bit patterns (Rust `half::f16` is repr(transparent) u16).
  * All strides are in ELEMENTS.  `x` is the last tensor dimension, `y` the second to last,
@@ -43,7 +44,8 @@ enum {
   ADR_EUNSUPPORTED_LAYOUT = -7, /* adr_attention_f16: head dimension, stride or alignment that the
                                    fused kernel does not cover; use the three-call sequence */
   ADR_ESCRATCH = -8             /* adr_matmul_f16_noalloc: the product needs more scratch than
-                                   ADR_NOALLOC_SCRATCH_BYTES */
+                                   ADR_NOALLOC_SCRATCH_BYTES (kept for ABI stability: products are
+                                   cut to fit instead) */
 };
 
 /* adrastea_models/src/kernels.rs:81-135, adrastea_kernels/cpp/matmul.cu:26-36 */
@@ -130,8 +132,9 @@ int64_t adr_matmul_f16_workspace_bytes(int32_t batches, int32_t m, int32_t k, in
  * on, held until the process ends; the entry point allocates and frees nothing (its first call
  * on a device looks the array's address up once: make that call before a graph capture begins).  Same arguments, validation and result as
  * adr_matmul_f16_ws given a workspace of at least adr_matmul_f16_workspace_bytes bytes.
- * A product that would use more than ADR_NOALLOC_SCRATCH_BYTES (16 MiB: the LLaMA-7B down
- * projection up to 256 rows fits) returns ADR_ESCRATCH and launches nothing.
+ * A product that would like more than ADR_NOALLOC_SCRATCH_BYTES (16 MiB: the LLaMA-7B down
+ * projection up to 256 rows fits) is cut into as many pieces as fit, or runs unsplit: the result
+ * is then that of adr_matmul_f16_ws given a workspace of exactly ADR_NOALLOC_SCRATCH_BYTES.
  * All calls on one GPU share that GPU's array: calls that may overlap in time (different streams)
  * race on it and must be serialised by the caller or use adr_matmul_f16_ws with buffers of their
  * own.  Nothing in the array has to start at zero and nothing is kept from one call to the next
@@ -147,32 +150,53 @@ int adr_matmul_f16_noalloc(adr_stream_t stream, uint16_t* output, const uint16_t
                            uint32_t load, uint32_t mask);
 
 /*
- * The workspace that adr_matmul_f16, adr_matmul_nt_f16 and adr_matmul_nt_fp16u8 hold themselves
- * (no counterpart in the reference).  Those entry points keep the reference's argument tuples and
- * so have no workspace argument; where a workspace pays -- the products adr_matmul_f16_ws splits
- * along K, and the u8 products adr_matmul_nt_fp16u8_ws runs on a matrix dequantised once -- they
- * take one from a cache inside the library: one buffer per (device, stream), allocated with
- * hipMalloc at the first call that wants it, replaced by a larger one when a later call wants more
- * (16 MiB doubling up to the limit; a replaced buffer is not freed, kernels in flight may still use
- * it), kept until the process ends.  Calls on one stream share a buffer and run in stream order;
- * the cache is locked while a call that uses it launches, so any thread may call on any stream.
- * No buffer is used or allocated -- and the call runs exactly as with a limit of 0 -- while the
- * stream is being captured into a graph (the launches would tie the buffer to a graph that may be
- * replayed on another stream), on hipStreamPerThread, when a product wants more than the limit
- * (adr_matmul_f16: it is split into fewer pieces instead), or when the allocation fails.
+ * The workspaces that adr_matmul_f16 and adr_matmul_nt_f16 hold themselves (no counterpart in the
+ * reference).  Those entry points keep the reference's argument tuples and so have no workspace
+ * argument; where a workspace pays -- the products adr_matmul_f16_ws splits along K -- they take
+ * one from a pool inside the library.  A buffer belongs to a (device, stream) pair: it is allocated
+ * with hipMalloc at the first call on that stream that wants one (16 MiB doubling up to the limit)
+ * and carries an event recorded behind the last launches that used it.  When a stream wants more
+ * than its buffer holds it gets a larger one and the old buffer stays in the pool for any stream
+ * that wants less; when all 16 entries of the pool are taken, a stream without a buffer takes over
+ * the least recently used one that is large enough.  A buffer changes hands by making the new
+ * owner's stream wait for the buffer's event (hipStreamWaitEvent): nothing is freed, allocated or
+ * synchronised inside a matmul call beyond those first allocations, and the pool never holds more
+ * than 16 buffers of at most the limit each.  Calls on one stream share a buffer and run in stream
+ * order; the pool is locked while a call that uses it launches, so any thread may call on any
+ * stream.  No buffer is used or allocated -- the call runs exactly as with a limit of 0 -- while
+ * the stream is being captured into a graph (the launches would tie the buffer to a graph that may
+ * be replayed on another stream), on hipStreamPerThread, when the allocation fails, or when the
+ * pool is full and holds no buffer large enough; a product that wants more than the limit is split
+ * into fewer pieces instead.  adr_held_workspace_declined counts the calls that wanted a buffer and
+ * ran without one.
  * Results: the split products sum K in pieces, so on inexact data the last bits may differ from
- * the unsplit launch (both within the stated tolerance); the u8 products from 257 rows on give
- * the same bits either way.
+ * the unsplit launch (both within the stated tolerance).
+ *
  * adr_set_held_workspace_limit: bytes per buffer (default ADR_HELD_WORKSPACE_DEFAULT_BYTES =
- * 128 MiB: the LLaMA-7B qkv matrix dequantised, 100.7 MB, fits); 0 switches the cache off for
- * later calls (buffers already allocated stay).  adr_held_workspace_bytes: bytes allocated so
- * far in this process, replaced buffers included.  Callers that must not allocate at all use
- * adr_matmul_f16_noalloc or the _ws forms, which never touch the cache.
+ * 128 MiB); 0 switches the pool off for later calls (buffers already allocated stay until
+ * released).  adr_held_workspace_bytes: bytes the pool holds now.
+ * adr_release_held_workspace(stream): waits for the last launches that used them (the buffers'
+ * events, not the device) and frees, on the current device, the buffers `stream` owns and those no
+ * stream owns any more; call it before destroying a stream.  adr_release_held_workspace_all: the
+ * same for every buffer on every device.  (hipFree itself may wait for other work on the device:
+ * these two are not for the hot path.)  Later calls allocate afresh.
+ * Callers that must not allocate at all use adr_matmul_f16_noalloc or the _ws forms, which never
+ * touch the pool.
+ *
+ * adr_set_u8_dequantise_first(1): lets adr_matmul_nt_fp16u8 take the route of
+ * adr_matmul_nt_fp16u8_ws by itself, with the dequantised matrix (n * p * 2 bytes, which must fit
+ * the limit above: the LLaMA-7B qkv matrix is 100.7 MB) in a buffer of this pool.  Off by default:
+ * the plain entry point then always runs its fused kernels, eagerly and under capture alike.
  */
 #define ADR_HELD_WORKSPACE_DEFAULT_BYTES ((int64_t)128 * 1024 * 1024)
 int adr_set_held_workspace_limit(int64_t bytes);
 int64_t adr_held_workspace_limit(void);
 int64_t adr_held_workspace_bytes(void);
+int64_t adr_held_workspace_declined(void);
+int adr_release_held_workspace(adr_stream_t stream);
+int adr_release_held_workspace_all(void);
+int adr_set_u8_dequantise_first(int enabled);
+int adr_u8_dequantise_first(void);
 
 /* `matmul_f16_raw` (matmul.cu:515-517): identity operators, the 16 common arguments. */
 int adr_matmul_f16_raw(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
@@ -200,6 +224,8 @@ int adr_matmul_nt_f16(adr_stream_t stream, uint16_t* output, const uint16_t* lhs
  *
  * lhs [m,p] fp16, rhs [n,p] u8, scales [n, p/block_size] fp16, out [m,n] fp16, all contiguous.
  * Any m >= 1 and n >= 1; p % block_size == 0; block_size a multiple of 8.
+ * Always the fused kernels (weights dequantised between the load and the matrix cores, nothing
+ * written back), eagerly and under graph capture alike, unless adr_set_u8_dequantise_first(1).
  */
 int adr_matmul_nt_fp16u8(adr_stream_t stream, uint16_t* output, const uint16_t* lhs,
                          const uint8_t* rhs, const uint16_t* scales, int32_t m, int32_t p,
@@ -328,12 +354,16 @@ int adr_attention_f16(adr_stream_t stream, uint16_t* output, const uint16_t* que
  * Diagnostics (no counterpart in the reference).
  *
  * adr_matmul_f16_plan: writes the name of the kernel adr_matmul_f16 would launch for these
- * arguments into `name` (at most `cap` bytes, NUL-terminated) without touching the device.
+ * arguments -- on a stream that is not being captured and with the held-workspace limit as it is
+ * now ("..._splitk4": K in four pieces through a held buffer; with a limit of 0, or under
+ * capture, the unsplit kernel that adr_matmul_f16_ws_plan names for a workspace of 0 bytes) --
+ * into `name` (at most `cap` bytes, NUL-terminated) without touching the device.
  * Same validation and return codes as adr_matmul_f16 minus the pointer checks.  Without pointers
  * the plan assumes 16-byte aligned operands; a call with unaligned ones runs on the general
  * (u8: the per-output) kernel whatever the plan says.  On a machine without a device the plan
  * is the one for an MI355X.  adr_matmul_nt_fp16u8_plan names the tile of a tiled kernel
- * ("gemm_nt_u8_mfma_256x192x64", "gemm_nt_u8_stage_128x128x32", ...).
+ * ("gemm_nt_u8_mfma_256x192x64", "gemm_nt_u8_stage_128x128x32", ...), or
+ * "dequantize_absmax_u8 + fp16 gemm" where adr_set_u8_dequantise_first(1) routes the product.
  */
 int adr_matmul_f16_plan(char* name, int32_t cap, int32_t batches, int32_t m, int32_t k,
                         int32_t n, int32_t stride_ox, int32_t stride_oy, int32_t stride_oz,

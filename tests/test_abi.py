@@ -163,8 +163,16 @@ def test_workspace_plan_and_size():
     # less workspace: fewer pieces (or smaller tiles), then none
     less = plan_ws(128, 11008, 4096, b - 16)
     assert "_splitk" in less and less != full
-    assert plan_ws(128, 11008, 4096, b // 8) == plan_ws(128, 11008, 4096, 0) == _plan(
-        1, 128, 11008, 4096, (1, 4096, 0), (1, 11008, 0), (11008, 1, 0))[1]
+    assert plan_ws(128, 11008, 4096, b // 8) == plan_ws(128, 11008, 4096, 0)
+    # the plain entry point's plan follows the held-workspace limit as it is now
+    before = lib.adr_held_workspace_limit()
+    try:
+        for limit in (0, b - 16, _ffi.HELD_WORKSPACE_DEFAULT_BYTES):
+            lib.adr_set_held_workspace_limit(limit)
+            assert _plan(1, 128, 11008, 4096, (1, 4096, 0), (1, 11008, 0), (11008, 1, 0))[1] == \
+                plan_ws(128, 11008, 4096, limit)
+    finally:
+        lib.adr_set_held_workspace_limit(before)
     # the prefill shapes and the decode shapes are never split
     assert need(2048, 4096, 12288) == 0 and need(2048, 11008, 4096) == 0
     assert need(1, 4096, 4096) == 0 and need(16, 11008, 4096) == 0
@@ -196,6 +204,28 @@ def test_u8_workspace_size_and_validation():
     assert ws(None, 8, 8, 8, 8, 0, 64, 64, 32, 0.0, None, 0) == 0                              # empty
 
 
+def test_u8_plan_follows_the_dequantise_first_switch():
+    lib = _ffi.lib()
+    buf = C.create_string_buffer(96)
+
+    def plan_u8(m, p, n):
+        assert lib.adr_matmul_nt_fp16u8_plan(buf, 96, m, p, n, 32) == 0
+        return buf.value.decode()
+    before = lib.adr_held_workspace_limit()
+    try:
+        lib.adr_set_held_workspace_limit(_ffi.HELD_WORKSPACE_DEFAULT_BYTES)
+        assert lib.adr_u8_dequantise_first() == 0
+        assert plan_u8(2048, 4096, 12288) == "gemm_nt_u8_mfma_256x192x64"      # the default: fused
+        assert lib.adr_set_u8_dequantise_first(1) == 0 and lib.adr_u8_dequantise_first() == 1
+        assert plan_u8(2048, 4096, 12288) == "dequantize_absmax_u8 + fp16 gemm"
+        assert plan_u8(16, 4096, 12288) == "gemv_u8_mfma16_regstream"          # never for decode
+        lib.adr_set_held_workspace_limit(64 << 20)                              # the matrix does not fit
+        assert plan_u8(2048, 4096, 12288) == "gemm_nt_u8_mfma_256x192x64"
+    finally:
+        lib.adr_set_u8_dequantise_first(0)
+        lib.adr_set_held_workspace_limit(before)
+
+
 def test_held_workspace_controls():
     import adrastea_amd as A
     lib = _ffi.lib()
@@ -210,5 +240,6 @@ def test_held_workspace_controls():
             A.set_held_workspace_limit(-1)
         # nothing is allocated by asking
         assert A.held_workspace_bytes() == lib.adr_held_workspace_bytes() >= 0
+        assert A.held_workspace_declined() == lib.adr_held_workspace_declined() >= 0
     finally:
         lib.adr_set_held_workspace_limit(before)

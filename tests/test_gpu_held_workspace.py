@@ -1,9 +1,10 @@
-"""The workspace the plain entry points hold themselves (adr_set_held_workspace_limit): products
-that adr_matmul_f16_ws splits along K and u8 products that adr_matmul_nt_fp16u8_ws runs on a
-matrix dequantised once take their buffer from a cache inside the library when they come through
-adr_matmul_f16 / adr_matmul_nt_f16 / adr_matmul_nt_fp16u8.  Bars: the same bits as the _ws entry
-point given a buffer of the same size; one allocation per (device, stream), growing on demand,
-none under stream capture, none with the limit at 0."""
+"""The workspaces the plain entry points hold themselves (adr_set_held_workspace_limit): products
+that adr_matmul_f16_ws splits along K -- and, after adr_set_u8_dequantise_first(1), u8 products that
+adr_matmul_nt_fp16u8_ws runs on a matrix dequantised once -- take their buffer from a pool inside
+the library when they come through adr_matmul_f16 / adr_matmul_nt_f16 / adr_matmul_nt_fp16u8.
+Bars: the same bits as the _ws entry point given a buffer of the same size; one allocation per
+(device, stream), growing on demand, none under stream capture, none with the limit at 0; buffers
+given back by adr_release_held_workspace*, a bounded pool however many streams come and go."""
 import ctypes as C
 
 import numpy as np
@@ -21,9 +22,15 @@ MIB = 1 << 20
 @pytest.fixture
 def held_on():
     lib = _ffi.lib()
+    torch.cuda.synchronize()
+    assert lib.adr_release_held_workspace_all() == 0   # every test starts from an empty pool
     lib.adr_set_held_workspace_limit(_ffi.HELD_WORKSPACE_DEFAULT_BYTES)
     yield lib
     lib.adr_set_held_workspace_limit(0)
+    lib.adr_set_u8_dequantise_first(0)
+    torch.cuda.synchronize()
+    assert lib.adr_release_held_workspace_all() == 0
+    assert lib.adr_held_workspace_bytes() == 0
 
 
 def _nt_args(o, a, w, M, K, N, store=0, bias=None, beta=0.0):
@@ -167,6 +174,26 @@ def test_u8_products_by_way_of_the_held_workspace(held_on):
     lib = held_on
     g = rng(10)
     main = torch.cuda.current_stream().cuda_stream
+    # the default: the fused kernels whatever the pool would allow, nothing allocated
+    m, p, n, bs = 300, 4096, 4096, 32
+    q = torch.from_numpy(g.integers(0, 256, size=(n, p), dtype=np.uint8)).cuda()
+    sc = torch.from_numpy((g.random((n, p // bs)) * 0.019 + 0.001).astype(np.float16)).cuda()
+    x = torch.from_numpy(randn_f16(g, (m, p))).cuda()
+    o_default = torch.zeros(m, n, dtype=torch.float16, device="cuda")
+    o_fused = torch.zeros_like(o_default)
+    assert lib.adr_u8_dequantise_first() == 0
+    name = C.create_string_buffer(96)
+    assert lib.adr_matmul_nt_fp16u8_plan(name, 96, m, p, n, bs) == 0 and name.value.startswith(b"gemm_nt_u8")
+    assert lib.adr_matmul_nt_fp16u8(main, o_default.data_ptr(), x.data_ptr(), q.data_ptr(), sc.data_ptr(), m, p, n, bs, 0.0) == 0
+    lib.adr_set_held_workspace_limit(0)
+    assert lib.adr_matmul_nt_fp16u8(main, o_fused.data_ptr(), x.data_ptr(), q.data_ptr(), sc.data_ptr(), m, p, n, bs, 0.0) == 0
+    lib.adr_set_held_workspace_limit(_ffi.HELD_WORKSPACE_DEFAULT_BYTES)
+    torch.cuda.synchronize()
+    assert torch.equal(o_default.view(torch.int16), o_fused.view(torch.int16))
+    assert lib.adr_held_workspace_bytes() == 0
+    # on request: the matrix dequantised once into a buffer of the pool
+    assert lib.adr_set_u8_dequantise_first(1) == 0 and lib.adr_u8_dequantise_first() == 1
+    assert lib.adr_matmul_nt_fp16u8_plan(name, 96, m, p, n, bs) == 0 and name.value == b"dequantize_absmax_u8 + fp16 gemm"
     for m, p, n, bs in [(300, 4096, 4096, 32), (2048, 4096, 4096, 32), (128, 4096, 8192, 32), (1100, 1024, 5120, 64),
                         (256, 11008, 4096, 32)]:
         need = lib.adr_matmul_nt_fp16u8_workspace_bytes(m, p, n, bs)
@@ -240,3 +267,79 @@ def test_threads_on_their_own_streams(held_on):
         assert torch.equal(o.view(torch.int16), outs[0].view(torch.int16))
     ref = a.double() @ w.double().t()
     assert float((outs[0].double() - ref).abs().max() / ref.pow(2).mean().sqrt()) < 1e-2
+
+
+def test_release_gives_the_memory_back_and_later_calls_allocate_afresh(held_on):
+    lib = held_on
+    g = rng(12)
+    M, K, N = 128, 11008, 4096
+    a = torch.from_numpy(randn_f16(g, (M, K))).cuda()
+    w = torch.from_numpy(randn_f16(g, (N, K), K ** -0.5)).cuda()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    o1 = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+    o2, o3 = torch.zeros_like(o1), torch.zeros_like(o1)
+    torch.cuda.synchronize()
+    _plain(lib, s1.cuda_stream, *_nt_args(o1, a, w, M, K, N))
+    _plain(lib, s2.cuda_stream, *_nt_args(o2, a, w, M, K, N))
+    assert lib.adr_held_workspace_bytes() == 32 * MIB
+    # released right behind the launch: the call waits for the buffer's last use, not for the caller
+    assert lib.adr_release_held_workspace(s1.cuda_stream) == 0
+    assert lib.adr_held_workspace_bytes() == 16 * MIB          # s2 keeps its own
+    assert lib.adr_release_held_workspace(s1.cuda_stream) == 0  # nothing left to release: fine
+    _plain(lib, s1.cuda_stream, *_nt_args(o3, a, w, M, K, N))   # allocates afresh
+    assert lib.adr_held_workspace_bytes() == 32 * MIB
+    torch.cuda.synchronize()
+    assert torch.equal(o1.view(torch.int16), o2.view(torch.int16))
+    assert torch.equal(o1.view(torch.int16), o3.view(torch.int16))
+    assert lib.adr_release_held_workspace_all() == 0
+    assert lib.adr_held_workspace_bytes() == 0
+
+
+def test_streams_that_come_and_go_leave_a_bounded_pool(held_on):
+    lib = held_on
+    g = rng(13)
+    M, K, N = 128, 11008, 4096
+    a = torch.from_numpy(randn_f16(g, (M, K))).cuda()
+    w = torch.from_numpy(randn_f16(g, (N, K), K ** -0.5)).cuda()
+    want = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+    _plain(lib, torch.cuda.current_stream().cuda_stream, *_nt_args(want, a, w, M, K, N))
+    torch.cuda.synchronize()
+    declined = lib.adr_held_workspace_declined()
+    # a host that releases before it destroys a stream holds nothing afterwards
+    base = lib.adr_held_workspace_bytes()
+    for _ in range(20):
+        s = torch.cuda.Stream()
+        o = torch.zeros_like(want)
+        _plain(lib, s.cuda_stream, *_nt_args(o, a, w, M, K, N))
+        assert lib.adr_release_held_workspace(s.cuda_stream) == 0
+        assert lib.adr_held_workspace_bytes() == base
+        assert torch.equal(o.view(torch.int16), want.view(torch.int16))
+        del s
+    # a host that does not: the pool stops at 16 buffers and hands the least recently used one on
+    streams, outs = [], []
+    for i in range(100):
+        s = torch.cuda.Stream()
+        o = torch.zeros_like(want) if i % 10 == 0 else outs[-1]
+        _plain(lib, s.cuda_stream, *_nt_args(o, a, w, M, K, N))
+        streams.append(s)
+        outs.append(o)
+        assert lib.adr_held_workspace_bytes() <= 16 * 16 * MIB
+    torch.cuda.synchronize()
+    assert lib.adr_held_workspace_bytes() == 16 * 16 * MIB
+    assert lib.adr_held_workspace_declined() == declined       # every call found a buffer
+    for o in outs[::10]:
+        assert torch.equal(o.view(torch.int16), want.view(torch.int16))
+    # the pool is full of 16 MiB buffers: a product that wants more runs without one, and is counted
+    big = (640, 22016, 4096)
+    assert _need(lib, *big) > 16 * MIB
+    ab = torch.from_numpy(randn_f16(g, big[:2])).cuda()
+    wb = torch.from_numpy(randn_f16(g, (big[2], big[1]), big[1] ** -0.5)).cuda()
+    o_full, o_off = (torch.zeros(big[0], big[2], dtype=torch.float16, device="cuda") for _ in range(2))
+    fresh = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    _plain(lib, fresh.cuda_stream, *_nt_args(o_full, ab, wb, *big))
+    assert lib.adr_held_workspace_declined() == declined + 1
+    lib.adr_set_held_workspace_limit(0)
+    _plain(lib, fresh.cuda_stream, *_nt_args(o_off, ab, wb, *big))
+    torch.cuda.synchronize()
+    assert torch.equal(o_full.view(torch.int16), o_off.view(torch.int16))

@@ -95,8 +95,10 @@ def held(request):
     """The library's own workspace cache switched on (default size) or left off for the test."""
     L = _ffi.lib()
     L.adr_set_held_workspace_limit(_ffi.HELD_WORKSPACE_DEFAULT_BYTES if request.param else 0)
+    L.adr_set_u8_dequantise_first(1 if request.param else 0)
     yield request.param
     L.adr_set_held_workspace_limit(0)
+    L.adr_set_u8_dequantise_first(0)
 
 
 @pytest.mark.parametrize("seed,held", [(11, False), (12, False), (13, False), (14, True), (15, True)],

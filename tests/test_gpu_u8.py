@@ -330,14 +330,18 @@ CFG5_U8 = [("qkv", 4096, 12288, "256x192"), ("o", 4096, 4096, "256x128"),
            ("gate_up", 4096, 11008, "256x192"), ("down", 11008, 4096, "256x128")]
 
 
+@pytest.mark.parametrize("workspace_mode", ["pool_off", "shipped_default", "u8_dequantise_first"], indirect=True)
 @pytest.mark.parametrize("case", CFG5_U8, ids=[c[0] for c in CFG5_U8])
-def test_prefill_u8_gemm_layer_set_full_size(kern, case):
+def test_prefill_u8_gemm_layer_set_full_size(kern, case, workspace_mode):
     """benchmark config 5 (u8 half) at full size, M = 2048: every product of the layer set on the
     tile the benchmark measures (asserted through the plan), against an fp32 GEMM on the
-    bit-exactly dequantised weights, both on the device; plus f(2a) = 2 f(a) exactly."""
+    bit-exactly dequantised weights, both on the device; plus f(2a) = 2 f(a) exactly.  With the
+    workspace pool off, as the library ships (the fused kernel either way), and on the route that
+    adr_set_u8_dequantise_first(1) opens."""
     _, p, n, tile = case
     m = 2048
-    assert u8_plan(m, p, n, 32) == f"gemm_nt_u8_mfma_{tile}x64"
+    assert u8_plan(m, p, n, 32) == ("dequantize_absmax_u8 + fp16 gemm" if workspace_mode == "u8_dequantise_first"
+                                    else f"gemm_nt_u8_mfma_{tile}x64")
     gen = torch.Generator(device="cuda").manual_seed(45 + n)
     q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)
     s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
@@ -390,11 +394,12 @@ def test_u8_other_block_sizes_and_fallbacks(kern):
 DECODE = [(4096, 4096), (4096, 11008), (4096, 12288), (11008, 4096)]
 
 
+@pytest.mark.parametrize("workspace_mode", ["pool_off", "shipped_default"], indirect=True)
 @pytest.mark.parametrize("kn", DECODE, ids=[f"K{k}_N{n}" for k, n in DECODE])
 @pytest.mark.parametrize("m", [1, 4, 16])
-def test_decode_shapes_full_size(kern, kn, m):
+def test_decode_shapes_full_size(kern, kn, m, workspace_mode):
     """benchmark config 3 at full size against an fp32 GEMM on the (bit-exactly) dequantised
-    weights, computed on the device."""
+    weights, computed on the device; with the workspace pool off and as the library ships."""
     p, n = kn
     gen = torch.Generator(device="cuda").manual_seed(44)
     q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)

@@ -1,7 +1,10 @@
 """adr_matmul_f16_noalloc (the entry point that allocates nothing: its scratch is a fixed array
 inside the library's device code) against adr_matmul_f16_ws (the same kernels with a
 caller-provided workspace), through the C ABI: bit-identical results on two calls in a row, the
-second with a smaller input; the size limit; products that need no scratch."""
+second with a smaller input; a product that would like more than the scratch holds; products
+that need no scratch."""
+import ctypes as C
+
 import pytest
 import torch
 
@@ -62,17 +65,26 @@ def test_noalloc_matches_workspace_entry_point_on_two_calls_in_a_row():
 
 def test_noalloc_size_limit_and_products_without_scratch():
     lib = _ffi.lib()
-    # a product whose split would need more than the built-in scratch: rejected, nothing written
+    # a product whose best split would need more than the built-in scratch is cut into as many
+    # pieces as fit: the result of adr_matmul_f16_ws given a workspace of exactly that size
     M, K, N = 300, 22016, 4096
     so, sl, sr = nt(M, K, N)
     assert lib.adr_matmul_f16_workspace_bytes(1, M, K, N, *so, *sl, *sr, 0, 0, 0) > _ffi.NOALLOC_SCRATCH_BYTES
-    a = torch.zeros(M, K, dtype=torch.float16, device="cuda")
-    w = torch.zeros(N, K, dtype=torch.float16, device="cuda")
-    out = torch.full((M, N), 3.0, dtype=torch.float16, device="cuda")
-    rc = call("adr_matmul_f16_noalloc", out, a, w, M, K, N)
-    assert rc == _ffi.ADR_ESCRATCH and "ADR_NOALLOC_SCRATCH_BYTES" in _ffi.strerror(rc)
+    name = C.create_string_buffer(96)
+    assert lib.adr_matmul_f16_ws_plan(name, 96, 1, M, K, N, *so, *sl, *sr, 0, 0, 0, _ffi.NOALLOC_SCRATCH_BYTES) == 0
+    gen = torch.Generator(device="cuda").manual_seed(94)
+    a = torch.randn(M, K, generator=gen, device="cuda").half()
+    w = (torch.randn(N, K, generator=gen, device="cuda") * K ** -0.5).half()
+    ws = torch.empty(_ffi.NOALLOC_SCRATCH_BYTES, dtype=torch.uint8, device="cuda")
+    want = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+    got = torch.zeros_like(want)
+    assert call("adr_matmul_f16_ws", want, a, w, M, K, N, ws=ws) == 0
+    assert call("adr_matmul_f16_noalloc", got, a, w, M, K, N) == 0
     torch.cuda.synchronize()
-    assert torch.all(out == 3.0)
+    assert torch.equal(got, want), name.value
+    ref = a.float() @ w.float().t()
+    rms = ref.pow(2).mean().sqrt()
+    assert ((got.float() - ref).abs() / torch.maximum(ref.abs(), rms)).max().item() <= 2e-3
     # products that are not split run as adr_matmul_f16 does: prefill, decode, empty
     gen = torch.Generator(device="cuda").manual_seed(92)
     for M, K, N in ((512, 1024, 768), (4, 4096, 4096), (0, 64, 64)):
