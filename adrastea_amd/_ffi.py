@@ -19,13 +19,14 @@ SYMBOLS = (
     "adr_dequantize_absmax_u8", "adr_quantize_absmax_u8",
     "adr_dequantize_absmax_uint8", "adr_quantize_absmax_uint8", "adr_matmul_f16_plan",
     "adr_matmul_nt_fp16u8_plan", "adr_softmax_rows", "adr_error_stats_f16", "adr_error_stats_f32", "adr_attention_f16", "adr_embed_uint8",
-    "adr_microbench_empty", "adr_microbench_mfma_f16", "adr_microbench_stream_read",
+    "adr_debug_knob", "adr_microbench_empty", "adr_microbench_mfma_f16", "adr_microbench_stream_read",
     "adr_strerror", "adr_abi_version",
 )
 
 ADR_OK, ADR_EINVAL_SHAPE, ADR_EINVAL_ENUM, ADR_ENOTIMPL, ADR_ENULL, ADR_EDIVISIBILITY = (
     0, -1, -2, -3, -4, -5)
 ADR_EUNSUPPORTED_DEVICE, ADR_EUNSUPPORTED_LAYOUT, ADR_ESCRATCH = -6, -7, -8
+KNOB_GEMM_TILE = 0
 NOALLOC_SCRATCH_BYTES = 16 * 1024 * 1024
 HELD_WORKSPACE_DEFAULT_BYTES = 128 * 1024 * 1024
 
@@ -85,6 +86,7 @@ def lib():
     L.adr_matmul_f16_plan.argtypes = [C.c_char_p, i32] + [i32] * 13 + [u32, u32, u32]
     L.adr_matmul_nt_fp16u8_plan.argtypes = [C.c_char_p, i32, i32, i32, i32, i32]
     L.adr_softmax_rows.argtypes = [vp, vp, vp, i32, i32, i32, f32]
+    L.adr_debug_knob.argtypes = [i32, i32]
     L.adr_microbench_empty.argtypes = [vp]
     L.adr_microbench_mfma_f16.argtypes = [vp, i32, i32, i32, vp]
     L.adr_microbench_stream_read.argtypes = [vp, vp, C.c_int64, i32, vp]

@@ -209,6 +209,17 @@ struct DeviceInfo {
 DeviceInfo device_info();
 DeviceInfo device_info_for_plan();  // as above, but an MI355X where no usable device is current
 
+// Switches for tests and benchmarks (adr_debug_knob): they force a kernel choice that the
+// dispatch would make by itself from the arguments.  0 = the dispatch decides.
+enum Knob {
+  KNOB_GEMM_TILE = 0,  // fp16 tiled GEMM: 1 + index into the tile list (gemm_mfma.hip: forced tile)
+  KNOB_LAB_A,          // (free for lab builds)
+  KNOB_LAB_B,
+  KNOB_LAB_C,
+  KNOB_COUNT
+};
+int knob(int id);
+
 // Launchers implemented in the kernel translation units; all return a hipError_t.
 hipError_t launch_matmul_general(hipStream_t stream, const MatmulArgs& a);
 // Returns true and fills `name` when the MFMA kernel family covers these arguments.

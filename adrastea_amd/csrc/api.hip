@@ -9,6 +9,10 @@
 
 using namespace adr;
 
+namespace adr {
+int set_knob(int id, int value);  // device.hip
+}
+
 namespace {
 
 constexpr int ABI_VERSION = 1;
@@ -712,6 +716,8 @@ static int error_stats_common(adr_stream_t stream, adr_tensor_desc output, adr_t
   return (int)launch_error_stats((hipStream_t)stream, (float*)output.ptr, lhs.ptr, rhs.ptr,
                                  lhs.shape[0], lhs.strides[0], rhs.strides[0], f32);
 }
+
+int adr_debug_knob(int32_t id, int32_t value) { return set_knob(id, value); }
 
 int adr_microbench_empty(adr_stream_t stream) {
   if (int rc = check_device()) return rc;

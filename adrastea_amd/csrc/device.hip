@@ -68,6 +68,16 @@ DeviceInfo device_info() {
   return d;  // (a thread that lost the race returns its own, identical, copy)
 }
 
+namespace {
+std::atomic<int> knobs[KNOB_COUNT];
+}
+int knob(int id) { return id >= 0 && id < KNOB_COUNT ? knobs[id].load(std::memory_order_relaxed) : 0; }
+int set_knob(int id, int value) {
+  if (id < 0 || id >= KNOB_COUNT) return ADR_EINVAL_ENUM;
+  knobs[id].store(value, std::memory_order_relaxed);
+  return ADR_OK;
+}
+
 DeviceInfo device_info_for_plan() {
   // the plan queries answer without a device too (a build machine): then for an MI355X
   DeviceInfo d = device_info();

@@ -552,6 +552,10 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   __shared__ __attribute__((aligned(1024))) unsigned char sB2[NSTAGE >= 3 ? BN * BK * 2 : 1024];
   __shared__ __attribute__((aligned(1024))) unsigned char sB3[NSTAGE == 6 ? BN * BK * 2 : 1024];
 
+#ifdef ADR_LAB_STAMPS
+  const uint64_t st_c0 = __builtin_readcyclecounter(), st_r0 = __builtin_amdgcn_s_memrealtime();
+  uint64_t st_c1 = 0, st_r1 = 0, st_c2 = 0, st_r2 = 0;
+#endif
   int batch, tile_m, tile_n;
   const int tile_id = SPLIT ? (int)(blockIdx.x % (unsigned)map.total) : (int)blockIdx.x;
   const int piece = SPLIT ? (int)(blockIdx.x / (unsigned)map.total) : 0;
@@ -695,6 +699,22 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
                                                              0, 0, 0);
       }
   };
+  // MFMAs [lo, hi) of a k-step, in the order of mfmas()
+  auto mfmas_range = [&](int slot, auto lo_tag, auto hi_tag) {
+    constexpr int lo = decltype(lo_tag)::value, hi = decltype(hi_tag)::value;
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+      for (int j = 0; j < FN; j++) {
+        if (i * FN + j < lo || i * FN + j >= hi) continue;
+        if constexpr (MI16)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[slot][j], fa[slot][i], acc[i][j],
+                                                             0, 0, 0);
+        else
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[slot][j], fa[slot][i], acc[i][j],
+                                                             0, 0, 0);
+      }
+  };
   // s_waitcnt vmcnt(n) lgkmcnt(0): n outstanding DMA instructions may remain in flight
   auto wait_dma_barrier = [&](auto n_tag) {
     constexpr int n = decltype(n_tag)::value;
@@ -746,6 +766,11 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
     // instruction stream; both pass the same barriers.
     auto run = [&](auto role_tag) {
       constexpr bool LEFT = decltype(role_tag)::value;
+      // (measured on the qkv product, same box, us with the weights rewritten by other launches in
+      // between / multiplied again and again: the compiler's own choice, 38 of 48 behind the
+      // barrier, 173 / 165; 4 or 8: 167 / 167; 12: 159 / 161; 16: 162 / 160; 20, 24: 162-164 / 162)
+      constexpr int KEEP = 12;
+
       int kA = 0, kB = 0;
       auto slice6 = [&](const unsigned char* cA, const unsigned char* cB, const unsigned char* nA,
                         const unsigned char* nB, unsigned char* dA, unsigned char* dB) {
@@ -762,11 +787,23 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
               if (kk * FM * FN + q < (LEFT ? IA : IB)) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
             }
           } else {
-            mfmas(kk & 1);
+            // The slice's last MFMAs: all but KEEP of them in front of the wait and the barrier
+            // (pinned: left to itself the compiler sinks most of the k-step behind the barrier,
+            // and the wait for the left operand's transfers, issued at the head of this very
+            // slice, then comes a few MFMAs after their issue), KEEP behind it, where they cover
+            // the latency of the next slice's first fragment reads.
+            mfmas_range(kk & 1, std::integral_constant<int, 0>{}, std::integral_constant<int, FM * FN - KEEP>{});
+            __builtin_amdgcn_sched_barrier(0);
           }
         }
         wait_dma_barrier(std::integral_constant<int, LEFT ? 0 : 2 * IB>{});
         load_frags(0, nA, nB, 0);
+        mfmas_range((KK - 1) & 1, std::integral_constant<int, FM * FN - KEEP>{}, std::integral_constant<int, FM * FN>{});
+#pragma unroll
+        for (int q = 0; q < KEEP; q++) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, (FM + FN + KEEP - 1) / KEEP, 0);
+        }
         __builtin_amdgcn_sched_barrier(0);
       };
       if (LEFT) {
@@ -778,6 +815,9 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
       }
       wait_dma_barrier(std::integral_constant<int, LEFT ? 0 : 2 * IB>{});
       load_frags(0, sA0, sB0, 0);
+#ifdef ADR_LAB_STAMPS
+      st_c1 = __builtin_readcyclecounter(); st_r1 = __builtin_amdgcn_s_memrealtime();
+#endif
       int kt = 0;
       for (; kt + 4 <= KT; kt += 4) {
         slice6(sA0, sB0, sA1, sB1, sA1, sB3);
@@ -795,6 +835,9 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
     dma(sA1, sB1);
     wait_dma_barrier(std::integral_constant<int, INFLIGHT>{});
     load_frags(0, sA0, sB0, 0);
+#ifdef ADR_LAB_STAMPS
+    st_c1 = __builtin_readcyclecounter(); st_r1 = __builtin_amdgcn_s_memrealtime();
+#endif
     int kt = 0;
     for (; kt + 3 <= KT; kt += 3) {
       slice(sA0, sB0, sA1, sB1, sA2, sB2);
@@ -814,6 +857,9 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
     }
     if (kt < KT) slice(sA0, sB0, sA1, sB1, sA1, sB1);
   }
+#ifdef ADR_LAB_STAMPS
+  st_c2 = __builtin_readcyclecounter(); st_r2 = __builtin_amdgcn_s_memrealtime();
+#endif
   // drain the trailing (redundant) DMA before the stages are reused by the epilogue
   wait_dma_barrier(std::integral_constant<int, 0>{});
 
@@ -835,6 +881,19 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   unsigned char* const slot = (SLOTS_IN_B ? (wave < NW / 2 ? sB0 : sB1) : (wave < NW / 2 ? sA0 : sA1)) +
                               (wave % (NW / 2)) * SLOT;
   wave_epilogue<TM, TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, slot, (half_t)a.scale, lane);
+#ifdef ADR_LAB_STAMPS
+  if (a.workspace && !SPLIT) {
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0): the tile is written
+    const uint64_t st_c3 = __builtin_readcyclecounter(), st_r3 = __builtin_amdgcn_s_memrealtime();
+    if (lane == 0) {
+      uint64_t* st = (uint64_t*)a.workspace + ((int64_t)blockIdx.x * NW + wave) * 10;
+      st[0] = st_c0; st[1] = st_c1; st[2] = st_c2; st[3] = st_c3;
+      st[4] = st_r0; st[5] = st_r1; st[6] = st_r2; st[7] = st_r3;
+      st[8] = __builtin_amdgcn_s_getreg((4 << 0) | (0 << 6) | (31 << 11));   // HW_ID
+      st[9] = __builtin_amdgcn_s_getreg((20 << 0) | (0 << 6) | (31 << 11));  // XCC_ID
+    }
+  }
+#endif
 }
 
 // Second launch of a split product: one workgroup per tile, with the geometry of the kernel that
@@ -1636,7 +1695,7 @@ enum GemmChoice {
   GEMM_NONE = 0,
   SHORTK_64, SHORTK_128,
   U8_256x192, U8_256x128,
-  DMA_256x192, DMA_256x128, DMA_128x256, DMA_128x192, DMA_128x128, DMA_128x64, DMA_64x64, DMA_64x64_K128, DMA_128x64_K128,
+  DMA_256x192, DMA_256x128, DMA_256x128_ROLES, DMA_128x256, DMA_128x192, DMA_128x128, DMA_128x64, DMA_64x64, DMA_64x64_K128, DMA_128x64_K128,
   DMA_NN_256x128, DMA_NN_128x128,
   STAGE_256x128, STAGE_128x128, STAGE_64x64,
 };
@@ -1711,6 +1770,10 @@ GemmChoice choose(const MatmulArgs& a) {
                                          {DMA_64x64, 64, 64, 4, 0.50f}};
       return pick(a, shortk, 2);
     }
+    // (tests and benchmarks can force a tile: adr_debug_knob)
+    const int forced = knob(KNOB_GEMM_TILE);
+    if (forced >= 1 && forced <= N_DMA_TILES) return DMA_TILES[forced - 1].id;
+    if (forced == N_DMA_TILES + 1) return DMA_256x128_ROLES;
     GemmChoice c = pick(a, DMA_TILES, N_DMA_TILES);
     // At most one 64 x 64 tile per CU (a few dozen to a few hundred rows against a weight
     // matrix): the product is bound by how DRAM serves the weight requests -- one piece of every
@@ -1824,6 +1887,7 @@ static bool choice_name(GemmChoice c, const char** name, bool u8 = false) {
     case U8_256x128: *name = "gemm_nt_u8_mfma_256x128x64"; return true;
     case DMA_256x192: *name = "gemm_nt_mfma_dma_256x192x64"; return true;
     case DMA_256x128: *name = "gemm_nt_mfma_dma_256x128x64"; return true;
+    case DMA_256x128_ROLES: *name = "gemm_nt_mfma_dma_256x128x64_roles"; return true;
     case DMA_128x256: *name = "gemm_nt_mfma_dma_128x256x64"; return true;
     case DMA_128x192: *name = "gemm_nt_mfma_dma_128x192x64"; return true;
     case DMA_128x128: *name = "gemm_nt_mfma_dma_128x128x64"; return true;
@@ -1848,6 +1912,7 @@ static hipError_t launch_choice(hipStream_t stream, const MatmulArgs& a, GemmCho
     case U8_256x128: return launch_u8<256, 128, 4, 2, true>(stream, a);
     case DMA_256x192: return launch_dma<256, 192, 4, 2, 6, 1, false, 64, true>(stream, a);
     case DMA_256x128: return launch_dma<256, 128, 4, 2, 3, 1, false, 64, true>(stream, a);
+    case DMA_256x128_ROLES: return launch_dma<256, 128, 4, 2, 6, 1, false, 64, true>(stream, a);
     case DMA_128x256: return launch_dma<128, 256, 2, 4, 3, 1, false, 64, true>(stream, a);
     case DMA_128x192: return launch_dma<128, 192, 2, 2, 3, 1>(stream, a);
     case DMA_128x128: return launch_dma<128, 128, 2, 2, 3, 1>(stream, a);

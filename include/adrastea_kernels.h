@@ -380,6 +380,15 @@ int adr_matmul_f16_ws_plan(char* name, int32_t cap, int32_t batches, int32_t m, 
                            uint32_t load, uint32_t mask, int64_t workspace_bytes);
 
 /*
+ * For tests and benchmarks only (no counterpart in the reference): forces a kernel choice that
+ * the dispatch otherwise makes from the arguments, process-wide, so that the chosen kernel can be
+ * compared with the others on the same operands.  id 0: the tile of the fp16 tiled GEMM (value 0:
+ * the dispatch decides; 1 + i: tile i of 256x192, 256x128, 128x256, 128x192, 128x128, 128x64, 64x64
+ * where the product is one the tiled kernels cover).  Unknown ids return ADR_EINVAL_ENUM.
+ */
+int adr_debug_knob(int32_t id, int32_t value);
+
+/*
  * Microbenchmark aids (the device kernels of adrastea_kernels/cpp/microbench.cu:28-51 -- empty_kernel,
  * wmma_loop_f32_f16 -- as adrastea/src/main.rs:486-553 drives them, plus a streaming read): the
  * measured peaks that the fractions of the 2516.6 TFLOP/s and 8 TB/s figures are put beside.
