@@ -83,6 +83,9 @@ def main():
     ap.add_argument("--step-trace", action="store_true",
                     help="time each of the first 300 replays of the step graph on its own (HIP events), "
                          "from a cold start, and print them: shows how long the device takes to settle")
+    ap.add_argument("--forced-tiles", action="store_true",
+                    help="every fp16 tile forced (adr_debug_knob) on the benchmark's fp16 GEMM shapes "
+                         "beside the tile the dispatch chooses: guards the dispatch's fitted constants")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run only a plain 256 MiB device copy (reference point for the "
                          "FETCH_SIZE / WRITE_SIZE counters of rocprofv3 --pmc)")
@@ -569,6 +572,49 @@ def main():
                         "frac_mfma_peak": round(2.0 * m * K * N / t / 1e12 / PEAK_F16_TFLOPS, 4)}
         return clip
 
+    TILE_NAMES = ["256x192", "256x128", "128x256", "128x192", "128x128", "128x64", "64x64"]
+    FP16_GEMM_SHAPES = [("clip_text_qkv", 77, 768, 2304), ("clip_mlp_up", 2056, 1024, 4096),
+                        ("clip_mlp_down", 2056, 4096, 1024), ("llama_qkv", 2048, 4096, 12288),
+                        ("llama_o", 2048, 4096, 4096), ("llama_gate_up", 2048, 4096, 11008),
+                        ("llama_down", 2048, 11008, 4096)]
+
+    def forced_tiles_set(shapes=FP16_GEMM_SHAPES, rounds=3):
+        """For every fp16 GEMM shape of the benchmark: the dispatch's own choice and every tile
+        forced, interleaved over `rounds` passes (best of the passes per variant, so that clock
+        drift between variants cancels).  `chosen_over_best` near 1 says the fitted tile model
+        still picks well on this machine."""
+        import ctypes
+        rows = []
+        for nm, m, K, N in shapes:
+            a, w = randn_h(m, K), randn_h(N, K, std=K ** -0.5)
+            o = torch.zeros(m, N, dtype=torch.float16, device=dev)
+            buf = ctypes.create_string_buffer(96)
+            lib.adr_matmul_f16_plan(buf, 96, 1, m, K, N, 1, N, 0, 1, K, 0, K, 1, 0, 0, 0, 0)
+            f = lambda: mm(o, a, w, m, K, N)   # noqa: E731
+            iters = max(40, int(0.010 / max(timed(f, 20, 5), 1e-6)))
+            best = {}
+            try:
+                for _ in range(rounds):
+                    for t in range(len(TILE_NAMES) + 1):
+                        lib.adr_debug_knob(0, t)
+                        # (every measurement spans some ten milliseconds: shorter ones see the
+                        # clock wander by a few percent)
+                        us = (timed_graph(f, 50, 40) if m < 256 else timed(f, iters, 10)) * 1e6
+                        key = "chosen" if t == 0 else TILE_NAMES[t - 1]
+                        best[key] = min(best.get(key, 1e30), us)
+            finally:
+                lib.adr_debug_knob(0, 0)
+            fastest = min(v for k, v in best.items() if k != "chosen")
+            rows.append({"shape": nm, "M": m, "K": K, "N": N, "plan": buf.value.decode(),
+                         "chosen_us": round(best["chosen"], 2),
+                         "forced_us": {k: round(v, 2) for k, v in best.items() if k != "chosen"},
+                         "chosen_over_best": round(best["chosen"] / fastest, 3)})
+        return rows
+
+    if args.forced_tiles:
+        print(json.dumps({"forced_tiles": forced_tiles_set()}))
+        return
+
     if args.u8_prefill_only:
         print(json.dumps({"llama7b_prefill_u8": u8_prefill_set()}))
         return
@@ -818,7 +864,33 @@ def main():
         rms = np.sqrt(np.mean(ref ** 2))
         faithful["max_rel_err_gpu_vs_cpu"] = float(
             np.max(np.abs(got - ref) / np.maximum(np.abs(ref), rms)))
+        # The reference's own GPU kernel on this device (its matmul.cu compiled as it lies into
+        # oracle/_ref/matmul.co, launched with the grid its host code uses, kernels.rs:849-863), and
+        # this build's module with the same symbols at that same grid: what a host that keeps
+        # calling `matmul_f16_fast` gets.  A baseline beside the figures above, never timed inside
+        # the step.
+        reference_gpu = None
+        try:
+            from oracle import refgpu
+            if refgpu.available():
+                name, K, N = LAYER_SET[0]
+                so, sl, sr = (1, N, 0), (1, K, 0), (K, 1, 0)
+                reference_gpu = {"shape": f"qkv M{M} K{K} N{N}, NT weights, grid of kernels.rs:849-863"}
+                for label, directory in (("reference_matmul_f16_fast", refgpu.REF_DIR),
+                                         ("this_build_legacy_symbol_matmul_f16_fast", refgpu.LEGACY_DIR)):
+                    if not os.path.exists(os.path.join(directory, "matmul.co")):
+                        continue
+                    rk = refgpu.RefKernels(directory)
+                    call = lambda: rk.matmul_f16_fast(outs[name].data_ptr(), acts[K].data_ptr(),   # noqa: E731
+                                                      weights[name].data_ptr(), 1, M, K, N, so, sl, sr)
+                    t = timed(call, 5, 2)
+                    reference_gpu[label] = {"ms": round(t * 1e3, 3),
+                                            "tflops": round(2.0 * M * K * N / t / 1e12, 2)}
+                reference_gpu["adr_matmul_f16_ms"] = round(t_qkv * 1e3, 4)
+        except Exception as e:  # noqa: BLE001  (a baseline leg: report, never fail the benchmark)
+            reference_gpu = {"error": repr(e)}
         cpu_baseline = {
+            "reference_gpu_kernel_same_device": reference_gpu,
             "value": round(torch_value, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
             "threads": threads, "nproc": nproc,
             "sample": per_config["configs[4] llama7b_layer_set_fp16_M2048"]["sample"] +

@@ -1,0 +1,96 @@
+"""Guard of the dispatch's fitted constants (tile efficiencies, cost model): on the benchmark's
+fp16 GEMM shapes the tile the dispatch chooses must be within 5 % of the best tile forced through
+adr_debug_knob, timed on this machine.  A timing test: variants are interleaved and the best of
+several passes is taken per variant; a miss is measured again before it counts.  Runs late in the
+suite (file name) so that a slow machine cannot hide the parity tests behind it."""
+import ctypes as C
+
+import pytest
+import torch
+
+from adrastea_amd import _ffi
+
+pytestmark = pytest.mark.gpu
+
+TILES = ["256x192", "256x128", "128x256", "128x192", "128x128", "128x64", "64x64"]
+SHAPES = [("clip_mlp_up", 2056, 1024, 4096), ("clip_mlp_down", 2056, 4096, 1024),
+          ("llama_qkv", 2048, 4096, 12288), ("llama_o", 2048, 4096, 4096),
+          ("llama_gate_up", 2048, 4096, 11008), ("llama_down", 2048, 11008, 4096)]
+
+
+def _time(fn, iters, warm=8):
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def _measure(lib, fn, passes):
+    # (every measurement spans some ten milliseconds: shorter ones see the clock wander)
+    iters = max(40, int(10.0 / max(_time(fn, 20), 1e-3)))
+    best = {}
+    try:
+        for _ in range(passes):
+            for t in range(len(TILES) + 1):
+                assert lib.adr_debug_knob(0, t) == 0
+                best[t] = min(best.get(t, 1e30), _time(fn, iters))
+    finally:
+        lib.adr_debug_knob(0, 0)
+    return best
+
+
+def test_forced_tile_changes_the_plan_and_not_the_result():
+    lib = _ffi.lib()
+    M, K, N = 512, 1024, 768
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    a = (torch.randint(-8, 9, (M, K), generator=gen, device="cuda").float() / 64).half()
+    w = (torch.randint(-8, 9, (N, K), generator=gen, device="cuda").float() / 64).half()
+    want = (a.double() @ w.double().t()).half()
+    buf = C.create_string_buffer(96)
+    names = set()
+    try:
+        for t in range(len(TILES) + 1):
+            assert lib.adr_debug_knob(0, t) == 0
+            assert lib.adr_matmul_f16_plan(buf, 96, 1, M, K, N, 1, N, 0, 1, K, 0, K, 1, 0, 0, 0, 0) == 0
+            if t:
+                names.add(buf.value.decode())
+                assert buf.value.decode() == f"gemm_nt_mfma_dma_{TILES[t - 1]}x64"
+            out = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+            assert lib.adr_matmul_f16(torch.cuda.current_stream().cuda_stream, out.data_ptr(), a.data_ptr(),
+                                      w.data_ptr(), 1, M, K, N, 1, N, 0, 1, K, 0, K, 1, 0, None, 0.0, 1.0,
+                                      0, 0, 0) == 0
+            assert torch.equal(out.view(torch.int16), want.view(torch.int16)), buf.value
+    finally:
+        lib.adr_debug_knob(0, 0)
+    assert len(names) == len(TILES)
+    assert lib.adr_debug_knob(99, 1) == _ffi.ADR_EINVAL_ENUM
+
+
+@pytest.mark.parametrize("case", SHAPES, ids=[c[0] for c in SHAPES])
+def test_chosen_tile_is_within_five_percent_of_the_best_forced_one(case):
+    lib = _ffi.lib()
+    _, M, K, N = case
+    gen = torch.Generator(device="cuda").manual_seed(6)
+    a = torch.randn(M, K, generator=gen, device="cuda").half()
+    w = (torch.randn(N, K, generator=gen, device="cuda") * K ** -0.5).half()
+    out = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+
+    def fn():
+        rc = lib.adr_matmul_f16(torch.cuda.current_stream().cuda_stream, out.data_ptr(), a.data_ptr(),
+                                w.data_ptr(), 1, M, K, N, 1, N, 0, 1, K, 0, K, 1, 0, None, 0.0, 1.0, 0, 0, 0)
+        assert rc == 0
+    for _ in range(100):   # the clocks settle under load
+        fn()
+    ratio = None
+    for attempt in range(3):
+        best = _measure(lib, fn, passes=3)
+        ratio = best[0] / min(v for t, v in best.items() if t)
+        if ratio <= 1.05:
+            break
+    assert ratio <= 1.05, (case, {("chosen" if t == 0 else TILES[t - 1]): round(v * 1e3, 1) for t, v in best.items()})
