@@ -75,6 +75,31 @@ def build_library(force: bool = False, extra_flags=()) -> str:
     return LIB
 
 
+STAMPS_LIB = os.path.join(LIBDIR, "libadrastea_kernels_hip_stamps.so")
+
+
+def build_stamps_library(force: bool = False) -> str:
+    """The diagnostic twin of the library: gemm_mfma.hip compiled with -DADR_PHASE_STAMPS (its tiled
+    GEMM kernels then leave per-wavefront time stamps of prologue / K loop / epilogue in the
+    buffer passed as workspace), linked with the other objects of build_library().  Read by
+    `bench.py --phase-stamps`; nothing else loads it."""
+    build_library(force=False)
+    if (not force and os.path.exists(STAMPS_LIB)
+            and all(os.path.getmtime(f) <= os.path.getmtime(STAMPS_LIB) for f in _deps())):
+        return STAMPS_LIB
+    obj = os.path.join(LIBDIR, "gemm_mfma_stamps.o")
+    cmd = [HIPCC, *CXXFLAGS, "-DADR_PHASE_STAMPS", "-c", os.path.join(CSRC, "gemm_mfma.hip"), "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed for the stamps build:\n{r.stdout}\n{r.stderr}")
+    objs = [os.path.join(LIBDIR, os.path.splitext(src)[0] + ".o") for src in SOURCES if src != "gemm_mfma.hip"]
+    cmd = [HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", STAMPS_LIB, obj, *objs]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
+    return STAMPS_LIB
+
+
 # Code objects for an unmodified host of the reference: module name -> source.  Each exports the
 # device symbols that host looks up in its module of that name, with the same kernel arguments.
 LEGACY_DIR = os.path.join(LIBDIR, "legacy")
@@ -121,5 +146,6 @@ def build_host_test(force: bool = False) -> str:
 
 if __name__ == "__main__":
     print(build_library(force="--force" in sys.argv))
+    print(build_stamps_library(force="--force" in sys.argv))
     print(build_legacy_modules(force="--force" in sys.argv))
     print(build_host_test(force="--force" in sys.argv))

@@ -552,7 +552,11 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   __shared__ __attribute__((aligned(1024))) unsigned char sB2[NSTAGE >= 3 ? BN * BK * 2 : 1024];
   __shared__ __attribute__((aligned(1024))) unsigned char sB3[NSTAGE == 6 ? BN * BK * 2 : 1024];
 
-#ifdef ADR_LAB_STAMPS
+  // Diagnostic build only (-DADR_PHASE_STAMPS, adrastea_amd.build.build_stamps_library, read by
+  // bench.py --phase-stamps): every wavefront leaves the shader-clock and 100 MHz real-time
+  // counters at its start, behind its prologue, behind its K loop and behind its stores in the
+  // buffer passed as workspace ([workgroup][wavefront][10] 64-bit words).
+#ifdef ADR_PHASE_STAMPS
   const uint64_t st_c0 = __builtin_readcyclecounter(), st_r0 = __builtin_amdgcn_s_memrealtime();
   uint64_t st_c1 = 0, st_r1 = 0, st_c2 = 0, st_r2 = 0;
 #endif
@@ -815,7 +819,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
       }
       wait_dma_barrier(std::integral_constant<int, LEFT ? 0 : 2 * IB>{});
       load_frags(0, sA0, sB0, 0);
-#ifdef ADR_LAB_STAMPS
+#ifdef ADR_PHASE_STAMPS
       st_c1 = __builtin_readcyclecounter(); st_r1 = __builtin_amdgcn_s_memrealtime();
 #endif
       int kt = 0;
@@ -835,7 +839,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
     dma(sA1, sB1);
     wait_dma_barrier(std::integral_constant<int, INFLIGHT>{});
     load_frags(0, sA0, sB0, 0);
-#ifdef ADR_LAB_STAMPS
+#ifdef ADR_PHASE_STAMPS
     st_c1 = __builtin_readcyclecounter(); st_r1 = __builtin_amdgcn_s_memrealtime();
 #endif
     int kt = 0;
@@ -857,7 +861,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
     }
     if (kt < KT) slice(sA0, sB0, sA1, sB1, sA1, sB1);
   }
-#ifdef ADR_LAB_STAMPS
+#ifdef ADR_PHASE_STAMPS
   st_c2 = __builtin_readcyclecounter(); st_r2 = __builtin_amdgcn_s_memrealtime();
 #endif
   // drain the trailing (redundant) DMA before the stages are reused by the epilogue
@@ -881,7 +885,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   unsigned char* const slot = (SLOTS_IN_B ? (wave < NW / 2 ? sB0 : sB1) : (wave < NW / 2 ? sA0 : sA1)) +
                               (wave % (NW / 2)) * SLOT;
   wave_epilogue<TM, TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, slot, (half_t)a.scale, lane);
-#ifdef ADR_LAB_STAMPS
+#ifdef ADR_PHASE_STAMPS
   if (a.workspace && !SPLIT) {
     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0): the tile is written
     const uint64_t st_c3 = __builtin_readcyclecounter(), st_r3 = __builtin_amdgcn_s_memrealtime();
@@ -1823,6 +1827,9 @@ struct SplitChoice {
 
 SplitChoice choose_split(const MatmulArgs& a, int64_t avail_bytes) {
   const SplitChoice none = {GEMM_NONE, 1, 0, 0};
+#ifdef ADR_PHASE_STAMPS
+  return none;  // (the diagnostic build: the workspace argument receives the stamps)
+#endif
   if (avail_bytes <= 0 || a.rhs_q || a.load != ADR_LOAD_IDENTITY || a.k % 64 != 0 || a.k < 1024)
     return none;
   const GemmChoice whole = choose(a);

@@ -83,6 +83,9 @@ def main():
     ap.add_argument("--step-trace", action="store_true",
                     help="time each of the first 300 replays of the step graph on its own (HIP events), "
                          "from a cold start, and print them: shows how long the device takes to settle")
+    ap.add_argument("--phase-stamps", action="store_true",
+                    help="per-workgroup timeline of the tiled fp16 GEMM on the layer set (prologue, K loop, "
+                         "epilogue, rounds), from the diagnostic build of the library that stamps them")
     ap.add_argument("--forced-tiles", action="store_true",
                     help="every fp16 tile forced (adr_debug_knob) on the benchmark's fp16 GEMM shapes "
                          "beside the tile the dispatch chooses: guards the dispatch's fitted constants")
@@ -98,6 +101,9 @@ def main():
 
     import torch
     from adrastea_amd import _ffi
+    if args.phase_stamps:
+        # the diagnostic twin (adrastea_amd.build.build_stamps_library): same kernels, plus stamps
+        _ffi.LIB_PATH = os.path.join(os.path.dirname(_ffi.LIB_PATH), "libadrastea_kernels_hip_stamps.so")
     lib = _ffi.lib()  # raises if the HIP library is not built: there is no fallback
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -613,6 +619,68 @@ def main():
 
     if args.forced_tiles:
         print(json.dumps({"forced_tiles": forced_tiles_set()}))
+        return
+
+    def phase_stamps_set():
+        """Where the time of a tiled fp16 GEMM launch goes: every workgroup's start, prologue, K
+        loop and epilogue (100 MHz real-time counter, averaged over its wavefronts), the loop's
+        length in shader-clock cycles, and the rounds of workgroups over the compute units."""
+        import numpy as np
+        lib.adr_set_held_workspace_limit(0)
+        M = 2048
+        rows = []
+        for name, K, N in LAYER_SET:
+            if name == "up":
+                continue
+            a, w = randn_h(M, K), randn_h(N, K, std=K ** -0.5)
+            o = torch.zeros(M, N, dtype=torch.float16, device=dev)
+            wide = N > 4096
+            bm, bn, nw = 256, (192 if wide else 128), 8
+            tiles = ((M + bm - 1) // bm) * ((N + bn - 1) // bn)
+            # MFMA issue cycles of one K slice on one SIMD: two wavefronts, each bm * bn / 8 outputs as
+            # 16 x 16 blocks over two k-steps of 32, sixteen clocks per v_mfma_f32_16x16x32_f16
+            ideal = bm * bn // 32
+            st_buf = torch.zeros(tiles * nw * 10, dtype=torch.int64, device=dev)
+
+            def call(ws):
+                rc = (lib.adr_matmul_f16(stream(), o.data_ptr(), a.data_ptr(), w.data_ptr(), 1, M, K, N, 1, N, 0, 1, K, 0,
+                                         K, 1, 0, None, 0.0, 1.0, 0, 0, 0) if ws is None else
+                      lib.adr_matmul_f16_ws(stream(), o.data_ptr(), a.data_ptr(), w.data_ptr(), 1, M, K, N, 1, N, 0, 1, K,
+                                            0, K, 1, 0, None, 0.0, 1.0, 0, 0, 0, ws.data_ptr(), ws.numel() * 8))
+                if rc != 0:
+                    raise RuntimeError(_ffi.strerror(rc))
+            timed(lambda: call(None), 300, 10)   # the clocks settle under this load
+            t_event = timed(lambda: call(st_buf), 20, 5) * 1e6
+            torch.cuda.synchronize()
+            st = st_buf.cpu().numpy().reshape(tiles, nw, 10).astype(np.float64)
+            r, c = st[:, :, 4:8] * 0.01, st[:, :, 0:4]   # microseconds; shader-clock cycles
+            t0 = r[:, :, 0].min()
+            start, end = r[:, 0, 0] - t0, r[:, :, 3].max(axis=1) - t0
+            pro = (r[:, :, 1] - r[:, :, 0]).mean(axis=1)
+            loop = (r[:, :, 2] - r[:, :, 1]).mean(axis=1)
+            epi = (r[:, :, 3] - r[:, :, 2]).mean(axis=1)
+            cyc = (c[:, :, 2] - c[:, :, 1]).mean(axis=1)
+            order = np.argsort(start)
+            cus = 256
+            row = {"product": name, "M": M, "K": K, "N": N, "tile": f"{bm}x{bn}", "workgroups": tiles,
+                   "launch_us_hip_events": round(t_event, 1), "first_start_to_last_end_us": round(float(end.max()), 1),
+                   "mfma_issue_cycles_per_slice": ideal, "rounds": []}
+            for lo in range(0, tiles, cus):
+                sel = order[lo:lo + cus]
+                row["rounds"].append({
+                    "workgroups": int(len(sel)), "start_us_mean": round(float(start[sel].mean()), 2),
+                    "prologue_us": round(float(pro[sel].mean()), 2), "k_loop_us": round(float(loop[sel].mean()), 2),
+                    "epilogue_us_stores_acknowledged": round(float(epi[sel].mean()), 2),
+                    "end_us_min_mean_max": [round(float(end[sel].min()), 2), round(float(end[sel].mean()), 2),
+                                            round(float(end[sel].max()), 2)],
+                    "k_loop_cycles_per_slice": round(float(cyc[sel].mean()) / (K // 64)),
+                    "shader_clock_ghz_in_k_loop": round(float((cyc[sel] / loop[sel]).mean()) / 1e3, 3)})
+            row["wavefront_skew_at_loop_end_us"] = round(float((r[:, :, 2].max(axis=1) - r[:, :, 2].min(axis=1)).mean()), 2)
+            rows.append(row)
+        return rows
+
+    if args.phase_stamps:
+        print(json.dumps({"phase_stamps": phase_stamps_set()}))
         return
 
     if args.u8_prefill_only:
