@@ -9,9 +9,9 @@
 //
 //  gemm_nt_dma_kernel   K % 64 == 0, plain fp16 operands.  K slices of depth 64 go from global
 //                       memory straight into LDS (global_load_lds_dwordx4, no register round
-//                       trip) into statically separate LDS stages (three per operand, or two of
-//                       the left and four of the right operand with the transfers split by
-//                       wavefront role), so the loads of the next slices are in flight while
+//                       trip) into statically separate LDS stages (three per operand, or two /
+//                       three of the left and four of the right operand with the transfers split
+//                       by wavefront role), so the loads of the next slices are in flight while
 //                       the current slice feeds the MFMAs; one barrier per slice.  MFMA
 //                       fragments are prefetched one k-step ahead and interleaved with the
 //                       MFMAs by scheduling-group barriers.
@@ -525,7 +525,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   constexpr int NW = WM * WN, NT = NW * 64;
   // DMA instructions per thread and slice.  NSTAGE == 6: the first half of the wavefronts issues
   // all transfers of the left operand, the second half all of the right one (NWD each)
-  constexpr int NWD = NSTAGE == 6 ? NW / 2 : NW;
+  constexpr int NWD = NSTAGE >= 6 ? NW / 2 : NW;
   constexpr int IA = BM * CPR / (NWD * 64), IB = BN * CPR / (NWD * 64);
   constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
   constexpr int FM = WTM / MI, FN = WTN / MI;  // MFMA blocks of the wavefront's sub-tile
@@ -538,19 +538,19 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   constexpr bool SLOTS_IN_B = BN > BM;
   static_assert((NW / 2) * SLOT <= (SLOTS_IN_B ? BN : BM) * BK * 2,
                 "epilogue slots must fit in the stage buffers");
-  static_assert(NSTAGE == 2 || NSTAGE == 3 || NSTAGE == 6,
+  static_assert(NSTAGE == 2 || NSTAGE == 3 || NSTAGE == 6 || NSTAGE == 7,
                 "2 or 3 LDS stages, or 6: two stages of the left and four of the right operand");
-  static_assert(NSTAGE != 6 || (!NN && !SPLIT && NW % 2 == 0), "role split: plain NT products");
+  static_assert(NSTAGE < 6 || (!NN && !SPLIT && NW % 2 == 0), "role split: plain NT products");
   static_assert(!NN || BN == 128, "the N-contiguous right operand is staged as [64][128] tiles");
   // Separate objects per stage: the compiler's alias analysis then knows that the asynchronous
   // LDS writes of one stage cannot touch the stage being read, and does not serialise them.
   __shared__ __attribute__((aligned(1024))) unsigned char sA0[BM * BK * 2];
   __shared__ __attribute__((aligned(1024))) unsigned char sA1[BM * BK * 2];
-  __shared__ __attribute__((aligned(1024))) unsigned char sA2[NSTAGE == 3 ? BM * BK * 2 : 1024];
+  __shared__ __attribute__((aligned(1024))) unsigned char sA2[NSTAGE == 3 || NSTAGE == 7 ? BM * BK * 2 : 1024];
   __shared__ __attribute__((aligned(1024))) unsigned char sB0[BN * BK * 2];
   __shared__ __attribute__((aligned(1024))) unsigned char sB1[BN * BK * 2];
   __shared__ __attribute__((aligned(1024))) unsigned char sB2[NSTAGE >= 3 ? BN * BK * 2 : 1024];
-  __shared__ __attribute__((aligned(1024))) unsigned char sB3[NSTAGE == 6 ? BN * BK * 2 : 1024];
+  __shared__ __attribute__((aligned(1024))) unsigned char sB3[NSTAGE >= 6 ? BN * BK * 2 : 1024];
 
   // Diagnostic build only (-DADR_PHASE_STAMPS, adrastea_amd.build.build_stamps_library, read by
   // bench.py --phase-stamps): every wavefront leaves the shader-clock and 100 MHz real-time
@@ -588,7 +588,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   // DMA instruction i of this wavefront fills LDS chunks [(i*NW + wave)*64, +64) of a stage,
   // lane l the l-th of them; the lane fetches whatever (row, k-chunk) the swizzle puts there.
   // Rows beyond the matrix are clamped to the last row (their results are never stored).
-  const int dwave = NSTAGE == 6 ? wave % NWD : wave;  // index among the wavefronts issuing an operand
+  const int dwave = NSTAGE >= 6 ? wave % NWD : wave;  // index among the wavefronts issuing an operand
   const half_t* gA[IA];
   const half_t* gB[IB];
 #pragma unroll
@@ -759,8 +759,8 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  if constexpr (NSTAGE == 6) {
-    // Two stages of the left and four of the right operand, and two roles.  A wavefront's
+  if constexpr (NSTAGE >= 6) {
+    // Two (NSTAGE 6) or three (NSTAGE 7) stages of the left and four of the right operand, and two roles.  A wavefront's
     // transfers complete in the order it issued them, so a wavefront that issues both operands
     // cannot leave a right-operand slice in flight across the wait for the next left-operand
     // slice.  Here wavefronts 0 .. NW/2-1 issue every transfer of the left operand (slice kt+1 at
@@ -768,11 +768,16 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
     // (slice kt+3 at the head of slice kt; at its end slices kt+2 and kt+3 may still be in
     // flight): weights that no cache holds get three slices to arrive.  Each role has its own
     // instruction stream; both pass the same barriers.
+    constexpr int SA = NSTAGE == 6 ? 2 : 3, SB = 4, P = NSTAGE == 6 ? 4 : 12;  // P: the stages' common period
+    auto stA = [&](int i) -> unsigned char* { return i == 0 ? sA0 : i == 1 ? sA1 : sA2; };
+    auto stB = [&](int i) -> unsigned char* { return i == 0 ? sB0 : i == 1 ? sB1 : i == 2 ? sB2 : sB3; };
     auto run = [&](auto role_tag) {
       constexpr bool LEFT = decltype(role_tag)::value;
       // (measured on the qkv product, same box, us with the weights rewritten by other launches in
       // between / multiplied again and again: the compiler's own choice, 38 of 48 behind the
       // barrier, 173 / 165; 4 or 8: 167 / 167; 12: 159 / 161; 16: 162 / 160; 20, 24: 162-164 / 162)
+      // (the 256 x 128 tile with three left and four right stages: 4 behind the barrier o 58.6 us, 8
+      // 57.2, 12 and 16 55.8; with three stages of both operands and every wavefront issuing both 57.4)
       constexpr int KEEP = 12;
 
       int kA = 0, kB = 0;
@@ -800,7 +805,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
             __builtin_amdgcn_sched_barrier(0);
           }
         }
-        wait_dma_barrier(std::integral_constant<int, LEFT ? 0 : 2 * IB>{});
+        wait_dma_barrier(std::integral_constant<int, LEFT ? (SA - 2) * IA : (SB - 2) * IB>{});
         load_frags(0, nA, nB, 0);
         mfmas_range((KK - 1) & 1, std::integral_constant<int, FM * FN - KEEP>{}, std::integral_constant<int, FM * FN>{});
 #pragma unroll
@@ -810,28 +815,32 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
         }
         __builtin_amdgcn_sched_barrier(0);
       };
+      // slice kt (kt % P == p) reads stages p % SA and p % SB; the transfers issued at its head
+      // refill the stages read one slice earlier: left slice kt + SA - 1, right slice kt + SB - 1
+      auto slice_p = [&](int p) {
+        slice6(stA(p % SA), stB(p % SB), stA((p + 1) % SA), stB((p + 1) % SB), stA((p + SA - 1) % SA),
+               stB((p + SB - 1) % SB));
+      };
       if (LEFT) {
-        dmaA(min(kA++, KT - 1), sA0);
+#pragma unroll
+        for (int i = 0; i < SA - 1; i++) dmaA(min(kA++, KT - 1), stA(i));
       } else {
-        dmaB(min(kB++, KT - 1), sB0);
-        dmaB(min(kB++, KT - 1), sB1);
-        dmaB(min(kB++, KT - 1), sB2);
+#pragma unroll
+        for (int i = 0; i < SB - 1; i++) dmaB(min(kB++, KT - 1), stB(i));
       }
-      wait_dma_barrier(std::integral_constant<int, LEFT ? 0 : 2 * IB>{});
+      wait_dma_barrier(std::integral_constant<int, LEFT ? (SA - 2) * IA : (SB - 2) * IB>{});
       load_frags(0, sA0, sB0, 0);
 #ifdef ADR_PHASE_STAMPS
       st_c1 = __builtin_readcyclecounter(); st_r1 = __builtin_amdgcn_s_memrealtime();
 #endif
       int kt = 0;
-      for (; kt + 4 <= KT; kt += 4) {
-        slice6(sA0, sB0, sA1, sB1, sA1, sB3);
-        slice6(sA1, sB1, sA0, sB2, sA0, sB0);
-        slice6(sA0, sB2, sA1, sB3, sA1, sB1);
-        slice6(sA1, sB3, sA0, sB0, sA0, sB2);
+      for (; kt + P <= KT; kt += P) {
+#pragma unroll
+        for (int p = 0; p < P; p++) slice_p(p);
       }
-      if (kt < KT) { slice6(sA0, sB0, sA1, sB1, sA1, sB3); kt++; }
-      if (kt < KT) { slice6(sA1, sB1, sA0, sB2, sA0, sB0); kt++; }
-      if (kt < KT) { slice6(sA0, sB2, sA1, sB3, sA1, sB1); kt++; }
+#pragma unroll
+      for (int p = 0; p < P - 1; p++)
+        if (kt < KT) { slice_p(p); kt++; }
     };
     if (__builtin_amdgcn_readfirstlane(wave) < NW / 2) run(std::true_type{}); else run(std::false_type{});
   } else if (NSTAGE == 3) {
@@ -1699,7 +1708,7 @@ enum GemmChoice {
   GEMM_NONE = 0,
   SHORTK_64, SHORTK_128,
   U8_256x192, U8_256x128,
-  DMA_256x192, DMA_256x128, DMA_256x128_ROLES, DMA_128x256, DMA_128x192, DMA_128x128, DMA_128x64, DMA_64x64, DMA_64x64_K128, DMA_128x64_K128,
+  DMA_256x192, DMA_256x128, DMA_128x256, DMA_128x192, DMA_128x128, DMA_128x64, DMA_64x64, DMA_64x64_K128, DMA_128x64_K128,
   DMA_NN_256x128, DMA_NN_128x128,
   STAGE_256x128, STAGE_128x128, STAGE_64x64,
 };
@@ -1777,7 +1786,6 @@ GemmChoice choose(const MatmulArgs& a) {
     // (tests and benchmarks can force a tile: adr_debug_knob)
     const int forced = knob(KNOB_GEMM_TILE);
     if (forced >= 1 && forced <= N_DMA_TILES) return DMA_TILES[forced - 1].id;
-    if (forced == N_DMA_TILES + 1) return DMA_256x128_ROLES;
     GemmChoice c = pick(a, DMA_TILES, N_DMA_TILES);
     // At most one 64 x 64 tile per CU (a few dozen to a few hundred rows against a weight
     // matrix): the product is bound by how DRAM serves the weight requests -- one piece of every
@@ -1894,7 +1902,6 @@ static bool choice_name(GemmChoice c, const char** name, bool u8 = false) {
     case U8_256x128: *name = "gemm_nt_u8_mfma_256x128x64"; return true;
     case DMA_256x192: *name = "gemm_nt_mfma_dma_256x192x64"; return true;
     case DMA_256x128: *name = "gemm_nt_mfma_dma_256x128x64"; return true;
-    case DMA_256x128_ROLES: *name = "gemm_nt_mfma_dma_256x128x64_roles"; return true;
     case DMA_128x256: *name = "gemm_nt_mfma_dma_128x256x64"; return true;
     case DMA_128x192: *name = "gemm_nt_mfma_dma_128x192x64"; return true;
     case DMA_128x128: *name = "gemm_nt_mfma_dma_128x128x64"; return true;
@@ -1918,8 +1925,7 @@ static hipError_t launch_choice(hipStream_t stream, const MatmulArgs& a, GemmCho
     case U8_256x192: return launch_u8<256, 192, 4, 2, false>(stream, a);
     case U8_256x128: return launch_u8<256, 128, 4, 2, true>(stream, a);
     case DMA_256x192: return launch_dma<256, 192, 4, 2, 6, 1, false, 64, true>(stream, a);
-    case DMA_256x128: return launch_dma<256, 128, 4, 2, 3, 1, false, 64, true>(stream, a);
-    case DMA_256x128_ROLES: return launch_dma<256, 128, 4, 2, 6, 1, false, 64, true>(stream, a);
+    case DMA_256x128: return launch_dma<256, 128, 4, 2, 7, 1, false, 64, true>(stream, a);
     case DMA_128x256: return launch_dma<128, 256, 2, 4, 3, 1, false, 64, true>(stream, a);
     case DMA_128x192: return launch_dma<128, 192, 2, 2, 3, 1>(stream, a);
     case DMA_128x128: return launch_dma<128, 128, 2, 2, 3, 1>(stream, a);

@@ -557,6 +557,23 @@ def test_large_tiles_every_k_tail_exact(K, M, N, tile):
     assert torch.equal(out.view(torch.int16), want.view(torch.int16))
 
 
+@pytest.mark.parametrize("K", [1536 + 64 * i for i in range(12)])
+def test_256x128_tile_every_remainder_of_its_twelve_slice_period(K):
+    """The 256 x 128 kernel rotates three left and four right LDS stages (period twelve slices), half
+    of its wavefronts issuing the left and half the right operand's transfers: every remainder of
+    that loop on inputs whose fp32 sums are exact, ragged last tile row and column."""
+    M, N = 2000, 8184
+    so, sl, sr = nt_strides(M, K, N)
+    assert plan(1, M, K, N, so, sl, sr) == "gemm_nt_mfma_dma_256x128x64"
+    gen = torch.Generator(device="cuda").manual_seed(K)
+    a = (torch.randint(-4, 5, (M, K), generator=gen, device="cuda").float() / 64).half()
+    w = (torch.randint(-4, 5, (N, K), generator=gen, device="cuda").float() / 64).half()
+    out = torch.full((M, N), 9.0, dtype=torch.float16, device="cuda")
+    assert raw_matmul("adr_matmul_f16", out, a, w, 1, M, K, N, so, sl, sr) == 0
+    want = (a.double() @ w.double().t()).half()
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+
+
 @pytest.mark.parametrize("store", STORES_EXACT + STORES_F32)
 @pytest.mark.parametrize("mask", [oracle.MASK_NONE, oracle.MASK_CAUSAL])
 @pytest.mark.parametrize("M,N,tile", [(4000, 4088, "256x128"), (630, 12280, "128x256"), (380, 12280, "128x192")])
