@@ -523,8 +523,9 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   constexpr int CPR = BK / 8, KK = CPR / KG;   // k-steps per slice: of 16 k (32x32x16) or 32 k
   static_assert(BK == 64 || (BK == 128 && !NN && NSTAGE == 3), "slices of 64, or 128 with three stages");
   constexpr int NW = WM * WN, NT = NW * 64;
-  // DMA instructions per thread and slice.  NSTAGE == 6: the first half of the wavefronts issues
-  // all transfers of the left operand, the second half all of the right one (NWD each)
+  // DMA instructions per thread and slice.  NSTAGE == 6 (two left + four right stages) and
+  // NSTAGE == 7 (three left + four right): the first half of the wavefronts issues all transfers
+  // of the left operand, the second half all of the right one (NWD each)
   constexpr int NWD = NSTAGE >= 6 ? NW / 2 : NW;
   constexpr int IA = BM * CPR / (NWD * 64), IB = BN * CPR / (NWD * 64);
   constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
@@ -958,32 +959,81 @@ __global__ __launch_bounds__(WM* WN * 64) void splitk_reduce_kernel(MatmulArgs a
 // Short-K persistent kernel (K == 64 or K == 128): QK^T-shaped products
 // =============================================================================================
 // With one or two K slices a tile is all load latency and epilogue, and the job is bound by the
-// output writes.  One workgroup per CU walks segments of tile rows (128 x 128 tiles): the left
-// panel of the segment stays in LDS, the right panels stream through a ring of three buffers,
-// and the wavefronts have three roles:
-//   0..3  multiply: MFMAs of tile j (2 x 2, 64 x 64 each), then the narrowed result goes into a
-//         128 x 128 fp16 staging tile in LDS;
-//   4..7  write: read tile j-1 from the staging tile as whole 256-byte rows, apply the store
-//         operator, issue the global stores.  Output writes stall the wavefront that issues
-//         them (the job is write bound), so they come from wavefronts that feed nothing else;
-//   8..11 load: keep the DMA two tiles ahead and wait for it.  A wavefront's memory counter
-//         covers its loads and stores alike, which is why loading and writing are not combined.
-// Two barriers per tile: X(j) (panel j landed, staging tile j-1 complete) and Y(j) (tile j
-// multiplied, staging tile j-1 read): between X(j) and Y(j) the MFMAs of tile j overlap the writes
-// of tile j-1.
+// output writes.  One workgroup per CU walks segments of tile rows (128 x 128 tiles).  The left
+// panel of a segment is copied from LDS into registers once, the right panels stream through a
+// ring of three LDS buffers, and the twelve wavefronts have four roles:
+//   0..3   upper group: rows 0..63 of every tile, 32 columns each;
+//   4..7   lower group: rows 64..127.  A group alternates between multiplying its half of a tile
+//          (32 MFMAs of 16x16x32 per wavefront, eight independent accumulators) and narrowing the result into its half of a 128 x 128 fp16
+//          staging tile in LDS; the two groups run half a tile apart, so that while one
+//          multiplies the other narrows, and the matrix pipes see a multiplying wavefront all the time;
+//   8..9   write: read a staged half tile as whole 256-byte rows, apply the store operator,
+//          issue the global stores.  Output writes stall the wavefront that issues them, so
+//          they come from wavefronts that feed nothing else;
+//   10..11 load: keep the DMA two tiles ahead and wait for it.  A wavefront's memory counter
+//          covers its loads and stores alike, which is why loading and writing are not combined.
+// One barrier per half tile.  Between barrier p and barrier p+1 (phase p), with tile j = p / 2:
+//   even p: upper multiplies tile j        | lower narrows tile j-1 | writers: upper half of j-1
+//   odd p:  upper narrows tile j           | lower multiplies tile j | writers: lower half of j-1
+// A workgroup with T tiles passes 2T + 2 barriers in every role.  The right panel of tile j is read
+// in phases 2j and 2j+1 and its buffer refilled (tile j+3) in phase 2j+2.  Both groups copy the
+// left panel of a new segment in the even phase of its first tile (the lower group's registers
+// are free by then), and the loader refills that buffer for the next segment one phase later.
 struct ShortKMap {
   int tiles_m, tiles_n, rows;   // rows = batches * tiles_m
   int seg, segs_per_row, units; // a unit is `seg` consecutive tiles of one tile row
   int xcds;                     // dies of the device
+  int prefilled;                // the tiles above the diagonal of a causal product are written
 };
 
+// The 128-column tiles that lie entirely above the diagonal of a causal product, as whole runs
+// of a row (one wavefront per row): -inf without any arithmetic (matmul.cu:182-184).  Runs of up
+// to a whole row are what the memory likes best; the same bytes written tile by tile from inside
+// the persistent kernel hold up its barriers.
+__global__ __launch_bounds__(256) void fill_causal_rows_kernel(MatmulArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t r = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);  // row, over all batches
+  if (r >= (int64_t)a.batches * a.m) return;
+  const int batch = (int)(r / a.m), y = (int)(r - (int64_t)batch * a.m);
+  const int x0 = (y / 128 + 1) * 128;  // first column right of the tile that holds the diagonal
+  half_t* const out = a.output + (int64_t)batch * a.stride_oz;
+  half_t* const row = out + (int64_t)y * a.stride_oy;
+  const half_t ninf = neg_inf_half();
+  if (out_vectorizable(a, out)) {
+    const half8_t v = {ninf, ninf, ninf, ninf, ninf, ninf, ninf, ninf};
+    for (int x = x0 + lane * 8; x < a.n; x += 512) {
+      if (x + 8 <= a.n) {
+        __builtin_nontemporal_store(v, (half8_t*)(row + x));
+      } else {
+        for (int q = 0; x + q < a.n; q++) row[x + q] = ninf;
+      }
+    }
+  } else {
+    for (int x = x0 + lane; x < a.n; x += 64) row[x] = ninf;
+  }
+}
+
+// (four writers instead of two leave the multiplying wavefronts 128 registers, nine short, and
+// measure the same: the stores wait for the memory, not for wavefronts to issue them)
+constexpr int SHORTK_WRITERS = 2, SHORTK_LOADERS = 2;
+constexpr int SHORTK_THREADS = (8 + SHORTK_WRITERS + SHORTK_LOADERS) * 64;
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt_at_most() {
+  static_assert(N >= 0 && N < 64, "vmcnt is a six-bit counter");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 0xF) | ((N >> 4) << 14));
+}
+
 template <int CPR>  // 16-byte chunks per row: 8 (K = 64) or 16 (K = 128)
-__global__ __launch_bounds__(1024, 1) void gemm_nt_shortk_kernel(MatmulArgs a, ShortKMap map) {
-  constexpr int BM = 128, BN = 128, NWL = 4, KK = CPR / 2;
-  constexpr int TM = 2, TN = 2, RING = 3;
+__global__ __launch_bounds__(SHORTK_THREADS, 1) void gemm_nt_shortk_kernel(MatmulArgs a,
+                                                                           ShortKMap map) {
+  constexpr int BM = 128, BN = 128, NWL = SHORTK_LOADERS, NWW = SHORTK_WRITERS;
+  constexpr int WROWS = 64 / NWW, WIT = WROWS / 4;  // rows and read rounds of a writer per half tile
+  constexpr int RING = 3;
   constexpr int IT = BM * CPR / (NWL * 64);    // DMA instructions per loader lane and panel
   constexpr int ROWS_PER_I = NWL * 64 / CPR;   // rows between a lane's successive instructions
   constexpr int PANEL = BM * CPR * 16;         // bytes of one 128-row panel
+  static_assert(3 * IT < 64, "three panels in flight must fit the memory counter");
   __shared__ __attribute__((aligned(1024))) unsigned char sA[PANEL];
   __shared__ __attribute__((aligned(1024))) unsigned char sB[RING * PANEL];
   // staging tile: row r = 256 bytes, 16-byte chunk c at position c ^ (r & 15)
@@ -1000,7 +1050,7 @@ __global__ __launch_bounds__(1024, 1) void gemm_nt_shortk_kernel(MatmulArgs a, S
   // Cursor over this workgroup's units and the tiles in them, in processing order.
   struct Cursor {
     int t, unit, batch, m0, n, n_end, n_vis_end;  // tiles [n, n_vis_end) computed, [.., n_end) filled
-    bool valid;
+    bool valid, first;                            // first: no earlier computed tile in this unit
   };
   auto load_unit = [&](Cursor& c) {
     c.unit = c.t * G + ((c.t & 1) ? G - 1 - gl : gl);
@@ -1020,110 +1070,136 @@ __global__ __launch_bounds__(1024, 1) void gemm_nt_shortk_kernel(MatmulArgs a, S
     c.t = 0;
     load_unit(c);
     while (c.valid && c.n >= c.n_vis_end) { c.t++; load_unit(c); }
+    c.first = true;
   };
   auto next_item = [&](Cursor& c) {
     c.n++;
-    while (c.valid && c.n >= c.n_vis_end) { c.t++; load_unit(c); }
+    c.first = false;
+    while (c.valid && c.n >= c.n_vis_end) { c.t++; load_unit(c); c.first = true; }
   };
 
-  if (wave >= 12) {
+  if (wave >= 8 + NWW) {
     // ---------------------------------------------------------------- loader wavefronts
-    const int lw = wave - 12;
-    int drow, dkc;  // the lane's place in a DMA instruction does not depend on the instruction
+    const int lw = wave - 8 - NWW;
+    // The lane's place in DMA instruction 0.  Instruction i fills the 256-byte lines 4 * NWL * i
+    // further down: the row moves with it, and the chunk by what those lines add to the swizzle.
+    int drow, dkc;
     lds_chunk_inv<CPR>(lw * 64 + lane, drow, dkc);
     auto panel = [&](const half_t* base, int64_t row_stride, int r0, int rmax, unsigned char* dst) {
 #pragma unroll
       for (int i = 0; i < IT; i++) {
         const int row = drow + i * ROWS_PER_I;
+        const int kc = dkc ^ ((i * NWL * 4) & (CPR - 1));
         __builtin_amdgcn_global_load_lds(
-            ADR_GLB_PTR(base + (int64_t)min(r0 + row, rmax) * row_stride + dkc * 8),
+            ADR_GLB_PTR(base + (int64_t)min(r0 + row, rmax) * row_stride + kc * 8),
             ADR_LDS_PTR(dst + (i * NWL + lw) * 1024), 16, 0, 0);
       }
     };
-    auto issueA = [&](const Cursor& c) {
+    Cursor cur;  // tile of the current phase
+    first_item(cur);
+    if (!cur.valid) return;
+    // Panels are issued as groups of IT instructions; a group has landed once at most the
+    // groups issued after it are outstanding.  `age` counts, one byte each, the groups issued
+    // after the right panel in ring buffer 0, 1, 2 and after the youngest left panel (a buffer
+    // is refilled every third right panel, so the counts stay small).  Kept in one register on
+    // purpose: three variables picked by the buffer number end up in scratch memory, and a load
+    // from there waits for every DMA in flight.
+    uint32_t age = 0;
+    int right_issued = 0;
+    Cursor is = cur;  // next right panel to issue
+    auto issued_into = [&](int byte) { age = (age + 0x01010101u) & ~(0xFFu << (8 * byte)); };
+    auto younger_than = [&](int byte) { return (int)((age >> (8 * byte)) & 0xFFu); };
+    auto issue_left = [&](const Cursor& c) {
       panel(a.lhs + (int64_t)c.batch * a.stride_lz, a.stride_ly, c.m0, a.m - 1, sA);
+      issued_into(3);
     };
-    auto issueB = [&](const Cursor& c, int slot) {
-      panel(a.rhs + (int64_t)c.batch * a.stride_rz, a.stride_rx, c.n * BN, a.n - 1,
+    auto issue_right = [&]() {
+      if (!is.valid) return;
+      const int slot = right_issued % RING;
+      panel(a.rhs + (int64_t)is.batch * a.stride_rz, a.stride_rx, is.n * BN, a.n - 1,
             sB + slot * PANEL);
+      issued_into(slot);
+      right_issued++;
+      next_item(is);
     };
-    Cursor w;  // tile being waited for
-    first_item(w);
-    if (w.valid) {
-      Cursor is = w;  // next tile to issue
-      int issued = 0;
-      bool a_young = false;  // a left panel was issued after the youngest right panel
-      issueA(w);
-      for (int k = 0; k < RING - 1 && is.valid; k++) {
-        issueB(is, issued % RING);
-        issued++;
-        next_item(is);
-      }
-      for (int j = 0; w.valid; j++) {
-        // the panel of tile j has landed; at most the one of tile j+1 is still in flight
-        if (issued - j - 1 >= 1 && !a_young)
-          __builtin_amdgcn_s_waitcnt(0x0070 | (IT & 0xF) | ((IT >> 4) << 14));
-        else
-          __builtin_amdgcn_s_waitcnt(0x0070);
-        a_young = false;
-        __builtin_amdgcn_s_barrier();  // X(j)
-        if (is.valid) {
-          issueB(is, issued % RING);  // into the buffer of tile j-1, read before Y(j-1)
-          issued++;
-          next_item(is);
+    auto wait_landed = [&](int younger) {
+      if (younger <= 0) wait_vmcnt_at_most<0>();
+      else if (younger == 1) wait_vmcnt_at_most<IT>();
+      else if (younger == 2) wait_vmcnt_at_most<2 * IT>();
+      else wait_vmcnt_at_most<3 * IT>();
+    };
+    issue_left(cur);
+    for (int k = 0; k < RING; k++) issue_right();
+    wait_landed(min(younger_than(3), younger_than(0)));
+    __builtin_amdgcn_s_barrier();  // barrier 0
+    for (int p = 0;; p++) {
+      const int j = p >> 1;
+      if (p & 1) {
+        // both groups copied the left panel of this unit in phase 2j: the next unit's may come
+        if (cur.first) {
+          Cursor nu = cur;
+          do { next_item(nu); } while (nu.valid && !nu.first);
+          if (nu.valid) issue_left(nu);
         }
-        __builtin_amdgcn_s_barrier();  // Y(j): tile j has been multiplied, the left panel is free
-        Cursor nx = w;
-        next_item(nx);
-        if (nx.valid && nx.unit != w.unit) {
-          issueA(nx);
-          a_young = true;
+        next_item(cur);  // tile j+1 starts after the next barrier
+        if (cur.valid) {
+          const int y = younger_than((j + 1) % RING);
+          wait_landed(cur.first ? min(y, younger_than(3)) : y);
         }
-        w = nx;
+        __builtin_amdgcn_s_barrier();  // barrier 2j+2
+      } else {
+        if (j >= 1) issue_right();  // tile j+2, into the buffer of tile j-1
+        __builtin_amdgcn_s_barrier();  // barrier 2j+1
+        if (!cur.valid) break;         // that was barrier 2T+1
       }
     }
-    __builtin_amdgcn_s_barrier();  // Z: last staging tile complete
     return;
   }
 
-  if (wave >= 4) {
+  if (wave >= 8) {
     // ---------------------------------------------------------------- writer wavefronts
-    const int sw = wave - 4;                       // rows sw*16 .. +15 of a tile
+    const int sw = wave - 8;                       // rows sw*WROWS .. of a half tile
     const int rrow = lane >> 4, rc = lane & 15;    // read round it: row it*4 + rrow, chunk rc
     const half_t hscale = (half_t)a.scale;
     Epilogue ep{a.bias, a.beta, hscale, a.store, true};
     const bool vec = out_vectorizable(a, a.output) && !(a.stride_oz & 7);
     const bool plain = vec && (a.store == ADR_STORE_IDENTITY || a.store == ADR_STORE_SCALE);
     const half_t mul = a.store == ADR_STORE_SCALE ? hscale : (half_t)1.0f;
-    auto write_tile = [&](int batch, int m0, int n0) {
-      half8_t v[4];
-#pragma unroll
-      for (int it = 0; it < 4; it++) {
-        const int row = sw * 16 + it * 4 + rrow;
-        v[it] = *(const half8_t*)(sC + row * 256 + ((rc ^ (row & 15)) << 4));
-      }
+    auto write_half = [&](int batch, int m0, int n0, int half) {
+      const int r0 = half * 64 + sw * WROWS;  // first of this wavefront's rows in the tile
+      auto staged = [&](int it) {
+        const int row = r0 + it * 4 + rrow;
+        return *(const half8_t*)(sC + row * 256 + ((rc ^ (row & 15)) << 4));
+      };
       half_t* const out = a.output + (int64_t)batch * a.stride_oz;
-      const int y0 = m0 + sw * 16 + rrow, x = n0 + rc * 8;
-      const bool inside = m0 + sw * 16 + 16 <= a.m && n0 + BN <= a.n;
-      const bool unmasked = a.mask != ADR_MASK_CAUSAL || n0 + BN - 1 <= m0 + sw * 16;
+      const int y0 = m0 + r0 + rrow, x = n0 + rc * 8;
+      const bool inside = m0 + r0 + WROWS <= a.m && n0 + BN <= a.n;
+      const bool unmasked = a.mask != ADR_MASK_CAUSAL || n0 + BN - 1 <= m0 + r0;
       if (plain && inside && unmasked) {
+        half8_t v[WIT];
+#pragma unroll
+        for (int it = 0; it < WIT; it++) v[it] = staged(it);
         // x * 1 is exact: one multiply serves Identity and Scale (fp16 product, matmul.cu)
         half_t* const p = out + (int64_t)y0 * a.stride_oy + x;
 #pragma unroll
-        for (int it = 0; it < 4; it++)
+        for (int it = 0; it < WIT; it++)
           __builtin_nontemporal_store(v[it] * mul, (half8_t*)(p + (int64_t)(it * 4) * a.stride_oy));
       } else if (vec) {
+        // (the rolled loops read the staging tile round by round: an array of rounds indexed by
+        // the loop counter would live in scratch memory)
 #pragma unroll 1
-        for (int it = 0; it < 4; it++) {
+        for (int it = 0; it < WIT; it++) {
           const int y = y0 + it * 4;
-          if (y < a.m && x < a.n) store_chunk(a, ep, out, y, x, v[it]);
+          const half8_t v = staged(it);
+          if (y < a.m && x < a.n) store_chunk(a, ep, out, y, x, v);
         }
       } else {
         const bool need_prev = Epilogue::needs_prev(a.store);
         const bool need_bias = Epilogue::needs_bias(a.store);
 #pragma unroll 1
-        for (int it = 0; it < 4; it++) {
+        for (int it = 0; it < WIT; it++) {
           const int y = y0 + it * 4;
+          const half8_t v = staged(it);
           if (y >= a.m) continue;
 #pragma unroll
           for (int e = 0; e < 8; e++) {
@@ -1134,7 +1210,7 @@ __global__ __launch_bounds__(1024, 1) void gemm_nt_shortk_kernel(MatmulArgs a, S
             } else {
               const half_t prev = need_prev ? *p : (half_t)0;
               const half_t bias = need_bias ? a.bias[x + e] : (half_t)0;
-              *p = ep.apply_s16(v[it][e], prev, bias);
+              *p = ep.apply_s16(v[e], prev, bias);
             }
           }
         }
@@ -1143,96 +1219,128 @@ __global__ __launch_bounds__(1024, 1) void gemm_nt_shortk_kernel(MatmulArgs a, S
     Cursor c;
     c.t = 0;
     load_unit(c);
-    bool have_prev = false;
-    int pb = 0, pm = 0, pn = 0;
+    bool started = false;
     while (c.valid) {
       const int first = c.n;
       for (; c.n < c.n_vis_end; c.n++) {
-        __builtin_amdgcn_s_barrier();  // X(j): staging tile j-1 complete
-        if (have_prev) write_tile(pb, pm, pn);
-        __builtin_amdgcn_s_barrier();  // Y(j): staging tile j-1 read
-        have_prev = true;
-        pb = c.batch; pm = c.m0; pn = c.n * BN;
+        if (!started) {
+          __builtin_amdgcn_s_barrier();  // barrier 0
+          __builtin_amdgcn_s_barrier();  // barrier 1
+          started = true;
+        }
+        __builtin_amdgcn_s_barrier();  // barrier 2j+2: the upper half of tile j is staged
+        write_half(c.batch, c.m0, c.n * BN, 0);
+        __builtin_amdgcn_s_barrier();  // barrier 2j+3: the lower half
+        write_half(c.batch, c.m0, c.n * BN, 1);
       }
-      // fully masked tiles of this unit
-      for (int n = max(first, c.n_vis_end); n < c.n_end; n++)
-        fill_masked_tile<BM, BN, 512>(a, a.output + (int64_t)c.batch * a.stride_oz, c.m0, n * BN,
-                                      tid - 256);
+      // fully masked tiles of this unit, unless fill_causal_rows_kernel wrote them already
+      if (!map.prefilled)
+        for (int n = max(first, c.n_vis_end); n < c.n_end; n++)
+          fill_masked_tile<BM, BN, NWW * 64>(a, a.output + (int64_t)c.batch * a.stride_oz, c.m0, n * BN,
+                                        tid - 512);
       c.t++;
       load_unit(c);
     }
-    __builtin_amdgcn_s_barrier();  // Z
-    if (have_prev) write_tile(pb, pm, pn);
     return;
   }
 
   // ------------------------------------------------------------------ multiplying wavefronts
-  const int wm = wave >> 1, wn = wave & 1;
-  const int frow = lane & 31, fkg = lane >> 5;
-  int offA[TM], offB[TN];  // k-step 0; k-step kk is at (off ^ (kk << 5))
+  // 16x16x32 MFMAs: the 64 x 32 block of a wavefront is 4 x 2 independent accumulators, so that
+  // no MFMA waits for the one before it
+  constexpr int KS = CPR / 4;                // k-steps of 32
+  const int grp = wave >> 2, wn = wave & 3;  // rows grp*64 .. +63, columns wn*32 .. +31 of a tile
+  const int frow = lane & 15, fkg = lane >> 4;
+  // k-step 0 of the first block; k-step kk is at (off ^ (kk << 6)), and sixteen rows further down
+  // the swizzle repeats: block i is R16 bytes times i further on
+  constexpr int R16 = 16 * CPR * 16;
+  const int offQ = lds_chunk_off<CPR>(grp * 64 + frow, fkg);
+  const int offB = lds_chunk_off<CPR>(wn * 32 + frow, fkg);
+  half8_t qa[KS][4];   // this wavefront's rows of the left panel
+  float4_t acc[4][2];
+  auto copy_left = [&]() {
 #pragma unroll
-  for (int i = 0; i < TM; i++) offA[i] = lds_chunk_off<CPR>(wm * 64 + i * 32 + frow, fkg);
+    for (int kk = 0; kk < KS; kk++)
 #pragma unroll
-  for (int j = 0; j < TN; j++) offB[j] = lds_chunk_off<CPR>(wn * 64 + j * 32 + frow, fkg);
+      for (int i = 0; i < 4; i++) qa[kk][i] = *(const half8_t*)(sA + (offQ ^ (kk << 6)) + i * R16);
+  };
+  auto multiply = [&](const unsigned char* cB) {
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+      for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+        for (int r = 0; r < 4; r++) acc[i][jj][r] = 0.0f;
+    half8_t fb[2][2];
+#pragma unroll
+    for (int jj = 0; jj < 2; jj++) fb[0][jj] = *(const half8_t*)(cB + offB + jj * R16);
+#pragma unroll
+    for (int kk = 0; kk < KS; kk++) {
+      if (kk + 1 < KS) {
+#pragma unroll
+        for (int jj = 0; jj < 2; jj++)
+          fb[(kk + 1) & 1][jj] = *(const half8_t*)(cB + (offB ^ ((kk + 1) << 6)) + jj * R16);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int jj = 0; jj < 2; jj++)
+          acc[i][jj] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[kk & 1][jj], qa[kk][i], acc[i][jj],
+                                                              0, 0, 0);
+    }
+    // a barrier orders memory operations only: without this the compiler sinks MFMAs below the
+    // barrier that ends the phase, into the time that belongs to the other group's
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // narrow and write the wavefront's 64 x 32 block: lane l of block (i, jj) holds row l % 16,
+  // columns 4 * (l / 16) .. +3 of the block
+  auto narrow = [&]() {
+    const int lrow = lane & 15, cg = lane >> 4;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const int row = grp * 64 + i * 16 + lrow;
+#pragma unroll
+      for (int jj = 0; jj < 2; jj++) {
+        half4_t h;
+#pragma unroll
+        for (int e = 0; e < 4; e++) h[e] = (half_t)acc[i][jj][e];
+        const int cc = wn * 4 + jj * 2 + (cg >> 1);
+        *(half4_t*)(sC + row * 256 + ((cc ^ (row & 15)) << 4) + (cg & 1) * 8) = h;
+      }
+    }
+  };
 
   Cursor c;
   first_item(c);
-  for (int j = 0; c.valid; j++) {
-    const unsigned char* cB = sB + (j % RING) * PANEL;
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // the staging tile of tile j-1 is written (lgkmcnt 0)
-    __builtin_amdgcn_s_barrier();        // X(j): panels of tile j ready
-    float16_t acc[TM][TN];
-#pragma unroll
-    for (int i = 0; i < TM; i++)
-#pragma unroll
-      for (int jj = 0; jj < TN; jj++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) acc[i][jj][r] = 0.0f;
-    half8_t fa[2][TM], fb[2][TN];
-#pragma unroll
-    for (int i = 0; i < TM; i++) fa[0][i] = *(const half8_t*)(sA + offA[i]);
-#pragma unroll
-    for (int jj = 0; jj < TN; jj++) fb[0][jj] = *(const half8_t*)(cB + offB[jj]);
-#pragma unroll
-    for (int kk = 0; kk < KK; kk++) {
-      if (kk + 1 < KK) {
-#pragma unroll
-        for (int i = 0; i < TM; i++)
-          fa[(kk + 1) & 1][i] = *(const half8_t*)(sA + (offA[i] ^ ((kk + 1) << 5)));
-#pragma unroll
-        for (int jj = 0; jj < TN; jj++)
-          fb[(kk + 1) & 1][jj] = *(const half8_t*)(cB + (offB[jj] ^ ((kk + 1) << 5)));
-      }
-#pragma unroll
-      for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int jj = 0; jj < TN; jj++)
-          acc[i][jj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[kk & 1][jj], fa[kk & 1][i],
-                                                              acc[i][jj], 0, 0, 0);
+  if (!c.valid) return;
+  if (grp == 0) {
+    for (int j = 0; c.valid; j++) {
+      __builtin_amdgcn_s_barrier();  // barrier 2j: the panels of tile j have landed
+      if (c.first) copy_left();
+      multiply(sB + (j % RING) * PANEL);
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // the panel has been read (lgkmcnt 0)
+      __builtin_amdgcn_s_barrier();  // barrier 2j+1: this half of the staging tile is free
+      narrow();
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // staged
+      next_item(c);
     }
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // the panels have been read
-    __builtin_amdgcn_s_barrier();        // Y(j): the staging tile has been read
-    // narrow and write the wavefront's 64 x 64 block: lane (row l % 32, half l / 32) of block
-    // (i, jj) holds columns 8q + 4*(l/32) .. +3 in elements 4q .. 4q+3
-    const int lrow = lane & 31, g = lane >> 5;
-#pragma unroll
-    for (int i = 0; i < TM; i++) {
-      const int row = wm * 64 + i * 32 + lrow;
-#pragma unroll
-      for (int jj = 0; jj < TN; jj++)
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-          half4_t h;
-#pragma unroll
-          for (int e = 0; e < 4; e++) h[e] = (half_t)acc[i][jj][4 * q + e];
-          const int cc = wn * 8 + jj * 4 + q;
-          *(half4_t*)(sC + row * 256 + ((cc ^ (row & 15)) << 4) + g * 8) = h;
-        }
+    __builtin_amdgcn_s_barrier();  // barrier 2T
+    __builtin_amdgcn_s_barrier();  // barrier 2T+1
+  } else {
+    __builtin_amdgcn_s_barrier();  // barrier 0
+    copy_left();
+    for (int j = 0; c.valid; j++) {
+      __builtin_amdgcn_s_waitcnt(0xC07F);
+      __builtin_amdgcn_s_barrier();  // barrier 2j+1
+      multiply(sB + (j % RING) * PANEL);
+      __builtin_amdgcn_s_waitcnt(0xC07F);
+      __builtin_amdgcn_s_barrier();  // barrier 2j+2: the ring buffer of tile j is free
+      next_item(c);
+      narrow();
+      if (c.valid && c.first) copy_left();  // tile j+1 opens a unit: its left panel has landed
     }
-    next_item(c);
+    __builtin_amdgcn_s_waitcnt(0xC07F);
+    __builtin_amdgcn_s_barrier();  // barrier 2T+1
   }
-  __builtin_amdgcn_s_waitcnt(0xC07F);
-  __builtin_amdgcn_s_barrier();  // Z: last staging tile complete
 }
 
 // =============================================================================================
@@ -1700,7 +1808,16 @@ hipError_t launch_shortk(hipStream_t stream, const MatmulArgs& a) {
   map.segs_per_row = (map.tiles_n + map.seg - 1) / map.seg;
   map.units = map.rows * map.segs_per_row;
   const unsigned grid = map.units < NUM_CU ? (unsigned)map.units : NUM_CU;
-  hipLaunchKernelGGL((gemm_nt_shortk_kernel<CPR>), dim3(grid), dim3(1024), 0, stream, a, map);
+  map.prefilled = 0;
+  const int64_t all_rows = (int64_t)a.m * a.batches;
+  if (a.mask == ADR_MASK_CAUSAL && map.tiles_n > 1 && all_rows <= 0x7fffffffLL) {
+    hipLaunchKernelGGL(fill_causal_rows_kernel, dim3((unsigned)((all_rows + 3) / 4)), dim3(256), 0,
+                       stream, a);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    map.prefilled = 1;
+  }
+  hipLaunchKernelGGL((gemm_nt_shortk_kernel<CPR>), dim3(grid), dim3(SHORTK_THREADS), 0, stream, a, map);
   return hipGetLastError();
 }
 

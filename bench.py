@@ -321,10 +321,10 @@ def main():
         q_, k_, v_ = randn_h(S, HD), randn_h(S, HD), randn_h(S, HD)
         qk = torch.zeros(H, S, S, dtype=torch.float16, device=dev)
 
-        def f_qk():
+        def f_qk(mask=0):
             rc = lib.adr_matmul_f16(stream(), qk.data_ptr(), q_.data_ptr(), k_.data_ptr(), H, S, D,
                                     S, 1, S, S * S, 1, HD, D, HD, 1, D, None, 0.0,
-                                    1.0 / D ** 0.5, 4, 0, 0)
+                                    1.0 / D ** 0.5, 4, 0, mask)
             if rc != 0:
                 raise RuntimeError(_ffi.strerror(rc))
         t = timed(f_qk, 50, 5)
@@ -332,6 +332,12 @@ def main():
         attn = {"qk_t": {"us": round(t * 1e6, 1), "tflops": round(2.0 * H * S * S * D / t / 1e12, 1),
                          "gbs": round(byts / t / 1e9, 1),
                          "frac_hbm_peak": round(byts / t / 1e9 / PEAK_HBM_GBS, 4)}}
+        # the same product under the causal mask (llama.rs:534-545): the same bytes are written,
+        # half of them -inf by a fill launch of their own, and half the arithmetic is done
+        t = timed(lambda: f_qk(1), 50, 5)
+        attn["qk_t_causal"] = {"us": round(t * 1e6, 1), "gbs": round(byts / t / 1e9, 1),
+                               "frac_hbm_peak": round(byts / t / 1e9 / PEAK_HBM_GBS, 4),
+                               "launches": "fill_causal_rows_kernel + gemm_nt_shortk_kernel"}
         # softmax_rows in place on the scores (read + write of the [32, 2048, 2048] tensor)
         def f_sm():
             rc = lib.adr_softmax_rows(stream(), qk.data_ptr(), qk.data_ptr(), H, S, S, 1.0)

@@ -280,6 +280,29 @@ def test_persistent_short_k_kernel_head_views(shape, mask):
     assert np.array_equal(to_np(o_t).view(np.uint16), want.view(np.uint16))
 
 
+@pytest.mark.parametrize("pad", [1, 4], ids=["odd_pitch", "pitch_8_bytes"])
+def test_persistent_short_k_kernel_causal_rows_not_16_byte_aligned(pad):
+    """The causal score product into rows that no 16-byte store may touch: the run of -inf right
+    of the diagonal tile and the tiles themselves go element by element, to the same bits."""
+    B, M, K, N = 9, 1000, 128, 1003
+    g = rng(930 + pad)
+    HD = B * K
+    NP = N + pad
+    so, sl, sr = (1, NP, M * NP), (1, HD, K), (HD, 1, K)
+    kw = dict(store=oracle.STORE_SCALE, scale=0.125, mask=oracle.MASK_CAUSAL)
+    assert plan(B, M, K, N, so, sl, sr, store=oracle.STORE_SCALE,
+                mask=oracle.MASK_CAUSAL).startswith("gemm_nt_mfma_persistent")
+    l, r = dyadic(g, M * HD), dyadic(g, N * HD)
+    prev = randn_f16(g, B * M * NP)
+    want = oracle_matmul(prev, l, r, B, M, K, N, so, sl, sr, mode=oracle.EXACT, **kw)
+    o_t = to_dev(prev)
+    assert raw_matmul("adr_matmul_f16", o_t, to_dev(l), to_dev(r), B, M, K, N, so, sl, sr, **kw) == 0
+    got = to_np(o_t)
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    # the padding between rows keeps what it held
+    assert np.array_equal(got.reshape(B, M, NP)[:, :, N:], prev.reshape(B, M, NP)[:, :, N:])
+
+
 @pytest.mark.parametrize("store", [oracle.STORE_ADD] + STORES_F32)
 def test_persistent_short_k_kernel_epilogues(store):
     g = rng(950 + store)
@@ -543,9 +566,9 @@ TILE_SHAPES = [(2000, 8184, "256x128"), (630, 12280, "128x256"), (380, 12280, "1
 @pytest.mark.parametrize("K", [2048, 2112, 2176, 2240, 2304, 2368])
 @pytest.mark.parametrize("M,N,tile", TILE_SHAPES)
 def test_large_tiles_every_k_tail_exact(K, M, N, tile):
-    """The 256 x 128 and 128 x 256 kernels (16x16x32 MFMAs) and the 128 x 192 kernel (32x32x16),
-    three LDS stages each: every remainder of the three-slice loop on inputs whose fp32 sums are
-    exact, ragged last tile row and column."""
+    """The 256 x 128 and 128 x 256 kernels (16x16x32 MFMAs) and the 128 x 192 kernel (32x32x16):
+    six consecutive K tails (every remainder of the three-slice loop of the three-stage tiles)
+    on inputs whose fp32 sums are exact, ragged last tile row and column."""
     so, sl, sr = nt_strides(M, K, N)
     assert plan(1, M, K, N, so, sl, sr) == f"gemm_nt_mfma_dma_{tile}x64"
     gen = torch.Generator(device="cuda").manual_seed(K)
