@@ -170,38 +170,39 @@ __device__ __forceinline__ void store_chunk(const MatmulArgs& a, const Epilogue&
 // Epilogue of one wavefront.  acc[i][j] is the TRANSPOSED 32x32 accumulator of row block i,
 // column block j: lane l holds output row l % 32 and, in element r, column
 // 8*(r/4) + 4*(l/32) + r%4.  (y0, x0) is the origin of the wavefront's sub-tile; `slot` is an
-// LDS region private to this wavefront of at least 32 * (TN*64 + 16) bytes.
+// LDS region private to this wavefront of at least 32 * (TN2*32 + 16) bytes.  TN2: the sub-tile's
+// width in blocks of 16 columns (even for the 32x32x16 layout).
 // The straight-line epilogue applies: the sub-tile begins inside the matrix and every 16-byte chunk
 // of its rows lies wholly inside or wholly outside (all of them inside, or n a multiple of 8; rows
 // and chunks past the matrix are read from the last row / chunk and not stored), it is on or below
 // the diagonal of a causal product, rows are 16-byte aligned.
-template <int TM, int TN>
+template <int TM, int TN2>
 __device__ __forceinline__ bool epilogue_is_straight(const MatmulArgs& a, const half_t* out, int y0,
                                                      int x0) {
-  const bool inside = y0 < a.m && x0 < a.n && (x0 + TN * 32 <= a.n || (a.n & 7) == 0);
-  const bool unmasked = a.mask != ADR_MASK_CAUSAL || x0 + TN * 32 - 1 <= y0;
+  const bool inside = y0 < a.m && x0 < a.n && (x0 + TN2 * 16 <= a.n || (a.n & 7) == 0);
+  const bool unmasked = a.mask != ADR_MASK_CAUSAL || x0 + TN2 * 16 - 1 <= y0;
   return inside && unmasked && out_vectorizable(a, out);
 }
 
 // Accumulators of a wavefront's sub-tile come in two register layouts.  32x32x16 MFMA
-// (float16_t acc[TM][TN]): see above.  16x16x32 MFMA (float4_t acc[2*TM][2*TN], transposed the
+// (float16_t acc[TM][TN2/2]): see above.  16x16x32 MFMA (float4_t acc[2*TM][TN2], transposed the
 // same way): acc[i][j] is the 16 x 16 block of rows 16*i.., columns 16*j..; lane l holds output
 // row l % 16 and, in element e, column 4*(l/16) + e.  The epilogues see both through these two
 // helpers, which put 32-row block i of the sub-tile into the wavefront's LDS slot.
 template <class T> struct is_mi16 { static constexpr bool value = false; };
 template <int A, int B> struct is_mi16<float4_t[A][B]> { static constexpr bool value = true; };
 
-// [32 rows][TN*32 halves], PITCH bytes per row; `mul` multiplies when `scaled`
-template <int TM, int TN, class Acc>
+// [32 rows][TN2*16 halves], PITCH bytes per row; `mul` multiplies when `scaled`
+template <int TM, int TN2, class Acc>
 __device__ __forceinline__ void stage_block_f16(Acc& acc, int i, unsigned char* slot, int lane,
                                                 bool scaled, half_t mul) {
-  constexpr int PITCH = TN * 64 + 16;
+  constexpr int PITCH = TN2 * 32 + 16;
   if constexpr (is_mi16<Acc>::value) {
     const int lrow = lane & 15, g = lane >> 4;
 #pragma unroll
     for (int h2 = 0; h2 < 2; h2++)
 #pragma unroll
-      for (int j = 0; j < 2 * TN; j++) {
+      for (int j = 0; j < TN2; j++) {
         half4_t h;
 #pragma unroll
         for (int e = 0; e < 4; e++) h[e] = (half_t)acc[2 * i + h2][j][e];
@@ -210,7 +211,7 @@ __device__ __forceinline__ void stage_block_f16(Acc& acc, int i, unsigned char* 
   } else {
     const int lrow = lane & 31, g = lane >> 5;
 #pragma unroll
-    for (int j = 0; j < TN; j++)
+    for (int j = 0; j < TN2 / 2; j++)
 #pragma unroll
       for (int q = 0; q < 4; q++) {
         half4_t h;
@@ -250,7 +251,7 @@ __device__ __forceinline__ void stage_block_f32(Acc& acc, int i, int j, int qh, 
 // operator gets its own compact instruction stream; with the operator switch inside the chunk
 // loop the code of all of them, exp and tanh included, sat between any two stores, and the
 // operators that are not Identity paid for it in instruction fetch).
-template <int TM, int TN, uint32_t OP, class Acc>
+template <int TM, int TN2, uint32_t OP, class Acc>
 __device__ __forceinline__ void straight_epilogue(const MatmulArgs& a, half_t* out, Acc& acc, int y0,
                                                   int x0, unsigned char* slot, half_t hscale,
                                                   int lane) {
@@ -260,27 +261,27 @@ __device__ __forceinline__ void straight_epilogue(const MatmulArgs& a, half_t* o
   constexpr bool nb = OP == ADR_STORE_BETA_BIAS || OP == ADR_STORE_BETA_GELU_BIAS ||
                       OP == ADR_STORE_QUICK_GELU_BIAS;
   const Epilogue ep{a.bias, a.beta, hscale, OP, true};
-  constexpr int PITCH = TN * 64 + 16;  // bytes per staged row (TN*32 halves + pad)
-  constexpr int CPW = TN * 4;          // 16-byte chunks per staged row
+  constexpr int PITCH = TN2 * 32 + 16;  // bytes per staged row (TN2*16 halves + pad)
+  constexpr int CPW = TN2 * 2;          // 16-byte chunks per staged row
   const half_t mul = OP == ADR_STORE_SCALE ? hscale : (half_t)1.0f;
   // store round `it` of a 32-row block: lane -> 16-byte chunk it*64 + lane of the staged block
   // (scol: the chunk's first column, clamped to the last chunk of the matrix for the loads;
   // colin: the chunk lies inside the matrix)
-  int rd[TN * 2], srow[TN * 2], scol[TN * 2];
-  bool colin[TN * 2];
+  int rd[TN2], srow[TN2], scol[TN2];
+  bool colin[TN2];
   const int cmax = a.n - 8 - x0;  // first column of the matrix's last chunk, relative to the sub-tile
 #pragma unroll
-  for (int it = 0; it < TN * 2; it++) {
+  for (int it = 0; it < TN2; it++) {
     const int idx = it * 64 + lane, row = idx / CPW, c = idx % CPW;
     rd[it] = row * PITCH + c * 16;
     srow[it] = row;
     colin[it] = c * 8 <= cmax;
     scol[it] = min(c * 8, cmax);
   }
-  half8_t bias[TN * 2];
+  half8_t bias[TN2];
   if (nb) {
 #pragma unroll
-    for (int it = 0; it < TN * 2; it++) bias[it] = *(const half8_t*)(a.bias + x0 + scol[it]);
+    for (int it = 0; it < TN2; it++) bias[it] = *(const half8_t*)(a.bias + x0 + scol[it]);
   }
   half_t* const p0 = out + (int64_t)y0 * a.stride_oy + x0;
   const int last = a.m - y0 - 1;  // last row of the matrix, relative to the sub-tile
@@ -291,20 +292,20 @@ __device__ __forceinline__ void straight_epilogue(const MatmulArgs& a, half_t* o
   };
   // all of the sub-tile's previous output in one burst: with one workgroup per compute unit
   // nothing else hides this latency
-  half8_t prev[TM][TN * 2];
+  half8_t prev[TM][TN2];
   if (np) {
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
-      for (int it = 0; it < TN * 2; it++) prev[i][it] = *(const half8_t*)at(i, it);
+      for (int it = 0; it < TN2; it++) prev[i][it] = *(const half8_t*)at(i, it);
   }
 #pragma unroll
   for (int i = 0; i < TM; i++) {
     // x * 1 is exact, so one multiply serves Identity and Scale (matmul.cu Scale: fp16
     // product); the other operators take the narrowed sum as it is
-    stage_block_f16<TM, TN>(acc, i, slot, lane, plain_op, mul);
+    stage_block_f16<TM, TN2>(acc, i, slot, lane, plain_op, mul);
 #pragma unroll
-    for (int it = 0; it < TN * 2; it++) {
+    for (int it = 0; it < TN2; it++) {
       half8_t v = *(const half8_t*)(slot + rd[it]);
       if (OP == ADR_STORE_ADD) {
         v = v + prev[i][it];
@@ -333,23 +334,25 @@ __device__ __forceinline__ void straight_epilogue(const MatmulArgs& a, half_t* o
 // LDS slot, QN groups of eight columns of a 32 x 32 block at a time; a lane then owns whole
 // 16-byte chunks of the output, whose previous values were all requested up front.  Same
 // conditions as epilogue_is_straight, minus the restriction to beta == 0.
-template <int TM, int TN>
+template <int TM, int TN2>
 __device__ __forceinline__ bool acc_beta_is_straight(const MatmulArgs& a, const half_t* out, int y0,
                                                      int x0) {
   return a.store == STORE_ACC_BETA && a.beta != 0.0f && a.mask == ADR_MASK_NONE && y0 < a.m &&
-         x0 < a.n && (x0 + TN * 32 <= a.n || (a.n & 7) == 0) && !(a.stride_oy & 7) &&
+         x0 < a.n && (x0 + TN2 * 16 <= a.n || (a.n & 7) == 0) && !(a.stride_oy & 7) &&
          !((uintptr_t)out & 15);
 }
 
-template <int TM, int TN, class Acc>
+template <int TM, int TN2, class Acc>
 __device__ __forceinline__ void straight_epilogue_acc_beta(const MatmulArgs& a, half_t* out, Acc& acc,
                                                            int y0, int x0, unsigned char* slot,
                                                            int lane) {
-  constexpr int QN = TN >= 2 ? 4 : 2;     // 32 rows x (QN * 32 + 16) bytes fit the slot
+  // QN groups of eight columns at a time: a whole 32 x 32 block, or 16 columns where the sub-tile
+  // is narrow or an odd number of 16-column blocks wide
+  constexpr int QN = (TN2 >= 4 && TN2 % 2 == 0) ? 4 : 2;  // 32 rows x (QN * 32 + 16) bytes fit the slot
   constexpr int FP = QN * 32 + 16;        // bytes per staged row
-  constexpr int QH = 4 / QN;              // column groups per 32 x 32 block
+  constexpr int G = TN2 * 2 / QN;         // column groups of the sub-tile
   constexpr int H = QN * 32 / 64;         // chunks per lane and group
-  static_assert(32 * FP <= 32 * (TN * 64 + 16), "fp32 staging must fit the wavefront's slot");
+  static_assert(32 * FP <= 32 * (TN2 * 32 + 16), "fp32 staging must fit the wavefront's slot");
   const int cmax = a.n - 8 - x0;          // first column of the matrix's last chunk, relative to the sub-tile
   const int last = a.m - y0 - 1;          // last row of the matrix, relative to the sub-tile
   half_t* const p0 = out + (int64_t)y0 * a.stride_oy + x0;
@@ -361,76 +364,72 @@ __device__ __forceinline__ void straight_epilogue_acc_beta(const MatmulArgs& a, 
     rcol[h] = (idx % QN) * 8;
   }
   // rows and chunks past the matrix are clamped for the loads and skipped for the stores
-  auto at = [&](int i, int j, int qh, int h) {
-    return p0 + (int64_t)min(i * 32 + rrow[h], last) * a.stride_oy + min(j * 32 + qh * QN * 8 + rcol[h], cmax);
+  auto at = [&](int i, int g, int h) {
+    return p0 + (int64_t)min(i * 32 + rrow[h], last) * a.stride_oy + min(g * QN * 8 + rcol[h], cmax);
   };
-  half8_t prev[TM][TN][QH][H];
+  half8_t prev[TM][G][H];
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
-    for (int j = 0; j < TN; j++)
+    for (int g = 0; g < G; g++)
 #pragma unroll
-      for (int qh = 0; qh < QH; qh++)
-#pragma unroll
-        for (int h = 0; h < H; h++) prev[i][j][qh][h] = *(const half8_t*)at(i, j, qh, h);
+      for (int h = 0; h < H; h++) prev[i][g][h] = *(const half8_t*)at(i, g, h);
   const float beta = a.beta;
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
-    for (int j = 0; j < TN; j++)
+    for (int g = 0; g < G; g++) {
+      stage_block_f32<QN>(acc, i, QN == 4 ? g : g >> 1, QN == 4 ? 0 : g & 1, slot, lane);
 #pragma unroll
-      for (int qh = 0; qh < QH; qh++) {
-        stage_block_f32<QN>(acc, i, j, qh, slot, lane);
+      for (int h = 0; h < H; h++) {
+        const float4_t lo = *(const float4_t*)(slot + rrow[h] * FP + rcol[h] * 4);
+        const float4_t hi = *(const float4_t*)(slot + rrow[h] * FP + rcol[h] * 4 + 16);
+        half8_t v;
 #pragma unroll
-        for (int h = 0; h < H; h++) {
-          const float4_t lo = *(const float4_t*)(slot + rrow[h] * FP + rcol[h] * 4);
-          const float4_t hi = *(const float4_t*)(slot + rrow[h] * FP + rcol[h] * 4 + 16);
-          half8_t v;
-#pragma unroll
-          for (int e = 0; e < 4; e++) {
-            v[e] = (half_t)(lo[e] + beta * (float)prev[i][j][qh][h][e]);
-            v[4 + e] = (half_t)(hi[e] + beta * (float)prev[i][j][qh][h][4 + e]);
-          }
-          if (i * 32 + rrow[h] <= last && j * 32 + qh * QN * 8 + rcol[h] <= cmax)
-            __builtin_nontemporal_store(v, (half8_t*)at(i, j, qh, h));
+        for (int e = 0; e < 4; e++) {
+          v[e] = (half_t)(lo[e] + beta * (float)prev[i][g][h][e]);
+          v[4 + e] = (half_t)(hi[e] + beta * (float)prev[i][g][h][4 + e]);
         }
+        if (i * 32 + rrow[h] <= last && g * QN * 8 + rcol[h] <= cmax)
+          __builtin_nontemporal_store(v, (half8_t*)at(i, g, h));
       }
+    }
 }
 
-template <int TM, int TN, class Acc>
+template <int TM, int TN2, class Acc>
 __device__ __forceinline__ void wave_epilogue(const MatmulArgs& a, half_t* out, Acc& acc, int y0,
                                               int x0, unsigned char* slot, half_t hscale, int lane) {
   Epilogue ep{a.bias, a.beta, hscale, a.store, true};
-  constexpr int PITCH = TN * 64 + 16;  // bytes per staged row (TN*32 halves + pad)
-  constexpr int CPW = TN * 4;          // 16-byte chunks per staged row
-  if (acc_beta_is_straight<TM, TN>(a, out, y0, x0))
-    return straight_epilogue_acc_beta<TM, TN>(a, out, acc, y0, x0, slot, lane);
+  constexpr int PITCH = TN2 * 32 + 16;  // bytes per staged row (TN2*16 halves + pad)
+  constexpr int CPW = TN2 * 2;          // 16-byte chunks per staged row
+  if (acc_beta_is_straight<TM, TN2>(a, out, y0, x0))
+    return straight_epilogue_acc_beta<TM, TN2>(a, out, acc, y0, x0, slot, lane);
   // Common case, straight-line: the sub-tile's columns lie inside the matrix, it is (for a
   // causal product) on or below the diagonal, rows are 16-byte aligned.
-  if (epilogue_is_straight<TM, TN>(a, out, y0, x0)) {
+  if (epilogue_is_straight<TM, TN2>(a, out, y0, x0)) {
     switch (a.store) {
       case ADR_STORE_SCALE:
-        return straight_epilogue<TM, TN, ADR_STORE_SCALE>(a, out, acc, y0, x0, slot, hscale, lane);
+        return straight_epilogue<TM, TN2, ADR_STORE_SCALE>(a, out, acc, y0, x0, slot, hscale, lane);
       case ADR_STORE_ADD:
-        return straight_epilogue<TM, TN, ADR_STORE_ADD>(a, out, acc, y0, x0, slot, hscale, lane);
+        return straight_epilogue<TM, TN2, ADR_STORE_ADD>(a, out, acc, y0, x0, slot, hscale, lane);
       case ADR_STORE_BETA_BIAS:
-        return straight_epilogue<TM, TN, ADR_STORE_BETA_BIAS>(a, out, acc, y0, x0, slot, hscale, lane);
+        return straight_epilogue<TM, TN2, ADR_STORE_BETA_BIAS>(a, out, acc, y0, x0, slot, hscale, lane);
       case ADR_STORE_QUICK_GELU_BIAS:
-        return straight_epilogue<TM, TN, ADR_STORE_QUICK_GELU_BIAS>(a, out, acc, y0, x0, slot, hscale, lane);
+        return straight_epilogue<TM, TN2, ADR_STORE_QUICK_GELU_BIAS>(a, out, acc, y0, x0, slot, hscale, lane);
       case ADR_STORE_BETA_GELU_BIAS:
-        return straight_epilogue<TM, TN, ADR_STORE_BETA_GELU_BIAS>(a, out, acc, y0, x0, slot, hscale, lane);
+        return straight_epilogue<TM, TN2, ADR_STORE_BETA_GELU_BIAS>(a, out, acc, y0, x0, slot, hscale, lane);
       case STORE_ACC_BETA:
-        return straight_epilogue<TM, TN, STORE_ACC_BETA>(a, out, acc, y0, x0, slot, hscale, lane);
+        return straight_epilogue<TM, TN2, STORE_ACC_BETA>(a, out, acc, y0, x0, slot, hscale, lane);
       default:
-        return straight_epilogue<TM, TN, ADR_STORE_IDENTITY>(a, out, acc, y0, x0, slot, hscale, lane);
+        return straight_epilogue<TM, TN2, ADR_STORE_IDENTITY>(a, out, acc, y0, x0, slot, hscale, lane);
     }
   }
   if (out_vectorizable(a, out)) {
 #pragma unroll
     for (int i = 0; i < TM; i++) {
-      stage_block_f16<TM, TN>(acc, i, slot, lane, false, (half_t)1.0f);
+      stage_block_f16<TM, TN2>(acc, i, slot, lane, false, (half_t)1.0f);
 #pragma unroll 1
-      for (int it = 0; it < TN * 2; it++) {
+      for (int it = 0; it < TN2; it++) {
         const int idx = it * 64 + lane;
         const int row = idx / CPW, c = idx % CPW;
         const half8_t v = *(const half8_t*)(slot + row * PITCH + c * 16);
@@ -447,32 +446,30 @@ __device__ __forceinline__ void wave_epilogue(const MatmulArgs& a, half_t* out, 
     const bool need_prev = Epilogue::needs_prev(a.store);
     const bool need_bias = Epilogue::needs_bias(a.store);
     const bool causal = a.mask == ADR_MASK_CAUSAL;
-    constexpr int QN = TN >= 2 ? 4 : 2;     // 32 rows x (QN * 32 + 16) bytes fit the slot
+    constexpr int QN = (TN2 >= 4 && TN2 % 2 == 0) ? 4 : 2;  // 32 rows x (QN * 32 + 16) bytes fit the slot
     constexpr int FP = QN * 32 + 16;        // bytes per staged row
     static_assert(32 * FP <= 32 * PITCH, "fp32 staging must fit the wavefront's slot");
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
-      for (int j = 0; j < TN; j++)
-#pragma unroll
-        for (int qh = 0; qh < 4 / QN; qh++) {
-          stage_block_f32<QN>(acc, i, j, qh, slot, lane);
+      for (int g = 0; g < TN2 * 2 / QN; g++) {
+        stage_block_f32<QN>(acc, i, QN == 4 ? g : g >> 1, QN == 4 ? 0 : g & 1, slot, lane);
 #pragma unroll 1
-          for (int e = lane; e < 32 * 8 * QN; e += 64) {
-            const int row = e / (8 * QN), c = e % (8 * QN);
-            const int y = y0 + i * 32 + row, x = x0 + j * 32 + qh * QN * 8 + c;
-            if (y >= a.m || x >= a.n) continue;
-            const float sum = *(const float*)(slot + row * FP + c * 4);
-            half_t* p = out + (int64_t)y * a.stride_oy + x;
-            if (causal && x > y) {
-              *p = neg_inf_half();
-            } else {
-              half_t prev = need_prev ? *p : (half_t)0;
-              half_t bias = need_bias ? a.bias[x] : (half_t)0;
-              *p = ep.apply(sum, prev, bias);
-            }
+        for (int e = lane; e < 32 * 8 * QN; e += 64) {
+          const int row = e / (8 * QN), c = e % (8 * QN);
+          const int y = y0 + i * 32 + row, x = x0 + g * QN * 8 + c;
+          if (y >= a.m || x >= a.n) continue;
+          const float sum = *(const float*)(slot + row * FP + c * 4);
+          half_t* p = out + (int64_t)y * a.stride_oy + x;
+          if (causal && x > y) {
+            *p = neg_inf_half();
+          } else {
+            half_t prev = need_prev ? *p : (half_t)0;
+            half_t bias = need_bias ? a.bias[x] : (half_t)0;
+            *p = ep.apply(sum, prev, bias);
           }
         }
+      }
   }
 }
 
@@ -894,7 +891,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   }
   unsigned char* const slot = (SLOTS_IN_B ? (wave < NW / 2 ? sB0 : sB1) : (wave < NW / 2 ? sA0 : sA1)) +
                               (wave % (NW / 2)) * SLOT;
-  wave_epilogue<TM, TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, slot, (half_t)a.scale, lane);
+  wave_epilogue<TM, 2 * TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, slot, (half_t)a.scale, lane);
 #ifdef ADR_PHASE_STAMPS
   if (a.workspace && !SPLIT) {
     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0): the tile is written
@@ -951,7 +948,7 @@ __global__ __launch_bounds__(WM* WN * 64) void splitk_reduce_kernel(MatmulArgs a
           for (int e = 0; e < 4; e++) acc[i][j][4 * c + e] += v[e];
         }
   }
-  wave_epilogue<TM, TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, slots + wave * SLOT,
+  wave_epilogue<TM, 2 * TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, slots + wave * SLOT,
                         (half_t)a.scale, lane);
 }
 
@@ -1543,7 +1540,7 @@ __global__ __launch_bounds__(WM* WN * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a
   __builtin_amdgcn_s_barrier();
 
   unsigned char* slot = (wave < NW / 2 ? sA0 : sA1) + (wave % (NW / 2)) * SLOT;
-  wave_epilogue<TM, TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, slot, (half_t)a.scale, lane);
+  wave_epilogue<TM, 2 * TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, slot, (half_t)a.scale, lane);
 }
 
 // =============================================================================================
@@ -1705,7 +1702,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_stage_kernel(Matmul
     __syncthreads();
   }
 
-  wave_epilogue<TM, TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, smem + wave * SLOT, hscale,
+  wave_epilogue<TM, 2 * TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, smem + wave * SLOT, hscale,
                         lane);
 }
 
