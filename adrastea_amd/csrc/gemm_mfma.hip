@@ -527,11 +527,13 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   constexpr int IA = BM * CPR / (NWD * 64), IB = BN * CPR / (NWD * 64);
   constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
   constexpr int FM = WTM / MI, FN = WTN / MI;  // MFMA blocks of the wavefront's sub-tile
-  constexpr int SLOT = 32 * (TN * 64 + 16);
+  constexpr int TN2 = WTN / 16;                // the sub-tile's width in 16-column blocks
+  constexpr int SLOT = 32 * (TN2 * 32 + 16);
   static_assert(!MI16 || (!NN && !SPLIT), "16x16x32: plain NT products");
   static_assert(BM * CPR % (NWD * 64) == 0 && BN * CPR % (NWD * 64) == 0,
                 "slices must split evenly over lanes");
-  static_assert(WTM % 32 == 0 && WTN % 32 == 0, "MFMA 32x32x16 tiling");
+  static_assert(WTM % 32 == 0 && WTN % (MI16 ? 16 : 32) == 0,
+                "whole MFMA blocks (with 16x16x32 the sub-tile may be an odd number of them wide)");
   // epilogue slots: half of the wavefronts in each of the first two stages of the larger operand
   constexpr bool SLOTS_IN_B = BN > BM;
   static_assert((NW / 2) * SLOT <= (SLOTS_IN_B ? BN : BM) * BK * 2,
@@ -891,7 +893,7 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_dma_kernel(MatmulAr
   }
   unsigned char* const slot = (SLOTS_IN_B ? (wave < NW / 2 ? sB0 : sB1) : (wave < NW / 2 ? sA0 : sA1)) +
                               (wave % (NW / 2)) * SLOT;
-  wave_epilogue<TM, 2 * TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, slot, (half_t)a.scale, lane);
+  wave_epilogue<TM, TN2>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, slot, (half_t)a.scale, lane);
 #ifdef ADR_PHASE_STAMPS
   if (a.workspace && !SPLIT) {
     __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0): the tile is written
@@ -1822,7 +1824,7 @@ enum GemmChoice {
   GEMM_NONE = 0,
   SHORTK_64, SHORTK_128,
   U8_256x192, U8_256x128,
-  DMA_256x192, DMA_256x128, DMA_128x256, DMA_128x192, DMA_128x128, DMA_128x64, DMA_64x64, DMA_64x64_K128, DMA_128x64_K128,
+  DMA_256x192, DMA_256x160, DMA_256x128, DMA_128x256, DMA_128x192, DMA_128x128, DMA_128x64, DMA_64x64, DMA_64x64_K128, DMA_128x64_K128,
   DMA_NN_256x128, DMA_NN_128x128,
   STAGE_256x128, STAGE_128x128, STAGE_64x64,
 };
@@ -1864,7 +1866,7 @@ GemmChoice pick(const MatmulArgs& a, const Candidate* c, int n, double* cost_out
 const Candidate DMA_TILES[] = {
     {DMA_256x192, 256, 192, 1, 1.24f}, {DMA_256x128, 256, 128, 1, 1.13f},
     {DMA_128x256, 128, 256, 1, 1.13f}, {DMA_128x192, 128, 192, 1, 0.85f}, {DMA_128x128, 128, 128, 2, 0.80f}, {DMA_128x64, 128, 64, 2, 0.60f},
-    {DMA_64x64, 64, 64, 4, 0.40f}};
+    {DMA_64x64, 64, 64, 4, 0.40f}, {DMA_256x160, 256, 160, 1, 1.19f}};
 constexpr int N_DMA_TILES = sizeof(DMA_TILES) / sizeof(DMA_TILES[0]);
 
 // The MFMA family needs 16-byte aligned, K-contiguous rows on both operands.
@@ -2015,6 +2017,7 @@ static bool choice_name(GemmChoice c, const char** name, bool u8 = false) {
     case U8_256x192: *name = "gemm_nt_u8_mfma_256x192x64"; return true;
     case U8_256x128: *name = "gemm_nt_u8_mfma_256x128x64"; return true;
     case DMA_256x192: *name = "gemm_nt_mfma_dma_256x192x64"; return true;
+    case DMA_256x160: *name = "gemm_nt_mfma_dma_256x160x64"; return true;
     case DMA_256x128: *name = "gemm_nt_mfma_dma_256x128x64"; return true;
     case DMA_128x256: *name = "gemm_nt_mfma_dma_128x256x64"; return true;
     case DMA_128x192: *name = "gemm_nt_mfma_dma_128x192x64"; return true;
@@ -2039,6 +2042,7 @@ static hipError_t launch_choice(hipStream_t stream, const MatmulArgs& a, GemmCho
     case U8_256x192: return launch_u8<256, 192, 4, 2, false>(stream, a);
     case U8_256x128: return launch_u8<256, 128, 4, 2, true>(stream, a);
     case DMA_256x192: return launch_dma<256, 192, 4, 2, 6, 1, false, 64, true>(stream, a);
+    case DMA_256x160: return launch_dma<256, 160, 4, 2, 6, 1, false, 64, true>(stream, a);
     case DMA_256x128: return launch_dma<256, 128, 4, 2, 7, 1, false, 64, true>(stream, a);
     case DMA_128x256: return launch_dma<128, 256, 2, 4, 3, 1, false, 64, true>(stream, a);
     case DMA_128x192: return launch_dma<128, 192, 2, 2, 3, 1>(stream, a);
@@ -2074,7 +2078,7 @@ static bool split_m_tail(const MatmulArgs& a, MatmulArgs& head, MatmulArgs& tail
   tail.output = a.output ? a.output + (int64_t)head.m * a.stride_oy : nullptr;
   const GemmChoice ca = choose(a), ch = choose(head), ct = choose(tail);
   auto dma_tile = [](GemmChoice c) {
-    return c == DMA_256x192 || c == DMA_256x128 || c == DMA_128x256 || c == DMA_128x192 || c == DMA_128x128 ||
+    return c == DMA_256x192 || c == DMA_256x160 || c == DMA_256x128 || c == DMA_128x256 || c == DMA_128x192 || c == DMA_128x128 ||
            c == DMA_128x64 || c == DMA_64x64;
   };
   if (!dma_tile(ca) || !dma_tile(ch) || !dma_tile(ct)) return false;

@@ -584,7 +584,7 @@ def main():
                         "frac_mfma_peak": round(2.0 * m * K * N / t / 1e12 / PEAK_F16_TFLOPS, 4)}
         return clip
 
-    TILE_NAMES = ["256x192", "256x128", "128x256", "128x192", "128x128", "128x64", "64x64"]
+    TILE_NAMES = ["256x192", "256x128", "128x256", "128x192", "128x128", "128x64", "64x64", "256x160"]
     FP16_GEMM_SHAPES = [("clip_text_qkv", 77, 768, 2304), ("clip_mlp_up", 2056, 1024, 4096),
                         ("clip_mlp_down", 2056, 4096, 1024), ("llama_qkv", 2048, 4096, 12288),
                         ("llama_o", 2048, 4096, 4096), ("llama_gate_up", 2048, 4096, 11008),

@@ -383,8 +383,8 @@ int adr_matmul_f16_ws_plan(char* name, int32_t cap, int32_t batches, int32_t m, 
  * For tests and benchmarks only (no counterpart in the reference): forces a kernel choice that
  * the dispatch otherwise makes from the arguments, process-wide, so that the chosen kernel can be
  * compared with the others on the same operands.  id 0: the tile of the fp16 tiled GEMM (value 0:
- * the dispatch decides; 1 + i: tile i of 256x192, 256x128, 128x256, 128x192, 128x128, 128x64, 64x64
- * where the product is one the tiled kernels cover).  Unknown ids return ADR_EINVAL_ENUM.
+ * the dispatch decides; 1 + i: tile i of 256x192, 256x128, 128x256, 128x192, 128x128, 128x64, 64x64,
+ * 256x160 where the product is one the tiled kernels cover).  Unknown ids return ADR_EINVAL_ENUM.
  */
 int adr_debug_knob(int32_t id, int32_t value);
 

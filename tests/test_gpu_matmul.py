@@ -368,7 +368,8 @@ def test_row_and_batch_strides_with_padding_on_the_fast_path():
 
 
 @pytest.mark.parametrize("B,M,K,N,tile", [(2, 600, 1088, 6136, "128x256"), (2, 380, 1088, 6136, "128x192"),
-                                          (2, 1000, 1088, 4088, "256x128"), (3, 1000, 1088, 3064, "256x192")])
+                                          (2, 1000, 1088, 4088, "256x128"), (4, 1000, 1088, 3064, "256x192"),
+                                          (3, 1000, 1088, 3064, "256x160")])
 def test_batched_padded_operands_on_the_large_tiles(B, M, K, N, tile):
     """Batches with row pitches wider than the rows and batch strides wider than the matrices on
     every large tile (16 x 16 and 32 x 32 accumulator blocks), exact inputs; whatever lies between
@@ -560,14 +561,15 @@ def test_large_tile_kernel_every_k_tail_exact(K):
 
 
 # (M, N, the tile the choice model gives the shape at K >= 2048)
-TILE_SHAPES = [(2000, 8184, "256x128"), (630, 12280, "128x256"), (380, 12280, "128x192")]
+TILE_SHAPES = [(2000, 8184, "256x128"), (630, 12280, "128x256"), (380, 12280, "128x192"),
+               (2000, 5112, "256x160")]
 
 
 @pytest.mark.parametrize("K", [2048, 2112, 2176, 2240, 2304, 2368])
 @pytest.mark.parametrize("M,N,tile", TILE_SHAPES)
 def test_large_tiles_every_k_tail_exact(K, M, N, tile):
-    """The 256 x 128 and 128 x 256 kernels (16x16x32 MFMAs) and the 128 x 192 kernel (32x32x16):
-    six consecutive K tails (every remainder of the three-slice loop of the three-stage tiles)
+    """The 256 x 128, 128 x 256 and 256 x 160 kernels (16x16x32 MFMAs; the last with sub-tiles five
+    16-column blocks wide) and the 128 x 192 kernel (32x32x16): six consecutive K tails (every remainder of the three-slice loop of the three-stage tiles)
     on inputs whose fp32 sums are exact, ragged last tile row and column."""
     so, sl, sr = nt_strides(M, K, N)
     assert plan(1, M, K, N, so, sl, sr) == f"gemm_nt_mfma_dma_{tile}x64"
@@ -599,7 +601,8 @@ def test_256x128_tile_every_remainder_of_its_twelve_slice_period(K):
 
 @pytest.mark.parametrize("store", STORES_EXACT + STORES_F32)
 @pytest.mark.parametrize("mask", [oracle.MASK_NONE, oracle.MASK_CAUSAL])
-@pytest.mark.parametrize("M,N,tile", [(4000, 4088, "256x128"), (630, 12280, "128x256"), (380, 12280, "128x192")])
+@pytest.mark.parametrize("M,N,tile", [(4000, 4088, "256x128"), (630, 12280, "128x256"), (380, 12280, "128x192"),
+                                      (2000, 5112, "256x160")])
 def test_large_tile_epilogues_against_the_slow_kernel(store, mask, M, N, tile):
     """Every store operator and the causal mask through the epilogues of the 256 x 128 and
     128 x 256 tiles (accumulators in 16 x 16 blocks, the latter's staging slots in the right

@@ -12,7 +12,7 @@ from adrastea_amd import _ffi
 
 pytestmark = pytest.mark.gpu
 
-TILES = ["256x192", "256x128", "128x256", "128x192", "128x128", "128x64", "64x64"]
+TILES = ["256x192", "256x128", "128x256", "128x192", "128x128", "128x64", "64x64", "256x160"]
 SHAPES = [("clip_mlp_up", 2056, 1024, 4096), ("clip_mlp_down", 2056, 4096, 1024),
           ("llama_qkv", 2048, 4096, 12288), ("llama_o", 2048, 4096, 4096),
           ("llama_gate_up", 2048, 4096, 11008), ("llama_down", 2048, 11008, 4096)]
