@@ -16,10 +16,13 @@
 //                       fragments are prefetched one k-step ahead and interleaved with the
 //                       MFMAs by scheduling-group barriers.
 //  gemm_nt_u8_kernel    the same with u8 weights dequantised on their way into LDS.
-//  gemm_nt_shortk_kernel  K = 64 / 128 (the attention score product): persistent workgroups.
+//  gemm_nt_shortk_kernel  K = 64 / 128 (the attention score product): persistent workgroups;
+//                       also with the Load Scale operator (both operands scaled in fp16 on the
+//                       way into the MFMAs) and for score rows that are not 16-byte aligned.
 //  gemm_nt_stage_kernel any K % 8 == 0, and the variants that must touch the data on the way
 //                       in: u8 weights dequantised while staging (adr_matmul_nt_fp16u8), and
-//                       the Load Scale operator.  Global -> registers -> LDS, two LDS stages.
+//                       the Load Scale operator on other K.  Global -> registers -> LDS, two
+//                       LDS stages.
 //
 // One workgroup owns a BM x BN output tile, WM x WN wavefronts each own a (BM/WM) x (BN/WN)
 // sub-tile as fp32 accumulator blocks: 16 x 16 blocks of v_mfma_f32_16x16x32_f16 in the tiles
@@ -134,14 +137,25 @@ __device__ __forceinline__ half8_t apply_chunk(const MatmulArgs& a, const Epilog
   return r;
 }
 
-// One 16-byte chunk (8 consecutive columns x..x+7 of output row y) through the store operator.
+// One chunk of 8 consecutive columns x..x+7 of output row y through the store operator, read and
+// written W halves at a time: 8 where rows are 16-byte aligned, 4 or 2 where they are aligned to
+// that many halves only (a score tensor whose row length is not a multiple of 8).
+template <int W = 8>
 __device__ __forceinline__ void store_chunk(const MatmulArgs& a, const Epilogue& ep, half_t* out,
                                             int y, int x, half8_t v) {
+  typedef half_t piece_t __attribute__((ext_vector_type(W)));
   half_t* p = out + (int64_t)y * a.stride_oy + x;
   const bool full = x + 8 <= a.n;
   half8_t prev = {0, 0, 0, 0, 0, 0, 0, 0}, bias = {0, 0, 0, 0, 0, 0, 0, 0};
   if (full) {
-    if (Epilogue::needs_prev(a.store)) prev = *(const half8_t*)p;
+    if (Epilogue::needs_prev(a.store)) {
+#pragma unroll
+      for (int q = 0; q < 8 / W; q++) {
+        const piece_t t = *(const piece_t*)(p + q * W);
+#pragma unroll
+        for (int e = 0; e < W; e++) prev[q * W + e] = t[e];
+      }
+    }
     if (Epilogue::needs_bias(a.store)) bias = *(const half8_t*)(a.bias + x);
   } else {
 #pragma unroll
@@ -159,12 +173,27 @@ __device__ __forceinline__ void store_chunk(const MatmulArgs& a, const Epilogue&
       if (x + e > y) r[e] = neg_inf_half();
   }
   if (full) {
-    __builtin_nontemporal_store(r, (half8_t*)p);
+#pragma unroll
+    for (int q = 0; q < 8 / W; q++) {
+      piece_t t;
+#pragma unroll
+      for (int e = 0; e < W; e++) t[e] = r[q * W + e];
+      __builtin_nontemporal_store(t, (piece_t*)(p + q * W));
+    }
   } else {
 #pragma unroll
     for (int e = 0; e < 8; e++)
       if (x + e < a.n) p[e] = r[e];
   }
+}
+
+// Halves per access that every row chunk of the output (8 columns from a column that is a multiple
+// of 8) is aligned to: 8, 4, 2, or 1 (element by element).  As out_vectorizable() for 8.
+__device__ __forceinline__ int out_chunk_alignment(const MatmulArgs& a, const half_t* out) {
+  if (Epilogue::needs_bias(a.store) && ((uintptr_t)a.bias & 15)) return 1;
+  if (a.store == STORE_ACC_BETA && a.beta != 0.0f) return 1;
+  const uintptr_t bits = (uintptr_t)a.stride_oy | (uintptr_t)a.stride_oz | ((uintptr_t)out >> 1);
+  return (bits & 7) == 0 ? 8 : (bits & 3) == 0 ? 4 : (bits & 1) == 0 ? 2 : 1;
 }
 
 // Epilogue of one wavefront.  acc[i][j] is the TRANSPOSED 32x32 accumulator of row block i,
@@ -1161,7 +1190,8 @@ __global__ __launch_bounds__(SHORTK_THREADS, 1) void gemm_nt_shortk_kernel(Matmu
     const int rrow = lane >> 4, rc = lane & 15;    // read round it: row it*4 + rrow, chunk rc
     const half_t hscale = (half_t)a.scale;
     Epilogue ep{a.bias, a.beta, hscale, a.store, true};
-    const bool vec = out_vectorizable(a, a.output) && !(a.stride_oz & 7);
+    const int walign = out_chunk_alignment(a, a.output);
+    const bool vec = walign >= 2;
     const bool plain = vec && (a.store == ADR_STORE_IDENTITY || a.store == ADR_STORE_SCALE);
     const half_t mul = a.store == ADR_STORE_SCALE ? hscale : (half_t)1.0f;
     auto write_half = [&](int batch, int m0, int n0, int half) {
@@ -1174,15 +1204,40 @@ __global__ __launch_bounds__(SHORTK_THREADS, 1) void gemm_nt_shortk_kernel(Matmu
       const int y0 = m0 + r0 + rrow, x = n0 + rc * 8;
       const bool inside = m0 + r0 + WROWS <= a.m && n0 + BN <= a.n;
       const bool unmasked = a.mask != ADR_MASK_CAUSAL || n0 + BN - 1 <= m0 + r0;
-      if (plain && inside && unmasked) {
+      if (plain && walign >= 4 && unmasked) {
         half8_t v[WIT];
 #pragma unroll
         for (int it = 0; it < WIT; it++) v[it] = staged(it);
         // x * 1 is exact: one multiply serves Identity and Scale (fp16 product, matmul.cu)
         half_t* const p = out + (int64_t)y0 * a.stride_oy + x;
+        if (inside && walign == 8) {
 #pragma unroll
-        for (int it = 0; it < WIT; it++)
-          __builtin_nontemporal_store(v[it] * mul, (half8_t*)(p + (int64_t)(it * 4) * a.stride_oy));
+          for (int it = 0; it < WIT; it++)
+            __builtin_nontemporal_store(v[it] * mul, (half8_t*)(p + (int64_t)(it * 4) * a.stride_oy));
+        } else {
+          // a ragged tile (rows or chunks past the matrix are skipped, a chunk across its last
+          // column goes element by element), or rows aligned to 8 bytes only (a row length that
+          // is a multiple of 4, not of 8: two stores per chunk)
+          const bool whole = x + 8 <= a.n, part = !whole && x < a.n;
+#pragma unroll
+          for (int it = 0; it < WIT; it++) {
+            if (y0 + it * 4 >= a.m) continue;
+            const half8_t r = v[it] * mul;
+            half_t* const q = p + (int64_t)(it * 4) * a.stride_oy;
+            if (whole) {
+              if (walign == 8) {
+                __builtin_nontemporal_store(r, (half8_t*)q);
+              } else {
+                __builtin_nontemporal_store(half4_t{r[0], r[1], r[2], r[3]}, (half4_t*)q);
+                __builtin_nontemporal_store(half4_t{r[4], r[5], r[6], r[7]}, (half4_t*)(q + 4));
+              }
+            } else if (part) {
+#pragma unroll
+              for (int e = 0; e < 8; e++)
+                if (x + e < a.n) q[e] = r[e];
+            }
+          }
+        }
       } else if (vec) {
         // (the rolled loops read the staging tile round by round: an array of rounds indexed by
         // the loop counter would live in scratch memory)
@@ -1190,7 +1245,11 @@ __global__ __launch_bounds__(SHORTK_THREADS, 1) void gemm_nt_shortk_kernel(Matmu
         for (int it = 0; it < WIT; it++) {
           const int y = y0 + it * 4;
           const half8_t v = staged(it);
-          if (y < a.m && x < a.n) store_chunk(a, ep, out, y, x, v);
+          if (y < a.m && x < a.n) {
+            if (walign == 8) store_chunk<8>(a, ep, out, y, x, v);
+            else if (walign == 4) store_chunk<4>(a, ep, out, y, x, v);
+            else store_chunk<2>(a, ep, out, y, x, v);
+          }
         }
       } else {
         const bool need_prev = Epilogue::needs_prev(a.store);
@@ -1256,11 +1315,21 @@ __global__ __launch_bounds__(SHORTK_THREADS, 1) void gemm_nt_shortk_kernel(Matmu
   const int offB = lds_chunk_off<CPR>(wn * 32 + frow, fkg);
   half8_t qa[KS][4];   // this wavefront's rows of the left panel
   float4_t acc[4][2];
+  // Load Scale (matmul.cu:439-443): both operands are multiplied by the scale, in fp16, before the
+  // product -- the left panel once per segment, the right fragments as they are read
+  const bool load_scale = a.load == ADR_LOAD_SCALE;
+  const half_t ls = (half_t)a.scale;
   auto copy_left = [&]() {
 #pragma unroll
     for (int kk = 0; kk < KS; kk++)
 #pragma unroll
       for (int i = 0; i < 4; i++) qa[kk][i] = *(const half8_t*)(sA + (offQ ^ (kk << 6)) + i * R16);
+    if (load_scale) {
+#pragma unroll
+      for (int kk = 0; kk < KS; kk++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) qa[kk][i] = qa[kk][i] * ls;
+    }
   };
   auto multiply = [&](const unsigned char* cB) {
 #pragma unroll
@@ -1278,6 +1347,10 @@ __global__ __launch_bounds__(SHORTK_THREADS, 1) void gemm_nt_shortk_kernel(Matmu
 #pragma unroll
         for (int jj = 0; jj < 2; jj++)
           fb[(kk + 1) & 1][jj] = *(const half8_t*)(cB + (offB ^ ((kk + 1) << 6)) + jj * R16);
+      }
+      if (load_scale) {
+#pragma unroll
+        for (int jj = 0; jj < 2; jj++) fb[kk & 1][jj] = fb[kk & 1][jj] * ls;
       }
 #pragma unroll
       for (int i = 0; i < 4; i++)
@@ -1888,12 +1961,14 @@ GemmChoice choose(const MatmulArgs& a) {
   if (a.lhs && ((uintptr_t)a.lhs % 16 != 0 || (uintptr_t)a.rhs % 16 != 0 ||
                 (uintptr_t)a.rhs_q % 8 != 0)) return GEMM_NONE;
   const bool plain = !a.rhs_q && a.load == ADR_LOAD_IDENTITY;
+  // One or two K slices (the attention score product): the persistent kernel, which also scales
+  // its operands on the way in where the caller asks for that (whisper.rs:424-430)
+  if (!a.rhs_q && (a.k == 64 || a.k == 128) && !(a.store == STORE_ACC_BETA && a.beta != 0.0f) &&
+      (int64_t)((a.m + 127) / 128) * ((a.n + 127) / 128) * a.batches >= 2 * NUM_CU)
+    return a.k == 64 ? SHORTK_64 : SHORTK_128;
   if (plain && a.k % 64 == 0) {
-    // Few K slices: the tile is dominated by its load latency and its epilogue; two resident
-    // workgroups per CU overlap those phases, which one large tile cannot.
-    if ((a.k == 64 || a.k == 128) && !(a.store == STORE_ACC_BETA && a.beta != 0.0f) &&
-        (int64_t)((a.m + 127) / 128) * ((a.n + 127) / 128) * a.batches >= 2 * NUM_CU)
-      return a.k == 64 ? SHORTK_64 : SHORTK_128;
+    // Few K slices and too few tiles for the persistent kernel: a tile is dominated by its load
+    // latency and its epilogue; two resident workgroups per CU overlap those phases
     if (a.k <= 256) {
       static const Candidate shortk[] = {{DMA_128x128, 128, 128, 2, 1.00f},
                                          {DMA_64x64, 64, 64, 4, 0.50f}};

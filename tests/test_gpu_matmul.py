@@ -280,10 +280,11 @@ def test_persistent_short_k_kernel_head_views(shape, mask):
     assert np.array_equal(to_np(o_t).view(np.uint16), want.view(np.uint16))
 
 
-@pytest.mark.parametrize("pad", [1, 4], ids=["odd_pitch", "pitch_8_bytes"])
+@pytest.mark.parametrize("pad", [1, 3, 4], ids=["rows_aligned_to_8_bytes", "to_4_bytes", "to_2_bytes"])
 def test_persistent_short_k_kernel_causal_rows_not_16_byte_aligned(pad):
-    """The causal score product into rows that no 16-byte store may touch: the run of -inf right
-    of the diagonal tile and the tiles themselves go element by element, to the same bits."""
+    """The causal score product into rows that no 16-byte store may touch (a sequence length that
+    is not a multiple of 8): the tiles go out in 8-, 4- or 2-byte pieces, the run of -inf right of
+    the diagonal tile element by element, to the same bits."""
     B, M, K, N = 9, 1000, 128, 1003
     g = rng(930 + pad)
     HD = B * K
@@ -301,6 +302,31 @@ def test_persistent_short_k_kernel_causal_rows_not_16_byte_aligned(pad):
     assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
     # the padding between rows keeps what it held
     assert np.array_equal(got.reshape(B, M, NP)[:, :, N:], prev.reshape(B, M, NP)[:, :, N:])
+
+
+@pytest.mark.parametrize("K,N", [(64, 1500), (128, 1000)])
+def test_persistent_short_k_kernel_load_scale(K, N):
+    """Whisper's score product (whisper.rs:424-430: both operands times d_head^-0.25 in fp16 before
+    the product) on the persistent kernel: 1500 positions, rows of the score tensor aligned to
+    8 bytes only."""
+    B, M = 6, 1500
+    g = rng(960 + K)
+    HD = B * K
+    so, sl, sr = (1, N, M * N), (1, HD, K), (HD, 1, K)
+    scale = float(K) ** -0.25
+    assert plan(B, M, K, N, so, sl, sr, load=oracle.LOAD_SCALE).startswith("gemm_nt_mfma_persistent")
+    l, r = randn_f16(g, M * HD), randn_f16(g, N * HD)
+    want = oracle_matmul(np.zeros(B * M * N, np.float16), l, r, B, M, K, N, so, sl, sr,
+                         load=oracle.LOAD_SCALE, scale=scale, mode=oracle.EXACT)
+    o_t = to_dev(np.zeros(B * M * N, np.float16))
+    assert raw_matmul("adr_matmul_f16", o_t, to_dev(l), to_dev(r), B, M, K, N, so, sl, sr,
+                      load=oracle.LOAD_SCALE, scale=scale) == 0
+    # the scaled operands are the same fp16 numbers; the fp32 sums run in another order, which
+    # shows as a second step only where products cancel to almost nothing
+    got, ref = to_np(o_t).astype(np.float64), want.astype(np.float64)
+    floor = 1e-2 * np.sqrt(np.mean(ref * ref))
+    assert np.max(np.abs(got - ref) / np.maximum(np.abs(ref), floor)) <= 2.0 ** -10
+    assert np.count_nonzero(ulp_diff_f16(to_np(o_t), want) > 1) <= 1e-4 * want.size
 
 
 @pytest.mark.parametrize("store", [oracle.STORE_ADD] + STORES_F32)
