@@ -19,6 +19,9 @@
 //  gemm_nt_shortk_kernel  K = 64 / 128 (the attention score product): persistent workgroups;
 //                       also with the Load Scale operator (both operands scaled in fp16 on the
 //                       way into the MFMAs) and for score rows that are not 16-byte aligned.
+//  gemm_nn_anyrow_kernel  row-major x row-major products (P.V) whose left rows start at any even
+//                       address and whose K is no multiple of 64 (sequence lengths like 77, 257,
+//                       1500): left operand through registers, shifted into place.
 //  gemm_nt_stage_kernel any K % 8 == 0, and the variants that must touch the data on the way
 //                       in: u8 weights dequantised while staging (adr_matmul_nt_fp16u8), and
 //                       the Load Scale operator on other K.  Global -> registers -> LDS, two
@@ -1782,6 +1785,186 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_stage_kernel(Matmul
 }
 
 // =============================================================================================
+// Register-staged kernel for row-major x row-major products whose left rows have any alignment
+// =============================================================================================
+// P.V of the attention call sites (llama.rs:552-554, clip.rs:385-388, whisper.rs:433-436) when
+// the sequence length is no multiple of 64: the probabilities [heads, S, T] are a dense tensor,
+// so their rows start at any even byte address (T = 77, 257, 1500, 2001 ...) and K = T ends in the
+// middle of a slice, or of a 16-byte chunk.  The left operand goes through registers: a lane
+// loads the dwords around its chunk from a 4-byte aligned address and shifts them into place
+// (v_alignbyte_b32), zeroes what lies beyond K, and writes the chunk to LDS in the layout of the
+// other kernels.  The right operand ([K][N], N contiguous, 16-byte aligned rows: V on its head
+// view) is staged as [64][128] tiles and read with the transposing LDS reads of the DMA kernel's
+// row-major form.  Two LDS stages, one barrier per slice, 128 x BN tiles of 2 x 2 wavefronts
+// (BN = 64 for heads of 64 columns).
+template <int BN>
+__global__ __launch_bounds__(256, 2) void gemm_nn_anyrow_kernel(MatmulArgs a, TileMap map) {
+  constexpr int BM = 128, BK = 64, WM = 2, WN = 2, NT = 256, CPR = 8;
+  constexpr int LA = BM * CPR / NT, LB = BK * (BN / 8) / NT;  // chunks each thread stages
+  constexpr int WTM = 64, WTN = BN / 2, TM = 2, TN = WTN / 32, KK = BK / 16;
+  constexpr int SLOT = 32 * (TN * 64 + 16);
+  static_assert(BN == 128 || BN == 64, "one or half a 256-byte line per k row");
+  // chunk c of k row r of the right tile sits at position c ^ swz(r) of its row: the 16 chunks a
+  // transposing read touches (4 rows x 4 chunks per 32 lanes) then fall into 16 bank groups
+  auto swz = [](int krow) { return BN == 128 ? (krow & 3) << 2 : ((krow >> 1) & 1) << 2; };
+  static_assert(WM * WN * SLOT <= 2 * (BM + BN) * BK * 2, "epilogue slots must fit in LDS");
+  __shared__ __attribute__((aligned(1024))) unsigned char sA[2][BM * BK * 2];
+  __shared__ __attribute__((aligned(1024))) unsigned char sB[2][BK * BN * 2];
+
+  int batch, tile_m, tile_n;
+  map_tile(map, batch, tile_m, tile_n);
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / WN, wn = wave % WN;
+  half_t* const out = a.output + (int64_t)batch * a.stride_oz;
+  if (a.mask == ADR_MASK_CAUSAL && n0 > m0 + BM - 1) {
+    fill_masked_tile<BM, BN, NT>(a, out, m0, n0, tid);
+    return;
+  }
+  const half_t* const A = a.lhs + (int64_t)batch * a.stride_lz;
+  const half_t* const B = a.rhs + (int64_t)batch * a.stride_rz;
+  const int K = a.k, KT = (K + BK - 1) / BK;
+
+  // Left operand.  Chunk c = tid + i * NT -> (row, kc).  Rows beyond the matrix read the last
+  // row again (their products are never stored).  `last` is the last dword of the left operand
+  // that may be read: no load goes past the tensor, whatever comes after it in memory.
+  const half_t* gA[LA];
+  int offA[LA], kcA[LA];
+#pragma unroll
+  for (int i = 0; i < LA; i++) {
+    const int c = tid + i * NT, row = c / CPR, kc = c % CPR;
+    gA[i] = A + (int64_t)min(m0 + row, a.m - 1) * a.stride_ly + kc * 8;
+    offA[i] = lds_chunk_off<CPR>(row, kc);
+    kcA[i] = kc * 8;
+  }
+  const uintptr_t a_end = (uintptr_t)(a.lhs + (int64_t)(a.batches - 1) * a.stride_lz +
+                                      (int64_t)(a.m - 1) * a.stride_ly + K);  // one past the last element
+  const uintptr_t last = ((a_end + 3) & ~(uintptr_t)3) - 4;
+  // Right operand.  Chunk c -> (k row, column chunk) of the [64][128] tile; k rows beyond K and
+  // columns beyond N are zero.
+  int krB[LB], ncB[LB], offB[LB];
+#pragma unroll
+  for (int i = 0; i < LB; i++) {
+    const int c = tid + i * NT;
+    krB[i] = c / (BN / 8);
+    ncB[i] = (c % (BN / 8)) * 8;
+    offB[i] = krB[i] * (BN * 2) + (((ncB[i] >> 3) ^ swz(krB[i])) << 4);
+  }
+
+  u32x4_t ra[LA], rb[LB];
+  // eight halves from any even address: five dwords from the aligned address below it, shifted
+  // by 0 or 2 bytes; elements from `valid` on are zero
+  auto load_left = [&](const half_t* p, int valid) -> u32x4_t {
+    const uintptr_t u = (uintptr_t)p, base = u & ~(uintptr_t)3;
+    const uint32_t shift = (uint32_t)(u & 2);
+    uint32_t d[5];
+    // (global, not generic, addresses: a generic load also waits on the LDS counter)
+    typedef const __attribute__((address_space(1))) uint32_t* gptr32_t;
+    typedef uint32_t u32x4_dword_aligned_t __attribute__((ext_vector_type(4), aligned(4)));
+    typedef const __attribute__((address_space(1))) u32x4_dword_aligned_t* gptr128_t;
+    // (a wavefront-uniform branch: a load under a lane mask is waited for where the lanes rejoin)
+    if (__builtin_amdgcn_ballot_w64(base + 16 > last) == 0) {
+      const u32x4_t q = *(gptr128_t)base;
+      d[0] = q[0]; d[1] = q[1]; d[2] = q[2]; d[3] = q[3];
+      d[4] = *(gptr32_t)(base + 16);
+    } else {
+#pragma unroll
+      for (int j = 0; j < 5; j++) d[j] = *(gptr32_t)(base + 4 * j < last ? base + 4 * j : last);
+    }
+    u32x4_t r;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      uint32_t w = __builtin_amdgcn_alignbyte(d[j + 1], d[j], shift);
+      // elements 2j and 2j+1 of the chunk
+      w = 2 * j + 1 < valid ? w : 2 * j < valid ? (w & 0xffffu) : 0u;
+      r[j] = w;
+    }
+    return r;
+  };
+  auto load_slice = [&](int kt) {
+    const int k0 = kt * BK;
+#pragma unroll
+    for (int i = 0; i < LA; i++) ra[i] = load_left(gA[i] + k0, K - k0 - kcA[i]);
+#pragma unroll
+    for (int i = 0; i < LB; i++) {
+      const int kr = k0 + krB[i], col = n0 + ncB[i];
+      const bool in = kr < K && col < a.n;
+      const u32x4_t v = *(const u32x4_t*)(B + (int64_t)min(kr, K - 1) * a.stride_ry + (col < a.n ? col : 0));
+      rb[i] = in ? v : u32x4_t{0, 0, 0, 0};
+    }
+  };
+  auto store_slice = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < LA; i++) *(u32x4_t*)(sA[buf] + offA[i]) = ra[i];
+#pragma unroll
+    for (int i = 0; i < LB; i++) *(u32x4_t*)(sB[buf] + offB[i]) = rb[i];
+  };
+
+  float16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+  // fragment addressing.  Left: lane -> (row lane % 32, k-group lane / 32).  Right: the
+  // transposing read of the DMA kernel's row-major form (ds_read_b64_tr_b16): inside each group of
+  // 16 lanes, lanes 4r..4r+3 address 16 consecutive halves of k-row r and lane i receives column
+  // i of that 4 x 16 block.
+  const int frow = lane & 31, fkg = lane >> 5;
+  int offFB[TN][KK];
+  {
+    const int q = lane >> 4, r = (lane >> 2) & 3, jj = lane & 3;
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++)
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        const int krow = kk * 16 + (q >> 1) * 8 + r;
+        const int col = wn * WTN + j * 32 + 16 * (q & 1) + 4 * jj;
+        offFB[j][kk] = krow * (BN * 2) + (((col >> 3) ^ swz(krow)) << 4) + (jj & 1) * 8;
+      }
+  }
+  typedef short short4_t __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) short4_t lds_short4_t;
+
+  load_slice(0);
+  store_slice(0);
+  __syncthreads();
+  for (int kt = 0; kt < KT; kt++) {
+    const int buf = kt & 1;
+    if (kt + 1 < KT) load_slice(kt + 1);
+    const unsigned char* cA = sA[buf];
+    const unsigned char* cB = sB[buf];
+#pragma unroll
+    for (int kk = 0; kk < KK; kk++) {
+      half8_t fa[TM], fb[TN];
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+        fa[i] = *(const half8_t*)(cA + lds_chunk_off<CPR>(wm * WTM + i * 32 + frow, kk * 2 + fkg));
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        const short4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (lds_short4_t*)ADR_LDS_PTR(cB + offFB[j][kk]));
+        const short4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (lds_short4_t*)ADR_LDS_PTR(cB + offFB[j][kk] + 4 * (BN * 2)));  // k-rows + 4
+        fb[j] = __builtin_shufflevector(__builtin_bit_cast(half4_t, lo),
+                                        __builtin_bit_cast(half4_t, hi), 0, 1, 2, 3, 4, 5, 6, 7);
+      }
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < KT) store_slice(buf ^ 1);
+    __syncthreads();
+  }
+  wave_epilogue<TM, 2 * TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, &sA[0][0] + wave * SLOT,
+                            (half_t)a.scale, lane);
+}
+
+// =============================================================================================
 // Host side: configuration choice and launch
 // =============================================================================================
 TileMap make_map(const MatmulArgs& a, int bm, int bn) {
@@ -1860,6 +2043,14 @@ hipError_t launch_u8(hipStream_t stream, const MatmulArgs& a) {
   return hipGetLastError();
 }
 
+template <int BN>
+hipError_t launch_nn_anyrow(hipStream_t stream, const MatmulArgs& a) {
+  TileMap map = make_map(a, 128, BN);
+  if (map.total < 0) return hipErrorInvalidConfiguration;
+  hipLaunchKernelGGL(gemm_nn_anyrow_kernel<BN>, dim3((unsigned)map.total), dim3(256), 0, stream, a, map);
+  return hipGetLastError();
+}
+
 // compute units of the current device (MI355X: 256)
 static int num_cu() { return device_info_for_plan().cus; }
 
@@ -1898,7 +2089,7 @@ enum GemmChoice {
   SHORTK_64, SHORTK_128,
   U8_256x192, U8_256x128,
   DMA_256x192, DMA_256x160, DMA_256x128, DMA_128x256, DMA_128x192, DMA_128x128, DMA_128x64, DMA_64x64, DMA_64x64_K128, DMA_128x64_K128,
-  DMA_NN_256x128, DMA_NN_128x128,
+  DMA_NN_256x128, DMA_NN_128x128, NN_ANYROW_128x128, NN_ANYROW_128x64,
   STAGE_256x128, STAGE_128x128, STAGE_64x64,
 };
 
@@ -1955,6 +2146,13 @@ GemmChoice choose(const MatmulArgs& a) {
                                    {DMA_NN_128x128, 128, 128, 2, 0.80f}};
     return pick(a, nn, 2);
   }
+  // the same layout with left rows of any alignment or a K that is no multiple of 64: P.V of a
+  // sequence length like 77, 257, 1500 or 2001
+  if (a.stride_lx == 1 && a.stride_rx == 1 && a.stride_ry != 1 && a.stride_ox == 1 && !a.rhs_q &&
+      a.load == ADR_LOAD_IDENTITY && a.k >= 1 && a.n % 8 == 0 && a.n >= 8 && a.stride_ly > 0 &&
+      a.stride_lz >= 0 && !((a.stride_ry % 8) | (a.stride_rz % 8)) &&
+      !(a.lhs && (uintptr_t)a.rhs % 16 != 0))
+    return a.n <= 64 || (a.n > 128 && a.n % 128 != 0 && a.n % 128 <= 64) ? NN_ANYROW_128x64 : NN_ANYROW_128x128;
   if (a.stride_lx != 1 || a.stride_ry != 1 || a.stride_ox != 1) return GEMM_NONE;
   if (a.k % 8 != 0 || a.k < 8) return GEMM_NONE;
   if ((a.stride_ly % 8) | (a.stride_rx % 8) | (a.stride_lz % 8) | (a.stride_rz % 8)) return GEMM_NONE;
@@ -2103,6 +2301,8 @@ static bool choice_name(GemmChoice c, const char** name, bool u8 = false) {
     case DMA_128x64_K128: *name = "gemm_nt_mfma_dma_128x64x128"; return true;
     case DMA_NN_256x128: *name = "gemm_nn_mfma_dma_256x128x64"; return true;
     case DMA_NN_128x128: *name = "gemm_nn_mfma_dma_128x128x64"; return true;
+    case NN_ANYROW_128x128: *name = "gemm_nn_mfma_anyrow_128x128x64"; return true;
+    case NN_ANYROW_128x64: *name = "gemm_nn_mfma_anyrow_128x64x64"; return true;
     case STAGE_256x128: *name = "gemm_nt_mfma_stage_256x128x32"; return true;
     case STAGE_128x128: *name = "gemm_nt_mfma_stage_128x128x32"; return true;
     case STAGE_64x64: *name = "gemm_nt_mfma_stage_64x64x64"; return true;
@@ -2128,6 +2328,8 @@ static hipError_t launch_choice(hipStream_t stream, const MatmulArgs& a, GemmCho
     case DMA_128x64_K128: return launch_dma<128, 64, 2, 2, 3, 1, false, 128>(stream, a);
     case DMA_NN_256x128: return launch_dma<256, 128, 4, 2, 3, 1, true>(stream, a);
     case DMA_NN_128x128: return launch_dma<128, 128, 2, 2, 2, 2, true>(stream, a);
+    case NN_ANYROW_128x128: return launch_nn_anyrow<128>(stream, a);
+    case NN_ANYROW_128x64: return launch_nn_anyrow<64>(stream, a);
     case STAGE_256x128: return launch_stage<256, 128, 32, 2, 2, 2>(stream, a);
     case STAGE_128x128: return launch_stage<128, 128, 32, 2, 2, 2>(stream, a);
     case STAGE_64x64: return launch_stage<64, 64, 64, 2, 2, 2>(stream, a);

@@ -250,6 +250,55 @@ def test_attention_views_qk_and_pv():
     assert np.array_equal(to_np(o_t).view(np.uint16), want.view(np.uint16))
 
 
+PV_SHAPES = [
+    # (heads, S, T, D, extra elements before the first probability)
+    (12, 77, 77, 64, 0),      # CLIP text: rows of 154 bytes
+    (16, 257, 257, 64, 0),    # CLIP vision, one image
+    (3, 300, 301, 128, 1),    # odd pitch and an odd first address
+    (2, 1500, 1500, 64, 0),   # Whisper: rows aligned to 8 bytes, K ends inside a chunk
+    (2, 130, 1999, 128, 3),   # a long odd K
+    (2, 200, 1000, 128, 0),   # 16-byte aligned rows, K no multiple of 64
+]
+
+
+@pytest.mark.parametrize("H,S,T,D,off", PV_SHAPES, ids=lambda v: str(v))
+def test_pv_of_sequence_lengths_that_are_no_multiple_of_64(H, S, T, D, off):
+    """P.V on the views of llama.rs:552-554 / clip.rs:385-388 / whisper.rs:433-436 when the
+    probabilities' rows start at any even address and K = T ends inside a slice: the tiled kernel
+    that shifts the left operand into place, on inputs whose fp32 sums are exact; the last
+    probability is the last element of its buffer (nothing may be read past it that matters)."""
+    HD = H * D
+    gen = torch.Generator(device="cuda").manual_seed(H * S + T)
+    pbuf = (torch.randint(0, 9, (off + H * S * T,), generator=gen, device="cuda").float() / 64).half()
+    v = (torch.randint(-8, 9, (T, HD), generator=gen, device="cuda").float() / 16).half()
+    out = torch.full((S, HD), 3.0, dtype=torch.float16, device="cuda")
+    so, sl, sr = (1, HD, D), (1, T, S * T), (1, HD, D)
+    assert plan(H, S, T, D, so, sl, sr) == f"gemm_nn_mfma_anyrow_128x{D}x64"
+    assert raw_matmul("adr_matmul_f16", out, pbuf, v, H, S, T, D, so, sl, sr, offsets=(0, off, 0)) == 0
+    p = pbuf[off:].view(H, S, T).double()
+    want = torch.bmm(p, v.view(T, H, D).permute(1, 0, 2).double()).permute(1, 0, 2).reshape(S, HD).half()
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+
+
+def test_pv_anyrow_kernel_ignores_what_follows_k():
+    """Non-finite values right behind a row's K elements (the next row's first probabilities, or
+    whatever follows the tensor) must not reach the sums: rows of T = 70 probabilities inside a
+    pitch of 75, the five elements in between set to NaN."""
+    H, S, T, D, pitch = 2, 140, 70, 64, 75
+    HD = H * D
+    gen = torch.Generator(device="cuda").manual_seed(3)
+    pbuf = torch.full((H * S * pitch,), float("nan"), dtype=torch.float16, device="cuda")
+    p = (torch.randint(0, 9, (H, S, T), generator=gen, device="cuda").float() / 64).half()
+    pbuf.view(H, S, pitch)[:, :, :T] = p
+    v = (torch.randint(-8, 9, (T, HD), generator=gen, device="cuda").float() / 16).half()
+    out = torch.zeros(S, HD, dtype=torch.float16, device="cuda")
+    so, sl, sr = (1, HD, D), (1, pitch, S * pitch), (1, HD, D)
+    assert plan(H, S, T, D, so, sl, sr) == "gemm_nn_mfma_anyrow_128x64x64"
+    assert raw_matmul("adr_matmul_f16", out, pbuf, v, H, S, T, D, so, sl, sr) == 0
+    want = torch.bmm(p.double(), v.view(T, H, D).permute(1, 0, 2).double()).permute(1, 0, 2).reshape(S, HD).half()
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+
+
 SHORTK = [
     # (B, M, K, N): at least 512 tiles of 128x128 so that the persistent kernel is selected
     (9, 1000, 128, 1000),    # ragged tiles in M and N, 64 tiles per batch
