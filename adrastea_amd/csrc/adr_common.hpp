@@ -181,6 +181,53 @@ __device__ __forceinline__ half8_t dequant8(uint32_t w0, uint32_t w1, half2_t s2
 
 typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
 
+// Eight halves from / to any even address in global memory, for tensors whose rows are not 16-byte
+// aligned (a score tensor [heads, S, T] with T no multiple of 8).  Vector accesses need 4-byte
+// alignment only: a chunk at a 4-byte aligned address moves as one dwordx4; a chunk 2 bytes off
+// is read as the five dwords around it and shifted (v_alignbyte_b32), and written as its first
+// half, three dwords and its last half -- whole dwords across a chunk's ends would touch halves that
+// other lanes or other workgroups own.
+typedef uint32_t u32x4_dword_aligned_t __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint32_t u32x2_dword_aligned_t __attribute__((ext_vector_type(2), aligned(4)));
+#define ADR_GLOBAL_AS __attribute__((address_space(1)))
+
+// `last`: the last dword that may be read (loads past it read it again: what they return lies
+// beyond the row's end and must be masked by the caller)
+__device__ __forceinline__ half8_t load8_any(const half_t* p, uintptr_t last) {
+  const uintptr_t u = (uintptr_t)p, base = u & ~(uintptr_t)3;
+  const uint32_t shift = (uint32_t)(u & 2);
+  uint32_t d[5];
+  // (a wavefront-uniform branch: a load under a lane mask is waited for where the lanes rejoin)
+  if (__builtin_amdgcn_ballot_w64(base + 16 > last) == 0) {
+    const u32x4_t q = *(const ADR_GLOBAL_AS u32x4_dword_aligned_t*)base;
+    d[0] = q[0]; d[1] = q[1]; d[2] = q[2]; d[3] = q[3];
+    d[4] = *(const ADR_GLOBAL_AS uint32_t*)(base + 16);
+  } else {
+#pragma unroll
+    for (int j = 0; j < 5; j++)
+      d[j] = *(const ADR_GLOBAL_AS uint32_t*)(base + 4 * j < last ? base + 4 * j : last);
+  }
+  u32x4_t r;
+#pragma unroll
+  for (int j = 0; j < 4; j++) r[j] = __builtin_amdgcn_alignbyte(d[j + 1], d[j], shift);
+  return __builtin_bit_cast(half8_t, r);
+}
+
+__device__ __forceinline__ void store8_any(half_t* p, half8_t v) {
+  const uintptr_t u = (uintptr_t)p;
+  const u32x4_t r = __builtin_bit_cast(u32x4_t, v);
+  if ((u & 2) == 0) {
+    __builtin_nontemporal_store(r, (ADR_GLOBAL_AS u32x4_dword_aligned_t*)u);
+  } else {
+    typedef uint16_t ADR_GLOBAL_AS* gptr16_t;
+    __builtin_nontemporal_store((uint16_t)(r[0] & 0xffffu), (gptr16_t)u);
+    const u32x2_t m01 = {__builtin_amdgcn_alignbyte(r[1], r[0], 2u), __builtin_amdgcn_alignbyte(r[2], r[1], 2u)};
+    __builtin_nontemporal_store(m01, (ADR_GLOBAL_AS u32x2_dword_aligned_t*)(u + 2));
+    __builtin_nontemporal_store(__builtin_amdgcn_alignbyte(r[3], r[2], 2u), (ADR_GLOBAL_AS uint32_t*)(u + 10));
+    __builtin_nontemporal_store((uint16_t)(r[3] >> 16), (gptr16_t)(u + 14));
+  }
+}
+
 template <int CTRL, int ROWMASK>
 __device__ __forceinline__ float dpp_add(float v) {
   int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROWMASK, 0xf, true);

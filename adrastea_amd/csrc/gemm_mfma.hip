@@ -1030,17 +1030,15 @@ __global__ __launch_bounds__(256) void fill_causal_rows_kernel(MatmulArgs a) {
   half_t* const out = a.output + (int64_t)batch * a.stride_oz;
   half_t* const row = out + (int64_t)y * a.stride_oy;
   const half_t ninf = neg_inf_half();
-  if (out_vectorizable(a, out)) {
-    const half8_t v = {ninf, ninf, ninf, ninf, ninf, ninf, ninf, ninf};
-    for (int x = x0 + lane * 8; x < a.n; x += 512) {
-      if (x + 8 <= a.n) {
-        __builtin_nontemporal_store(v, (half8_t*)(row + x));
-      } else {
-        for (int q = 0; x + q < a.n; q++) row[x + q] = ninf;
-      }
+  const half8_t v = {ninf, ninf, ninf, ninf, ninf, ninf, ninf, ninf};
+  const bool aligned = out_vectorizable(a, out);
+  for (int x = x0 + lane * 8; x < a.n; x += 512) {
+    if (x + 8 <= a.n) {
+      if (aligned) __builtin_nontemporal_store(v, (half8_t*)(row + x));
+      else store8_any(row + x, v);
+    } else {
+      for (int q = 0; x + q < a.n; q++) row[x + q] = ninf;
     }
-  } else {
-    for (int x = x0 + lane; x < a.n; x += 64) row[x] = ninf;
   }
 }
 
@@ -1195,7 +1193,8 @@ __global__ __launch_bounds__(SHORTK_THREADS, 1) void gemm_nt_shortk_kernel(Matmu
     Epilogue ep{a.bias, a.beta, hscale, a.store, true};
     const int walign = out_chunk_alignment(a, a.output);
     const bool vec = walign >= 2;
-    const bool plain = vec && (a.store == ADR_STORE_IDENTITY || a.store == ADR_STORE_SCALE);
+    // (Identity and Scale need neither the previous output nor the bias: any alignment)
+    const bool plain = a.store == ADR_STORE_IDENTITY || a.store == ADR_STORE_SCALE;
     const half_t mul = a.store == ADR_STORE_SCALE ? hscale : (half_t)1.0f;
     auto write_half = [&](int batch, int m0, int n0, int half) {
       const int r0 = half * 64 + sw * WROWS;  // first of this wavefront's rows in the tile
@@ -1207,7 +1206,7 @@ __global__ __launch_bounds__(SHORTK_THREADS, 1) void gemm_nt_shortk_kernel(Matmu
       const int y0 = m0 + r0 + rrow, x = n0 + rc * 8;
       const bool inside = m0 + r0 + WROWS <= a.m && n0 + BN <= a.n;
       const bool unmasked = a.mask != ADR_MASK_CAUSAL || n0 + BN - 1 <= m0 + r0;
-      if (plain && walign >= 4 && unmasked) {
+      if (plain && unmasked) {
         half8_t v[WIT];
 #pragma unroll
         for (int it = 0; it < WIT; it++) v[it] = staged(it);
@@ -1219,8 +1218,8 @@ __global__ __launch_bounds__(SHORTK_THREADS, 1) void gemm_nt_shortk_kernel(Matmu
             __builtin_nontemporal_store(v[it] * mul, (half8_t*)(p + (int64_t)(it * 4) * a.stride_oy));
         } else {
           // a ragged tile (rows or chunks past the matrix are skipped, a chunk across its last
-          // column goes element by element), or rows aligned to 8 bytes only (a row length that
-          // is a multiple of 4, not of 8: two stores per chunk)
+          // column goes element by element), or rows that are not 16-byte aligned (a row length
+          // that is no multiple of 8: store8_any)
           const bool whole = x + 8 <= a.n, part = !whole && x < a.n;
 #pragma unroll
           for (int it = 0; it < WIT; it++) {
@@ -1228,12 +1227,8 @@ __global__ __launch_bounds__(SHORTK_THREADS, 1) void gemm_nt_shortk_kernel(Matmu
             const half8_t r = v[it] * mul;
             half_t* const q = p + (int64_t)(it * 4) * a.stride_oy;
             if (whole) {
-              if (walign == 8) {
-                __builtin_nontemporal_store(r, (half8_t*)q);
-              } else {
-                __builtin_nontemporal_store(half4_t{r[0], r[1], r[2], r[3]}, (half4_t*)q);
-                __builtin_nontemporal_store(half4_t{r[4], r[5], r[6], r[7]}, (half4_t*)(q + 4));
-              }
+              if (walign == 8) __builtin_nontemporal_store(r, (half8_t*)q);
+              else store8_any(q, r);
             } else if (part) {
 #pragma unroll
               for (int e = 0; e < 8; e++)
@@ -1852,33 +1847,12 @@ __global__ __launch_bounds__(256, 2) void gemm_nn_anyrow_kernel(MatmulArgs a, Ti
   }
 
   u32x4_t ra[LA], rb[LB];
-  // eight halves from any even address: five dwords from the aligned address below it, shifted
-  // by 0 or 2 bytes; elements from `valid` on are zero
+  // eight halves from any even address (load8_any); elements from `valid` on are zero
   auto load_left = [&](const half_t* p, int valid) -> u32x4_t {
-    const uintptr_t u = (uintptr_t)p, base = u & ~(uintptr_t)3;
-    const uint32_t shift = (uint32_t)(u & 2);
-    uint32_t d[5];
-    // (global, not generic, addresses: a generic load also waits on the LDS counter)
-    typedef const __attribute__((address_space(1))) uint32_t* gptr32_t;
-    typedef uint32_t u32x4_dword_aligned_t __attribute__((ext_vector_type(4), aligned(4)));
-    typedef const __attribute__((address_space(1))) u32x4_dword_aligned_t* gptr128_t;
-    // (a wavefront-uniform branch: a load under a lane mask is waited for where the lanes rejoin)
-    if (__builtin_amdgcn_ballot_w64(base + 16 > last) == 0) {
-      const u32x4_t q = *(gptr128_t)base;
-      d[0] = q[0]; d[1] = q[1]; d[2] = q[2]; d[3] = q[3];
-      d[4] = *(gptr32_t)(base + 16);
-    } else {
+    u32x4_t r = __builtin_bit_cast(u32x4_t, load8_any(p, last));
 #pragma unroll
-      for (int j = 0; j < 5; j++) d[j] = *(gptr32_t)(base + 4 * j < last ? base + 4 * j : last);
-    }
-    u32x4_t r;
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-      uint32_t w = __builtin_amdgcn_alignbyte(d[j + 1], d[j], shift);
-      // elements 2j and 2j+1 of the chunk
-      w = 2 * j + 1 < valid ? w : 2 * j < valid ? (w & 0xffffu) : 0u;
-      r[j] = w;
-    }
+    for (int j = 0; j < 4; j++)  // elements 2j and 2j+1 of the chunk
+      r[j] = 2 * j + 1 < valid ? r[j] : 2 * j < valid ? (r[j] & 0xffffu) : 0u;
     return r;
   };
   auto load_slice = [&](int kt) {

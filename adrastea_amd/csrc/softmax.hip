@@ -4,8 +4,10 @@
 //   v_i   = float(in_i) / temp
 //   out_i = fp16( expf(v_i - max_j v_j) / sum_j expf(v_j - max_j v_j) )
 // The operation is bound by reading and writing the tensor once each.  Rows of up to 4096
-// elements are held in registers by one wavefront (16-byte loads, one pass over memory, shuffle
-// reductions); anything else takes a three-pass kernel with one workgroup per row.
+// elements are held in registers by one wavefront (one pass over memory, shuffle reductions):
+// 16-byte accesses where the rows are 16-byte aligned, shifted dword accesses where they start
+// at any even address (a row length that is no multiple of 8); longer rows take a three-pass
+// kernel with one workgroup per row.
 #include "adr_common.hpp"
 
 namespace adr {
@@ -92,6 +94,62 @@ __global__ __launch_bounds__(256) void softmax_rows_reg_kernel(half_t* out, cons
   }
 }
 
+// The same for rows that start at any even address and hold any number of elements (w <= 512 * NV):
+// a sequence length that is no multiple of 8 (Whisper's 1500 positions, CLIP's 77 and 257, any odd
+// prompt length).  Chunks of eight halves counted from the row's first element, moved with
+// load8_any / store8_any; the row's last, partial chunk is stored element by element.
+template <int NV>
+__global__ __launch_bounds__(256) void softmax_rows_anyrow_kernel(half_t* out, const half_t* in,
+                                                                  int64_t rows, int w, float temp) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+  if (row >= rows) return;
+  const half_t* src = in + row * w;
+  half_t* dst = out + row * w;
+  const uintptr_t end = (uintptr_t)(in + rows * w);  // one past the tensor's last element
+  const uintptr_t last = ((end + 3) & ~(uintptr_t)3) - 4;
+  float v[NV][8];
+  float mx = -INFINITY;
+  const bool unit_temp = temp == 1.0f;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const int c = (i * 64 + lane) * 8;
+    // (chunks past the row read the row's first chunk again: no load under a lane mask)
+    const half8_t x = load8_any(src + (c < w ? c : 0), last);
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const float t = unit_temp ? (float)x[e] : (float)x[e] / temp;
+      v[i][e] = c + e < w ? t : -INFINITY;
+      mx = fmaxf(mx, v[i][e]);
+    }
+  }
+  mx = wave_max(mx);
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NV; i++)
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      v[i][e] = exp_neg(v[i][e] - mx);  // (-inf - mx: 0 for the elements past the row)
+      sum += v[i][e];
+    }
+  sum = wave_sum(sum);
+  const float rs = 1.0f / sum;
+#pragma unroll
+  for (int i = 0; i < NV; i++) {
+    const int c = (i * 64 + lane) * 8;
+    half8_t r;
+#pragma unroll
+    for (int e = 0; e < 8; e++) r[e] = (half_t)(v[i][e] * rs);
+    if (c + 8 <= w) {
+      store8_any(dst + c, r);
+    } else if (c < w) {
+#pragma unroll
+      for (int e = 0; e < 8; e++)
+        if (c + e < w) dst[c + e] = r[e];
+    }
+  }
+}
+
 // Any width and alignment: one workgroup per row, three passes over the row.
 __global__ __launch_bounds__(256) void softmax_rows_general_kernel(half_t* out, const half_t* in,
                                                                    int w, float temp) {
@@ -134,6 +192,18 @@ hipError_t launch_softmax_rows(hipStream_t stream, half_t* out, const half_t* in
       hipLaunchKernelGGL(softmax_rows_reg_kernel<4>, grid, block, 0, stream, out, in, rows, w, temp);
     else
       hipLaunchKernelGGL(softmax_rows_reg_kernel<8>, grid, block, 0, stream, out, in, rows, w, temp);
+  } else if (w <= 4096) {
+    const int64_t blocks = (rows + 3) / 4;
+    if (blocks > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+    const dim3 grid((unsigned)blocks), block(256);
+    if (w <= 512)
+      hipLaunchKernelGGL(softmax_rows_anyrow_kernel<1>, grid, block, 0, stream, out, in, rows, w, temp);
+    else if (w <= 1024)
+      hipLaunchKernelGGL(softmax_rows_anyrow_kernel<2>, grid, block, 0, stream, out, in, rows, w, temp);
+    else if (w <= 2048)
+      hipLaunchKernelGGL(softmax_rows_anyrow_kernel<4>, grid, block, 0, stream, out, in, rows, w, temp);
+    else
+      hipLaunchKernelGGL(softmax_rows_anyrow_kernel<8>, grid, block, 0, stream, out, in, rows, w, temp);
   } else {
     if (rows > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     hipLaunchKernelGGL(softmax_rows_general_kernel, dim3((unsigned)rows), dim3(256), 0, stream, out,

@@ -31,7 +31,9 @@ def call(out_t, in_t, heads, h, w, temp):
 
 
 SHAPES = [(1, 1, 1), (2, 3, 8), (3, 5, 77), (2, 9, 257), (4, 16, 512), (2, 7, 520), (1, 33, 1024),
-          (2, 10, 2048), (1, 6, 3000), (1, 5, 4096), (1, 3, 4104), (1, 2, 10000)]
+          (2, 10, 2048), (1, 6, 3000), (1, 5, 4096), (1, 3, 4104), (1, 2, 10000),
+          # rows that are not 16-byte aligned: aligned to 8 bytes (1500), 4 bytes (1002), 2 bytes
+          (2, 11, 1500), (3, 4, 1002), (1, 9, 2001), (1, 7, 4095)]
 
 
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
@@ -61,6 +63,30 @@ def test_softmax_matches_oracle_and_reference_kernel(ref, shape, temp):
     inplace = x_t.clone()
     assert call(inplace, inplace, heads, h, w, temp) == 0
     assert torch.equal(inplace, out)
+
+
+@pytest.mark.parametrize("w", [77, 1500, 2001])
+def test_softmax_of_a_tensor_that_starts_at_an_odd_element(w):
+    """A score tensor inside a larger buffer, its first element at an odd index: the guard
+    elements before and behind it keep their bits, in place and out of place."""
+    heads, h = 2, 5
+    g = rng(830 + w)
+    x = (g.standard_normal((heads, h, w)) * 4).astype(np.float16)
+    want = oracle.softmax_rows(x, 1.0, 0)
+    n = heads * h * w
+    buf = torch.full((n + 8,), 5.0, dtype=torch.float16, device="cuda")
+    buf[3:3 + n] = to_dev(x).flatten()
+    out = torch.full((n + 8,), 9.0, dtype=torch.float16, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    lib = _ffi.lib()
+    assert lib.adr_softmax_rows(stream, out.data_ptr() + 2, buf.data_ptr() + 6, heads, h, w, 1.0) == 0
+    got = to_np(out)
+    assert np.max(ulp_diff_f16(got[1:1 + n].reshape(heads, h, w), want)) <= 1
+    assert np.all(got[:1] == 9.0) and np.all(got[1 + n:] == 9.0)
+    assert lib.adr_softmax_rows(stream, buf.data_ptr() + 6, buf.data_ptr() + 6, heads, h, w, 1.0) == 0
+    got = to_np(buf)
+    assert np.max(ulp_diff_f16(got[3:3 + n].reshape(heads, h, w), want)) <= 1
+    assert np.all(got[:3] == 5.0) and np.all(got[3 + n:] == 5.0)
 
 
 def test_softmax_closed_forms_and_errors(kern):
