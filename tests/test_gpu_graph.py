@@ -66,3 +66,54 @@ def test_graph_replays_equal_eager():
         torch.cuda.synchronize()
         for got, ref in zip((x, qkv, att, hidden, probs), want):
             assert torch.equal(got, ref), replay
+
+
+def test_three_launch_attention_of_an_odd_length_replays_equal_eager():
+    """The separate launches of llama.rs:541-554 at a sequence length that is no multiple of 8
+    (score rows at any even address): causal score product (its fill launch and the persistent
+    kernel), softmax_rows in place, P.V through the kernel that shifts its left operand into place
+    -- captured once, replayed with eager work in between, bit for bit the eager result and close
+    to the fused launch."""
+    k = GpuKernels()
+    gen = torch.Generator(device="cuda").manual_seed(22)
+    heads, S, hd = 32, 1001, 128
+    dim = heads * hd
+    q, kk, v = (torch.randn(S, dim, generator=gen, device="cuda", dtype=torch.float16) for _ in range(3))
+    scores = torch.zeros(heads, S, S, dtype=torch.float16, device="cuda")
+    out = torch.zeros(S, dim, dtype=torch.float16, device="cuda")
+
+    def hv(t):
+        return TensorView.of(t).shape_cast([S, heads, -1]).permute([1, 0, 2])
+
+    def chain():
+        k_view = TensorView.of(kk).shape_cast([S, heads, -1]).permute([1, 2, 0])
+        k.matmul_f16(TensorView.of(scores), hv(q), k_view,
+                     MatmulOptions.new().store(MatmulStore.Scale(1.0 / hd ** 0.5)).mask(MatmulMask.CAUSAL))
+        k.softmax_rows_inplace(TensorView.of(scores), 1.0)
+        k.matmul_f16(hv(out), TensorView.of(scores), hv(v), MatmulOptions.new())
+
+    chain()
+    torch.cuda.synchronize()
+    want_scores, want_out = scores.clone(), out.clone()
+    fused = torch.zeros_like(out)
+    k.attention_f16(hv(fused), hv(q), hv(kk), hv(v), 1.0 / hd ** 0.5, 1.0, MatmulMask.CAUSAL)
+    torch.cuda.synchronize()
+    assert (fused.float() - want_out.float()).abs().max().item() <= 4e-3
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        chain()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        chain()
+    for replay in range(3):
+        scores.fill_(float(replay))
+        out.fill_(float(replay))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(scores, want_scores), replay
+        assert torch.equal(out, want_out), replay
