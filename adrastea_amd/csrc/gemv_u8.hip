@@ -776,7 +776,7 @@ hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, co
     // 17 rows and more against 4 MiB of weights and more: passes of up to 64 rows, each reading
     // the weights once for two to four blocks of sixteen rows (p is a multiple of 256 here, so
     // every pass starts 16-byte aligned).  Row groups per workgroup as the register file allows:
-    // three with two blocks, two with three, one with four.  K11008 N4096 m=32 / 64 / 128:
+    // two with two or three blocks, one with four.  K11008 N4096 m=32 / 64 / 128:
     // 28.5 / 55.1 / 112 us in passes of sixteen rows -> 19.0 / 26.4 / 53.
     const int rg = regstream_row_groups(n);
     for (int r0 = 0; r0 < m; r0 += 64) {
@@ -805,8 +805,9 @@ hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, co
                              0, stream, o, l, rhs, scales, mb, p, n, beta);
         e = hipGetLastError();
       } else if (mb <= 32) {
-        e = rg == 3 ? launch_blocks<3, 2>(stream, o, l, rhs, scales, mb, p, n, beta)
-          : rg == 2 ? launch_blocks<2, 2>(stream, o, l, rhs, scales, mb, p, n, beta)
+        // (three row groups with two blocks spill four registers and are no faster: K5120 N13824
+        // m=32 29.8-31.7 against 29.7-30.1 us)
+        e = rg >= 2 ? launch_blocks<2, 2>(stream, o, l, rhs, scales, mb, p, n, beta)
                     : launch_blocks<1, 2>(stream, o, l, rhs, scales, mb, p, n, beta);
       } else if (mb <= 48) {
         e = rg >= 2 ? launch_blocks<2, 3>(stream, o, l, rhs, scales, mb, p, n, beta)
