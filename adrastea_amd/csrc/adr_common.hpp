@@ -260,7 +260,7 @@ DeviceInfo device_info_for_plan();  // as above, but an MI355X where no usable d
 // dispatch would make by itself from the arguments.  0 = the dispatch decides.
 enum Knob {
   KNOB_GEMM_TILE = 0,  // fp16 tiled GEMM: 1 + index into the tile list (gemm_mfma.hip: forced tile)
-  KNOB_LAB_A,          // (free for lab builds)
+  KNOB_U8_TILE,        // u8-weight tiled GEMM: 1 + index into its tile list; one past the list: the staged kernels
   KNOB_LAB_B,
   KNOB_LAB_C,
   KNOB_COUNT

@@ -510,17 +510,14 @@ int adr_matmul_nt_f16(adr_stream_t stream, uint16_t* output, const uint16_t* lhs
 }
 
 // Where dequantising the matrix once and running the fp16 kernels beats the fused kernels
-// (measured over M 33 .. 4096 on N 4096 / 8192 / 12288, K 4096 and 11008): always on narrow
-// matrices, and on wide ones except where one round of the fused 256-row tiles covers the product
-// (N12288: M512 72 against 81 us, M1024 112 against 120; N8192: M768 72 against 75).
+// (measured over M 64 .. 4096 on (K, N) of the LLaMA-7B and 13B layers): from 768 rows on.  Below,
+// the fused kernel's small tiles are 5-80 % ahead (K11008 N4096 M512 73 against 84 us, M256 46
+// against 63; K4096 N12288 M128 31 against 50); at 768 and 1024 rows the two are within 5 % of each
+// other either way; from 1536 rows on the fused kernel dequantises every weight six times and more
+// and is 6-25 % behind (K4096 N12288 M2048 218 against 185 us).
 static bool u8_dequantise_first(int m, int p, int n) {
-  // To 95 rows the streaming kernels, which read the bytes once per 64 rows, stay ahead; to 159
-  // rows they still do on narrow matrices (K11008 N4096 M128 53 against 62 us, K4096 N4096 26
-  // against 28) but not on wide ones (K4096 N12288 M96 54 against 49, N8192 M128 46 against 37).
-  if (m < 96 || p == 0) return false;
-  if (m < 160) return n >= 8192;
-  if (m <= 256 || m >= 1536) return true;
-  return m <= 512 ? n <= 10240 : n < 8192;
+  (void)n;
+  return m >= 768 && p > 0;
 }
 
 static int validate_u8(const uint16_t* output, const uint16_t* lhs, const uint8_t* rhs,

@@ -1424,11 +1424,11 @@ __global__ __launch_bounds__(SHORTK_THREADS, 1) void gemm_nt_shortk_kernel(Matmu
 // dequantised once per workgroup and the MFMA loop is the one of the fp16 kernel.
 // MI16: 16x16x32 MFMAs, two k-steps per slice, all chunks dequantised in the first (the 256 x 128
 // tile: 5-6 % faster; the 256 x 192 tile has no registers for the second set of fragments)
-template <int BM, int BN, int WM, int WN, bool MI16>
-__global__ __launch_bounds__(WM* WN * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a, TileMap map,
-                                                                   int block_shift) {
-  constexpr int BK = 64, CPR = 8, MI = MI16 ? 16 : 32, KG = 64 / MI, KK = CPR / KG;
-  constexpr int NW = WM * WN, NT = NW * 64;
+template <int BM, int BN, int WM, int WN, bool MI16, int BK = 64, int G = 1>
+__global__ __launch_bounds__(WM* WN* G * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a, TileMap map,
+                                                                      int block_shift) {
+  constexpr int CPR = BK / 8, MI = MI16 ? 16 : 32, KG = 64 / MI, KK = CPR / KG;
+  constexpr int NW = WM * WN, NT = NW * 64;  // wavefronts and lanes of one group
   constexpr int IA = BM * CPR / NT;   // DMA instructions per lane and slice
   constexpr int LB = BN * CPR / NT;   // 8-weight chunks per lane and slice
   constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
@@ -1436,18 +1436,31 @@ __global__ __launch_bounds__(WM* WN * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a
   constexpr int FSTEP = MI * CPR * 16;         // bytes between the fragments of consecutive blocks
   constexpr int SLOT = 32 * (TN * 64 + 16);
   static_assert(BM * CPR % NT == 0 && BN * CPR % NT == 0, "slices must split evenly over lanes");
-  static_assert((NW / 2) * SLOT <= BM * BK * 2, "epilogue slots must fit in two A stages");
-  static_assert(MI16 ? LB <= 3 : LB < KK, "no chunk is dequantised in the last k-step");
-  __shared__ __attribute__((aligned(1024))) unsigned char sA0[BM * BK * 2];
-  __shared__ __attribute__((aligned(1024))) unsigned char sA1[BM * BK * 2];
-  __shared__ __attribute__((aligned(1024))) unsigned char sA2[BM * BK * 2];
-  __shared__ __attribute__((aligned(1024))) unsigned char sB0[BN * BK * 2];
-  __shared__ __attribute__((aligned(1024))) unsigned char sB1[BN * BK * 2];
+  // epilogue slots lie in the stages of the operand with the larger ones, per stage half the
+  // wavefronts where they fit (the 256-row tiles), else as many as fit
+  constexpr bool SLOTS_IN_B = BN > BM;
+  constexpr int SLOT_STAGE = (SLOTS_IN_B ? BN : BM) * BK * 2;
+  constexpr int SLOTS = (NW / 2) * SLOT <= SLOT_STAGE ? NW / 2 : SLOT_STAGE / SLOT;
+  static_assert(SLOTS >= 1 && (NW + SLOTS - 1) / SLOTS <= (SLOTS_IN_B ? 2 : 3),
+                "epilogue slots must fit in the stages");
+  static_assert(MI16 ? LB <= 8 && FM * FN % LB == 0 : LB < KK, "no chunk is dequantised in the last k-step");
+  __shared__ __attribute__((aligned(1024))) unsigned char sA0[G * BM * BK * 2];
+  __shared__ __attribute__((aligned(1024))) unsigned char sA1[G * BM * BK * 2];
+  __shared__ __attribute__((aligned(1024))) unsigned char sA2[G * BM * BK * 2];
+  __shared__ __attribute__((aligned(1024))) unsigned char sB0[G * BN * BK * 2];
+  __shared__ __attribute__((aligned(1024))) unsigned char sB1[G * BN * BK * 2];
 
   int batch, tile_m, tile_n;
   map_tile(map, batch, tile_m, tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
-  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // G groups of NW wavefronts: every group multiplies the whole tile over its own slices of K
+  // (slice s of the tile's walk is the G slices s*G .. s*G+G-1 of K, one per group, in stages of
+  // its own), all groups pass the same barriers, and their sums meet in LDS behind the loop
+  const int lane = threadIdx.x & 63;
+  const int wave_all = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int grp = G > 1 ? wave_all / NW : 0, wave = G > 1 ? wave_all % NW : wave_all;
+  const int tid = wave * 64 + lane;
+  const int goA = grp * (BM * BK * 2), goB = grp * (BN * BK * 2);
   const int wm = wave / WN, wn = wave % WN;
   half_t* const out = a.output;
 
@@ -1467,20 +1480,20 @@ __global__ __launch_bounds__(WM* WN * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a
     const int c = tid + i * NT, row = c / CPR, kc = c % CPR;
     const int brow = min(n0 + row, a.n - 1);
     gQ[i] = a.rhs_q + (int64_t)brow * a.k + kc * 8;
-    // block of weight k0 + 8*kc: k0 is a multiple of 64 and 8*kc < 64, so the two parts of the
+    // block of weight k0 + 8*kc: k0 is a multiple of BK and 8*kc < BK, so the two parts of the
     // index add up exactly for any power-of-two block size
     gS[i] = a.scales + (int64_t)brow * (a.k >> block_shift) + ((kc * 8) >> block_shift);
     offB[i] = lds_chunk_off<CPR>(row, kc);
   }
-  const int KT = a.k / BK;
+  const int KT = a.k / (BK * G);
   int kloadA = 0, kloadQ = 0;
   auto dmaA = [&](unsigned char* dA) {
-    const int k0 = min(kloadA, KT - 1) * BK;
+    const int k0 = (min(kloadA, KT - 1) * G + grp) * BK;
     kloadA++;
 #pragma unroll
     for (int i = 0; i < IA; i++)
       __builtin_amdgcn_global_load_lds(ADR_GLB_PTR(gA[i] + k0),
-                                       ADR_LDS_PTR(dA + (i * NW + wave) * 1024), 16, 0, 0);
+                                       ADR_LDS_PTR(dA + goA + (i * NW + wave) * 1024), 16, 0, 0);
   };
   // three register sets: the weights consumed in slice kt+1 were requested at the head of slice
   // kt-1, so the wait at the end of slice kt-1 (everything but that slice's own requests)
@@ -1488,7 +1501,7 @@ __global__ __launch_bounds__(WM* WN * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a
   u32x2_t rq[3][LB];
   half_t rs[3][LB];
   auto fetchQ = [&](int set) {
-    const int ks = min(kloadQ, KT - 1);
+    const int ks = min(kloadQ, KT - 1) * G + grp;
     kloadQ++;
 #pragma unroll
     for (int i = 0; i < LB; i++) {
@@ -1498,7 +1511,7 @@ __global__ __launch_bounds__(WM* WN * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a
   };
   auto dequant_store1 = [&](int set, unsigned char* dB, int i) {
     const half2_t s2 = {rs[set][i], rs[set][i]};
-    *(half8_t*)(dB + offB[i]) = dequant8(rq[set][i][0], rq[set][i][1], s2);
+    *(half8_t*)(dB + goB + offB[i]) = dequant8(rq[set][i][0], rq[set][i][1], s2);
   };
   auto dequant_store = [&](int set, unsigned char* dB) {
 #pragma unroll
@@ -1525,9 +1538,9 @@ __global__ __launch_bounds__(WM* WN * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a
   half8_t fa[2][FM], fb[2][FN];
   auto load_frags = [&](int slot, const unsigned char* cA, const unsigned char* cB, int kk) {
 #pragma unroll
-    for (int i = 0; i < FM; i++) fa[slot][i] = *(const half8_t*)(cA + offFA[kk] + i * FSTEP);
+    for (int i = 0; i < FM; i++) fa[slot][i] = *(const half8_t*)(cA + goA + offFA[kk] + i * FSTEP);
 #pragma unroll
-    for (int j = 0; j < FN; j++) fb[slot][j] = *(const half8_t*)(cB + offFB[kk] + j * FSTEP);
+    for (int j = 0; j < FN; j++) fb[slot][j] = *(const half8_t*)(cB + goB + offFB[kk] + j * FSTEP);
   };
   auto mfmas = [&](int slot) {
 #pragma unroll
@@ -1612,7 +1625,38 @@ __global__ __launch_bounds__(WM* WN * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a
   __builtin_amdgcn_s_waitcnt(0x0070);
   __builtin_amdgcn_s_barrier();
 
-  unsigned char* slot = (wave < NW / 2 ? sA0 : sA1) + (wave % (NW / 2)) * SLOT;
+  if constexpr (G > 1) {
+    // the groups' sums, group by group in group order, through the first A stage: a lane's
+    // accumulator registers four at a time (a wavefront's four registers are 1 KiB)
+    constexpr int AR = MI16 ? 4 : 16, QUADS = FM * FN * AR / 4;
+    constexpr int PIECE = QUADS * NW * 1024 <= G * BM * BK * 2 ? QUADS : G * BM * BK * 2 / (NW * 1024);
+    static_assert(PIECE >= 1 && QUADS % PIECE == 0, "the sums pass through the first A stage in equal pieces");
+    float4_t* const red = (float4_t*)sA0 + (wave * PIECE) * 64 + lane;
+    auto quad = [&](int q) -> float4_t& {  // quad q of the lane's accumulators
+      constexpr int PER = AR / 4;
+      return *((float4_t*)&acc[q / PER / FN][q / PER % FN] + q % PER);
+    };
+    for (int g = 1; g < G; g++) {
+#pragma unroll
+      for (int p0 = 0; p0 < QUADS; p0 += PIECE) {
+        if (grp == g) {
+#pragma unroll
+          for (int q = 0; q < PIECE; q++) red[q * 64] = quad(p0 + q);
+        }
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        __builtin_amdgcn_s_barrier();
+        if (grp == 0) {
+#pragma unroll
+          for (int q = 0; q < PIECE; q++) quad(p0 + q) += red[q * 64];
+        }
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        __builtin_amdgcn_s_barrier();
+      }
+    }
+    if (grp != 0) return;
+  }
+  unsigned char* slot = (SLOTS_IN_B ? (wave < SLOTS ? sB0 : sB1)
+                                    : (wave < SLOTS ? sA0 : wave < 2 * SLOTS ? sA1 : sA2)) + (wave % SLOTS) * SLOT;
   wave_epilogue<TM, 2 * TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, slot, (half_t)a.scale, lane);
 }
 
@@ -2008,12 +2052,12 @@ hipError_t launch_stage(hipStream_t stream, const MatmulArgs& a) {
   return hipGetLastError();
 }
 
-template <int BM, int BN, int WM, int WN, bool MI16>
+template <int BM, int BN, int WM, int WN, bool MI16, int BK = 64, int G = 1>
 hipError_t launch_u8(hipStream_t stream, const MatmulArgs& a) {
   TileMap map = make_map(a, BM, BN);
-  if (map.total < 0) return hipErrorInvalidConfiguration;
-  hipLaunchKernelGGL((gemm_nt_u8_kernel<BM, BN, WM, WN, MI16>), dim3((unsigned)map.total),
-                     dim3(WM * WN * 64), 0, stream, a, map, __builtin_ctz(a.block_size));
+  if (map.total < 0 || a.k % (BK * G) != 0) return hipErrorInvalidConfiguration;
+  hipLaunchKernelGGL((gemm_nt_u8_kernel<BM, BN, WM, WN, MI16, BK, G>), dim3((unsigned)map.total),
+                     dim3(WM * WN * G * 64), 0, stream, a, map, __builtin_ctz(a.block_size));
   return hipGetLastError();
 }
 
@@ -2061,7 +2105,7 @@ hipError_t launch_shortk(hipStream_t stream, const MatmulArgs& a) {
 enum GemmChoice {
   GEMM_NONE = 0,
   SHORTK_64, SHORTK_128,
-  U8_256x192, U8_256x128,
+  U8_256x192, U8_256x128, U8_128x128, U8_128x64, U8_64x64, U8_128x64_G2, U8_64x64_G4,
   DMA_256x192, DMA_256x160, DMA_256x128, DMA_128x256, DMA_128x192, DMA_128x128, DMA_128x64, DMA_64x64, DMA_64x64_K128, DMA_128x64_K128,
   DMA_NN_256x128, DMA_NN_128x128, NN_ANYROW_128x128, NN_ANYROW_128x64,
   STAGE_256x128, STAGE_128x128, STAGE_64x64,
@@ -2106,6 +2150,29 @@ const Candidate DMA_TILES[] = {
     {DMA_128x256, 128, 256, 1, 1.13f}, {DMA_128x192, 128, 192, 1, 0.85f}, {DMA_128x128, 128, 128, 2, 0.80f}, {DMA_128x64, 128, 64, 2, 0.60f},
     {DMA_64x64, 64, 64, 4, 0.40f}, {DMA_256x160, 256, 160, 1, 1.19f}};
 constexpr int N_DMA_TILES = sizeof(DMA_TILES) / sizeof(DMA_TILES[0]);
+
+// The tiles of the u8-weight kernel.  One tile per CU, time per tile at K 11008 / K 4096 in us:
+// 256x192 195 / 78, 256x128 140 / 56, 128x128 97 / 41, 128x64 68 / 30 (two K groups; one: 73 / 32),
+// 64x64 47 / 22 (four K groups; one: 58 / 25).  The two smallest tiles are bound by what the L2s
+// deliver to all CUs together (M256 K11008 N4096 on 64x64: 540 MB in 47 us), the larger ones by
+// the path into one CU.  Over M 128..1536 x (K, N) of the LLaMA-7B and 13B layers the choice by
+// these constants is the fastest forced tile or within 5 % of it.
+const Candidate U8_TILES[] = {{U8_256x192, 256, 192, 1, 1.10f}, {U8_256x128, 256, 128, 1, 1.05f},
+                              {U8_128x128, 128, 128, 1, 0.74f}, {U8_128x64, 128, 64, 2, 0.52f},
+                              {U8_64x64, 64, 64, 4, 0.37f}};
+constexpr int N_U8_TILES = sizeof(U8_TILES) / sizeof(U8_TILES[0]);
+
+// With at most one tile per CU the two small tiles split K over groups of wavefronts inside the
+// workgroup (more slices in flight per CU; with more tiles than CUs several workgroups per CU do
+// the same).
+GemmChoice u8_k_groups(const MatmulArgs& a, GemmChoice c) {
+  const int bm = c == U8_128x64 ? 128 : 64;
+  const int64_t tiles = (int64_t)((a.m + bm - 1) / bm) * ((a.n + 63) / 64);
+  if (tiles > num_cu()) return c;
+  if (c == U8_128x64 && a.k % 128 == 0) return U8_128x64_G2;
+  if (c == U8_64x64 && a.k % 256 == 0) return U8_64x64_G4;
+  return c;
+}
 
 // The MFMA family needs 16-byte aligned, K-contiguous rows on both operands.
 GemmChoice choose(const MatmulArgs& a) {
@@ -2172,14 +2239,14 @@ GemmChoice choose(const MatmulArgs& a) {
     // instead of 128 x 128 is within +-4 % up to K 512 and 4-12 % behind above.)
     return c;
   }
-  if (a.rhs_q && a.k % 64 == 0 && a.block_size >= 8 && (a.block_size & (a.block_size - 1)) == 0 &&
-      (int64_t)a.m * a.n >= 256 * 1024 &&
-      // (with at most 64 of its 256 x 128 tiles the staged kernels' smaller tiles reach more CUs:
-      // N4096 m=129..512, K4096 59..65 -> 43..50 us, K11008 171..187 -> 129..141; with 96 tiles and
-      // more, N12288, they lose: 69..76 -> 91..126)
-      (int64_t)((a.m + 255) / 256) * ((a.n + 127) / 128) > 64) {
-    static const Candidate u8[] = {{U8_256x192, 256, 192, 1, 1.10f}, {U8_256x128, 256, 128, 1, 1.05f}};
-    return pick(a, u8, 2);
+  if (a.rhs_q && a.k % 64 == 0 && a.block_size >= 8 && (a.block_size & (a.block_size - 1)) == 0) {
+    // (tests and benchmarks can force a tile: adr_debug_knob; 1 + N_U8_TILES: 128 x 64 with two K
+    // groups, 2 + N_U8_TILES: 64 x 64 with four, 3 + N_U8_TILES: the staged kernels below)
+    const int forced = knob(KNOB_U8_TILE);
+    if (forced >= 1 && forced <= N_U8_TILES) return U8_TILES[forced - 1].id;
+    if (forced == N_U8_TILES + 1) return a.k % 128 == 0 ? U8_128x64_G2 : U8_128x64;
+    if (forced == N_U8_TILES + 2) return a.k % 256 == 0 ? U8_64x64_G4 : U8_64x64;
+    if (forced != N_U8_TILES + 3) return u8_k_groups(a, pick(a, U8_TILES, N_U8_TILES));
   }
   static const Candidate stage[] = {{STAGE_256x128, 256, 128, 2, 1.00f},
                                     {STAGE_128x128, 128, 128, 2, 0.85f},
@@ -2265,6 +2332,11 @@ static bool choice_name(GemmChoice c, const char** name, bool u8 = false) {
     case SHORTK_128: *name = "gemm_nt_mfma_persistent_128x128_k128"; return true;
     case U8_256x192: *name = "gemm_nt_u8_mfma_256x192x64"; return true;
     case U8_256x128: *name = "gemm_nt_u8_mfma_256x128x64"; return true;
+    case U8_128x128: *name = "gemm_nt_u8_mfma_128x128x64"; return true;
+    case U8_128x64: *name = "gemm_nt_u8_mfma_128x64x64"; return true;
+    case U8_64x64: *name = "gemm_nt_u8_mfma_64x64x64"; return true;
+    case U8_128x64_G2: *name = "gemm_nt_u8_mfma_128x64x64_k2"; return true;
+    case U8_64x64_G4: *name = "gemm_nt_u8_mfma_64x64x64_k4"; return true;
     case DMA_256x192: *name = "gemm_nt_mfma_dma_256x192x64"; return true;
     case DMA_256x160: *name = "gemm_nt_mfma_dma_256x160x64"; return true;
     case DMA_256x128: *name = "gemm_nt_mfma_dma_256x128x64"; return true;
@@ -2292,6 +2364,11 @@ static hipError_t launch_choice(hipStream_t stream, const MatmulArgs& a, GemmCho
     case SHORTK_128: return launch_shortk<16>(stream, a);
     case U8_256x192: return launch_u8<256, 192, 4, 2, false>(stream, a);
     case U8_256x128: return launch_u8<256, 128, 4, 2, true>(stream, a);
+    case U8_128x128: return launch_u8<128, 128, 4, 2, true>(stream, a);
+    case U8_128x64: return launch_u8<128, 64, 2, 2, true>(stream, a);
+    case U8_64x64: return launch_u8<64, 64, 2, 2, true>(stream, a);
+    case U8_128x64_G2: return launch_u8<128, 64, 2, 2, true, 64, 2>(stream, a);
+    case U8_64x64_G4: return launch_u8<64, 64, 2, 2, true, 64, 4>(stream, a);
     case DMA_256x192: return launch_dma<256, 192, 4, 2, 6, 1, false, 64, true>(stream, a);
     case DMA_256x160: return launch_dma<256, 160, 4, 2, 6, 1, false, 64, true>(stream, a);
     case DMA_256x128: return launch_dma<256, 128, 4, 2, 7, 1, false, 64, true>(stream, a);
@@ -2422,6 +2499,17 @@ const char* gemm_u8_mfma_plan(int m, int p, int n, int block_size) {
   const MatmulArgs a = u8_args(nullptr, nullptr, (const uint8_t*)16, nullptr, m, p, n, block_size, 0.0f);
   const char* name = nullptr;
   return choice_name(choose(a), &name, true) ? name : nullptr;
+}
+
+// Estimated time of the u8 product on the tiled u8 kernel, in us (negative: that kernel does not
+// cover it): pick()'s cost of the chosen tile times K.  4 us + 3.5e-7 us per unit fits one tile per
+// CU of 64 x 64 (K11008 47 us, K4096 21) and of 128 x 64 (68, 30).
+double gemm_u8_mfma_estimate_us(int m, int p, int n, int block_size) {
+  const MatmulArgs a = u8_args(nullptr, nullptr, (const uint8_t*)16, nullptr, m, p, n, block_size, 0.0f);
+  if (!(p % 64 == 0 && block_size >= 8 && (block_size & (block_size - 1)) == 0)) return -1.0;
+  double cost;
+  pick(a, U8_TILES, N_U8_TILES, &cost);
+  return 4.0 + cost * p * 3.5e-7;
 }
 
 bool gemm_u8_mfma_supported(const half_t* lhs, const uint8_t* rhs, const half_t* scales, int m, int p,

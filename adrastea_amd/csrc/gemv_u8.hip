@@ -35,6 +35,9 @@
 
 namespace adr {
 
+// (gemm_mfma.hip) estimated time of the product on the tiled u8 kernel, us; negative: not covered
+double gemm_u8_mfma_estimate_us(int m, int p, int n, int block_size);
+
 namespace {
 
 constexpr int MACRO_K = 256;  // k elements per macro step
@@ -722,27 +725,26 @@ U8Choice choose_u8(const void* lhs, const void* rhs, const void* scales, int m, 
 }
 
 // 17 activation rows and more against at least 4 MiB of weights: passes of up to 64 rows on the
-// matrix-core streaming kernels, each pass reading the weights once.  The tiled GEMM walks K on
-// N / 64 .. N / 128 CUs for these row counts, which takes about 10 + 0.0105 K us whatever the
-// rows (K4096 N4096 m=65..256: 49.6 .. 52.3 us, K11008 N4096 127 .. 132, K512 N9000 15.4; ten more
-// on N 12288).  A pass of 64 rows is one workgroup per sixteen weight rows, 2 + 0.0023 K us per
-// round of them over the CUs (K4096 N4096 13.1 us, N8192 23.5, N12288 33.9, K11008 N4096 26.4,
-// K5120 N5120 25.7); a last pass of r rows costs 0.55 + 0.45 r / 64 of that.  Up to 64 rows the
-// passes always win; above, where this estimate says so (measured: K4096 N4096 to 256 rows,
-// 25.7 us at m=128 against 49.6; K11008 N4096 m=256 105 against 132; K4096 N12288 to 96 rows, 54
-// against 63; K4096 N8192 and K5120 N5120 to 128, 46 against 53 and 51 against 64).
+// matrix-core streaming kernels, each pass reading the weights once.  A pass of 64 rows is one
+// workgroup per sixteen weight rows, 2 + 0.0023 K us per round of them over the CUs (K4096 N4096
+// 13.1 us, N8192 23.5, N12288 33.9, K11008 N4096 26.4, K5120 N5120 25.7); a last pass of r rows
+// costs 0.55 + 0.45 r / 64 of that.  Up to 64 rows the passes always win (the tiled kernel has
+// N / 64 tiles for them: K11008 N4096 43 us); above, where this estimate is below the tiled
+// kernel's own: K11008 N4096 m=70 41 against 44 us (m=128: 54 against 44, tiled), K4096 N4096
+// m=70 20.6 against 20.2, m=128 25 against 19; K5120 N5120 and K13824 N5120 are tiled from 65 rows.
 bool rows_in_passes(int m, int p, int n, int block_size) {
   if (m <= 16 || m > 256 || (int64_t)n * p < (1 << 22) ||
       choose_u8(nullptr, nullptr, nullptr, 16, p, n, block_size) != U8_GEMV)
     return false;
   if (m <= 64) return true;
+  if (knob(KNOB_U8_TILE)) return false;  // (a test or benchmark forces a tile of the tiled kernel)
   const int cus = device_info_for_plan().cus;
   const int rounds = ((n + ROWS - 1) / ROWS + cus - 1) / cus;
   const double t64 = fmax(12.0, rounds * (2.0 + 0.0023 * p));
   const int rem = m % 64;
   const double passes = (m / 64) * t64 + (rem ? t64 * (0.55 + 0.45 * rem / 64.0) : 0.0);
-  const double tiled = 10.0 + 0.0105 * p + (n > 10240 ? 10.0 : 0.0);
-  return passes < tiled;
+  const double tiled = gemm_u8_mfma_estimate_us(m, p, n, block_size);
+  return tiled < 0.0 || passes < tiled;
 }
 
 }  // namespace

@@ -84,19 +84,26 @@ def test_u8_plan():
     assert plan(32, 4096, 12288, 32) == (0, "gemv_u8_mfma16_dma_32rows")
     assert plan(32, 11008, 4096, 32) == (0, "gemv_u8_mfma16_blocks")
     assert plan(64, 4096, 12288, 32) == (0, "gemv_u8_mfma16_blocks")
-    # above 64 rows: passes of 64 rows where the estimate puts them ahead of the tiled kernels
-    assert plan(256, 11008, 4096, 32) == (0, "gemv_u8_mfma16_blocks")
-    assert plan(96, 4096, 12288, 32) == (0, "gemv_u8_mfma16_blocks")
-    assert plan(128, 4096, 12288, 32)[1].startswith("gemm_nt_u8_")
-    assert plan(100, 512, 9000, 32)[1].startswith("gemm_nt_u8_")
-    assert plan(257, 11008, 4096, 32)[1].startswith("gemm_nt_u8_")
-    # tiled kernels: the name carries the tile
+    # above 64 rows: passes of 64 rows where the estimate puts them ahead of the tiled kernel (a
+    # few rows past 64 against a narrow matrix)
+    assert plan(70, 11008, 4096, 32) == (0, "gemv_u8_mfma16_blocks")
+    assert plan(70, 4096, 4096, 32) == (0, "gemv_u8_mfma16_blocks")
+    assert plan(128, 11008, 4096, 32) == (0, "gemm_nt_u8_mfma_64x64x64_k4")
+    assert plan(256, 11008, 4096, 32) == (0, "gemm_nt_u8_mfma_64x64x64_k4")
+    assert plan(96, 4096, 12288, 32) == (0, "gemm_nt_u8_mfma_128x64x64_k2")
+    assert plan(100, 512, 9000, 32)[1].startswith("gemm_nt_u8_mfma_")
+    # tiled kernel: the name carries the tile, and the K groups of the two small ones where
+    # there is at most one tile per compute unit
     assert plan(2048, 4096, 4096, 32) == (0, "gemm_nt_u8_mfma_256x128x64")
     assert plan(2048, 4096, 12288, 32) == (0, "gemm_nt_u8_mfma_256x192x64")
     assert plan(2048, 4096, 11008, 32) == (0, "gemm_nt_u8_mfma_256x192x64")
     assert plan(2048, 11008, 4096, 32) == (0, "gemm_nt_u8_mfma_256x128x64")
-    assert plan(300, 4096, 4096, 32)[1].startswith("gemm_nt_u8_stage_")
-    assert plan(8, 4096, 4096, 64)[1].startswith("gemm_nt_u8_stage_")
+    assert plan(1024, 11008, 4096, 32) == (0, "gemm_nt_u8_mfma_128x128x64")
+    assert plan(300, 4096, 4096, 32) == (0, "gemm_nt_u8_mfma_128x64x64_k2")
+    assert plan(300, 4096 + 64, 4096, 32) == (0, "gemm_nt_u8_mfma_128x64x64")      # K % 128 != 0: one group
+    assert plan(600, 4096, 4096, 32)[1] in ("gemm_nt_u8_mfma_128x64x64", "gemm_nt_u8_mfma_128x128x64")
+    assert plan(8, 4096, 4096, 64) == (0, "gemm_nt_u8_mfma_64x64x64_k4")
+    assert plan(300, 4096 + 32, 4096, 32)[1].startswith("gemm_nt_u8_stage_")        # K % 64 != 0
     assert plan(8, 36, 64, 12) == (0, "gemm_u8_naive")
     assert plan(4, 4100, 64, 32)[0] == _ffi.ADR_EDIVISIBILITY
     assert plan(4, 64, 64, 0)[0] == _ffi.ADR_EINVAL_SHAPE
@@ -181,19 +188,16 @@ def test_workspace_plan_and_size():
 
 
 def test_u8_workspace_size_and_validation():
-    """adr_matmul_nt_fp16u8_ws dequantises the matrix first from 96 rows on (160 on narrow matrices; not where one round
-    of the fused kernel's tiles covers a wide product); the size query says when, and how much."""
+    """adr_matmul_nt_fp16u8_ws dequantises the matrix first from 768 rows on (below, the fused kernel's small tiles are
+    ahead); the size query says when, and how much."""
     lib = _ffi.lib()
     need = lib.adr_matmul_nt_fp16u8_workspace_bytes
     assert need(2048, 4096, 12288, 32) == 12288 * 4096 * 2
-    assert need(512, 11008, 4096, 32) == 4096 * 11008 * 2
+    assert need(768, 11008, 4096, 32) == 4096 * 11008 * 2
     assert need(1024, 4096, 4096, 32) == 4096 * 4096 * 2
-    assert need(1024, 4096, 12288, 32) == 0        # the fused 256-row tiles are ahead here
-    assert need(512, 4096, 12288, 32) == 0 and need(512, 4096, 8192, 32) == 8192 * 4096 * 2
-    assert need(1024, 4096, 8192, 32) == 0 and need(256, 4096, 12288, 32) == 12288 * 4096 * 2
-    assert need(95, 4096, 12288, 32) == 0 and need(1, 4096, 12288, 32) == 0
-    assert need(96, 4096, 12288, 32) == 12288 * 4096 * 2 and need(128, 4096, 8192, 32) == 8192 * 4096 * 2
-    assert need(159, 11008, 4096, 32) == 0 and need(160, 11008, 4096, 32) == 4096 * 11008 * 2
+    assert need(1024, 4096, 12288, 32) == 12288 * 4096 * 2
+    assert need(767, 4096, 12288, 32) == 0 and need(512, 11008, 4096, 32) == 0
+    assert need(256, 4096, 12288, 32) == 0 and need(1, 4096, 12288, 32) == 0
     assert need(2048, 0, 64, 32) == 0
     assert need(-1, 64, 64, 32) == _ffi.ADR_EINVAL_SHAPE
     assert need(256, 100, 64, 32) == _ffi.ADR_EDIVISIBILITY

@@ -175,7 +175,7 @@ def test_u8_products_by_way_of_the_held_workspace(held_on):
     g = rng(10)
     main = torch.cuda.current_stream().cuda_stream
     # the default: the fused kernels whatever the pool would allow, nothing allocated
-    m, p, n, bs = 300, 4096, 4096, 32
+    m, p, n, bs = 800, 4096, 4096, 32
     q = torch.from_numpy(g.integers(0, 256, size=(n, p), dtype=np.uint8)).cuda()
     sc = torch.from_numpy((g.random((n, p // bs)) * 0.019 + 0.001).astype(np.float16)).cuda()
     x = torch.from_numpy(randn_f16(g, (m, p))).cuda()
@@ -194,8 +194,8 @@ def test_u8_products_by_way_of_the_held_workspace(held_on):
     # on request: the matrix dequantised once into a buffer of the pool
     assert lib.adr_set_u8_dequantise_first(1) == 0 and lib.adr_u8_dequantise_first() == 1
     assert lib.adr_matmul_nt_fp16u8_plan(name, 96, m, p, n, bs) == 0 and name.value == b"dequantize_absmax_u8 + fp16 gemm"
-    for m, p, n, bs in [(300, 4096, 4096, 32), (2048, 4096, 4096, 32), (128, 4096, 8192, 32), (1100, 1024, 5120, 64),
-                        (256, 11008, 4096, 32)]:
+    for m, p, n, bs in [(800, 4096, 4096, 32), (2048, 4096, 4096, 32), (768, 4096, 8192, 32), (1100, 1024, 5120, 64),
+                        (1000, 11008, 4096, 32)]:
         need = lib.adr_matmul_nt_fp16u8_workspace_bytes(m, p, n, bs)
         assert need == n * p * 2
         q = torch.from_numpy(g.integers(0, 256, size=(n, p), dtype=np.uint8)).cuda()
@@ -227,7 +227,7 @@ def test_u8_products_by_way_of_the_held_workspace(held_on):
     lib.adr_set_held_workspace_limit(8 * MIB)
     before = lib.adr_held_workspace_bytes()
     s = torch.cuda.Stream()
-    m, p, n, bs = 300, 4096, 4096, 32
+    m, p, n, bs = 800, 4096, 4096, 32
     q = torch.from_numpy(g.integers(0, 256, size=(n, p), dtype=np.uint8)).cuda()
     sc = torch.from_numpy((g.random((n, p // bs)) * 0.019 + 0.001).astype(np.float16)).cuda()
     x = torch.from_numpy(randn_f16(g, (m, p))).cuda()

@@ -142,16 +142,38 @@ def test_fused_dequant_in_gemv_is_bit_exact_for_every_q_and_finite_scale(kern, m
         assert np.all((got[z] & 0x7FFF) == 0)
 
 
-@pytest.mark.parametrize("tile", ["256x128", "256x192"])
-def test_fused_dequant_in_u8_gemm_is_bit_exact_for_every_q_and_finite_scale(kern, tile):
+# the tiles of the u8 kernel in the order of adr_debug_knob(1, 1 + i); "_k2" / "_k4": K split over
+# two / four groups of wavefronts inside the workgroup
+U8_TILES = ["256x192x64", "256x128x64", "128x128x64", "128x64x64", "64x64x64", "128x64x64_k2", "64x64x64_k4"]
+U8_STAGED = len(U8_TILES) + 1   # knob value: the register-staged kernels
+
+
+@pytest.fixture
+def force_u8_tile():
+    """force_u8_tile(name) makes the tiled u8 kernel run that tile until the test ends."""
+    lib = _ffi.lib()
+
+    def force(tile):
+        assert lib.adr_debug_knob(1, U8_STAGED if tile == "staged" else 1 + U8_TILES.index(tile)) == 0
+    yield force
+    assert lib.adr_debug_knob(1, 0) == 0
+
+
+@pytest.mark.parametrize("tile", ["256x128x64", "256x192x64", "128x128x64", "128x64x64", "64x64x64", "128x64x64_k2",
+                                  "64x64x64_k4"])
+def test_fused_dequant_in_u8_gemm_is_bit_exact_for_every_q_and_finite_scale(kern, tile, force_u8_tile):
     """One-hot rows extract every weight of the tiled u8 kernel: all 49154 finite scales make 385
     tiles of 256 x 128; the first 49152 of them exactly 256 tiles of 256 x 192 (the two scales
-    left out are covered by the other tile and by the stand-alone kernel)."""
+    left out are covered by the other tile and by the stand-alone kernel).  The smaller tiles are
+    forced on the same product."""
     scales_bits = _finite_scale_rows()
-    if tile == "256x192":
+    if tile == "256x192x64":
         scales_bits = scales_bits[:192 * 256]
     n, p, bs, m = scales_bits.size, 256, 32, 256
-    assert u8_plan(m, p, n, bs) == f"gemm_nt_u8_mfma_{tile}x64"
+    if tile in ("256x128x64", "256x192x64"):
+        assert u8_plan(m, p, n, bs) == f"gemm_nt_u8_mfma_{tile}"   # what the dispatch runs here
+    force_u8_tile(tile)
+    assert u8_plan(m, p, n, bs) == f"gemm_nt_u8_mfma_{tile}"
     q = np.tile(np.arange(256, dtype=np.uint8), (n, 1))
     s = np.repeat(scales_bits.view(np.float16).reshape(n, 1), p // bs, axis=1)
     lhs = np.eye(m, dtype=np.float16)
@@ -235,7 +257,7 @@ def test_blocks_kernel_bit_exact_on_exact_inputs(kern, m, pn):
     both operands, a second pass for rows 65 .. 70, beta path."""
     p, n = pn
     g = rng(1700 + m + p)
-    if m <= 64 or p != 768:    # (70 rows on K 768 x N 8200 are estimated faster on the tiled kernel)
+    if m <= 64 or p >= 4096:   # (70 rows on a short K are estimated faster on the tiled kernel)
         assert u8_plan(m, p, n, 32) in ("gemv_u8_mfma16_blocks", "gemv_u8_mfma16_dma_32rows")
     a, q, s = _u8_case(g, m, p, n, 32, exact=True)
     for beta in (0.0, 1.0):
@@ -276,13 +298,19 @@ def test_u8_matmul_random_matches_oracle_and_reference_kernel(kern, ref, m):
                                   (260, 320, 1100, 64), (1024, 384, 300, 128), (1024, 448, 300, 64), (256, 832, 1024, 32),
                                   (700, 768, 400, 256)],
                          ids=lambda c: "M%d_K%d_N%d_bs%d" % c)
-def test_u8_staged_kernels_ragged_tiles_and_k_tails_bit_exact(kern, case):
-    """Products with at most 64 tiles of 256 x 128 run on the register-staged kernels (dequantised
-    while staging): partial tiles in M and N, K slices of 32 and 64 with and without a tail, block
-    sizes below, at and above the slice depth, and the beta path -- exact inputs, compared bit for
-    bit.  (The DMA kernel's tiles: test_u8_dma_kernel_* below.)"""
+@pytest.mark.parametrize("route", ["staged", "dispatch"])
+def test_u8_small_products_ragged_tiles_and_k_tails_bit_exact(kern, case, route, force_u8_tile):
+    """Small u8 products on the register-staged kernels (dequantised while staging; what a K
+    that is no multiple of 64 runs on, forced here) and on the tile the dispatch picks for them
+    (the small tiles of the DMA kernel): partial tiles in M and N, K of one to thirteen slices,
+    block sizes below, at and above the slice depth, and the beta path -- exact inputs, compared
+    bit for bit.  (Every tile of the DMA kernel: test_u8_dma_kernel_* below.)"""
     m, p, n, bs = case
-    assert u8_plan(m, p, n, bs).startswith("gemm_nt_u8_stage_")
+    if route == "staged":
+        force_u8_tile("staged")
+        assert u8_plan(m, p, n, bs).startswith("gemm_nt_u8_stage_")
+    else:
+        assert u8_plan(m, p, n, bs).startswith("gemm_nt_u8_mfma_")
     g = rng(640 + m + p)
     a, q, s = _u8_case(g, m, p, n, bs, exact=True)
     for beta in (0.0, 1.0):
@@ -294,24 +322,35 @@ def test_u8_staged_kernels_ragged_tiles_and_k_tails_bit_exact(kern, case):
         assert np.array_equal(to_np(out).view(np.uint16), want.view(np.uint16)), (case, beta)
 
 
-@pytest.mark.parametrize("p", [320, 384, 448, 512, 576, 640, 1024])
-@pytest.mark.parametrize("tile_mn", [("256x192", 520, 11000), ("256x128", 520, 2900)],
-                         ids=lambda t: t[0])
-def test_u8_dma_kernel_ragged_tiles_and_every_k_remainder_bit_exact(kern, tile_mn, p):
-    """gemm_nt_u8_kernel<256,192> and <256,128> (more than 64 tiles of 256 x 128): a ragged last
-    tile row (520 = 2 x 256 + 8) and tile column, K / 64 = 5 .. 10 and 16 slices, i.e. every
-    remainder of the six-slice unrolled loop, beta 0 and 1, block sizes 32 and 64 -- exact inputs,
-    compared bit for bit.  Expected values: one rounding of the float64 product on the oracle's
-    dequantised weights (every sum is exactly representable), cross-checked with the oracle's
-    own matmul on the rows around the tile borders."""
+_DMA_TILE_CASES = [("256x192x64", 520, 11000), ("256x128x64", 520, 2900), ("128x128x64", 520, 2900),
+                   ("128x64x64", 520, 1900), ("64x64x64", 200, 1900), ("128x64x64_k2", 520, 1900),
+                   ("64x64x64_k4", 200, 1900)]
+# (K, tile): every tile on K of 5 .. 10 and 16 slices; the tiles that split K also on 20 .. 40
+_DMA_TILE_K = [(t, p) for t in _DMA_TILE_CASES
+               for p in [320, 384, 448, 512, 576, 640, 1024] +
+               ([1280, 1536, 1792, 2048, 2304, 2560] if t[0].endswith(("_k2", "_k4")) else [])]
+
+
+@pytest.mark.parametrize("tile_mn,p", _DMA_TILE_K, ids=[f"{t[0]}-K{p}" for t, p in _DMA_TILE_K])
+def test_u8_dma_kernel_ragged_tiles_and_every_k_remainder_bit_exact(kern, tile_mn, p, force_u8_tile):
+    """Every tile of gemm_nt_u8_kernel, forced: a ragged last tile row (520 = 2 x 256 + 8,
+    200 = 3 x 64 + 8) and tile column, K / 64 = 5 .. 10 slices and 16 .. 40 in steps of four, i.e.
+    every remainder of the six-slice unrolled loop also for the tiles that split K over two or
+    four groups of wavefronts (which walk K / 128 or K / 256 steps; a K they do not divide runs
+    the tile without groups), beta 0 and 1, block sizes 32 and 64 -- exact inputs, compared bit
+    for bit.  Expected values: one rounding of the float64 product on the oracle's dequantised
+    weights (every sum is exactly representable), cross-checked with the oracle's own matmul on
+    the rows around the tile borders."""
     tile, m, n = tile_mn
     bs = 64 if p % 128 == 0 else 32
-    assert u8_plan(m, p, n, bs) == f"gemm_nt_u8_mfma_{tile}x64"
+    force_u8_tile(tile)
+    groups = 4 if tile.endswith("_k4") else 2 if tile.endswith("_k2") else 1
+    assert u8_plan(m, p, n, bs) == "gemm_nt_u8_mfma_" + (tile if p % (64 * groups) == 0 else tile[:-3])
     g = rng(1640 + p + n)
     a, q, s = _u8_case(g, m, p, n, bs, exact=True)
     w64 = oracle.dequantize_absmax_u8(q, s, bs).astype(np.float64)
     prod = a.astype(np.float64) @ w64.T
-    rows = np.array([0, 1, 31, 32, 255, 256, 257, 511, 512, 519])
+    rows = np.array([r for r in (0, 1, 31, 32, 63, 64, 127, 128, 199, 255, 256, 257, 511, 512, 519) if r < m])
     a_t, q_t, s_t = to_dev(a), to_dev(q), to_dev(s)
     for beta in (0.0, 1.0):
         prev = (g.integers(-8, 9, size=(m, n)) / 4.0).astype(np.float16)
@@ -460,9 +499,10 @@ def test_seventeen_and_more_rows_in_passes(kern, kn, m):
         assert name == ("gemv_u8_mfma16_dma_32rows" if p == 4096 and m <= 32 else "gemv_u8_mfma16_blocks")
     else:
         assert name == "gemv_u8_mfma16_blocks" or name.startswith("gemm_nt_u8_")
-    # decisions the estimate must make: a long K keeps the passes to 256 rows, a matrix of three
-    # rounds of workgroups leaves them at 64
-    assert u8_plan(256, 11008, 1000, 32) == "gemv_u8_mfma16_blocks"
+    # decisions the estimate must make: a few rows past 64 against a narrow matrix stay in passes,
+    # more rows or a matrix of several rounds of workgroups go to the tiled kernel
+    assert u8_plan(70, 11008, 4096, 32) == "gemv_u8_mfma16_blocks"
+    assert u8_plan(128, 11008, 4096, 32).startswith("gemm_nt_u8_mfma_64x64")
     assert u8_plan(100, 4096, 8200, 32).startswith("gemm_nt_u8_")
     assert u8_plan(257, 11008, 1000, 32).startswith("gemm_nt_u8_")
     gen = torch.Generator(device="cuda").manual_seed(47 + m + p)
@@ -482,12 +522,14 @@ def test_seventeen_and_more_rows_in_passes(kern, kn, m):
 
 
 @pytest.mark.parametrize("mpn", [(300, 4096, 4096), (512, 2048, 4090), (260, 11008, 1000)])
-def test_mid_row_counts_take_the_smaller_staged_tiles(kern, mpn):
-    """With at most 64 tiles of 256 x 128 the u8 product runs on the staged kernels' smaller tiles;
-    same arithmetic bar as the large-tile kernel."""
+def test_mid_row_counts_take_the_smaller_tiles(kern, mpn):
+    """A few hundred rows against a narrow matrix are too few 256-row tiles for the compute units:
+    the u8 kernel's 128 x 64 and 64 x 64 tiles take them, K split over groups of wavefronts where
+    there is at most one tile per compute unit; same arithmetic bar as the large tiles."""
     m, p, n = mpn
     assert (m + 255) // 256 * ((n + 127) // 128) <= 64
-    assert u8_plan(m, p, n, 32).startswith("gemm_nt_u8_stage_")
+    assert u8_plan(m, p, n, 32) in ("gemm_nt_u8_mfma_128x64x64_k2", "gemm_nt_u8_mfma_64x64x64_k4",
+                                    "gemm_nt_u8_mfma_128x64x64", "gemm_nt_u8_mfma_64x64x64")
     gen = torch.Generator(device="cuda").manual_seed(48 + m)
     q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)
     s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()

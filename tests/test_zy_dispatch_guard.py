@@ -31,17 +31,17 @@ def _time(fn, iters, warm=8):
     return e0.elapsed_time(e1) / iters
 
 
-def _measure(lib, fn, passes):
+def _measure(lib, fn, passes, knob=0, tiles=len(TILES)):
     # (every measurement spans some ten milliseconds: shorter ones see the clock wander)
     iters = max(40, int(10.0 / max(_time(fn, 20), 1e-3)))
     best = {}
     try:
         for _ in range(passes):
-            for t in range(len(TILES) + 1):
-                assert lib.adr_debug_knob(0, t) == 0
+            for t in range(tiles + 1):
+                assert lib.adr_debug_knob(knob, t) == 0
                 best[t] = min(best.get(t, 1e30), _time(fn, iters))
     finally:
-        lib.adr_debug_knob(0, 0)
+        lib.adr_debug_knob(knob, 0)
     return best
 
 
@@ -94,3 +94,37 @@ def test_chosen_tile_is_within_five_percent_of_the_best_forced_one(case):
         if ratio <= 1.05:
             break
     assert ratio <= 1.05, (case, {("chosen" if t == 0 else TILES[t - 1]): round(v * 1e3, 1) for t, v in best.items()})
+
+
+# the u8-weight kernel's tiles in the order of adr_debug_knob(1, 1 + i)
+U8_TILES = ["256x192", "256x128", "128x128", "128x64", "64x64", "128x64_k2", "64x64_k4"]
+U8_SHAPES = [("down_m256", 256, 11008, 4096), ("o_m512", 512, 4096, 4096), ("down_m1024", 1024, 11008, 4096),
+             ("qkv_m128", 128, 4096, 12288), ("gate_m384", 384, 4096, 11008), ("qkv_m2048", 2048, 4096, 12288)]
+
+
+@pytest.mark.parametrize("case", U8_SHAPES, ids=[c[0] for c in U8_SHAPES])
+def test_chosen_u8_tile_is_within_seven_percent_of_the_best_forced_one(case):
+    """The same guard for the u8-weight kernel over the row counts where its small tiles and the K
+    groups inside a workgroup decide the time (a forced tile also keeps the product off the
+    passes of 64 rows, so the passes are not among the candidates here)."""
+    lib = _ffi.lib()
+    _, M, K, N = case
+    gen = torch.Generator(device="cuda").manual_seed(7)
+    q = torch.randint(0, 256, (N, K), generator=gen, device="cuda", dtype=torch.uint8)
+    s = (torch.rand(N, K // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
+    a = torch.randn(M, K, generator=gen, device="cuda").half()
+    out = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+
+    def fn():
+        rc = lib.adr_matmul_nt_fp16u8(torch.cuda.current_stream().cuda_stream, out.data_ptr(), a.data_ptr(),
+                                      q.data_ptr(), s.data_ptr(), M, K, N, 32, 0.0)
+        assert rc == 0
+    for _ in range(100):   # the clocks settle under load
+        fn()
+    ratio = None
+    for attempt in range(3):
+        best = _measure(lib, fn, passes=3, knob=1, tiles=len(U8_TILES))
+        ratio = best[0] / min(v for t, v in best.items() if t)
+        if ratio <= 1.07:
+            break
+    assert ratio <= 1.07, (case, {("chosen" if t == 0 else U8_TILES[t - 1]): round(v * 1e3, 1) for t, v in best.items()})
