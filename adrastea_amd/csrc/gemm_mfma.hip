@@ -15,7 +15,8 @@
 //                       the current slice feeds the MFMAs; one barrier per slice.  MFMA
 //                       fragments are prefetched one k-step ahead and interleaved with the
 //                       MFMAs by scheduling-group barriers.
-//  gemm_nt_u8_kernel    the same with u8 weights dequantised on their way into LDS.
+//  gemm_nt_u8_kernel    the same with u8 weights dequantised on their way into LDS; its two small
+//                       tiles can split K over groups of wavefronts inside the workgroup.
 //  gemm_nt_shortk_kernel  K = 64 / 128 (the attention score product): persistent workgroups;
 //                       also with the Load Scale operator (both operands scaled in fp16 on the
 //                       way into the MFMAs) and for score rows that are not 16-byte aligned.
@@ -23,9 +24,9 @@
 //                       address and whose K is no multiple of 64 (sequence lengths like 77, 257,
 //                       1500): left operand through registers, shifted into place.
 //  gemm_nt_stage_kernel any K % 8 == 0, and the variants that must touch the data on the way
-//                       in: u8 weights dequantised while staging (adr_matmul_nt_fp16u8), and
-//                       the Load Scale operator on other K.  Global -> registers -> LDS, two
-//                       LDS stages.
+//                       in: u8 weights dequantised while staging (a K that is no multiple of 64,
+//                       block sizes that are no power of two), and the Load Scale operator on
+//                       other K.  Global -> registers -> LDS, two LDS stages.
 //
 // One workgroup owns a BM x BN output tile, WM x WN wavefronts each own a (BM/WM) x (BN/WN)
 // sub-tile as fp32 accumulator blocks: 16 x 16 blocks of v_mfma_f32_16x16x32_f16 in the tiles
@@ -1424,6 +1425,10 @@ __global__ __launch_bounds__(SHORTK_THREADS, 1) void gemm_nt_shortk_kernel(Matmu
 // dequantised once per workgroup and the MFMA loop is the one of the fp16 kernel.
 // MI16: 16x16x32 MFMAs, two k-steps per slice, all chunks dequantised in the first (the 256 x 128
 // tile: 5-6 % faster; the 256 x 192 tile has no registers for the second set of fragments)
+// G: groups of WM x WN wavefronts that split K between them (1: none).  A tile that has its compute
+// unit to itself is bound by the chain of one slice -- barrier, fragment reads, MFMAs, the wait for
+// the next slice: 0.3-0.4 us per slice of a 64 x 64 tile whatever its loads -- so with at most one
+// tile per compute unit the small tiles run G such chains side by side.
 template <int BM, int BN, int WM, int WN, bool MI16, int BK = 64, int G = 1>
 __global__ __launch_bounds__(WM* WN* G * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a, TileMap map,
                                                                       int block_shift) {

@@ -268,10 +268,10 @@ def main():
 
     def u8_short_prompt_set():
         """The same row counts against u8 weights: `us` as the entry point comes (the streaming
-        kernels in passes of 64 rows, or the tiled u8 kernels), `dequantise_first_us` after
-        adr_set_u8_dequantise_first(1) (from 96 rows on wide and 160 rows on narrow matrices the
-        matrix is dequantised once into a buffer of the library's pool and the fp16 kernels run
-        on it)."""
+        kernels in passes of 64 rows, or the tiled u8 kernel on its small tiles),
+        `dequantise_first_us` after adr_set_u8_dequantise_first(1) (from 768 rows on the matrix is
+        dequantised once into a buffer of the library's pool and the fp16 kernels run on it; below,
+        the switch changes nothing)."""
         rows = []
         for K, N in DECODE_SET:
             per = N * K + N * (K // 32) * 2
@@ -280,7 +280,7 @@ def main():
                   for _ in range(nbuf)]
             ss = [(torch.rand(N, K // 32, generator=gen, device=dev) * 0.019 + 0.001).half()
                   for _ in range(nbuf)]
-            for m in (96, 128, 256, 512):
+            for m in (96, 128, 256, 512, 1024):
                 a = randn_h(m, K)
                 o = torch.zeros(m, N, dtype=torch.float16, device=dev)
                 i = [0]
