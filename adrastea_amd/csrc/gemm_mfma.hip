@@ -2160,10 +2160,11 @@ constexpr int N_DMA_TILES = sizeof(DMA_TILES) / sizeof(DMA_TILES[0]);
 // 256x192 195 / 78, 256x128 140 / 56, 128x128 97 / 41, 128x64 68 / 30 (two K groups; one: 73 / 32),
 // 64x64 47 / 22 (four K groups; one: 58 / 25).  The two smallest tiles are bound by what the L2s
 // deliver to all CUs together (M256 K11008 N4096 on 64x64: 540 MB in 47 us), the larger ones by
-// the path into one CU.  Over M 128..1536 x (K, N) of the LLaMA-7B and 13B layers the choice by
-// these constants is the fastest forced tile or within 5 % of it.
+// the path into one CU.  Over M 70..1536 x (K, N) of the LLaMA-7B and 13B layers the choice by
+// these constants is the fastest forced tile or within 5 % of it, with the weights resident in
+// the Infinity Cache and with weights that come from HBM (rotated through 600 MB) alike.
 const Candidate U8_TILES[] = {{U8_256x192, 256, 192, 1, 1.10f}, {U8_256x128, 256, 128, 1, 1.05f},
-                              {U8_128x128, 128, 128, 1, 0.74f}, {U8_128x64, 128, 64, 2, 0.52f},
+                              {U8_128x128, 128, 128, 1, 0.72f}, {U8_128x64, 128, 64, 2, 0.52f},
                               {U8_64x64, 64, 64, 4, 0.37f}};
 constexpr int N_U8_TILES = sizeof(U8_TILES) / sizeof(U8_TILES[0]);
 
@@ -2507,14 +2508,15 @@ const char* gemm_u8_mfma_plan(int m, int p, int n, int block_size) {
 }
 
 // Estimated time of the u8 product on the tiled u8 kernel, in us (negative: that kernel does not
-// cover it): pick()'s cost of the chosen tile times K.  4 us + 3.5e-7 us per unit fits one tile per
-// CU of 64 x 64 (K11008 47 us, K4096 21) and of 128 x 64 (68, 30).
+// cover it): pick()'s cost of the chosen tile times K.  4 us + 4.3e-7 us per unit fits one tile per
+// CU of 64 x 64 (K11008 53-59 us, K4096 23-26) and of 128 x 64 (71-85, 30-35) on weights that come
+// from HBM (3.5e-7 where the Infinity Cache holds them: 47 / 21 and 68 / 30).
 double gemm_u8_mfma_estimate_us(int m, int p, int n, int block_size) {
   const MatmulArgs a = u8_args(nullptr, nullptr, (const uint8_t*)16, nullptr, m, p, n, block_size, 0.0f);
   if (!(p % 64 == 0 && block_size >= 8 && (block_size & (block_size - 1)) == 0)) return -1.0;
   double cost;
   pick(a, U8_TILES, N_U8_TILES, &cost);
-  return 4.0 + cost * p * 3.5e-7;
+  return 4.0 + cost * p * 4.3e-7;
 }
 
 bool gemm_u8_mfma_supported(const half_t* lhs, const uint8_t* rhs, const half_t* scales, int m, int p,

@@ -730,14 +730,17 @@ U8Choice choose_u8(const void* lhs, const void* rhs, const void* scales, int m, 
 // 13.1 us, N8192 23.5, N12288 33.9, K11008 N4096 26.4, K5120 N5120 25.7); a last pass of r rows
 // costs 0.55 + 0.45 r / 64 of that.  Up to 64 rows the passes always win (the tiled kernel has
 // N / 64 tiles for them: K11008 N4096 43 us); above, where this estimate is below the tiled
-// kernel's own: K11008 N4096 m=70 41 against 44 us (m=128: 54 against 44, tiled), K4096 N4096
-// m=70 20.6 against 20.2, m=128 25 against 19; K5120 N5120 and K13824 N5120 are tiled from 65 rows.
+// kernel's own.  Measured with weights that come from HBM: K11008 N4096 m=96 45 against 53 us,
+// m=128 53 against 59, m=160 71 against 53 (tiled); K4096 N4096 m=96 22.4 against 23.2, m=128 a
+// tie, m=160 36 against 23; wide or 13B-sized matrices are tiled from 65 rows (K4096 N12288 m=70
+// 47 against 31, K13824 N5120 m=70 78 against 57).
 bool rows_in_passes(int m, int p, int n, int block_size) {
   if (m <= 16 || m > 256 || (int64_t)n * p < (1 << 22) ||
       choose_u8(nullptr, nullptr, nullptr, 16, p, n, block_size) != U8_GEMV)
     return false;
   if (m <= 64) return true;
-  if (knob(KNOB_U8_TILE)) return false;  // (a test or benchmark forces a tile of the tiled kernel)
+  // (a test or benchmark forces a tile of the tiled kernel, or -- value 9 -- the passes)
+  if (knob(KNOB_U8_TILE)) return knob(KNOB_U8_TILE) == 9;
   const int cus = device_info_for_plan().cus;
   const int rounds = ((n + ROWS - 1) / ROWS + cus - 1) / cus;
   const double t64 = fmax(12.0, rounds * (2.0 + 0.0023 * p));

@@ -84,11 +84,12 @@ def test_u8_plan():
     assert plan(32, 4096, 12288, 32) == (0, "gemv_u8_mfma16_dma_32rows")
     assert plan(32, 11008, 4096, 32) == (0, "gemv_u8_mfma16_blocks")
     assert plan(64, 4096, 12288, 32) == (0, "gemv_u8_mfma16_blocks")
-    # above 64 rows: passes of 64 rows where the estimate puts them ahead of the tiled kernel (a
-    # few rows past 64 against a narrow matrix)
+    # above 64 rows: passes of 64 rows where the estimate puts them ahead of the tiled kernel (to
+    # 128 rows against a narrow matrix)
     assert plan(70, 11008, 4096, 32) == (0, "gemv_u8_mfma16_blocks")
     assert plan(70, 4096, 4096, 32) == (0, "gemv_u8_mfma16_blocks")
-    assert plan(128, 11008, 4096, 32) == (0, "gemm_nt_u8_mfma_64x64x64_k4")
+    assert plan(128, 11008, 4096, 32) == (0, "gemv_u8_mfma16_blocks")
+    assert plan(160, 11008, 4096, 32) == (0, "gemm_nt_u8_mfma_64x64x64_k4")
     assert plan(256, 11008, 4096, 32) == (0, "gemm_nt_u8_mfma_64x64x64_k4")
     assert plan(96, 4096, 12288, 32) == (0, "gemm_nt_u8_mfma_128x64x64_k2")
     assert plan(100, 512, 9000, 32)[1].startswith("gemm_nt_u8_mfma_")

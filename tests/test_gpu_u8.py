@@ -499,10 +499,10 @@ def test_seventeen_and_more_rows_in_passes(kern, kn, m):
         assert name == ("gemv_u8_mfma16_dma_32rows" if p == 4096 and m <= 32 else "gemv_u8_mfma16_blocks")
     else:
         assert name == "gemv_u8_mfma16_blocks" or name.startswith("gemm_nt_u8_")
-    # decisions the estimate must make: a few rows past 64 against a narrow matrix stay in passes,
+    # decisions the estimate must make: to 128 rows against a narrow matrix the passes stay,
     # more rows or a matrix of several rounds of workgroups go to the tiled kernel
-    assert u8_plan(70, 11008, 4096, 32) == "gemv_u8_mfma16_blocks"
-    assert u8_plan(128, 11008, 4096, 32).startswith("gemm_nt_u8_mfma_64x64")
+    assert u8_plan(128, 11008, 4096, 32) == "gemv_u8_mfma16_blocks"
+    assert u8_plan(160, 11008, 4096, 32).startswith("gemm_nt_u8_mfma_64x64")
     assert u8_plan(100, 4096, 8200, 32).startswith("gemm_nt_u8_")
     assert u8_plan(257, 11008, 1000, 32).startswith("gemm_nt_u8_")
     gen = torch.Generator(device="cuda").manual_seed(47 + m + p)
