@@ -728,19 +728,20 @@ U8Choice choose_u8(const void* lhs, const void* rhs, const void* scales, int m, 
 // matrix-core streaming kernels, each pass reading the weights once.  A pass of 64 rows is one
 // workgroup per sixteen weight rows, 2 + 0.0023 K us per round of them over the CUs (K4096 N4096
 // 13.1 us, N8192 23.5, N12288 33.9, K11008 N4096 26.4, K5120 N5120 25.7); a last pass of r rows
-// costs 0.55 + 0.45 r / 64 of that.  Up to 64 rows the passes always win (the tiled kernel has
-// N / 64 tiles for them: K11008 N4096 43 us); above, where this estimate is below the tiled
-// kernel's own.  Measured with weights that come from HBM: K11008 N4096 m=96 45 against 53 us,
-// m=128 53 against 59, m=160 71 against 53 (tiled); K4096 N4096 m=96 22.4 against 23.2, m=128 a
-// tie, m=160 36 against 23; wide or 13B-sized matrices are tiled from 65 rows (K4096 N12288 m=70
-// 47 against 31, K13824 N5120 m=70 78 against 57).
+// costs 0.55 + 0.45 r / 64 of that.  Up to 32 rows the passes always win (K4096 N12288 m=32 18 us
+// against 25 on 64 x 64 tiles); above, where this estimate is below the tiled kernel's own.
+// Measured with weights that come from HBM: K11008 N4096 m=64 27 against 61 us (passes), m=96 45
+// against 53, m=128 53 against 59, m=160 71 against 53 (tiled); K4096 N4096 m=96 22.4 against 23.2,
+// m=128 a tie, m=160 36 against 23; wide matrices are tiled from 33 rows (K4096 N12288 m=40 29
+// against 26, m=64 34 against 28, m=70 47 against 31; K5120 N13824 m=64 50 against 36), 13B-sized
+// narrow ones from 65 (K13824 N5120 m=64 58 against 77, m=70 78 against 57).
 bool rows_in_passes(int m, int p, int n, int block_size) {
   if (m <= 16 || m > 256 || (int64_t)n * p < (1 << 22) ||
       choose_u8(nullptr, nullptr, nullptr, 16, p, n, block_size) != U8_GEMV)
     return false;
-  if (m <= 64) return true;
   // (a test or benchmark forces a tile of the tiled kernel, or -- value 9 -- the passes)
   if (knob(KNOB_U8_TILE)) return knob(KNOB_U8_TILE) == 9;
+  if (m <= 32) return true;
   const int cus = device_info_for_plan().cus;
   const int rounds = ((n + ROWS - 1) / ROWS + cus - 1) / cus;
   const double t64 = fmax(12.0, rounds * (2.0 + 0.0023 * p));

@@ -388,7 +388,7 @@ int adr_matmul_f16_ws_plan(char* name, int32_t cap, int32_t batches, int32_t m, 
  * GEMM (0: the dispatch decides; 1 + i: tile i of 256x192, 256x128, 128x128, 128x64, 64x64, 128x64
  * with K split over two groups of wavefronts, 64x64 with K split over four; 8: the register-staged
  * kernels that otherwise serve a K that is no multiple of 64; 9: the passes of 64 rows for products
- * of 65 to 256 rows); a forced tile also keeps products of 65 to 256 rows off those passes.  Unknown
+ * of 17 to 256 rows); a forced tile also keeps products of 17 to 256 rows off those passes.  Unknown
  * ids return ADR_EINVAL_ENUM.
  */
 int adr_debug_knob(int32_t id, int32_t value);

@@ -83,7 +83,10 @@ def test_u8_plan():
     # 17 to 64 rows in blocks of rows: 32 per pass for K = 4096, 16 otherwise
     assert plan(32, 4096, 12288, 32) == (0, "gemv_u8_mfma16_dma_32rows")
     assert plan(32, 11008, 4096, 32) == (0, "gemv_u8_mfma16_blocks")
-    assert plan(64, 4096, 12288, 32) == (0, "gemv_u8_mfma16_blocks")
+    assert plan(64, 4096, 4096, 32) == (0, "gemv_u8_mfma16_blocks")
+    # 33 rows and more: passes where the estimate puts them ahead of the tiled kernel (narrow
+    # matrices), else the tiled kernel's small tiles
+    assert plan(64, 4096, 12288, 32) == (0, "gemm_nt_u8_mfma_64x64x64_k4")
     # above 64 rows: passes of 64 rows where the estimate puts them ahead of the tiled kernel (to
     # 128 rows against a narrow matrix)
     assert plan(70, 11008, 4096, 32) == (0, "gemv_u8_mfma16_blocks")

@@ -154,7 +154,8 @@ def force_u8_tile():
     lib = _ffi.lib()
 
     def force(tile):
-        assert lib.adr_debug_knob(1, U8_STAGED if tile == "staged" else 1 + U8_TILES.index(tile)) == 0
+        assert lib.adr_debug_knob(1, U8_STAGED if tile == "staged" else U8_STAGED + 1 if tile == "passes" else
+                                  1 + U8_TILES.index(tile)) == 0
     yield force
     assert lib.adr_debug_knob(1, 0) == 0
 
@@ -251,14 +252,17 @@ def test_wide_gemv_bit_exact_on_exact_inputs(kern, m, pn):
 
 @pytest.mark.parametrize("m", [17, 31, 32, 33, 48, 50, 64, 70])
 @pytest.mark.parametrize("pn", [(256, 16400), (768, 8200), (2304, 1900), (11008, 400), (4096, 1030)])
-def test_blocks_kernel_bit_exact_on_exact_inputs(kern, m, pn):
+def test_blocks_kernel_bit_exact_on_exact_inputs(kern, m, pn, force_u8_tile):
     """Two to four blocks of sixteen activation rows per workgroup: one, two and three groups of
     weight rows, macro-step counts from one (wavefronts without a step) to 43, ragged rows of
-    both operands, a second pass for rows 65 .. 70, beta path."""
+    both operands, a second pass for rows 65 .. 70, beta path.  The passes are forced: from 33 rows
+    on the dispatch sends wide matrices and short K to the tiled kernel."""
     p, n = pn
     g = rng(1700 + m + p)
-    if m <= 64 or p >= 4096:   # (70 rows on a short K are estimated faster on the tiled kernel)
+    if m <= 32 or (n <= 1900 and (m <= 64 or p >= 4096)):   # what the dispatch runs in passes by itself
         assert u8_plan(m, p, n, 32) in ("gemv_u8_mfma16_blocks", "gemv_u8_mfma16_dma_32rows")
+    force_u8_tile("passes")
+    assert u8_plan(m, p, n, 32) in ("gemv_u8_mfma16_blocks", "gemv_u8_mfma16_dma_32rows")
     a, q, s = _u8_case(g, m, p, n, 32, exact=True)
     for beta in (0.0, 1.0):
         prev = (g.integers(-8, 9, size=(m, n)) / 4.0).astype(np.float16)
@@ -491,18 +495,20 @@ def test_decode_ten_rows_and_more_long_k(kern, kn, m):
 def test_seventeen_and_more_rows_in_passes(kern, kn, m):
     """17 rows and more on matrices of 4 MiB and more run in passes of up to 64 rows, each
     reading the weights once for two to four blocks of sixteen rows (K = 4096 up to 32 rows: the
-    DMA-ring kernel; a last pass of up to sixteen rows: the sixteen-row kernels); above 64 rows
-    only where that is estimated to beat the tiled GEMM.  Previous output added, ragged N."""
+    DMA-ring kernel; a last pass of up to sixteen rows: the blocks kernel with one block); above
+    32 rows only where that is estimated to beat the tiled GEMM.  Previous output added, ragged N."""
     p, n = kn
     name = u8_plan(m, p, n, 32)
-    if m <= 64:
-        assert name == ("gemv_u8_mfma16_dma_32rows" if p == 4096 and m <= 32 else "gemv_u8_mfma16_blocks")
+    if m <= 32:
+        assert name == ("gemv_u8_mfma16_dma_32rows" if p == 4096 else "gemv_u8_mfma16_blocks")
     else:
         assert name == "gemv_u8_mfma16_blocks" or name.startswith("gemm_nt_u8_")
     # decisions the estimate must make: to 128 rows against a narrow matrix the passes stay,
     # more rows or a matrix of several rounds of workgroups go to the tiled kernel
+    assert u8_plan(64, 11008, 4096, 32) == "gemv_u8_mfma16_blocks"
     assert u8_plan(128, 11008, 4096, 32) == "gemv_u8_mfma16_blocks"
     assert u8_plan(160, 11008, 4096, 32).startswith("gemm_nt_u8_mfma_64x64")
+    assert u8_plan(48, 4096, 12288, 32).startswith("gemm_nt_u8_mfma_64x64")
     assert u8_plan(100, 4096, 8200, 32).startswith("gemm_nt_u8_")
     assert u8_plan(257, 11008, 1000, 32).startswith("gemm_nt_u8_")
     gen = torch.Generator(device="cuda").manual_seed(47 + m + p)
