@@ -73,7 +73,8 @@ def test_u8_plan():
         return rc, buf.value.decode()
     for m in (1, 2):
         assert plan(m, 4096, 4096, 32) == (0, "gemv_u8_dot2_stream")
-        assert plan(m, 11008, 4096, 32) == (0, "gemv_u8_dot2_stream")
+    assert plan(1, 11008, 4096, 32) == (0, "gemv_u8_dot2_stream")
+    assert plan(2, 11008, 4096, 32) == (0, "gemv_u8_mfma16_regstream")   # two rows over a long K
     for m in (3, 4, 16):
         assert plan(m, 4096, 4096, 32) == (0, "gemv_u8_mfma16_regstream")
         assert plan(m, 11008, 4096, 32) == (0, "gemv_u8_mfma16_regstream")

@@ -413,7 +413,7 @@ def test_prefill_u8_gemm_layer_set_full_size(kern, case, workspace_mode):
 def test_u8_other_block_sizes_and_fallbacks(kern):
     g = rng(630)
     for m, p, n, bs in [(4, 512, 40, 64), (4, 384, 40, 128), (3, 96, 20, 8), (2, 48, 10, 16),
-                        (40, 320, 70, 64)]:
+                        (40, 320, 70, 64), (2, 4608, 40, 64), (2, 4608, 40, 32)]:
         a, q, s = _u8_case(g, m, p, n, bs, exact=True)
         want = np.zeros((m, n), np.float16)
         oracle.matmul_nt_fp16u8(want, a, q, s, bs)
