@@ -527,6 +527,42 @@ def test_seventeen_and_more_rows_in_passes(kern, kn, m):
     assert rel <= 2e-3, rel
 
 
+@pytest.mark.parametrize("mpn", [(256, 11008, 4096), (500, 4096, 4090)])
+def test_tiles_that_split_k_over_wavefront_groups_give_the_same_bits_every_launch(kern, mpn):
+    """The groups' partial sums meet in LDS in group order, whichever group finishes first: twenty
+    launches (and one on another stream) of the 64 x 64 tile with four groups and of the 128 x 64
+    tile with two give one result, equal to the same tile without groups up to fp32 summation
+    order."""
+    m, p, n = mpn
+    name = u8_plan(m, p, n, 32)
+    assert name in ("gemm_nt_u8_mfma_64x64x64_k4", "gemm_nt_u8_mfma_128x64x64_k2")
+    gen = torch.Generator(device="cuda").manual_seed(49 + m)
+    q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)
+    s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
+    a = torch.randn(m, p, generator=gen, device="cuda").half()
+    lib = _ffi.lib()
+
+    def run(stream):
+        out = torch.zeros(m, n, dtype=torch.float16, device="cuda")
+        assert lib.adr_matmul_nt_fp16u8(stream, out.data_ptr(), a.data_ptr(), q.data_ptr(), s.data_ptr(),
+                                        m, p, n, 32, 0.0) == 0
+        return out
+    first = run(torch.cuda.current_stream().cuda_stream)
+    for _ in range(19):
+        assert torch.equal(run(torch.cuda.current_stream().cuda_stream), first)
+    side = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        other = run(side.cuda_stream)
+    torch.cuda.synchronize()
+    assert torch.equal(other, first)
+    w = torch.zeros(n, p, dtype=torch.float16, device="cuda")
+    kern.dequantize_absmax_uint8(w, s, q)
+    ref32 = a.float() @ w.float().t()
+    rms = ref32.pow(2).mean().sqrt()
+    assert ((first.float() - ref32).abs() / torch.maximum(ref32.abs(), rms)).max().item() <= 2e-3
+
+
 @pytest.mark.parametrize("mpn", [(300, 4096, 4096), (512, 2048, 4090), (260, 11008, 1000)])
 def test_mid_row_counts_take_the_smaller_tiles(kern, mpn):
     """A few hundred rows against a narrow matrix are too few 256-row tiles for the compute units:
