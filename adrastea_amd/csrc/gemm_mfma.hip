@@ -2389,8 +2389,11 @@ static hipError_t launch_choice(hipStream_t stream, const MatmulArgs& a, GemmCho
     case DMA_128x256: return launch_dma<128, 256, 2, 4, 3, 1, false, 64, true>(stream, a);
     case DMA_128x192: return launch_dma<128, 192, 2, 2, 3, 1>(stream, a);
     // (eight wavefronts of 32 x 64 on 16x16x32 MFMAs: two per SIMD overlap each other's slice
-    // chains; 2-7 % ahead of four wavefronts of 64 x 64 on 32x32x16: M1024 K4096 N4096 37.8 -> 35.3 us)
-    case DMA_128x128: return launch_dma<128, 128, 4, 2, 3, 1, false, 64, true>(stream, a);
+    // chains; 2-7 % ahead of four wavefronts of 64 x 64 on 32x32x16: M1024 K4096 N4096 37.8 -> 35.3 us.
+    // Three left and four right stages with the transfers split by wavefront role: another 2-9 %,
+    // M2056 K4096 N1024 29.2 -> 26.5, M768 K4096 N4096 30.4 -> 27.8; the same on the 128 x 256,
+    // 128 x 192, 128 x 64 and 64 x 64 tiles changed nothing or lost.)
+    case DMA_128x128: return launch_dma<128, 128, 4, 2, 7, 1, false, 64, true>(stream, a);
     case DMA_128x64: return launch_dma<128, 64, 2, 2, 3, 2>(stream, a);
     case DMA_64x64: return launch_dma<64, 64, 2, 2, 3, 3>(stream, a);
     case DMA_64x64_K128: return launch_dma<64, 64, 2, 2, 3, 1, false, 128>(stream, a);

@@ -674,6 +674,24 @@ def test_256x128_tile_every_remainder_of_its_twelve_slice_period(K):
     assert torch.equal(out.view(torch.int16), want.view(torch.int16))
 
 
+@pytest.mark.parametrize("K", [320 + 64 * i for i in range(14)])
+def test_128x128_tile_every_remainder_of_its_twelve_slice_period(K):
+    """The 128 x 128 kernel (eight wavefronts of 32 x 64 on 16x16x32 MFMAs) rotates three left and four
+    right LDS stages like the 256 x 128 one: K of 5 to 18 slices, i.e. fewer slices than the period,
+    every remainder of it and one full turn, on inputs whose fp32 sums are exact, ragged last tile
+    row and column."""
+    M, N = 1000, 3064
+    so, sl, sr = nt_strides(M, K, N)
+    assert plan(1, M, K, N, so, sl, sr) == "gemm_nt_mfma_dma_128x128x64"
+    gen = torch.Generator(device="cuda").manual_seed(K)
+    a = (torch.randint(-4, 5, (M, K), generator=gen, device="cuda").float() / 64).half()
+    w = (torch.randint(-4, 5, (N, K), generator=gen, device="cuda").float() / 64).half()
+    out = torch.full((M, N), 9.0, dtype=torch.float16, device="cuda")
+    assert raw_matmul("adr_matmul_f16", out, a, w, 1, M, K, N, so, sl, sr) == 0
+    want = (a.double() @ w.double().t()).half()
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+
+
 @pytest.mark.parametrize("store", STORES_EXACT + STORES_F32)
 @pytest.mark.parametrize("mask", [oracle.MASK_NONE, oracle.MASK_CAUSAL])
 @pytest.mark.parametrize("M,N,tile", [(4000, 4088, "256x128"), (630, 12280, "128x256"), (380, 12280, "128x192"),
