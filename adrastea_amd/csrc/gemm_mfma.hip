@@ -1426,7 +1426,7 @@ __global__ __launch_bounds__(SHORTK_THREADS, 1) void gemm_nt_shortk_kernel(Matmu
 // u8-weight kernel: left operand by DMA, weights dequantised on their way into LDS
 // =============================================================================================
 // K % 64 == 0, block size a power of two >= 8.  The fp16 left operand goes global -> LDS by DMA
-// through three stages (two slices ahead).  The u8 weights of slice kt+2 are fetched into
+// through three stages (two slices ahead; SA = 4: four stages, three ahead).  The u8 weights of slice kt+2 are fetched into
 // registers (8 weights + their scale per chunk, three chunks per lane) while slice kt runs; the
 // chunks of slice kt+1 are dequantised (bit-identical to quantize.cu:53-54) and written to one
 // of two fp16 LDS stages in the same swizzled layout the DMA produces, so that every weight is
@@ -1437,7 +1437,7 @@ __global__ __launch_bounds__(SHORTK_THREADS, 1) void gemm_nt_shortk_kernel(Matmu
 // unit to itself is bound by the chain of one slice -- barrier, fragment reads, MFMAs, the wait for
 // the next slice: 0.3-0.4 us per slice of a 64 x 64 tile whatever its loads -- so with at most one
 // tile per compute unit the small tiles run G such chains side by side.
-template <int BM, int BN, int WM, int WN, bool MI16, int BK = 64, int G = 1>
+template <int BM, int BN, int WM, int WN, bool MI16, int BK = 64, int G = 1, int SA = 3>
 __global__ __launch_bounds__(WM* WN* G * 64, 1) void gemm_nt_u8_kernel(MatmulArgs a, TileMap map,
                                                                       int block_shift) {
   constexpr int CPR = BK / 8, MI = MI16 ? 16 : 32, KG = 64 / MI, KK = CPR / KG;
@@ -1460,6 +1460,8 @@ __global__ __launch_bounds__(WM* WN* G * 64, 1) void gemm_nt_u8_kernel(MatmulArg
   __shared__ __attribute__((aligned(1024))) unsigned char sA0[G * BM * BK * 2];
   __shared__ __attribute__((aligned(1024))) unsigned char sA1[G * BM * BK * 2];
   __shared__ __attribute__((aligned(1024))) unsigned char sA2[G * BM * BK * 2];
+  __shared__ __attribute__((aligned(1024))) unsigned char sA3[SA == 4 ? G * BM * BK * 2 : 1024];
+  static_assert(SA == 3 || SA == 4, "three stages of the left operand (two slices ahead) or four (three ahead)");
   __shared__ __attribute__((aligned(1024))) unsigned char sB0[G * BN * BK * 2];
   __shared__ __attribute__((aligned(1024))) unsigned char sB1[G * BN * BK * 2];
 
@@ -1603,38 +1605,45 @@ __global__ __launch_bounds__(WM* WN* G * 64, 1) void gemm_nt_u8_kernel(MatmulArg
     }
     // A(kt+1) has landed: only the weight fetch and the DMA issued in this slice may still be
     // in flight; the dequantised weights of slice kt+1 are in LDS
-    constexpr int n = 2 * LB + IA;
+    // (four A stages: the transfer issued in the slice before, which is younger than that slice's
+    // weight requests, may stay in flight too)
+    constexpr int n = 2 * LB + (SA - 2) * IA;
     __builtin_amdgcn_s_waitcnt(0x0070 | (n & 0xF) | ((n >> 4) << 14));
     __builtin_amdgcn_s_barrier();
     load_frags(0, nA, nB, 0);
   };
 
+  // slice kt (kt % P == p) reads A stage p % SA and B stage p % 2, dequantises register set
+  // (p + 1) % 3 into the other B stage, refills the A stage read one slice earlier with slice
+  // kt + SA - 1 and register set p % 3 with the weights of slice kt + 3
+  auto stA = [&](int i) -> unsigned char* { return i == 0 ? sA0 : i == 1 ? sA1 : i == 2 ? sA2 : sA3; };
+  auto stB = [&](int i) -> unsigned char* { return i == 0 ? sB0 : sB1; };
+  constexpr int P = SA == 3 ? 6 : 12;  // the common period of the stages and the register sets
+  auto slice_p = [&](int p) {
+    slice(stA(p % SA), stB(p % 2), stA((p + 1) % SA), stB((p + 1) % 2), stA((p + SA - 1) % SA), p % 3,
+          (p + 1) % 3);
+  };
   fetchQ(0);
   fetchQ(1);
   dmaA(sA0);
   fetchQ(2);
   dmaA(sA1);
+  if (SA == 4) dmaA(sA2);
   dequant_store(0, sB0);
   {
-    constexpr int n = IA;
+    constexpr int n = (SA - 2) * IA;
     __builtin_amdgcn_s_waitcnt(0x0070 | (n & 0xF) | ((n >> 4) << 14));
     __builtin_amdgcn_s_barrier();
   }
   load_frags(0, sA0, sB0, 0);
   int kt = 0;
-  for (; kt + 6 <= KT; kt += 6) {
-    slice(sA0, sB0, sA1, sB1, sA2, 0, 1);
-    slice(sA1, sB1, sA2, sB0, sA0, 1, 2);
-    slice(sA2, sB0, sA0, sB1, sA1, 2, 0);
-    slice(sA0, sB1, sA1, sB0, sA2, 0, 1);
-    slice(sA1, sB0, sA2, sB1, sA0, 1, 2);
-    slice(sA2, sB1, sA0, sB0, sA1, 2, 0);
+  for (; kt + P <= KT; kt += P) {
+#pragma unroll
+    for (int p = 0; p < P; p++) slice_p(p);
   }
-  if (kt < KT) { slice(sA0, sB0, sA1, sB1, sA2, 0, 1); kt++; }
-  if (kt < KT) { slice(sA1, sB1, sA2, sB0, sA0, 1, 2); kt++; }
-  if (kt < KT) { slice(sA2, sB0, sA0, sB1, sA1, 2, 0); kt++; }
-  if (kt < KT) { slice(sA0, sB1, sA1, sB0, sA2, 0, 1); kt++; }
-  if (kt < KT) { slice(sA1, sB0, sA2, sB1, sA0, 1, 2); kt++; }
+#pragma unroll
+  for (int p = 0; p < P - 1; p++)
+    if (kt < KT) { slice_p(p); kt++; }
   __builtin_amdgcn_s_waitcnt(0x0070);
   __builtin_amdgcn_s_barrier();
 
@@ -2065,11 +2074,11 @@ hipError_t launch_stage(hipStream_t stream, const MatmulArgs& a) {
   return hipGetLastError();
 }
 
-template <int BM, int BN, int WM, int WN, bool MI16, int BK = 64, int G = 1>
+template <int BM, int BN, int WM, int WN, bool MI16, int BK = 64, int G = 1, int SA = 3>
 hipError_t launch_u8(hipStream_t stream, const MatmulArgs& a) {
   TileMap map = make_map(a, BM, BN);
   if (map.total < 0 || a.k % (BK * G) != 0) return hipErrorInvalidConfiguration;
-  hipLaunchKernelGGL((gemm_nt_u8_kernel<BM, BN, WM, WN, MI16, BK, G>), dim3((unsigned)map.total),
+  hipLaunchKernelGGL((gemm_nt_u8_kernel<BM, BN, WM, WN, MI16, BK, G, SA>), dim3((unsigned)map.total),
                      dim3(WM * WN * G * 64), 0, stream, a, map, __builtin_ctz(a.block_size));
   return hipGetLastError();
 }
@@ -2377,7 +2386,9 @@ static hipError_t launch_choice(hipStream_t stream, const MatmulArgs& a, GemmCho
     case SHORTK_64: return launch_shortk<8>(stream, a);
     case SHORTK_128: return launch_shortk<16>(stream, a);
     case U8_256x192: return launch_u8<256, 192, 4, 2, false>(stream, a);
-    case U8_256x128: return launch_u8<256, 128, 4, 2, true>(stream, a);
+    // (four stages of the left operand, three slices ahead, fill the 160 KB: K11008 N4096 M2048 with
+    // weights from HBM 202 -> 191 us, K4096 unchanged; the smaller tiles gain nothing from a fourth stage)
+    case U8_256x128: return launch_u8<256, 128, 4, 2, true, 64, 1, 4>(stream, a);
     case U8_128x128: return launch_u8<128, 128, 4, 2, true>(stream, a);
     case U8_128x64: return launch_u8<128, 64, 2, 2, true>(stream, a);
     case U8_64x64: return launch_u8<64, 64, 2, 2, true>(stream, a);

@@ -329,17 +329,18 @@ def test_u8_small_products_ragged_tiles_and_k_tails_bit_exact(kern, case, route,
 _DMA_TILE_CASES = [("256x192x64", 520, 11000), ("256x128x64", 520, 2900), ("128x128x64", 520, 2900),
                    ("128x64x64", 520, 1900), ("64x64x64", 200, 1900), ("128x64x64_k2", 520, 1900),
                    ("64x64x64_k4", 200, 1900)]
-# (K, tile): every tile on K of 5 .. 10 and 16 slices; the tiles that split K also on 20 .. 40
+# (K, tile): every tile on K of 5 .. 16 slices; the tiles that split K also on 20 .. 40
 _DMA_TILE_K = [(t, p) for t in _DMA_TILE_CASES
-               for p in [320, 384, 448, 512, 576, 640, 1024] +
+               for p in [320, 384, 448, 512, 576, 640, 704, 768, 832, 896, 960, 1024] +
                ([1280, 1536, 1792, 2048, 2304, 2560] if t[0].endswith(("_k2", "_k4")) else [])]
 
 
 @pytest.mark.parametrize("tile_mn,p", _DMA_TILE_K, ids=[f"{t[0]}-K{p}" for t, p in _DMA_TILE_K])
 def test_u8_dma_kernel_ragged_tiles_and_every_k_remainder_bit_exact(kern, tile_mn, p, force_u8_tile):
     """Every tile of gemm_nt_u8_kernel, forced: a ragged last tile row (520 = 2 x 256 + 8,
-    200 = 3 x 64 + 8) and tile column, K / 64 = 5 .. 10 slices and 16 .. 40 in steps of four, i.e.
-    every remainder of the six-slice unrolled loop also for the tiles that split K over two or
+    200 = 3 x 64 + 8) and tile column, K / 64 = 5 .. 16 slices and 20 .. 40 in steps of four, i.e.
+    every remainder of the six-slice loop (twelve for the 256 x 128 tile with its four stages of the
+    left operand), fewer slices than a period, and the same for the tiles that split K over two or
     four groups of wavefronts (which walk K / 128 or K / 256 steps; a K they do not divide runs
     the tile without groups), beta 0 and 1, block sizes 32 and 64 -- exact inputs, compared bit
     for bit.  Expected values: one rounding of the float64 product on the oracle's dequantised
