@@ -193,10 +193,8 @@ typedef uint32_t u32x2_dword_aligned_t __attribute__((ext_vector_type(2), aligne
 
 // `last`: the last dword that may be read (loads past it read it again: what they return lies
 // beyond the row's end and must be masked by the caller)
-__device__ __forceinline__ half8_t load8_any(const half_t* p, uintptr_t last) {
-  const uintptr_t u = (uintptr_t)p, base = u & ~(uintptr_t)3;
-  const uint32_t shift = (uint32_t)(u & 2);
-  uint32_t d[5];
+__device__ __forceinline__ void load5_any(const half_t* p, uintptr_t last, uint32_t (&d)[5]) {
+  const uintptr_t base = (uintptr_t)p & ~(uintptr_t)3;
   // (a wavefront-uniform branch: a load under a lane mask is waited for where the lanes rejoin)
   if (__builtin_amdgcn_ballot_w64(base + 16 > last) == 0) {
     const u32x4_t q = *(const ADR_GLOBAL_AS u32x4_dword_aligned_t*)base;
@@ -207,10 +205,47 @@ __device__ __forceinline__ half8_t load8_any(const half_t* p, uintptr_t last) {
     for (int j = 0; j < 5; j++)
       d[j] = *(const ADR_GLOBAL_AS uint32_t*)(base + 4 * j < last ? base + 4 * j : last);
   }
+}
+
+// the eight halves that begin `shift` (0 or 2) bytes into the five dwords of load5_any
+__device__ __forceinline__ u32x4_t align5(const uint32_t (&d)[5], uint32_t shift) {
   u32x4_t r;
 #pragma unroll
   for (int j = 0; j < 4; j++) r[j] = __builtin_amdgcn_alignbyte(d[j + 1], d[j], shift);
-  return __builtin_bit_cast(half8_t, r);
+  return r;
+}
+
+// load5_any in two halves with no branch around the loads, for loops that keep several slices of
+// loads in flight (a branch that holds loads makes every later wait count for all of them).  The
+// 16-byte load never starts beyond last - 12: near the end of the tensor it reads from further back
+// and load5_finish picks the dwords that belong to the chunk.  What lies beyond `last` is
+// unspecified, as for load5_any.  The tensor must hold at least 24 bytes.
+__device__ __forceinline__ void load5_issue(const half_t* p, uintptr_t last, uint32_t (&d)[5]) {
+  const uintptr_t base = (uintptr_t)p & ~(uintptr_t)3, lim = last - 12;
+  const u32x4_t q = *(const ADR_GLOBAL_AS u32x4_dword_aligned_t*)(base < lim ? base : lim);
+  d[0] = q[0]; d[1] = q[1]; d[2] = q[2]; d[3] = q[3];
+  d[4] = *(const ADR_GLOBAL_AS uint32_t*)(base + 16 < last ? base + 16 : last);
+}
+
+__device__ __forceinline__ u32x4_t load5_finish(const half_t* p, uintptr_t last, const uint32_t (&d)[5]) {
+  const uintptr_t base = (uintptr_t)p & ~(uintptr_t)3, lim = last - 12;
+  uint32_t e[5] = {d[0], d[1], d[2], d[3], d[4]};
+  if (__builtin_amdgcn_ballot_w64(base > lim) != 0) {
+    // the 16 bytes were read s dwords further back: dword j of the chunk is dword j + s of them
+    // (j + s <= 3 for every dword at or before `last`)
+    const uintptr_t back = base > lim ? (base - lim) >> 2 : 0;
+    const int s = back < 3 ? (int)back : 3;
+    e[0] = s == 0 ? d[0] : s == 1 ? d[1] : s == 2 ? d[2] : d[3];
+    e[1] = s == 0 ? d[1] : s == 1 ? d[2] : d[3];
+    e[2] = s == 0 ? d[2] : d[3];
+  }
+  return align5(e, (uint32_t)((uintptr_t)p & 2));
+}
+
+__device__ __forceinline__ half8_t load8_any(const half_t* p, uintptr_t last) {
+  uint32_t d[5];
+  load5_any(p, last, d);
+  return __builtin_bit_cast(half8_t, align5(d, (uint32_t)((uintptr_t)p & 2)));
 }
 
 __device__ __forceinline__ void store8_any(half_t* p, half8_t v) {

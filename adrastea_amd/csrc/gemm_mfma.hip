@@ -1855,36 +1855,51 @@ __global__ __launch_bounds__(WM* WN * 64, MINB) void gemm_nt_stage_kernel(Matmul
 // loads the dwords around its chunk from a 4-byte aligned address and shifts them into place
 // (v_alignbyte_b32), zeroes what lies beyond K, and writes the chunk to LDS in the layout of the
 // other kernels.  The right operand ([K][N], N contiguous, 16-byte aligned rows: V on its head
-// view) is staged as [64][128] tiles and read with the transposing LDS reads of the DMA kernel's
-// row-major form.  Two LDS stages, one barrier per slice, 128 x BN tiles of 2 x 2 wavefronts
-// (BN = 64 for heads of 64 columns).
-template <int BN>
-__global__ __launch_bounds__(256, 2) void gemm_nn_anyrow_kernel(MatmulArgs a, TileMap map) {
-  constexpr int BM = 128, BK = 64, WM = 2, WN = 2, NT = 256, CPR = 8;
-  constexpr int LA = BM * CPR / NT, LB = BK * (BN / 8) / NT;  // chunks each thread stages
-  constexpr int WTM = 64, WTN = BN / 2, TM = 2, TN = WTN / 32, KK = BK / 16;
+// view) is staged as [64][BN] tiles and read with the transposing LDS reads of the DMA kernel's
+// row-major form.  Two LDS stages, one barrier per slice, loads two slices ahead of the MFMAs,
+// BM x BN tiles of WM x WN wavefronts (eight for the 128-row tiles; BN = 64 for heads of 64
+// columns and wherever that gives a product of few tiles more workgroups).
+// G > 1: G groups of WM x WN wavefronts share the tile, group g multiplying the K slices
+// g, g + G, g + 2G ... in stages of its own (a slice past K is all zeros).  A compute unit does
+// not fetch much more than 100 GB/s, and a tile that has one to itself is bound by the chain of
+// one slice, load -> LDS -> barrier -> fragment reads -> MFMA: small tiles put a product of few
+// rows on many compute units and G chains in flight shorten each G-fold (20 heads x 1..200 rows
+// against 1500 frames: 24 -> 8 us).  Behind the loop the groups leave their accumulators in
+// their stages and group 0 adds them in group order (the same sum every launch).
+template <int BM, int BN, int WM, int WN, int G>
+__global__ __launch_bounds__(WM * WN * G * 64, (G == 1 ? 2 : 1)) void gemm_nn_anyrow_kernel(MatmulArgs a, TileMap map) {
+  constexpr int BK = 64, NW = WM * WN, NT = NW * 64, CPR = 8;
+  constexpr int LA = (BM * CPR + NT - 1) / NT, LB = BK * (BN / 8) / NT;  // chunks each thread stages
+  constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32, KK = BK / 16;
   constexpr int SLOT = 32 * (TN * 64 + 16);
+  constexpr int A_STAGE = BM * BK * 2, B_STAGE = BK * BN * 2, GROUP = 2 * (A_STAGE + B_STAGE);
   static_assert(BN == 128 || BN == 64, "one or half a 256-byte line per k row");
+  static_assert(TM >= 1 && TN >= 1 && BM * CPR % NT == 0 && BK * (BN / 8) % NT == 0, "tile shape");
   // chunk c of k row r of the right tile sits at position c ^ swz(r) of its row: the 16 chunks a
   // transposing read touches (4 rows x 4 chunks per 32 lanes) then fall into 16 bank groups
   auto swz = [](int krow) { return BN == 128 ? (krow & 3) << 2 : ((krow >> 1) & 1) << 2; };
-  static_assert(WM * WN * SLOT <= 2 * (BM + BN) * BK * 2, "epilogue slots must fit in LDS");
-  __shared__ __attribute__((aligned(1024))) unsigned char sA[2][BM * BK * 2];
-  __shared__ __attribute__((aligned(1024))) unsigned char sB[2][BK * BN * 2];
+  static_assert(NW * SLOT <= GROUP, "epilogue slots must fit in the stages of group 0");
+  static_assert(NT * TM * TN * 64 <= GROUP, "a group's accumulators must fit in its stages");
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[G][GROUP];
 
   int batch, tile_m, tile_n;
   map_tile(map, batch, tile_m, tile_n);
   const int m0 = tile_m * BM, n0 = tile_n * BN;
-  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = threadIdx.x & 63;
+  const int wave_all = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int grp = wave_all / NW, wave = wave_all % NW, tid = wave * 64 + lane;
   const int wm = wave / WN, wn = wave % WN;
   half_t* const out = a.output + (int64_t)batch * a.stride_oz;
   if (a.mask == ADR_MASK_CAUSAL && n0 > m0 + BM - 1) {
-    fill_masked_tile<BM, BN, NT>(a, out, m0, n0, tid);
+    fill_masked_tile<BM, BN, NT * G>(a, out, m0, n0, threadIdx.x);
     return;
   }
   const half_t* const A = a.lhs + (int64_t)batch * a.stride_lz;
   const half_t* const B = a.rhs + (int64_t)batch * a.stride_rz;
-  const int K = a.k, KT = (K + BK - 1) / BK;
+  const int K = a.k, KT = (K + BK - 1) / BK, ITERS = (KT + G - 1) / G;
+  unsigned char* const mine = lds[grp];
+  auto sA = [&](int buf) { return mine + buf * A_STAGE; };
+  auto sB = [&](int buf) { return mine + 2 * A_STAGE + buf * B_STAGE; };
 
   // Left operand.  Chunk c = tid + i * NT -> (row, kc).  Rows beyond the matrix read the last
   // row again (their products are never stored).  `last` is the last dword of the left operand
@@ -1904,40 +1919,79 @@ __global__ __launch_bounds__(256, 2) void gemm_nn_anyrow_kernel(MatmulArgs a, Ti
   // Right operand.  Chunk c -> (k row, column chunk) of the [64][128] tile; k rows beyond K and
   // columns beyond N are zero.
   int krB[LB], ncB[LB], offB[LB];
+  const half_t* gB[LB];  // the chunk in slice 0 (columns beyond N read column 0)
 #pragma unroll
   for (int i = 0; i < LB; i++) {
     const int c = tid + i * NT;
     krB[i] = c / (BN / 8);
     ncB[i] = (c % (BN / 8)) * 8;
     offB[i] = krB[i] * (BN * 2) + (((ncB[i] >> 3) ^ swz(krB[i])) << 4);
+    gB[i] = B + (int64_t)krB[i] * a.stride_ry + (n0 + ncB[i] < a.n ? n0 + ncB[i] : 0);
   }
+  const bool cols_full = n0 + BN <= a.n;
 
-  u32x4_t ra[LA], rb[LB];
-  // eight halves from any even address (load8_any); elements from `valid` on are zero
-  auto load_left = [&](const half_t* p, int valid) -> u32x4_t {
-    u32x4_t r = __builtin_bit_cast(u32x4_t, load8_any(p, last));
-#pragma unroll
-    for (int j = 0; j < 4; j++)  // elements 2j and 2j+1 of the chunk
-      r[j] = 2 * j + 1 < valid ? r[j] : 2 * j < valid ? (r[j] & 0xffffu) : 0u;
-    return r;
+  // What a thread holds of one slice between its loads and its LDS stores: the five dwords around
+  // each chunk of the left operand (shifted into place and cut at K only when they are stored, so
+  // that nothing waits for a load before the slice's MFMAs have been issued) and its chunks of the
+  // right operand.
+  struct Raw {
+    uint32_t a[LA][5];
+    u32x4_t b[LB];
   };
-  auto load_slice = [&](int kt) {
+  // A slice that ends at least two elements before K lies inside every row with the dword that
+  // follows each chunk: no address needs clamping and nothing needs cutting.  Both branches issue
+  // the same loads in the same order, so the waits counted behind them hold for either.
+  auto inside = [&](int k0) { return k0 + BK + 2 <= K; };
+  auto issue = [&](int kt, Raw& r) {
     const int k0 = kt * BK;
+    if (inside(k0)) {
 #pragma unroll
-    for (int i = 0; i < LA; i++) ra[i] = load_left(gA[i] + k0, K - k0 - kcA[i]);
+      for (int i = 0; i < LA; i++) {
+        const uintptr_t base = (uintptr_t)(gA[i] + k0) & ~(uintptr_t)3;
+        const u32x4_t q = *(const ADR_GLOBAL_AS u32x4_dword_aligned_t*)base;
+        r.a[i][0] = q[0]; r.a[i][1] = q[1]; r.a[i][2] = q[2]; r.a[i][3] = q[3];
+        r.a[i][4] = *(const ADR_GLOBAL_AS uint32_t*)(base + 16);
+      }
+      const int64_t step = (int64_t)k0 * a.stride_ry;
 #pragma unroll
-    for (int i = 0; i < LB; i++) {
-      const int kr = k0 + krB[i], col = n0 + ncB[i];
-      const bool in = kr < K && col < a.n;
-      const u32x4_t v = *(const u32x4_t*)(B + (int64_t)min(kr, K - 1) * a.stride_ry + (col < a.n ? col : 0));
-      rb[i] = in ? v : u32x4_t{0, 0, 0, 0};
+      for (int i = 0; i < LB; i++) r.b[i] = *(const u32x4_t*)(gB[i] + step);
+    } else {
+#pragma unroll
+      for (int i = 0; i < LA; i++) load5_issue(gA[i] + k0, last, r.a[i]);
+#pragma unroll
+      for (int i = 0; i < LB; i++) {
+        const int kr = k0 + krB[i], col = n0 + ncB[i];
+        r.b[i] = *(const u32x4_t*)(B + (int64_t)min(kr, K - 1) * a.stride_ry + (col < a.n ? col : 0));
+      }
     }
   };
-  auto store_slice = [&](int buf) {
+  auto finish = [&](int kt, int buf, const Raw& r) {
+    const int k0 = kt * BK;
+    if (inside(k0)) {
 #pragma unroll
-    for (int i = 0; i < LA; i++) *(u32x4_t*)(sA[buf] + offA[i]) = ra[i];
+      for (int i = 0; i < LA; i++)
+        *(u32x4_t*)(sA(buf) + offA[i]) = align5(r.a[i], (uint32_t)((uintptr_t)gA[i] & 2));
+    } else {
 #pragma unroll
-    for (int i = 0; i < LB; i++) *(u32x4_t*)(sB[buf] + offB[i]) = rb[i];
+      for (int i = 0; i < LA; i++) {
+        u32x4_t v = load5_finish(gA[i] + k0, last, r.a[i]);
+        const int valid = K - k0 - kcA[i];  // elements from `valid` on are zero
+#pragma unroll
+        for (int j = 0; j < 4; j++)  // elements 2j and 2j+1 of the chunk
+          v[j] = 2 * j + 1 < valid ? v[j] : 2 * j < valid ? (v[j] & 0xffffu) : 0u;
+        *(u32x4_t*)(sA(buf) + offA[i]) = v;
+      }
+    }
+    if (inside(k0) && cols_full) {
+#pragma unroll
+      for (int i = 0; i < LB; i++) *(u32x4_t*)(sB(buf) + offB[i]) = r.b[i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < LB; i++) {
+        const bool in = k0 + krB[i] < K && n0 + ncB[i] < a.n;
+        *(u32x4_t*)(sB(buf) + offB[i]) = in ? r.b[i] : u32x4_t{0, 0, 0, 0};
+      }
+    }
   };
 
   float16_t acc[TM][TN];
@@ -1968,14 +2022,9 @@ __global__ __launch_bounds__(256, 2) void gemm_nn_anyrow_kernel(MatmulArgs a, Ti
   typedef short short4_t __attribute__((ext_vector_type(4)));
   typedef __attribute__((address_space(3))) short4_t lds_short4_t;
 
-  load_slice(0);
-  store_slice(0);
-  __syncthreads();
-  for (int kt = 0; kt < KT; kt++) {
-    const int buf = kt & 1;
-    if (kt + 1 < KT) load_slice(kt + 1);
-    const unsigned char* cA = sA[buf];
-    const unsigned char* cB = sB[buf];
+  auto compute = [&](int buf) {
+    const unsigned char* cA = sA(buf);
+    const unsigned char* cB = sB(buf);
 #pragma unroll
     for (int kk = 0; kk < KK; kk++) {
       half8_t fa[TM], fb[TN];
@@ -1997,10 +2046,92 @@ __global__ __launch_bounds__(256, 2) void gemm_nn_anyrow_kernel(MatmulArgs a, Ti
         for (int j = 0; j < TN; j++)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[j], fa[i], acc[i][j], 0, 0, 0);
     }
-    if (kt + 1 < KT) store_slice(buf ^ 1);
+  };
+  // The group's slice number `it` is slice it * G + grp of K.  Loads run two slices ahead of the
+  // MFMAs: while slice `it` is multiplied out of one LDS stage, slice it + 1 waits in registers for
+  // the other stage and slice it + 2 is on its way (loads return in order, so storing the older
+  // set does not wait for the younger one).
+  auto at = [&](int it) { return it * G + grp; };
+  // The waits are counted statically, so inside the steady loop no branch holds a load and no exit
+  // leaves from its middle: either would make the loads of the two register sets pending in an
+  // order that depends on the path, and every wait would then drain them all.  Products of more
+  // than four slices run the steady loop down to their last three or four slices; the rest (and
+  // short products from the start) go through the tail, whose waits may be conservative.
+  Raw r0, r1;
+  int it = 0;
+  if (ITERS > 4) {
+    issue(at(0), r0);
+    issue(at(1), r1);
+    finish(at(0), 0, r0);
+    issue(at(2), r0);
+    __syncthreads();
+    for (; it + 4 < ITERS; it += 2) {
+      compute(0);
+      __builtin_amdgcn_sched_barrier(0);
+      finish(at(it + 1), 1, r1);
+      issue(at(it + 3), r1);
+      __syncthreads();
+      compute(1);
+      __builtin_amdgcn_sched_barrier(0);
+      finish(at(it + 2), 0, r0);
+      issue(at(it + 4), r0);
+      __syncthreads();
+    }
+  } else {
+    issue(at(0), r0);
+    if (ITERS > 1) issue(at(1), r1);
+    finish(at(0), 0, r0);
+    if (ITERS > 2) issue(at(2), r0);
     __syncthreads();
   }
-  wave_epilogue<TM, 2 * TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, &sA[0][0] + wave * SLOT,
+  // tail: slice `it` is in stage 0, r1 holds slice it + 1 and r0 slice it + 2 (where they exist);
+  // at most four slices are left
+  compute(0);
+  if (it + 1 < ITERS) finish(at(it + 1), 1, r1);
+  if (it + 3 < ITERS) issue(at(it + 3), r1);
+  __syncthreads();
+  if (it + 1 < ITERS) {
+    compute(1);
+    if (it + 2 < ITERS) finish(at(it + 2), 0, r0);
+    __syncthreads();
+  }
+  if (it + 2 < ITERS) {
+    compute(0);
+    if (it + 3 < ITERS) finish(at(it + 3), 1, r1);
+    __syncthreads();
+  }
+  if (it + 3 < ITERS) {
+    compute(1);
+    __syncthreads();
+  }
+  if constexpr (G > 1) {
+    // [register quad][thread] float4 in the group's own stages: consecutive lanes, consecutive 16 bytes
+    if (grp != 0) {
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int q = 0; q < 4; q++)
+            *(float4_t*)(mine + (((i * TN + j) * 4 + q) * NT + tid) * 16) =
+                float4_t{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+    }
+    __syncthreads();
+    if (grp != 0) return;
+#pragma unroll 1
+    for (int g = 1; g < G; g++)
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int q = 0; q < 4; q++) {
+            const float4_t v = *(const float4_t*)(lds[g] + (((i * TN + j) * 4 + q) * NT + tid) * 16);
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[i][j][4 * q + e] += v[e];
+          }
+  }
+  wave_epilogue<TM, 2 * TN>(a, out, acc, m0 + wm * WTM, n0 + wn * WTN, lds[0] + wave * SLOT,
                             (half_t)a.scale, lane);
 }
 
@@ -2083,11 +2214,12 @@ hipError_t launch_u8(hipStream_t stream, const MatmulArgs& a) {
   return hipGetLastError();
 }
 
-template <int BN>
+template <int BM, int BN, int WM, int WN, int G>
 hipError_t launch_nn_anyrow(hipStream_t stream, const MatmulArgs& a) {
-  TileMap map = make_map(a, 128, BN);
+  TileMap map = make_map(a, BM, BN);
   if (map.total < 0) return hipErrorInvalidConfiguration;
-  hipLaunchKernelGGL(gemm_nn_anyrow_kernel<BN>, dim3((unsigned)map.total), dim3(256), 0, stream, a, map);
+  hipLaunchKernelGGL((gemm_nn_anyrow_kernel<BM, BN, WM, WN, G>), dim3((unsigned)map.total),
+                     dim3(WM * WN * G * 64), 0, stream, a, map);
   return hipGetLastError();
 }
 
@@ -2130,6 +2262,7 @@ enum GemmChoice {
   U8_256x192, U8_256x128, U8_128x128, U8_128x64, U8_64x64, U8_128x64_G2, U8_64x64_G4,
   DMA_256x192, DMA_256x160, DMA_256x128, DMA_128x256, DMA_128x192, DMA_128x128, DMA_128x64, DMA_64x64, DMA_64x64_K128, DMA_128x64_K128,
   DMA_NN_256x128, DMA_NN_128x128, NN_ANYROW_128x128, NN_ANYROW_128x64,
+  NN_ANYROW_64x64_G4, NN_ANYROW_32x64_G4,
   STAGE_256x128, STAGE_128x128, STAGE_64x64,
 };
 
@@ -2201,22 +2334,43 @@ GemmChoice u8_k_groups(const MatmulArgs& a, GemmChoice c) {
 GemmChoice choose(const MatmulArgs& a) {
   const int NUM_CU = num_cu();
   // "NN": both the left operand (k contiguous) and the right operand (n contiguous) are row
-  // major, e.g. P.V on the head views of llama.rs:552-554
-  if (a.stride_lx == 1 && a.stride_rx == 1 && a.stride_ry != 1 && a.stride_ox == 1 && !a.rhs_q &&
+  // major, e.g. P.V on the head views of llama.rs:552-554.  Left rows of any alignment and any K
+  // (P.V of a sequence length like 77, 257, 1500 or 2001) go to the kernel that stages the left
+  // operand through registers.
+  const bool nn_anyrow =
+      a.stride_lx == 1 && a.stride_rx == 1 && a.stride_ry != 1 && a.stride_ox == 1 && !a.rhs_q &&
+      a.load == ADR_LOAD_IDENTITY && a.k >= 1 && a.n % 8 == 0 && a.n >= 8 && a.stride_ly > 0 &&
+      a.stride_lz >= 0 && !((a.stride_ry % 8) | (a.stride_rz % 8)) &&
+      !(a.lhs && (uintptr_t)a.rhs % 16 != 0) &&
+      // (its 16-byte loads near the end of the left operand start up to 12 bytes before the last dword)
+      (int64_t)(a.batches - 1) * a.stride_lz + (int64_t)(a.m - 1) * a.stride_ly + a.k >= 12;
+  // Few tiles and a long K (the first steps of whisper.rs:433-436 against 1500 frames, or a few
+  // query rows against a long context): a compute unit cannot fetch much more than 100 GB/s, so
+  // the product goes to the smallest row tile that still gives every workgroup a compute unit of
+  // its own, on 64 columns, with K split over four groups of wavefronts -- aligned or not.
+  const bool nn_dma =
+      a.stride_lx == 1 && a.stride_rx == 1 && a.stride_ry != 1 && a.stride_ox == 1 && !a.rhs_q &&
       a.load == ADR_LOAD_IDENTITY && a.k % 64 == 0 && a.k >= 64 && a.n % 8 == 0 && a.n >= 8 &&
       !((a.stride_ly % 8) | (a.stride_ry % 8) | (a.stride_lz % 8) | (a.stride_rz % 8)) &&
-      !(a.lhs && ((uintptr_t)a.lhs % 16 != 0 || (uintptr_t)a.rhs % 16 != 0))) {
+      !(a.lhs && ((uintptr_t)a.lhs % 16 != 0 || (uintptr_t)a.rhs % 16 != 0));
+  // (against the direct-to-LDS kernel the small tiles win from 16 slices on: 32 heads x 256 rows
+  // x K 256 take 5.4 us there and 6.1 here, one row x K 2048 16.2 and 9.1)
+  if (nn_anyrow && a.k > 192 && !(nn_dma && a.k < 1024)) {
+    const int64_t cols64 = (int64_t)((a.n + 63) / 64) * a.batches;
+    if ((int64_t)((a.m + 31) / 32) * cols64 <= NUM_CU) return NN_ANYROW_32x64_G4;
+    if ((int64_t)((a.m + 63) / 64) * cols64 <= NUM_CU) return NN_ANYROW_64x64_G4;
+  }
+  if (nn_dma) {
     static const Candidate nn[] = {{DMA_NN_256x128, 256, 128, 1, 1.00f},
                                    {DMA_NN_128x128, 128, 128, 2, 0.80f}};
     return pick(a, nn, 2);
   }
-  // the same layout with left rows of any alignment or a K that is no multiple of 64: P.V of a
-  // sequence length like 77, 257, 1500 or 2001
-  if (a.stride_lx == 1 && a.stride_rx == 1 && a.stride_ry != 1 && a.stride_ox == 1 && !a.rhs_q &&
-      a.load == ADR_LOAD_IDENTITY && a.k >= 1 && a.n % 8 == 0 && a.n >= 8 && a.stride_ly > 0 &&
-      a.stride_lz >= 0 && !((a.stride_ry % 8) | (a.stride_rz % 8)) &&
-      !(a.lhs && (uintptr_t)a.rhs % 16 != 0))
-    return a.n <= 64 || (a.n > 128 && a.n % 128 != 0 && a.n % 128 <= 64) ? NN_ANYROW_128x64 : NN_ANYROW_128x128;
+  if (nn_anyrow) {
+    const bool narrow = a.n <= 64 || (a.n > 128 && a.n % 128 != 0 && a.n % 128 <= 64);
+    // (half the compute units or fewer on 128 columns: twice the workgroups on 64)
+    const int64_t tiles128 = (int64_t)((a.m + 127) / 128) * ((a.n + 127) / 128) * a.batches;
+    return narrow || 2 * tiles128 <= NUM_CU ? NN_ANYROW_128x64 : NN_ANYROW_128x128;
+  }
   if (a.stride_lx != 1 || a.stride_ry != 1 || a.stride_ox != 1) return GEMM_NONE;
   if (a.k % 8 != 0 || a.k < 8) return GEMM_NONE;
   if ((a.stride_ly % 8) | (a.stride_rx % 8) | (a.stride_lz % 8) | (a.stride_rz % 8)) return GEMM_NONE;
@@ -2374,6 +2528,8 @@ static bool choice_name(GemmChoice c, const char** name, bool u8 = false) {
     case DMA_NN_128x128: *name = "gemm_nn_mfma_dma_128x128x64"; return true;
     case NN_ANYROW_128x128: *name = "gemm_nn_mfma_anyrow_128x128x64"; return true;
     case NN_ANYROW_128x64: *name = "gemm_nn_mfma_anyrow_128x64x64"; return true;
+    case NN_ANYROW_32x64_G4: *name = "gemm_nn_mfma_anyrow_32x64x64_k4"; return true;
+    case NN_ANYROW_64x64_G4: *name = "gemm_nn_mfma_anyrow_64x64x64_k4"; return true;
     case STAGE_256x128: *name = "gemm_nt_mfma_stage_256x128x32"; return true;
     case STAGE_128x128: *name = "gemm_nt_mfma_stage_128x128x32"; return true;
     case STAGE_64x64: *name = "gemm_nt_mfma_stage_64x64x64"; return true;
@@ -2411,8 +2567,10 @@ static hipError_t launch_choice(hipStream_t stream, const MatmulArgs& a, GemmCho
     case DMA_128x64_K128: return launch_dma<128, 64, 2, 2, 3, 1, false, 128>(stream, a);
     case DMA_NN_256x128: return launch_dma<256, 128, 4, 2, 3, 1, true>(stream, a);
     case DMA_NN_128x128: return launch_dma<128, 128, 2, 2, 2, 2, true>(stream, a);
-    case NN_ANYROW_128x128: return launch_nn_anyrow<128>(stream, a);
-    case NN_ANYROW_128x64: return launch_nn_anyrow<64>(stream, a);
+    case NN_ANYROW_128x128: return launch_nn_anyrow<128, 128, 4, 2, 1>(stream, a);
+    case NN_ANYROW_128x64: return launch_nn_anyrow<128, 64, 4, 2, 1>(stream, a);
+    case NN_ANYROW_32x64_G4: return launch_nn_anyrow<32, 64, 1, 2, 4>(stream, a);
+    case NN_ANYROW_64x64_G4: return launch_nn_anyrow<64, 64, 2, 2, 4>(stream, a);
     case STAGE_256x128: return launch_stage<256, 128, 32, 2, 2, 2>(stream, a);
     case STAGE_128x128: return launch_stage<128, 128, 32, 2, 2, 2>(stream, a);
     case STAGE_64x64: return launch_stage<64, 64, 64, 2, 2, 2>(stream, a);

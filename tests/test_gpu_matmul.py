@@ -251,40 +251,108 @@ def test_attention_views_qk_and_pv():
 
 
 PV_SHAPES = [
-    # (heads, S, T, D, extra elements before the first probability)
-    (12, 77, 77, 64, 0),      # CLIP text: rows of 154 bytes
-    (16, 257, 257, 64, 0),    # CLIP vision, one image
-    (3, 300, 301, 128, 1),    # odd pitch and an odd first address
-    (2, 1500, 1500, 64, 0),   # Whisper: rows aligned to 8 bytes, K ends inside a chunk
-    (2, 130, 1999, 128, 3),   # a long odd K
-    (2, 200, 1000, 128, 0),   # 16-byte aligned rows, K no multiple of 64
+    # (heads, S, T, D, extra elements before the first probability, kernel)
+    (12, 77, 77, 64, 0, "128x64x64"),        # CLIP text: rows of 154 bytes
+    (16, 257, 257, 64, 0, "32x64x64_k4"),    # CLIP vision, one image
+    (3, 300, 301, 128, 1, "32x64x64_k4"),    # odd pitch and an odd first address
+    (2, 1500, 1500, 64, 0, "32x64x64_k4"),   # Whisper: rows aligned to 8 bytes, K ends inside a chunk
+    (2, 130, 1999, 128, 3, "32x64x64_k4"),   # a long odd K
+    (2, 200, 1000, 128, 0, "32x64x64_k4"),   # 16-byte aligned rows, K no multiple of 64
+    (20, 5, 1500, 64, 0, "32x64x64_k4"),     # the first steps of the Whisper decoder against 1500 frames
+    (32, 1, 2047, 128, 1, "32x64x64_k4"),    # one query row against a long context
+    (32, 1, 2048, 128, 0, "32x64x64_k4"),    # ... whose length is a multiple of 64
+    (20, 448, 1536, 64, 0, "64x64x64_k4"),
+    (32, 300, 333, 64, 1, "64x64x64_k4"),    # more 32-row tiles than compute units
+    (20, 448, 1500, 64, 0, "64x64x64_k4"),   # the last steps of the Whisper decoder
+    (40, 500, 200, 64, 1, "128x64x64"),      # more 64-row tiles than compute units, heads of 64
+    (8, 1100, 257, 128, 0, "128x64x64"),     # heads of 128 on few tiles: 64-column tiles
+    (16, 1100, 321, 128, 1, "128x128x64"),
+    (4, 600, 130, 72, 0, "128x64x64"),       # 72 columns: a full and a ragged column tile
+    (3, 70, 500, 200, 1, "32x64x64_k4"),     # 200 columns: three full column tiles and 8 columns
 ]
 
 
-@pytest.mark.parametrize("H,S,T,D,off", PV_SHAPES, ids=lambda v: str(v))
-def test_pv_of_sequence_lengths_that_are_no_multiple_of_64(H, S, T, D, off):
-    """P.V on the views of llama.rs:552-554 / clip.rs:385-388 / whisper.rs:433-436 when the
-    probabilities' rows start at any even address and K = T ends inside a slice: the tiled kernel
-    that shifts the left operand into place, on inputs whose fp32 sums are exact; the last
-    probability is the last element of its buffer (nothing may be read past it that matters)."""
+def _pv_case(H, S, T, D, off, pitch=None, gen=None):
+    """Probabilities (multiples of 1/64 up to 1/8) as [H, S, T] rows of `pitch` elements that end
+    with the buffer, values (multiples of 1/16), the output and the strides of the head views."""
+    pitch = pitch or T
     HD = H * D
-    gen = torch.Generator(device="cuda").manual_seed(H * S + T)
-    pbuf = (torch.randint(0, 9, (off + H * S * T,), generator=gen, device="cuda").float() / 64).half()
+    pbuf = (torch.randint(0, 9, (off + (H * S - 1) * pitch + T,), generator=gen, device="cuda").float() / 64).half()
     v = (torch.randint(-8, 9, (T, HD), generator=gen, device="cuda").float() / 16).half()
     out = torch.full((S, HD), 3.0, dtype=torch.float16, device="cuda")
-    so, sl, sr = (1, HD, D), (1, T, S * T), (1, HD, D)
-    assert plan(H, S, T, D, so, sl, sr) == f"gemm_nn_mfma_anyrow_128x{D}x64"
+    return pbuf, v, out, ((1, HD, D), (1, pitch, S * pitch), (1, HD, D))
+
+
+def _pv_want(pbuf, v, H, S, T, D, off, pitch=None):
+    pitch = pitch or T
+    p = torch.as_strided(pbuf, (H, S, T), (S * pitch, pitch, 1), off).double()
+    return torch.bmm(p, v.view(T, H, D).permute(1, 0, 2).double()).permute(1, 0, 2).reshape(S, H * D).half()
+
+
+@pytest.mark.parametrize("H,S,T,D,off,kernel", PV_SHAPES, ids=lambda v: str(v))
+def test_pv_of_sequence_lengths_that_are_no_multiple_of_64(H, S, T, D, off, kernel):
+    """P.V on the views of llama.rs:552-554 / clip.rs:385-388 / whisper.rs:433-436 when the
+    probabilities' rows start at any even address and K = T ends inside a slice: the tiled kernel
+    that shifts the left operand into place, on every tile it has, on inputs whose fp32 sums are
+    exact; the last probability is the last element of its buffer (nothing may be read past it
+    that matters)."""
+    gen = torch.Generator(device="cuda").manual_seed(H * S + T)
+    pbuf, v, out, (so, sl, sr) = _pv_case(H, S, T, D, off, gen=gen)
+    assert plan(H, S, T, D, so, sl, sr) == "gemm_nn_mfma_anyrow_" + kernel
     assert raw_matmul("adr_matmul_f16", out, pbuf, v, H, S, T, D, so, sl, sr, offsets=(0, off, 0)) == 0
-    p = pbuf[off:].view(H, S, T).double()
-    want = torch.bmm(p, v.view(T, H, D).permute(1, 0, 2).double()).permute(1, 0, 2).reshape(S, HD).half()
+    want = _pv_want(pbuf, v, H, S, T, D, off)
     assert torch.equal(out.view(torch.int16), want.view(torch.int16))
 
 
-def test_pv_anyrow_kernel_ignores_what_follows_k():
+# K from one slice to many: the kernel runs a steady loop of two slices a trip from its fifth
+# slice on (per group of wavefronts: from K > 1024 where four groups share K) and a tail of up to
+# four; every remainder of both, K ending on a slice, one element behind and one before it
+_PV_K = {
+    "32x64x64_k4": (3, 40, 64, [193, 255, 257, 319, 511, 700, 1024, 1025, 1100, 1281, 1345,
+                                1537, 1601, 1857, 1999, 2305, 2560]),
+    "64x64x64_k4": (32, 300, 64, [193, 255, 321, 449, 1025, 1088, 1282, 1409]),
+    "128x64x64": (40, 500, 64, [193, 255, 257, 321, 385, 449, 513]),
+    "128x128x64": (16, 1100, 128, [193, 255, 258, 322, 385]),
+}
+
+
+@pytest.mark.parametrize("kernel,T", [(k, t) for k, (_, _, _, ts) in _PV_K.items() for t in ts],
+                         ids=lambda v: str(v))
+def test_pv_anyrow_tiles_every_remainder_of_their_loops(kernel, T):
+    H, S, D, _ = _PV_K[kernel]
+    gen = torch.Generator(device="cuda").manual_seed(T)
+    off = T % 2
+    pbuf, v, out, (so, sl, sr) = _pv_case(H, S, T, D, off, gen=gen)
+    assert plan(H, S, T, D, so, sl, sr) == "gemm_nn_mfma_anyrow_" + kernel
+    assert raw_matmul("adr_matmul_f16", out, pbuf, v, H, S, T, D, so, sl, sr, offsets=(0, off, 0)) == 0
+    want = _pv_want(pbuf, v, H, S, T, D, off)
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.parametrize("H,S,T,D,off", [(1, 1, 12, 8, 0), (1, 1, 13, 8, 1), (1, 2, 7, 8, 0),
+                                          (1, 3, 5, 16, 1), (2, 1, 9, 8, 0), (1, 1, 5, 8, 0),
+                                          (1, 2, 3, 8, 1), (1, 1, 1, 8, 0)], ids=lambda v: str(v))
+def test_pv_of_a_handful_of_probabilities(H, S, T, D, off):
+    """Left operands of a few bytes that end with their buffer: the tiled kernel (whose 16-byte
+    loads start up to 12 bytes before the last dword) from 12 elements on, another kernel below
+    that; the same sums either way."""
+    gen = torch.Generator(device="cuda").manual_seed(T)
+    pbuf, v, out, (so, sl, sr) = _pv_case(H, S, T, D, off, gen=gen)
+    tiled = plan(H, S, T, D, so, sl, sr).startswith("gemm_nn_mfma_anyrow")
+    assert tiled == ((H * S - 1) * T + T >= 12)
+    assert raw_matmul("adr_matmul_f16", out, pbuf, v, H, S, T, D, so, sl, sr, offsets=(0, off, 0)) == 0
+    want = _pv_want(pbuf, v, H, S, T, D, off)
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.parametrize("H,S,T,D,pitch,kernel", [(2, 140, 70, 64, 75, "128x64x64"),
+                                                  (2, 140, 326, 64, 331, "32x64x64_k4"),
+                                                  (40, 330, 1030, 64, 1033, "64x64x64_k4")],
+                         ids=lambda v: str(v))
+def test_pv_anyrow_kernel_ignores_what_follows_k(H, S, T, D, pitch, kernel):
     """Non-finite values right behind a row's K elements (the next row's first probabilities, or
-    whatever follows the tensor) must not reach the sums: rows of T = 70 probabilities inside a
-    pitch of 75, the five elements in between set to NaN."""
-    H, S, T, D, pitch = 2, 140, 70, 64, 75
+    whatever follows the tensor) must not reach the sums: rows of T probabilities inside a
+    longer pitch, the elements in between set to NaN."""
     HD = H * D
     gen = torch.Generator(device="cuda").manual_seed(3)
     pbuf = torch.full((H * S * pitch,), float("nan"), dtype=torch.float16, device="cuda")
@@ -293,7 +361,7 @@ def test_pv_anyrow_kernel_ignores_what_follows_k():
     v = (torch.randint(-8, 9, (T, HD), generator=gen, device="cuda").float() / 16).half()
     out = torch.zeros(S, HD, dtype=torch.float16, device="cuda")
     so, sl, sr = (1, HD, D), (1, pitch, S * pitch), (1, HD, D)
-    assert plan(H, S, T, D, so, sl, sr) == "gemm_nn_mfma_anyrow_128x64x64"
+    assert plan(H, S, T, D, so, sl, sr) == "gemm_nn_mfma_anyrow_" + kernel
     assert raw_matmul("adr_matmul_f16", out, pbuf, v, H, S, T, D, so, sl, sr) == 0
     want = torch.bmm(p.double(), v.view(T, H, D).permute(1, 0, 2).double()).permute(1, 0, 2).reshape(S, HD).half()
     assert torch.equal(out.view(torch.int16), want.view(torch.int16))
@@ -400,7 +468,9 @@ def test_persistent_short_k_kernel_epilogues(store):
 
 
 NN_SHAPES = [(2, 100, 128, 136), (1, 300, 64, 128), (3, 257, 192, 72), (1, 64, 64, 8),
-             (2, 513, 256, 264)]
+             (2, 513, 256, 264),
+             # few tiles and a long K: the small tiles whose wavefront groups share K
+             (2, 100, 1024, 136), (2, 90, 1030, 72), (3, 200, 300, 136), (40, 300, 1088, 64)]
 
 
 @pytest.mark.parametrize("shape", NN_SHAPES)
