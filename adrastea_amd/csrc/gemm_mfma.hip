@@ -191,6 +191,35 @@ __device__ __forceinline__ void store_chunk(const MatmulArgs& a, const Epilogue&
   }
 }
 
+// store_chunk for output rows that start at any even address (a dense [M, N] result with an odd N,
+// e.g. the 51865 logits of whisper.rs's decoder), for the store operators that do not read the
+// output: the chunk goes out as a half, three dwords and a half (store8_any) instead of eight halves.
+__device__ __forceinline__ void store_chunk_any(const MatmulArgs& a, const Epilogue& ep, half_t* out,
+                                                int y, int x, half8_t v) {
+  half_t* p = out + (int64_t)y * a.stride_oy + x;
+  const bool full = x + 8 <= a.n;
+  const half8_t prev = {0, 0, 0, 0, 0, 0, 0, 0};
+  half8_t bias = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (Epilogue::needs_bias(a.store)) {
+#pragma unroll
+    for (int e = 0; e < 8; e++)
+      if (x + e < a.n) bias[e] = a.bias[x + e];
+  }
+  half8_t r = apply_chunk(a, ep, v, prev, bias);
+  if (a.mask == ADR_MASK_CAUSAL && x + 7 > y) {
+#pragma unroll
+    for (int e = 0; e < 8; e++)
+      if (x + e > y) r[e] = neg_inf_half();
+  }
+  if (full) {
+    store8_any(p, r);
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; e++)
+      if (x + e < a.n) p[e] = r[e];
+  }
+}
+
 // Halves per access that every row chunk of the output (8 columns from a column that is a multiple
 // of 8) is aligned to: 8, 4, 2, or 1 (element by element).  As out_vectorizable() for 8.
 __device__ __forceinline__ int out_chunk_alignment(const MatmulArgs& a, const half_t* out) {
@@ -468,6 +497,20 @@ __device__ __forceinline__ void wave_epilogue(const MatmulArgs& a, half_t* out, 
         const half8_t v = *(const half8_t*)(slot + row * PITCH + c * 16);
         const int y = y0 + i * 32 + row, x = x0 + c * 8;
         if (y < a.m && x < a.n) store_chunk(a, ep, out, y, x, v);
+      }
+    }
+  } else if (!Epilogue::needs_prev(a.store) && a.store != STORE_ACC_BETA) {
+    // rows at any even address, nothing to read back: the same chunks, stored piecewise
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+      stage_block_f16<TM, TN2>(acc, i, slot, lane, false, (half_t)1.0f);
+#pragma unroll 1
+      for (int it = 0; it < TN2; it++) {
+        const int idx = it * 64 + lane;
+        const int row = idx / CPW, c = idx % CPW;
+        const half8_t v = *(const half8_t*)(slot + row * PITCH + c * 16);
+        const int y = y0 + i * 32 + row, x = x0 + c * 8;
+        if (y < a.m && x < a.n) store_chunk_any(a, ep, out, y, x, v);
       }
     }
   } else {

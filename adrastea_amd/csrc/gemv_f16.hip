@@ -277,6 +277,12 @@ static bool skinny_ok(const MatmulArgs& a) {
   // the same from 33 rows on where K is short of 8192 (K5120 N13824 m=48: 31.4 against 42.9 us,
   // K4096 N32000: 57.5 against 66.1; K8192 N22016 stays: 78.2 against 82.1)
   if (a.m > 32 && a.n >= 40 * device_info_for_plan().cus && a.k < 8192) return false;
+  // a short K splits badly over the eight wavefronts (ten steps: two rounds) and two blocks of
+  // activation rows double what each step re-reads: from 17 rows on, K < 4096 and more than one
+  // workgroup per CU the tiled kernels are ahead (weights from HBM; K1280 N51865 m=32: 43.3
+  // against 29.9 us, K1024 N16384: 15.8 against 9.3, K2048 N8192 m=64: 15.9 against 13.4, m=32:
+  // 12.3 against 12.0; N4096 stays: K1024 m=32 5.1 against 6.4)
+  if (a.m > 16 && a.k < 4096 && a.n > 16 * device_info_for_plan().cus) return false;
   // (one to four rows: only where the dot-product kernel does not reach, K > 12288 --
   // K13824 N5120 m=4: 53 us on the tiled kernels, 33 here)
   return a.m >= 1 && a.m <= 64;

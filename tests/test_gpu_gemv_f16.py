@@ -111,9 +111,21 @@ def test_nt_entry_point_with_beta():
     assert max_rel_err(to_np(o_t).reshape(m, N), want) <= 2e-3
 
 
+@pytest.mark.parametrize("m,K,N,tiled", [(32, 1280, 51865, True), (32, 2048, 12288, True), (64, 1536, 8192, True),
+                                         (17, 1024, 16384, True), (32, 1024, 4096, False),
+                                         (16, 1280, 51864, False), (32, 4096, 12288, False)])
+def test_short_k_from_17_rows_on_a_wide_matrix_takes_the_tiled_kernels(m, K, N, tiled):
+    """Ten macro steps split badly over the kernel's eight wavefronts: from 17 rows on, with
+    K < 4096 and more than one workgroup per compute unit, the product is a tiled one (the
+    Whisper decoder's logits for a 32-token prefix: 43 us here, 30 there)."""
+    so, sl, sr = nt(m, K, N)
+    name = plan(1, m, K, N, so, sl, sr)
+    assert name.startswith("gemm_nt_mfma") if tiled else name == PLAN_MFMA
+
+
 @pytest.mark.parametrize("m,K,N", [(9, 1024, 4100), (16, 4096, 1030), (13, 11008, 400), (17, 8192, 520),
-                                   (32, 11008, 390), (25, 12288, 350), (20, 1024, 6200),
-                                   (30, 1152, 10300),
+                                   (32, 11008, 390), (25, 12288, 350), (20, 1024, 4096),
+                                   (30, 1152, 4096),
                                    # one, two and three groups of 16 weight rows per workgroup
                                    (9, 2048, 4100), (16, 4096, 6200), (12, 5120, 10300),
                                    (11, 8192, 1000), (16, 4096, 12288),
@@ -122,12 +134,12 @@ def test_nt_entry_point_with_beta():
                                    (16, 11008, 4096), (10, 2176, 6200), (14, 4992, 10300), (9, 10368, 800),
                                    (16, 13824, 5120), (12, 6656, 700),
                                    # 17 to 32 rows: two blocks of activations
-                                   (17, 4096, 6200), (32, 2048, 12288), (25, 3072, 4100), (32, 4096, 12288),
-                                   (20, 3968, 10300), (32, 11008, 4096), (19, 8192, 6200), (27, 5120, 10300),
+                                   (17, 4096, 6200), (32, 2048, 4096), (25, 3072, 4000), (32, 4096, 12288),
+                                   (20, 3968, 4096), (32, 11008, 4096), (19, 8192, 6200), (27, 5120, 10300),
                                    # 33 to 64 rows: three and four blocks (four: at most two row groups)
-                                   (33, 4096, 4100), (48, 4096, 6200), (49, 3968, 8192), (64, 11008, 4096),
+                                   (33, 4096, 4100), (48, 4096, 6200), (49, 3968, 4000), (64, 11008, 4096),
                                    (40, 10368, 1000), (64, 4096, 8192), (48, 5120, 5000), (64, 13824, 1000),
-                                   (48, 8192, 12288), (33, 2048, 8192),
+                                   (48, 8192, 12288), (33, 2048, 4096),
                                    # one to four rows where K is beyond the dot-product kernel's reach
                                    (2, 13824, 1000), (4, 16384, 600), (1, 12416, 520),
                                    # three and four rows on narrow matrices, five to eight rows

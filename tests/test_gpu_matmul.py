@@ -209,6 +209,41 @@ def test_fast_nt_epilogues_match_oracle(store, mask):
         assert np.all(got.reshape(B, M, N).view(np.uint16)[:, x > y] == 0xFC00)
 
 
+@pytest.mark.parametrize("store", STORES_EXACT + STORES_F32)
+@pytest.mark.parametrize("mask", [oracle.MASK_NONE, oracle.MASK_CAUSAL])
+@pytest.mark.parametrize("shape", [(2, 150, 64, 201, 0), (1, 300, 128, 333, 1), (3, 70, 192, 1001, 1),
+                                   (1, 448, 128, 2047, 0)], ids=lambda v: str(v))
+def test_fast_nt_epilogues_into_rows_of_an_odd_length(store, mask, shape):
+    """A dense [M, N] result with an odd N (the 51865 logits of the Whisper decoder): its rows
+    start at any even address, so chunks go out piecewise (the operators that read nothing back)
+    or element by element; the output may start at an odd element too.  Same bits as aligned
+    rows would get, and nothing written outside the rows."""
+    B, M, K, N, off = shape
+    g = rng(700 + store * 2 + mask + N)
+    so, sl, sr = (1, N, M * N), (1, K, M * K), (K, 1, K * N)
+    assert plan(B, M, K, N, so, sl, sr, store=store, mask=mask).startswith("gemm_nt_mfma")
+    l = (g.integers(-16, 17, size=B * M * K) / 16.0).astype(np.float16)
+    r = (g.integers(-16, 17, size=B * K * N) / 16.0).astype(np.float16)
+    prev, bias = randn_f16(g, off + B * M * N + 3), randn_f16(g, N)
+    kw = dict(beta=0.7, scale=0.2, store=store, load=oracle.LOAD_IDENTITY, mask=mask)
+    want = oracle_matmul(prev, l, r, B, M, K, N, so, sl, sr, bias=bias, mode=oracle.EXACT,
+                         offsets=(off, 0, 0), **kw)
+    o_t = to_dev(prev)
+    assert raw_matmul("adr_matmul_f16", o_t, to_dev(l), to_dev(r), B, M, K, N, so, sl, sr,
+                      bias_t=to_dev(bias), offsets=(off, 0, 0), **kw) == 0
+    got = to_np(o_t)
+    assert np.array_equal(got[:off].view(np.uint16), prev[:off].view(np.uint16))
+    assert np.array_equal(got[-3:].view(np.uint16), prev[-3:].view(np.uint16))
+    if store in STORES_EXACT:
+        assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    else:
+        # (the fp32 operator may fuse its multiply and add: a third step only where v + beta * prev
+        # cancels to almost nothing)
+        steps = ulp_diff_f16(got, want)
+        assert np.count_nonzero(steps > 2) <= 1e-5 * steps.size
+        assert np.max(steps) <= 8
+
+
 def test_fast_nt_load_scale():
     g = rng(520)
     B, M, K, N = 1, 100, 128, 90
