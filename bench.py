@@ -22,6 +22,7 @@ u8 weights uniform with fp16 scales ~ U(0.001, 0.02) per 32 weights.
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -407,8 +408,39 @@ def main():
                           "frac_mfma_peak": round(fl / t / 1e12 / PEAK_F16_TFLOPS, 4)}
         return attn
 
+    def other_lengths_set():
+        # ---- P.V where the sequence length is no multiple of 64 (the probabilities' rows then
+        # start at any even address) or the query rows are few: the lengths the reference's models
+        # run at (llama.rs:552-554, whisper.rs:433-436, clip.rs:385-388); device time per launch
+        # from graph replays
+        out = {}
+        for name, H, S, T, D in (("llama_S2001", 32, 2001, 2001, 128), ("llama_S1000", 32, 1000, 1000, 128),
+                                 ("llama_1_row_T2047", 32, 1, 2047, 128),
+                                 ("whisper_encoder_1500", 20, 1500, 1500, 64),
+                                 ("whisper_cross_448_rows", 20, 448, 1500, 64),
+                                 ("whisper_cross_8_rows", 20, 8, 1500, 64),
+                                 ("clip_vision_257", 16, 257, 257, 64), ("clip_text_77", 12, 77, 77, 64)):
+            HD = H * D
+            p_ = torch.softmax(randn_h(H, S, T).float(), dim=-1).half()
+            v_, o_ = randn_h(T, HD), torch.zeros(S, HD, dtype=torch.float16, device=dev)
+
+            def f():
+                rc = lib.adr_matmul_f16(stream(), o_.data_ptr(), p_.data_ptr(), v_.data_ptr(), H, S, T,
+                                        D, 1, HD, D, 1, T, S * T, 1, HD, D, None, 0.0, 1.0, 0, 0, 0)
+                if rc != 0:
+                    raise RuntimeError(_ffi.strerror(rc))
+            plan = ctypes.create_string_buffer(96)
+            lib.adr_matmul_f16_plan(plan, 96, H, S, T, D, 1, HD, D, 1, T, S * T, 1, HD, D, 0, 0, 0)
+            t = timed_graph(f, 10, 10)
+            byts = (H * S * T + T * HD + S * HD) * 2
+            out["pv_" + name] = {"us": round(t * 1e6, 1), "kernel": plan.value.decode(),
+                                 "tflops": round(2.0 * H * S * T * D / t / 1e12, 1),
+                                 "gbs": round(byts / t / 1e9, 1)}
+        return out
+
     if args.attention_only:
-        print(json.dumps({"llama7b_attention_fp16": attention_set()}))
+        print(json.dumps({"llama7b_attention_fp16": attention_set(),
+                          "pv_other_lengths_fp16": other_lengths_set()}))
         return
 
     def microbenchmark():
@@ -835,6 +867,7 @@ def main():
 
         attn = attention_set()
         secondary["llama7b_attention_fp16"] = attn
+        secondary["pv_other_lengths_fp16"] = other_lengths_set()
 
     # ---------------- CPU baseline: every configuration on bounded samples, this machine's cores
     cpu_baseline = None
