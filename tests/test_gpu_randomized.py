@@ -146,6 +146,73 @@ def test_random_products_match_the_slow_kernel(seed, held):
     assert sum(v for k, v in plans.items() if k != "matmul_general") >= 40, plans
 
 
+def _pv_case(g):
+    """P.V on head views (llama.rs:552-554, whisper.rs:433-436): probabilities [H, S, T] with rows
+    of any pitch from any element, values [T, H * D] and the output [S, H * D] interleaved by head."""
+    pick = lambda xs: xs[int(g.integers(0, len(xs)))]
+    H = int(pick([1, 2, 3, 8, 12, 20, 32]))
+    D = int(pick([64, 64, 128, 128, 72, 200, 8, 136]))
+    r = g.random()
+    S = int(g.integers(1, 40)) if r < 0.35 else int(g.integers(40, 500)) if r < 0.8 else int(g.integers(500, 1600))
+    r = g.random()
+    T = int(g.integers(1, 200)) if r < 0.2 else int(g.integers(193, 1100)) if r < 0.6 else int(g.integers(1024, 2600))
+    if g.random() < 0.15:
+        T = 64 * int(g.integers(1, 40))
+    if H * S * T > 30e6:
+        return None
+    pitch = T + int(pick([0, 0, 0, 1, 5, 8]))
+    HD = H * D + int(pick([0, 0, 8, 64]))
+    offs = [int(pick([0, 8])), int(pick([0, 0, 1, 8, 3])), int(pick([0, 8]))]
+    return dict(B=H, M=S, K=T, N=D, so=(1, HD, D), sl=(1, pitch, S * pitch), sr=(1, HD, D), offs=offs,
+                boff=int(pick([0, 0, 8, 1])), store=int(pick(STORES)), load=0, mask=int(pick([0, 0, 0, 1])),
+                beta=float(pick([0.0, 1.0, 0.5, -2.0])), scale=float(pick([1.0, 0.5, 0.25, 2.0])))
+
+
+@pytest.mark.parametrize("seed", [41, 42, 43])
+def test_random_pv_products_match_the_slow_kernel(seed):
+    """Every tile of the kernel for left rows of any alignment (and the direct-to-LDS kernels where
+    the draw is aligned), every store operator and the causal mask on them."""
+    g = np.random.default_rng(seed)
+    L = _ffi.lib()
+    plans, failures = {}, []
+    for it in range(70):
+        c = _pv_case(g)
+        if c is None:
+            continue
+        B, M, K, N = c["B"], c["M"], c["K"], c["N"]
+        (ox, oy, oz), (lx, ly, lz), (rx, ry, rz), offs = c["so"], c["sl"], c["sr"], c["offs"]
+        l_len = offs[1] + (M - 1) * ly + (K - 1) * lx + (B - 1) * lz + 1   # the last probability ends the buffer
+        r_len = offs[2] + (K - 1) * ry + (N - 1) * rx + (B - 1) * rz + 1 + 8
+        o_len = offs[0] + (M - 1) * oy + (N - 1) * ox + (B - 1) * oz + 1 + 8
+        l_t = torch.from_numpy(g.integers(-3, 4, size=l_len).astype(np.float16)).cuda()
+        r_t = torch.from_numpy(g.integers(-2, 3, size=r_len).astype(np.float16)).cuda()
+        b_t = torch.from_numpy((g.integers(-8, 9, size=N + 8) / 4.0).astype(np.float16)).cuda()
+        o1 = torch.from_numpy((g.integers(-8, 9, size=o_len) / 4.0).astype(np.float16)).cuda()
+        o2 = o1.clone()
+        name = _plan(c)
+        plans[name] = plans.get(name, 0) + 1
+        print(f"seed {seed} case {it}: {c} -> {name}", flush=True)
+        rcs = [fn(_stream(), o.data_ptr() + 2 * offs[0], l_t.data_ptr() + 2 * offs[1], r_t.data_ptr() + 2 * offs[2],
+                  B, M, K, N, ox, oy, oz, lx, ly, lz, rx, ry, rz, b_t.data_ptr() + 2 * c["boff"],
+                  c["beta"], c["scale"], c["store"], c["load"], c["mask"])
+               for fn, o in ((L.adr_matmul_f16, o1), (L.adr_matmul_f16_slow, o2))]
+        torch.cuda.synchronize()
+        assert rcs == [0, 0], (c, rcs)
+        a, b = o1.view(torch.int16), o2.view(torch.int16)
+        if torch.equal(a, b):
+            continue
+        diff = (a != b) & ~(torch.isnan(o1) & torch.isnan(o2))
+        if c["store"] in GELU_STORES:
+            ka = torch.where(a < 0, -(a.int() & 0x7FFF), a.int())
+            kb = torch.where(b < 0, -(b.int() & 0x7FFF), b.int())
+            diff &= (ka - kb).abs() > 2
+        if bool(diff.any()):
+            failures.append((c, name, int(diff.sum())))
+    assert not failures, failures
+    for tile in ("128x128x64", "128x64x64", "64x64x64_k4", "32x64x64_k4"):
+        assert any(k == "gemm_nn_mfma_anyrow_" + tile for k in plans) or seed != 41, (tile, plans)
+
+
 def _u8_case(g):
     pick = lambda xs: xs[int(g.integers(0, len(xs)))]
     bs = int(pick([32, 32, 32, 64, 128, 8, 16]))
