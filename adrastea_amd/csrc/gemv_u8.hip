@@ -745,6 +745,10 @@ bool rows_in_passes(int m, int p, int n, int block_size) {
   if (knob(KNOB_U8_TILE)) return knob(KNOB_U8_TILE) == 9;
   if (m <= 32) return true;
   const int cus = device_info_for_plan().cus;
+  // one pass of up to three blocks of rows against a matrix so wide that the 64 x 64 tiles need a
+  // second round: K6656 N17920 m=40 57.5 us against 73.6, K8192 N22016 m=48 74 against 89 (weights
+  // from HBM; with four blocks the pass loses: m=64 104 against 92)
+  if (m <= 48 && (n + 63) / 64 > cus) return true;
   const int rounds = ((n + ROWS - 1) / ROWS + cus - 1) / cus;
   const double t64 = fmax(12.0, rounds * (2.0 + 0.0023 * p));
   const int rem = m % 64;

@@ -512,6 +512,11 @@ def test_seventeen_and_more_rows_in_passes(kern, kn, m):
     assert u8_plan(48, 4096, 12288, 32).startswith("gemm_nt_u8_mfma_64x64")
     assert u8_plan(100, 4096, 8200, 32).startswith("gemm_nt_u8_")
     assert u8_plan(257, 11008, 1000, 32).startswith("gemm_nt_u8_")
+    # one pass against a matrix whose 64 x 64 tiles would need a second round (LLaMA-30B's and
+    # 65B's gate / up projections): the pass
+    assert u8_plan(40, 6656, 17920, 32) == "gemv_u8_mfma16_blocks"
+    assert u8_plan(48, 8192, 22016, 32) == "gemv_u8_mfma16_blocks"
+    assert u8_plan(64, 8192, 22016, 32).startswith("gemm_nt_u8_")
     gen = torch.Generator(device="cuda").manual_seed(47 + m + p)
     q = torch.randint(0, 256, (n, p), generator=gen, device="cuda", dtype=torch.uint8)
     s = (torch.rand(n, p // 32, generator=gen, device="cuda") * 0.019 + 0.001).half()
