@@ -2439,6 +2439,14 @@ GemmChoice choose(const MatmulArgs& a) {
     const int forced = knob(KNOB_GEMM_TILE);
     if (forced >= 1 && forced <= N_DMA_TILES) return DMA_TILES[forced - 1].id;
     GemmChoice c = pick(a, DMA_TILES, N_DMA_TILES);
+    // Up to 64 rows against a matrix of a little more than one 64 x 64 tile per CU: the CUs that
+    // hold two tiles finish as late as one 128 x 128 tile would, and that tile is 0-16 % ahead
+    // (K6656 N17920 m=64: 72.8 -> 61.4 us, K3072 N24576: 37.9 -> 34.6, K8192 N22016: 86.2 -> 86.6);
+    // with two full rounds of the small tile it is the other way round (K4096 N32000: 54.5 / 62.0)
+    if (c == DMA_64x64 && a.m <= 64 && a.batches == 1 && a.k >= 3072) {
+      const int tiles64 = (a.n + 63) / 64;
+      if (tiles64 > NUM_CU && 2 * tiles64 <= 3 * NUM_CU) c = DMA_128x128;
+    }
     // At most one 64 x 64 tile per CU (a few dozen to a few hundred rows against a weight
     // matrix): the product is bound by how DRAM serves the weight requests -- one piece of every
     // tile row per slice, a whole weight row apart -- and pieces of 256 bytes (slices of 128)

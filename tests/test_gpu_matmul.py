@@ -244,6 +244,26 @@ def test_fast_nt_epilogues_into_rows_of_an_odd_length(store, mask, shape):
         assert np.max(steps) <= 8
 
 
+def test_up_to_64_rows_against_a_little_more_than_one_small_tile_per_cu():
+    """280 tiles of 64 x 64 on 256 compute units leave most of a second round empty: one 128 x 128
+    tile per CU takes such products; 500 tiles fill both rounds and stay."""
+    def nt(M, K, N):
+        return (1, N, 0), (1, K, 0), (K, 1, 0)
+    assert plan(1, 64, 4096, 17920, *nt(64, 4096, 17920)) == "gemm_nt_mfma_dma_128x128x64"
+    assert plan(1, 40, 3072, 24576, *nt(40, 3072, 24576)) == "gemm_nt_mfma_dma_128x128x64"
+    assert plan(1, 64, 4096, 32000, *nt(64, 4096, 32000)) == "gemm_nt_mfma_dma_64x64x64"
+    M, K, N = 50, 3072, 17000
+    so, sl, sr = nt(M, K, N)
+    assert plan(1, M, K, N, so, sl, sr) == "gemm_nt_mfma_dma_128x128x64"
+    gen = torch.Generator(device="cuda").manual_seed(77)   # small integers: every sum is exact
+    l = torch.randint(-3, 4, (M, K), generator=gen, device="cuda").half()
+    r = torch.randint(-2, 3, (N, K), generator=gen, device="cuda").half()
+    out = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+    assert raw_matmul("adr_matmul_f16", out, l, r, 1, M, K, N, so, sl, sr) == 0
+    want = (l.double() @ r.double().t()).half()
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+
+
 def test_fast_nt_load_scale():
     g = rng(520)
     B, M, K, N = 1, 100, 128, 90
