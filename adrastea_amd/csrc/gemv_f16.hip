@@ -292,16 +292,14 @@ enum SkinnyChoice { SKINNY_NONE, SKINNY_DOT, SKINNY_MFMA };
 
 static SkinnyChoice choose_skinny(const MatmulArgs& a) {
   if (!layout_ok(a)) return SKINNY_NONE;
-  // three and four rows on a matrix of at most 256 groups of 16 weight rows (one workgroup per
-  // CU) and K up to 4096: the matrix-core kernel is ahead already (m=4: K4096 N4096 9.4 -> 7.8 us, K2048
-  // N4096 6.9 -> 5.6, K3072 N3072 7.0 -> 5.3; with N 6000 12.3 -> 13.0 and with K 11008 19.3 ->
-  // 22.2, so not there; two rows: 7.7 either way)
-  const int cus = device_info_for_plan().cus;  // MI355X: 256
-  const bool narrow = a.m >= 3 && a.m <= 4 && a.n <= 16 * cus && a.k <= 4096 && a.k > 1024 &&
-                      a.k % 128 == 0 && (int64_t)a.n * a.k >= (1 << 22);
-  if (narrow) return SKINNY_MFMA;
-  if (a.m <= 4 && dot_ok(a)) return SKINNY_DOT;
-  if (skinny_ok(a) && (a.m >= 5 || !dot_ok(a))) return SKINNY_MFMA;
+  // One and two rows: dot products.  From three rows on the matrix cores wherever they apply: with
+  // weights that come from HBM they are level with the dot products at K 4096, 8192 and 12288 and
+  // well ahead where K fills the dot kernel's segments badly (m=4: K5120 N15360 41.5 -> 27.0 us,
+  // K6656 N19968 57.0 -> 43.5, K5120 N5120 17.3 -> 12.4, K4096 N12288 20.4 -> 18.7, K11008 N4096
+  // 19.4 -> 18.1).  (With the weights resident in the Infinity Cache the dot products had looked
+  // ahead at three and four rows on wide matrices, 12.3 against 13.0 us at N 6000.)
+  if (a.m <= 2 && dot_ok(a)) return SKINNY_DOT;
+  if (skinny_ok(a)) return SKINNY_MFMA;
   return dot_ok(a) ? SKINNY_DOT : SKINNY_NONE;
 }
 

@@ -25,11 +25,9 @@ def nt(M, K, N):
                                  (4096, 1100), (11008, 400)])
 def test_matches_oracle_and_is_exact_on_exact_inputs(m, K, N):
     so, sl, sr = nt(m, K, N)
-    # up to four rows: dot products, but for three and four rows on a narrow matrix with K up to
-    # 4096; five to eight: dot products only where K is no multiple of 128 (or the matrix is
-    # small); more: other kernels
-    mfma = K % 128 == 0 and K >= 1024 and N * K >= (1 << 22) and (
-        m >= 5 or (m >= 3 and N <= 4096 and 1024 < K <= 4096))
+    # one and two rows: dot products; three to eight: dot products only where K is no multiple
+    # of 128 (or the matrix is small); more: other kernels
+    mfma = K % 128 == 0 and K >= 1024 and N * K >= (1 << 22) and m >= 3
     if mfma:
         assert plan(1, m, K, N, so, sl, sr) == PLAN_MFMA
     elif m <= 8:
