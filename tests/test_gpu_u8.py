@@ -201,7 +201,9 @@ def _u8_case(g, m, p, n, bs, exact):
 
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 7, 8, 9, 12, 13, 16])
 @pytest.mark.parametrize("pn", [(256, 16), (512, 100), (1024, 33), (2816, 48), (4096, 52),
-                                (5120, 40), (11008, 24)])
+                                (5120, 40), (11008, 24),
+                                # five to eight segments of 1 KiB (one per wavefront for one row), whole and ragged
+                                (6656, 24), (8192, 20), (4128, 30), (7200, 18)])
 def test_gemv_bit_exact_on_exact_inputs(kern, m, pn):
     p, n = pn
     g = rng(610 + m + n)
@@ -435,7 +437,7 @@ def test_u8_other_block_sizes_and_fallbacks(kern):
         assert torch.all(prev == 1.0)
 
 
-DECODE = [(4096, 4096), (4096, 11008), (4096, 12288), (11008, 4096)]
+DECODE = [(4096, 4096), (4096, 11008), (4096, 12288), (11008, 4096), (5120, 13824), (8192, 4100)]
 
 
 @pytest.mark.parametrize("workspace_mode", ["pool_off", "shipped_default"], indirect=True)
