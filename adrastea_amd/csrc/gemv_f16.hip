@@ -352,6 +352,15 @@ hipError_t launch_gemv_f16(hipStream_t stream, const MatmulArgs& a) {
   // Weight rows per workgroup: every workgroup fetches the activations of all m rows again
   // (from L2), so with eight rows a workgroup has to cover more weight rows to keep that
   // traffic below the weights' own (m=8, K4096 N12288: 32.3 us with two rows, 25.0 with eight).
+  // One and two rows: a workgroup takes as long as its busiest wavefront, so five to sixteen
+  // segments go to eight wavefronts with one or two each instead of 4 x 2 and 8 x 3 (weights from
+  // HBM, m=1 / m=2: K5120 N13824 25.1 -> 22.8 / 28.4 -> 24.1 us, K5120 N5120 12.0 -> 10.5 / 13.4 ->
+  // 11.8, K6656 N17920 37.2 -> 36.0 / 40.7 -> 37.3, K4096 N12288 17.0 -> 16.8 / 17.9 -> 17.1; up to
+  // four segments the four wavefronts stay: K1280 N51864 27.4 against 27.7)
+  if (a.m <= 2 && nseg > 4 && nseg <= 16) {
+    if (a.m == 1) return small ? launch<1, 8, 4, 1>(stream, a) : launch<1, 8, 4, 2>(stream, a);
+    return small ? launch<2, 8, 4, 1>(stream, a) : launch<2, 8, 4, 2>(stream, a);
+  }
   switch (rows_class(a.m)) {
     case 1: return small ? launch<1, 4, 4, 2>(stream, a) : launch<1, 8, 4, 3>(stream, a);
     case 2: return small ? launch<2, 4, 4, 2>(stream, a) : launch<2, 8, 4, 3>(stream, a);

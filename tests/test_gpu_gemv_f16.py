@@ -22,6 +22,8 @@ def nt(M, K, N):
 
 @pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 8, 9, 16])
 @pytest.mark.parametrize("K,N", [(512, 1030), (4096, 259), (4104, 131), (11008, 50), (12288, 44),
+                                 # five to sixteen segments of 512: eight wavefronts with one or two each
+                                 (2560, 420), (5120, 230), (6664, 90), (8192, 140),
                                  (4096, 1100), (11008, 400)])
 def test_matches_oracle_and_is_exact_on_exact_inputs(m, K, N):
     so, sl, sr = nt(m, K, N)
