@@ -839,16 +839,16 @@ hipError_t launch_gemm_u8(hipStream_t stream, half_t* out, const half_t* lhs, co
                                 : launch_dot<1, 4, 2, 1>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
         return launch_dot<2, 4, 4, 1>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
       }
-      // up to 12 segments: 4 wavefronts, three segments each (K = 11008 has 11: one idle slot
-      // instead of five with 8 x 2)
       // up to 8 segments: 8 wavefronts, one segment each.  A workgroup takes as long as its busiest
       // wavefront, and 4 x 3 gives one of them two of K = 5120's five segments (LLaMA-13B: N13824
       // 21.6 -> 14.1 us, N5120 9.3 -> 7.4; K6656 N17920 26.0 -> 21.2, K8192 N8192 15.1 -> 13.3)
       if (m == 1 && p <= 8 * 1024)
         return launch_dot<1, 8, 4, 1>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
-      // (from 9 segments on 8 x 2 loses to 4 x 3: K11008 N4096 11.2 against 10.7 us, K9216 19.5 / 18.1)
+      // up to 12 segments: twelve wavefronts with one each (K11008 N4096 10.8 -> 10.4 us, K9216 N9216
+      // 17.9 -> 17.0, K12288 N12288 26.8 -> 25.7; four wavefronts with three each before, and
+      // 8 x 2 behind that: 11.2 and 19.5)
       if (m == 1 && p <= 12 * 1024)
-        return launch_dot<1, 4, 4, 3>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
+        return launch_dot<1, 12, 4, 1>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
       // up to 16 segments: 8 wavefronts, two segments each
       if (m == 1) return launch_dot<1, 8, 4, 2>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
       return launch_dot<2, 8, 4, 2>(stream, out, lhs, rhs, scales, m, p, n, block_size, beta);
